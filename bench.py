@@ -1,0 +1,179 @@
+"""Benchmark of the permutohedral-lattice filter on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--size 1024] [--no-cpu]
+
+One step = the hot path over one synthetic image: a bilateral filter (pd=5, vd=4) of a
+1024 x 1024 RGB image under itself as guide, forward then reverse (two filter() calls, each
+building its lattice from the positions, as the reference's op does).  Inputs are resident in
+HBM before the timed region.  Prints one JSON line.
+"""
+import argparse
+import json
+import os
+import statistics
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, vendor figure
+
+
+def algorithmic_bytes(n, m, pd, vd):
+    """Compulsory bytes of one filter() call, per kernel: positions, input and output streams once;
+    vertex keys once; the vertex value table written by splat, read and written once per blur axis,
+    read by slice.  Replay matrix, hash cells, neighbour table and clears are not counted."""
+    return {
+        "build": 4 * n * pd + 2 * pd * m,
+        "splat": 4 * n * (vd - 1) + 4 * vd * m,
+        "blur_axis": 2 * 4 * vd * m,
+        "slice": 4 * vd * m + 4 * n * (vd - 1),
+        "filter": 4 * n * (pd + 2 * (vd - 1)) + m * (2 * pd + 4 * vd * (2 * (pd + 1) + 2)),
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--size", type=int, default=1024, help="image side (default 1024)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and parity legs")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on exactly one GPU (got --gpus %d); there is no "
+                 "multi-GPU path to measure" % args.gpus)
+
+    import numpy as np
+    import torch
+
+    import permutohedral_lattice_amd as pla
+    from permutohedral_lattice_amd import synth
+
+    torch.cuda.set_device(0)
+    side = args.size
+    n, pd, vd = side * side, 5, 4
+    img = synth.blob_image(side, side, seed=0xC0FFEE)
+    pos = synth.bilateral_positions(img, 8.0, 0.125)
+    val = img.reshape(-1, 3)
+    grad = synth.normal_image((n, 3), 0xC0FFEE + 1)  # upstream gradient of the reverse pass
+
+    d_pos = torch.from_numpy(pos).cuda()
+    d_val = torch.from_numpy(val).cuda()
+    d_grad = torch.from_numpy(grad).cuda()
+    out_f = torch.empty_like(d_val)
+    out_r = torch.empty_like(d_val)
+    lat = pla.PermutohedralLattice(pd, vd, n)
+
+    def step():
+        lat.filter(out_f, d_val, d_pos, False)
+        lat.filter(out_r, d_grad, d_pos, True)
+
+    for _ in range(args.warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    seconds = time.perf_counter() - t0
+    ms_per_step = 1e3 * seconds / args.steps
+    m = lat.num_vertices
+    pixels_per_step = 2 * n
+    value = pixels_per_step / (ms_per_step * 1e-3) / 1e6
+
+    # build once, apply forward and reverse (what a caller that keeps the lattice gets)
+    lat.build(d_pos)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        lat.apply(out_f, d_val, False)
+        lat.apply(out_r, d_grad, True)
+    torch.cuda.synchronize()
+    reuse_ms = 1e3 * (time.perf_counter() - t0) / args.steps
+
+    # per-kernel durations from HIP events on the lattice's stream
+    lat.set_option(pla.PL_OPT_PROFILE, 1)
+    stage_samples = []
+    for _ in range(max(5, min(20, args.steps))):
+        for o, v, rev in ((out_f, d_val, False), (out_r, d_grad, True)):
+            lat.filter(o, v, d_pos, rev)
+            stage_samples.append(lat.stage_ms())
+    lat.set_option(pla.PL_OPT_PROFILE, 0)
+    stages = {k: statistics.mean(s[k] for s in stage_samples) for k in stage_samples[0]}
+    stages["blur_axis"] = stages["blur"] / (pd + 1)
+
+    alg = algorithmic_bytes(n, m, pd, vd)
+    per_launch_ms = {k: stages[k] for k in ("build", "splat", "blur_axis", "slice")}
+    dominant = max(("build", "splat", "slice"), key=lambda k: stages[k])
+    if stages["blur"] > stages[dominant]:
+        dominant = "blur_axis"
+    achieved = alg[dominant] / (per_launch_ms[dominant] * 1e-3) / 1e9
+    roofline = {"bound": "hbm", "kernel": dominant, "achieved": round(achieved, 2),
+                "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 5),
+                "traffic": None, "algorithmic_bytes_per_launch": alg[dominant],
+                "launch_ms": round(per_launch_ms[dominant], 5)}
+    gpu_kernel_ms = sum(stages[k] for k in ("clear", "build", "neighbours", "fill", "splat", "blur", "slice"))
+    filter_gbs = 2 * alg["filter"] / (ms_per_step * 1e-3) / 1e9
+
+    result = {
+        "metric": "Mpixels/sec, bilateral pd=5 vd=4 on 1 MI355X; % of HBM peak; CPU baseline",
+        "value": round(value, 3), "unit": "Mpixels/s", "n_gpus": 1, "steps": args.steps,
+        "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "bilateral RGB %dx%d, pd=5 vd=4, theta 8/0.125, filter() forward + "
+                               "filter() reverse per step, positions given" % (side, side),
+                   "pixels_per_step": pixels_per_step, "num_vertices": m},
+        "roofline": roofline,
+        "filter_roofline": {"algorithmic_bytes_per_step": 2 * alg["filter"],
+                            "achieved": round(filter_gbs, 2), "unit": "GB/s",
+                            "frac": round(filter_gbs / HBM_PEAK_GBS, 5)},
+        "stage_ms": {k: round(v, 5) for k, v in stages.items()},
+        "kernel_ms_per_filter": round(gpu_kernel_ms, 4),
+        "reuse": {"what": "build once, apply forward + reverse per step",
+                  "ms_per_step": round(reuse_ms, 4),
+                  "value": round(pixels_per_step / (reuse_ms * 1e-3) / 1e6, 3)},
+    }
+
+    if not args.no_cpu:
+        import oracle
+        ref = oracle.reference()
+        cores = 1
+        times, outs = [], None
+        reps = 3 if n >= (1 << 20) else 5
+        for rep in range(reps + 1):  # first repetition is the warm-up
+            t0 = time.perf_counter()
+            if ref is not None:
+                o_f = ref.filter(pd, vd, val, pos, False)[0]
+                o_r = ref.filter(pd, vd, grad, pos, True)[0]
+            else:
+                o_f = oracle.Lattice(pd, vd, n, reference_growth_quirk=True).filter(val, pos, False)
+                o_r = oracle.Lattice(pd, vd, n, reference_growth_quirk=True).filter(grad, pos, True)
+            dt = time.perf_counter() - t0
+            if rep:
+                times.append(dt)
+            outs = (o_f, o_r)
+        cpu_s = statistics.median(times)
+        result["cpu_baseline"] = {
+            "value": round(pixels_per_step / cpu_s / 1e6, 4), "unit": "Mpixels/s", "cores": cores,
+            "kind": "reference" if ref is not None else "port",
+            "sample": "the whole step (forward + reverse of the same %dx%d arrays), median of %d "
+                      "after one warm-up" % (side, side, reps),
+            "seconds_per_step": round(cpu_s, 4), "host_cpus": os.cpu_count()}
+        lat.filter(out_f, d_val, d_pos, False)
+        lat.filter(out_r, d_grad, d_pos, True)
+        torch.cuda.synchronize()
+        parity = {}
+        for name, got, want in (("forward", out_f.cpu().numpy(), outs[0]),
+                                ("reverse", out_r.cpu().numpy(), outs[1])):
+            parity[name] = {"max_abs": float(np.abs(got - want).max()),
+                            "rel_l2": float(np.linalg.norm(got - want) / np.linalg.norm(want))}
+        result["parity_vs_cpu"] = parity
+
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

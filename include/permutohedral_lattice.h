@@ -1,0 +1,155 @@
+/*
+ * C ABI of the gfx950 (MI355X) permutohedral-lattice filter.
+ *
+ * Plain pointers and sizes only.  Every pointer named "device" must be device memory of the
+ * GPU that is current when the call is made; all work is enqueued on the lattice's stream.
+ * Each entry point cites the reference interface it stands in for (paths are relative to the
+ * reference tree, MiguelMonteiro/permutohedral_lattice).
+ *
+ * Status codes: every function returns PL_OK (0) or a negative pl_status; nothing here calls
+ * exit() or throws (the reference GPU path exits the process on errors:
+ * src/PermutohedralLatticeGPU.cuh:49-55, src/DeviceMemoryAllocator.h:29-37).
+ */
+#ifndef PERMUTOHEDRAL_LATTICE_H
+#define PERMUTOHEDRAL_LATTICE_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef enum pl_status {
+    PL_OK = 0,
+    PL_EINVAL = -1,       /* null pointer, negative size, bad option */
+    PL_EUNSUPPORTED = -2, /* (pd, vd) outside what the kernels are built for */
+    PL_ENOMEM = -3,       /* allocator returned NULL */
+    PL_EOVERFLOW = -4,    /* sizes do not fit int32, or lattice coordinates do not fit the packed key */
+    PL_EHIP = -5,         /* a HIP runtime call failed; pl_last_hip_error() has the code */
+    PL_ESTATE = -6        /* pl_apply before pl_build, and the like */
+} pl_status;
+
+/* Opaque lattice object. */
+typedef struct pl_lattice *pl_handle;
+
+/* A hipStream_t passed as an untyped pointer (NULL = the default stream). */
+typedef void *pl_stream;
+
+/*
+ * Scratch-memory callbacks.  Stands in for DeviceMemoryAllocator (src/DeviceMemoryAllocator.h:47-120),
+ * which backs the lattice's scratch either with TensorFlow temporaries or with cudaMalloc.
+ * NULL in pl_create means hipMalloc/hipFree.
+ */
+typedef struct pl_alloc {
+    void *(*alloc)(void *ctx, size_t bytes); /* device memory, 256-byte aligned, or NULL */
+    void (*free)(void *ctx, void *ptr);
+    void *ctx;
+} pl_alloc;
+
+/* pl_set_option keys */
+typedef enum pl_option {
+    PL_OPT_NORMALIZE = 1,  /* 1 (default): slice divides by the homogeneous channel as the reference
+                              does (src/PermutohedralLatticeCPU.h:347-350).  0: input and output carry all
+                              vd channels and nothing is divided -- the bare linear operator, for tests. */
+    PL_OPT_PROFILE = 2,    /* 1: record per-stage HIP events, read with pl_stage_ms */
+    PL_OPT_TABLE_CELLS = 3 /* force the initial number of hash cells (power of two), 0 = automatic */
+} pl_option;
+
+/* 1 when a lattice can be built for these dimensions, else 0.
+ * Replaces the compile-time (pd, vd) pairs of src/LatticeFilterKernel.cu:87-100 by run-time dispatch. */
+int pl_supported(int pd, int vd);
+
+const char *pl_strerror(int status);
+
+/* hipError_t of the last failed HIP call on this thread (0 if none). */
+int pl_last_hip_error(void);
+
+/*
+ * Lattice for (pd, vd, N): pd feature dimensions, vd = value channels + 1 homogeneous, N points.
+ * Stands in for PermutohedralLatticeCPU<T>(pd, vd, N) (src/PermutohedralLatticeCPU.h:419) and
+ * PermutohedralLatticeGPU<T,pd,vd>(n, allocator, stream) (src/PermutohedralLatticeGPU.cuh:434).
+ * Unlike the reference objects, which are single-shot, a handle may be used for any number of
+ * filter calls; each behaves as if on a fresh lattice.
+ */
+int pl_create(int pd, int vd, int N, pl_stream stream, const pl_alloc *alloc, pl_handle *out);
+int pl_destroy(pl_handle h);
+
+/*
+ * output[N*(vd-1)] = filter(input[N*(vd-1)]) under positions[N*pd]; all three are device pointers,
+ * row-major, one row per point.  reverse != 0 visits the blur axes pd..0 (the gradient pass).
+ * Stands in for filter(output, input, positions, reverse)
+ * (src/PermutohedralLatticeCPU.h:442-446, src/PermutohedralLatticeGPU.cuh:453-479).
+ * Equivalent to pl_build followed by pl_apply.  Returns after the result of the build has been
+ * checked on the host (one stream synchronisation); the remaining work may still be in flight.
+ */
+int pl_filter(pl_handle h, float *output, const float *input, const float *positions, int reverse);
+
+/*
+ * Build the lattice for positions[N*pd] (embed, enclosing simplex, hash insertion, neighbour
+ * table) once; pl_apply then runs splat, blur, slice for any number of inputs, forward or reverse,
+ * under those positions.  The reference rebuilds for every call
+ * (src/LatticeFilterKernel.cpp:79, src/LatticeFilterKernel.cu:88); results are the same.
+ */
+int pl_build(pl_handle h, const float *positions);
+int pl_apply(pl_handle h, float *output, const float *input, int reverse);
+
+/* Number of lattice vertices of the last build (HashTableCPU::size(), src/PermutohedralLatticeCPU.h:151). */
+int pl_num_vertices(pl_handle h, int *num_vertices);
+
+int pl_set_option(pl_handle h, int option, long value);
+
+/* Milliseconds of the kernels of the last pl_build and pl_apply (or pl_filter) with
+ * PL_OPT_PROFILE on, from HIP events on the lattice's stream: ms[0] table clear, ms[1] build
+ * (embed + simplex + hash insertion), ms[2] neighbour table, ms[3] value clear, ms[4] splat,
+ * ms[5] blur (all pd+1 launches together), ms[6] slice.  Synchronises the stream. */
+int pl_stage_ms(pl_handle h, float ms[7]);
+
+/*
+ * Debug export of the per-point integer results of the last build, for parity checks; device
+ * pointers, any may be NULL: rem0[N*(pd+1)], rank[N*(pd+1)], keys[N*(pd+1)*pd] (vertex-major
+ * inside a point), barycentric[N*(pd+1)].  Same quantities as
+ * find_enclosing_simplex / compute_barycentric_coordinates / the key loop of splat_point
+ * (src/PermutohedralLatticeCPU.h:233-304).
+ */
+int pl_debug_simplex(pl_handle h, const float *positions, short *rem0, short *rank, short *keys,
+                     float *barycentric);
+
+/* Keys of the vertices of the last build, M*pd shorts to device memory, in vertex-index order
+ * (HashTableCPU::getKeys(), src/PermutohedralLatticeCPU.h:154; the order is not the reference's). */
+int pl_debug_keys(pl_handle h, short *keys);
+
+/* Vertex index (0..M-1) and weight of each point's simplex vertices after the last pl_apply or
+ * pl_filter: vertex[(pd+1)*N], weight[(pd+1)*N], laid out [r][n]; device pointers.  The replay
+ * matrix of src/PermutohedralLatticeCPU.h:187-191, 314-317. */
+int pl_debug_replay(pl_handle h, int *vertex, float *weight);
+
+/*
+ * Feature vectors of one batch item: positions[n][0..k) = coordinate / spatial_std (tensor order,
+ * last dimension fastest), positions[n][k..k+rc) = reference[n][c] / feature_std.
+ * reference and positions are device pointers; spatial_dims is a HOST array of n_spatial_dims ints.
+ * Stands in for compute_kernel_cpu / compute_kernel
+ * (src/PermutohedralLatticeCPU.h:452-474, src/PermutohedralLatticeGPU.cuh:482-506) and the
+ * ComputeKernel functor (src/LatticeFilterKernel.h:42-54).
+ */
+int pl_compute_positions(const float *reference, float *positions, int num_super_pixels,
+                         int n_reference_channels, int n_spatial_dims, const int *spatial_dims,
+                         float spatial_std, float feature_std, pl_stream stream);
+
+/*
+ * The LatticeFilter op on channels-last device tensors input[B, s_1..s_k, C_in],
+ * reference[B, s_1..s_k, C_ref] -> output (shape of input).  bilateral: features are
+ * (coords/theta_alpha, reference/theta_beta); otherwise coords/theta_gamma and the reference is
+ * ignored (may be NULL).  One lattice per batch item.  Stands in for LatticeFilterOp::Compute
+ * (src/LatticeFilterKernel.cpp:98-181); its gradient is the same call on the upstream gradient
+ * with reverse = 1 (lattice_filter_op_loader.py:32-54).  Scratch comes from alloc (NULL = hipMalloc).
+ */
+int pl_lattice_filter_op(const float *input, const float *reference, float *output, int batch,
+                         int n_spatial_dims, const int *spatial_dims, int n_input_channels,
+                         int n_reference_channels, int bilateral, float theta_alpha,
+                         float theta_beta, float theta_gamma, int reverse, pl_stream stream,
+                         const pl_alloc *alloc);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PERMUTOHEDRAL_LATTICE_H */

@@ -10,7 +10,11 @@
 #include <cstdlib>
 #include <ctime>
 
+// the header reports every growth of its hash table on stdout; keep stdout clean for callers
+// that print machine-readable results
+#define printf(...) ((void)0)
 #include "PermutohedralLatticeCPU.h"
+#undef printf
 
 namespace {
 double now_seconds() {

@@ -1,0 +1,250 @@
+"""MI355X (gfx950) permutohedral-lattice filter: Python mirror of the reference's interfaces over
+the C ABI of ``libpermutohedral_hip.so`` (declared in ``include/permutohedral_lattice.h``).
+
+* :class:`PermutohedralLattice` -- the lattice object ``(pd, vd, N)`` with
+  ``filter(output, input, positions, reverse)`` on device tensors
+  (reference: src/PermutohedralLatticeCPU.h:419-446, src/PermutohedralLatticeGPU.cuh:434-479).
+* :func:`compute_positions` -- the feature builder (reference: src/PermutohedralLatticeCPU.h:452-474).
+* :func:`lattice_filter` -- the ``LatticeFilter`` op with its registered gradient
+  (reference: src/LatticeFilterKernel.cpp:30-43, 98-181; lattice_filter_op_loader.py:32-54).
+
+torch is used for device memory, streams and autograd plumbing only; all computation is in the
+HIP library.  There is no CPU fallback: importing this package without the built library raises.
+"""
+import ctypes as C
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libpermutohedral_hip.so")
+
+PL_OK, PL_EINVAL, PL_EUNSUPPORTED, PL_ENOMEM, PL_EOVERFLOW, PL_EHIP, PL_ESTATE = 0, -1, -2, -3, -4, -5, -6
+PL_OPT_NORMALIZE, PL_OPT_PROFILE, PL_OPT_TABLE_CELLS = 1, 2, 3
+
+# every symbol include/permutohedral_lattice.h declares
+EXPORTS = (
+    "pl_supported", "pl_strerror", "pl_last_hip_error", "pl_create", "pl_destroy", "pl_filter",
+    "pl_build", "pl_apply", "pl_num_vertices", "pl_set_option", "pl_stage_ms", "pl_debug_simplex",
+    "pl_debug_keys", "pl_debug_replay", "pl_compute_positions", "pl_lattice_filter_op",
+)
+
+
+class PermutohedralError(RuntimeError):
+    def __init__(self, status, where):
+        self.status = status
+        msg = _lib.pl_strerror(status).decode()
+        if status == PL_EHIP:
+            msg += " (hipError %d)" % _lib.pl_last_hip_error()
+        super().__init__("%s: %s" % (where, msg))
+
+
+def _load():
+    if not os.path.exists(LIB_PATH):
+        raise ImportError(
+            "%s is missing: build it with `python -m permutohedral_lattice_amd.build` "
+            "(there is no CPU fallback)" % LIB_PATH)
+    lib = C.CDLL(LIB_PATH)
+    vp, ci, cf = C.c_void_p, C.c_int, C.c_float
+    lib.pl_supported.argtypes = [ci, ci]
+    lib.pl_strerror.argtypes = [ci]
+    lib.pl_strerror.restype = C.c_char_p
+    lib.pl_create.argtypes = [ci, ci, ci, vp, vp, C.POINTER(vp)]
+    lib.pl_destroy.argtypes = [vp]
+    lib.pl_filter.argtypes = [vp, vp, vp, vp, ci]
+    lib.pl_build.argtypes = [vp, vp]
+    lib.pl_apply.argtypes = [vp, vp, vp, ci]
+    lib.pl_num_vertices.argtypes = [vp, C.POINTER(ci)]
+    lib.pl_set_option.argtypes = [vp, ci, C.c_long]
+    lib.pl_stage_ms.argtypes = [vp, C.POINTER(cf)]
+    lib.pl_debug_simplex.argtypes = [vp, vp, vp, vp, vp, vp]
+    lib.pl_debug_keys.argtypes = [vp, vp]
+    lib.pl_debug_replay.argtypes = [vp, vp, vp]
+    lib.pl_compute_positions.argtypes = [vp, vp, ci, ci, ci, C.POINTER(ci), cf, cf, vp]
+    lib.pl_lattice_filter_op.argtypes = [vp, vp, vp, ci, ci, C.POINTER(ci), ci, ci, ci, cf, cf, cf,
+                                         ci, vp, vp]
+    return lib
+
+
+_lib = _load()
+
+
+def _check(status, where):
+    if status != PL_OK:
+        raise PermutohedralError(status, where)
+
+
+def _dev_f32(t, name, numel=None):
+    if not (isinstance(t, torch.Tensor) and t.is_cuda and t.dtype == torch.float32
+            and t.is_contiguous()):
+        raise TypeError("%s must be a contiguous float32 tensor on the GPU" % name)
+    if numel is not None and t.numel() != numel:
+        raise ValueError("%s has %d elements, expected %d" % (name, t.numel(), numel))
+    return C.c_void_p(t.data_ptr())
+
+
+def _stream_ptr(stream=None):
+    s = stream if stream is not None else torch.cuda.current_stream()
+    return C.c_void_p(s.cuda_stream)
+
+
+def supported(pd, vd):
+    return bool(_lib.pl_supported(pd, vd))
+
+
+class PermutohedralLattice:
+    """Lattice for ``(pd, vd, N)``; ``vd`` counts the homogeneous channel.  All tensors are
+    contiguous float32 on the GPU; work is enqueued on the stream current at construction."""
+
+    def __init__(self, pd, vd, N, stream=None):
+        self.pd, self.vd, self.N = int(pd), int(vd), int(N)
+        self._h = C.c_void_p()
+        self._stream = stream if stream is not None else torch.cuda.current_stream()
+        _check(_lib.pl_create(self.pd, self.vd, self.N, _stream_ptr(self._stream), None,
+                              C.byref(self._h)), "pl_create")
+        self._normalize = True
+
+    def close(self):
+        if getattr(self, "_h", None):
+            _lib.pl_destroy(self._h)
+            self._h = None
+
+    __del__ = close
+
+    # -- the reference's interface -------------------------------------------------------------
+    def filter(self, output, input, positions, reverse=False):
+        ch = self.vd - 1 if self._normalize else self.vd
+        _check(_lib.pl_filter(self._h, _dev_f32(output, "output", self.N * ch),
+                              _dev_f32(input, "input", self.N * ch),
+                              _dev_f32(positions, "positions", self.N * self.pd), int(bool(reverse))),
+               "pl_filter")
+        return output
+
+    # -- build once, apply many ----------------------------------------------------------------
+    def build(self, positions):
+        _check(_lib.pl_build(self._h, _dev_f32(positions, "positions", self.N * self.pd)), "pl_build")
+
+    def apply(self, output, input, reverse=False):
+        ch = self.vd - 1 if self._normalize else self.vd
+        _check(_lib.pl_apply(self._h, _dev_f32(output, "output", self.N * ch),
+                             _dev_f32(input, "input", self.N * ch), int(bool(reverse))), "pl_apply")
+        return output
+
+    @property
+    def num_vertices(self):
+        m = C.c_int()
+        _check(_lib.pl_num_vertices(self._h, C.byref(m)), "pl_num_vertices")
+        return m.value
+
+    def set_option(self, option, value):
+        _check(_lib.pl_set_option(self._h, option, int(value)), "pl_set_option")
+        if option == PL_OPT_NORMALIZE:
+            self._normalize = bool(value)
+
+    def stage_ms(self):
+        ms = (C.c_float * 7)()
+        _check(_lib.pl_stage_ms(self._h, ms), "pl_stage_ms")
+        return dict(zip(("clear", "build", "neighbours", "fill", "splat", "blur", "slice"), list(ms)))
+
+    # -- parity exports ------------------------------------------------------------------------
+    def debug_simplex(self, positions):
+        """-> dict of device tensors rem0 [N,pd+1] i16, rank [N,pd+1] i16, keys [N,pd+1,pd] i16,
+        barycentric [N,pd+1] f32."""
+        d1, dev = self.pd + 1, positions.device
+        out = dict(rem0=torch.empty((self.N, d1), dtype=torch.int16, device=dev),
+                   rank=torch.empty((self.N, d1), dtype=torch.int16, device=dev),
+                   keys=torch.empty((self.N, d1, self.pd), dtype=torch.int16, device=dev),
+                   barycentric=torch.empty((self.N, d1), dtype=torch.float32, device=dev))
+        _check(_lib.pl_debug_simplex(self._h, _dev_f32(positions, "positions", self.N * self.pd),
+                                     C.c_void_p(out["rem0"].data_ptr()),
+                                     C.c_void_p(out["rank"].data_ptr()),
+                                     C.c_void_p(out["keys"].data_ptr()),
+                                     C.c_void_p(out["barycentric"].data_ptr())), "pl_debug_simplex")
+        return out
+
+    def debug_keys(self):
+        keys = torch.empty((self.num_vertices, self.pd), dtype=torch.int16, device="cuda")
+        _check(_lib.pl_debug_keys(self._h, C.c_void_p(keys.data_ptr())), "pl_debug_keys")
+        return keys
+
+    def debug_replay(self):
+        """-> (vertex [pd+1, N] i32, weight [pd+1, N] f32) of the last apply/filter."""
+        v = torch.empty((self.pd + 1, self.N), dtype=torch.int32, device="cuda")
+        w = torch.empty((self.pd + 1, self.N), dtype=torch.float32, device="cuda")
+        _check(_lib.pl_debug_replay(self._h, C.c_void_p(v.data_ptr()), C.c_void_p(w.data_ptr())),
+               "pl_debug_replay")
+        return v, w
+
+
+def compute_positions(reference, spatial_dims, spatial_std, feature_std=1.0, out=None):
+    """Feature rows of one batch item.  ``reference``: ``[*spatial_dims, rc]`` device tensor, or
+    None for spatial-only features.  -> ``[N, k + rc]``."""
+    sd = [int(s) for s in spatial_dims]
+    n = 1
+    for s in sd:
+        n *= s
+    rc = 0 if reference is None else int(reference.shape[-1])
+    pd = len(sd) + rc
+    if out is None:
+        out = torch.empty((n, pd), dtype=torch.float32, device="cuda")
+    ref_ptr = None if reference is None else _dev_f32(reference, "reference", n * rc)
+    dims = (C.c_int * len(sd))(*sd)
+    _check(_lib.pl_compute_positions(ref_ptr, _dev_f32(out, "positions", n * pd), n, rc, len(sd), dims,
+                                     float(spatial_std), float(feature_std), _stream_ptr()),
+           "pl_compute_positions")
+    return out
+
+
+def _lattice_filter_raw(input_image, reference_image, bilateral, theta_alpha, theta_beta,
+                        theta_gamma, reverse):
+    if input_image.dim() < 3:
+        raise ValueError("input_image must be [batch, spatial..., channels]")
+    inp = input_image.contiguous()
+    sd = [int(s) for s in inp.shape[1:-1]]
+    out = torch.empty_like(inp)
+    ref_ptr, rc = None, 0
+    if reference_image is not None:
+        ref = reference_image.contiguous()
+        rc = int(ref.shape[-1])
+        if bilateral:
+            if list(ref.shape[:-1]) != list(inp.shape[:-1]):
+                raise ValueError("reference_image and input_image differ in batch or spatial shape")
+            ref_ptr = _dev_f32(ref, "reference_image")
+    dims = (C.c_int * len(sd))(*sd)
+    _check(_lib.pl_lattice_filter_op(_dev_f32(inp, "input_image"), ref_ptr,
+                                     C.c_void_p(out.data_ptr()), int(inp.shape[0]), len(sd), dims,
+                                     int(inp.shape[-1]), rc, int(bool(bilateral)),
+                                     float(theta_alpha), float(theta_beta), float(theta_gamma),
+                                     int(bool(reverse)), _stream_ptr(), None),
+           "pl_lattice_filter_op")
+    return out
+
+
+class _LatticeFilterFunction(torch.autograd.Function):
+    @staticmethod
+    def forward(ctx, input_image, reference_image, bilateral, theta_alpha, theta_beta, theta_gamma,
+                reverse):
+        ctx.save_for_backward(reference_image)
+        ctx.attrs = (bilateral, theta_alpha, theta_beta, theta_gamma)
+        return _lattice_filter_raw(input_image, reference_image, bilateral, theta_alpha, theta_beta,
+                                   theta_gamma, reverse)
+
+    @staticmethod
+    def backward(ctx, grad):
+        # the reference's registered gradient: the same op on the upstream gradient with
+        # reverse=True, and zeros for the reference image (lattice_filter_op_loader.py:46-54)
+        (reference_image,) = ctx.saved_tensors
+        bilateral, theta_alpha, theta_beta, theta_gamma = ctx.attrs
+        grad_vals = _lattice_filter_raw(grad, reference_image, bilateral, theta_alpha, theta_beta,
+                                        theta_gamma, True)
+        grad_ref = torch.zeros_like(reference_image) if ctx.needs_input_grad[1] else None
+        return grad_vals, grad_ref, None, None, None, None, None
+
+
+def lattice_filter(input_image, reference_image, bilateral=True, theta_alpha=1.0, theta_beta=1.0,
+                   theta_gamma=1.0, reverse=False):
+    """The ``LatticeFilter`` op: channels-last ``[B, s_1..s_k, C]`` device tensors, output shaped
+    like ``input_image``.  Differentiable in ``input_image`` by the reference's rule."""
+    return _LatticeFilterFunction.apply(input_image, reference_image, bool(bilateral),
+                                        float(theta_alpha), float(theta_beta), float(theta_gamma),
+                                        bool(reverse))

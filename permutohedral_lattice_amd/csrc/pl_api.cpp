@@ -1,0 +1,524 @@
+// Host side of the C ABI declared in include/permutohedral_lattice.h: the lattice object, its
+// scratch memory, the build/apply orchestration and the LatticeFilter op loop.
+#include "permutohedral_lattice.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdint>
+#include <cstring>
+#include <mutex>
+#include <new>
+#include <vector>
+
+#include "pl_kernels.h"
+
+namespace {
+
+thread_local int g_last_hip_error = 0;
+
+inline int hip_failed(hipError_t e) {
+    if (e == hipSuccess) return 0;
+    g_last_hip_error = (int)e;
+    return 1;
+}
+#define PL_HIP(call)                          \
+    do {                                      \
+        if (hip_failed((call))) return PL_EHIP; \
+    } while (0)
+
+void *default_alloc(void *, size_t bytes) {
+    void *p = nullptr;
+    if (hipMalloc(&p, bytes ? bytes : 1) != hipSuccess) return nullptr;
+    return p;
+}
+void default_free(void *, void *p) {
+    if (p) (void)hipFree(p);
+}
+
+uint32_t pow2_at_least(uint64_t x) {
+    uint64_t p = 1;
+    while (p < x) p <<= 1;
+    return (uint32_t)p;
+}
+
+// scale factors of the elevation, with the rounding of the reference CPU path
+// (src/PermutohedralLatticeCPU.h:209-214: double intermediates, float results)
+void compute_scale_factor(int pd, plk::ScaleFactor &sf) {
+    const float inv_std_dev = (float)((double)(pd + 1) * std::sqrt(2.0 / 3.0));
+    for (int i = 0; i < plk::kMaxPd; ++i) sf.v[i] = 0.0f;
+    for (int i = 0; i < pd; ++i)
+        sf.v[i] = (float)(1.0 / std::sqrt((double)((i + 1) * (i + 2))) * (double)inv_std_dev);
+}
+
+enum { EV_T0, EV_CLEAR, EV_BUILD, EV_NBR0, EV_NBR, EV_A0, EV_FILL, EV_SPLAT, EV_BLUR, EV_SLICE, EV_COUNT };
+
+}  // namespace
+
+struct pl_lattice {
+    int pd = 0, vd = 0, N = 0;
+    int device = 0;
+    hipStream_t stream = nullptr;
+    pl_alloc alloc{};
+    plk::ScaleFactor scale{};
+
+    // hash table
+    uint64_t *cell_keys = nullptr;
+    int *cell_vertex = nullptr;
+    uint64_t *vertex_keys = nullptr;  // n_cells_alloc / 2 entries
+    uint32_t n_cells_alloc = 0;       // allocated
+    uint32_t n_cells = 0;             // in use by the last build
+    uint32_t max_cells = 0;           // enough for N*(pd+1) vertices at load 1/2
+    long forced_cells = 0;
+
+    // per-vertex arrays, sized after the build
+    float *values[2] = {nullptr, nullptr};
+    int2 *neighbours = nullptr;
+    size_t vertex_capacity = 0;
+
+    // per-point arrays
+    int *replay_index = nullptr;
+    float *replay_weight = nullptr;
+
+    plk::Counters *d_counters = nullptr;
+    plk::Counters *h_counters = nullptr;  // pinned
+
+    int M = 0;
+    int last_M = -1;
+    bool built = false;
+    bool replay_holds_cells = false;
+    bool normalize = true;
+    bool profile = false;
+    hipEvent_t ev[EV_COUNT] = {};
+    bool ev_recorded[EV_COUNT] = {};
+
+    void *dmalloc(size_t bytes) { return alloc.alloc(alloc.ctx, bytes); }
+    void dfree(void *p) {
+        if (p) alloc.free(alloc.ctx, p);
+    }
+    void mark(int which) {
+        if (profile && ev[which]) {
+            ev_recorded[which] = hipEventRecord(ev[which], stream) == hipSuccess;
+        }
+    }
+};
+
+namespace {
+
+int ensure_table(pl_lattice *h, uint32_t cells) {
+    if (cells <= h->n_cells_alloc) return PL_OK;
+    h->dfree(h->cell_keys);
+    h->dfree(h->cell_vertex);
+    h->dfree(h->vertex_keys);
+    h->cell_keys = nullptr;
+    h->cell_vertex = nullptr;
+    h->vertex_keys = nullptr;
+    h->n_cells_alloc = 0;
+    h->cell_keys = (uint64_t *)h->dmalloc(sizeof(uint64_t) * (size_t)cells);
+    h->cell_vertex = (int *)h->dmalloc(sizeof(int) * (size_t)cells);
+    h->vertex_keys = (uint64_t *)h->dmalloc(sizeof(uint64_t) * (size_t)(cells / 2));
+    if (!h->cell_keys || !h->cell_vertex || !h->vertex_keys) return PL_ENOMEM;
+    h->n_cells_alloc = cells;
+    return PL_OK;
+}
+
+int ensure_vertices(pl_lattice *h, size_t m) {
+    if (m <= h->vertex_capacity) return PL_OK;
+    size_t cap = h->vertex_capacity ? h->vertex_capacity : 1024;
+    while (cap < m) cap *= 2;
+    h->dfree(h->values[0]);
+    h->dfree(h->values[1]);
+    h->dfree(h->neighbours);
+    h->values[0] = h->values[1] = nullptr;
+    h->neighbours = nullptr;
+    h->vertex_capacity = 0;
+    h->values[0] = (float *)h->dmalloc(sizeof(float) * cap * (size_t)h->vd);
+    h->values[1] = (float *)h->dmalloc(sizeof(float) * cap * (size_t)h->vd);
+    h->neighbours = (int2 *)h->dmalloc(sizeof(int2) * cap * (size_t)(h->pd + 1));
+    if (!h->values[0] || !h->values[1] || !h->neighbours) return PL_ENOMEM;
+    h->vertex_capacity = cap;
+    return PL_OK;
+}
+
+uint32_t initial_cells(const pl_lattice *h) {
+    uint64_t want;
+    if (h->forced_cells > 0) {
+        want = (uint64_t)h->forced_cells;
+    } else if (h->last_M > 0) {
+        want = (uint64_t)h->last_M * 5 / 2;  // load factor 0.4 if the next input resembles the last
+    } else {
+        want = (uint64_t)h->N * (uint64_t)(h->pd + 1) / 8;
+    }
+    if (want < 4096) want = 4096;
+    uint32_t cells = pow2_at_least(want);
+    if (cells > h->max_cells) cells = h->max_cells;
+    return cells;
+}
+
+}  // namespace
+
+extern "C" {
+
+int pl_supported(int pd, int vd) { return pd >= 1 && pd <= plk::kMaxPd && vd >= 2 ? 1 : 0; }
+
+const char *pl_strerror(int status) {
+    switch (status) {
+        case PL_OK: return "ok";
+        case PL_EINVAL: return "invalid argument";
+        case PL_EUNSUPPORTED: return "unsupported (pd, vd)";
+        case PL_ENOMEM: return "out of device memory";
+        case PL_EOVERFLOW: return "size or lattice coordinate out of range";
+        case PL_EHIP: return "HIP runtime error";
+        case PL_ESTATE: return "call out of order";
+        default: return "unknown status";
+    }
+}
+
+int pl_last_hip_error(void) { return g_last_hip_error; }
+
+int pl_create(int pd, int vd, int N, pl_stream stream, const pl_alloc *alloc, pl_handle *out) {
+    if (!out) return PL_EINVAL;
+    *out = nullptr;
+    if (N < 0 || pd < 1 || vd < 2) return PL_EINVAL;
+    if (!pl_supported(pd, vd)) return PL_EUNSUPPORTED;
+    if (alloc && (!alloc->alloc || !alloc->free)) return PL_EINVAL;
+    // N*(pd+1) replay rows and N*vd values must be addressable with the table sizes used here
+    const uint64_t rows = (uint64_t)N * (uint64_t)(pd + 1);
+    if (rows > (1ull << 30) || (uint64_t)N * (uint64_t)vd > (1ull << 31) - 1) return PL_EOVERFLOW;
+
+    pl_lattice *h = new (std::nothrow) pl_lattice();
+    if (!h) return PL_ENOMEM;
+    h->pd = pd;
+    h->vd = vd;
+    h->N = N;
+    h->stream = (hipStream_t)stream;
+    if (alloc) {
+        h->alloc = *alloc;
+    } else {
+        h->alloc.alloc = default_alloc;
+        h->alloc.free = default_free;
+        h->alloc.ctx = nullptr;
+    }
+    compute_scale_factor(pd, h->scale);
+    h->max_cells = pow2_at_least(rows * 2 < 4096 ? 4096 : rows * 2);
+
+    int rc = PL_OK;
+    if (hip_failed(hipGetDevice(&h->device))) rc = PL_EHIP;
+    if (rc == PL_OK) {
+        h->replay_index = (int *)h->dmalloc(sizeof(int) * (size_t)(rows ? rows : 1));
+        h->replay_weight = (float *)h->dmalloc(sizeof(float) * (size_t)(rows ? rows : 1));
+        h->d_counters = (plk::Counters *)h->dmalloc(sizeof(plk::Counters));
+        if (!h->replay_index || !h->replay_weight || !h->d_counters) rc = PL_ENOMEM;
+    }
+    if (rc == PL_OK && hip_failed(hipHostMalloc((void **)&h->h_counters, sizeof(plk::Counters), hipHostMallocDefault)))
+        rc = PL_EHIP;
+    if (rc != PL_OK) {
+        pl_destroy(h);
+        return rc;
+    }
+    *out = h;
+    return PL_OK;
+}
+
+int pl_destroy(pl_handle h) {
+    if (!h) return PL_OK;
+    (void)hipStreamSynchronize(h->stream);
+    h->dfree(h->cell_keys);
+    h->dfree(h->cell_vertex);
+    h->dfree(h->vertex_keys);
+    h->dfree(h->values[0]);
+    h->dfree(h->values[1]);
+    h->dfree(h->neighbours);
+    h->dfree(h->replay_index);
+    h->dfree(h->replay_weight);
+    h->dfree(h->d_counters);
+    if (h->h_counters) (void)hipHostFree(h->h_counters);
+    for (int i = 0; i < EV_COUNT; ++i)
+        if (h->ev[i]) (void)hipEventDestroy(h->ev[i]);
+    delete h;
+    return PL_OK;
+}
+
+int pl_set_option(pl_handle h, int option, long value) {
+    if (!h) return PL_EINVAL;
+    switch (option) {
+        case PL_OPT_NORMALIZE:
+            h->normalize = value != 0;
+            return PL_OK;
+        case PL_OPT_PROFILE:
+            h->profile = value != 0;
+            if (h->profile)
+                for (int i = 0; i < EV_COUNT; ++i)
+                    if (!h->ev[i]) PL_HIP(hipEventCreate(&h->ev[i]));
+            return PL_OK;
+        case PL_OPT_TABLE_CELLS:
+            if (value < 0 || (value & (value - 1)) != 0) return PL_EINVAL;
+            h->forced_cells = value;
+            h->last_M = -1;
+            return PL_OK;
+        default:
+            return PL_EINVAL;
+    }
+}
+
+int pl_build(pl_handle h, const float *positions) {
+    if (!h || (!positions && h->N > 0)) return PL_EINVAL;
+    h->built = false;
+    h->M = 0;
+    for (int i = 0; i <= EV_NBR; ++i) h->ev_recorded[i] = false;
+    if (h->N == 0) {
+        h->built = true;
+        return PL_OK;
+    }
+    uint32_t cells = initial_cells(h);
+    for (;;) {
+        int rc = ensure_table(h, cells);
+        if (rc != PL_OK) return rc;
+        h->mark(EV_T0);
+        PL_HIP(plk::clear_table(h->cell_keys, cells, h->d_counters, h->stream));
+        h->mark(EV_CLEAR);
+        PL_HIP(plk::build(h->pd, positions, h->N, h->scale, h->cell_keys, h->cell_vertex, cells,
+                          h->vertex_keys, h->d_counters, h->replay_index, h->replay_weight,
+                          h->stream));
+        h->mark(EV_BUILD);
+        PL_HIP(hipMemcpyAsync(h->h_counters, h->d_counters, sizeof(plk::Counters),
+                              hipMemcpyDeviceToHost, h->stream));
+        PL_HIP(hipStreamSynchronize(h->stream));
+        const int flags = h->h_counters->flags;
+        if (flags & plk::kFlagKeyRange) return PL_EOVERFLOW;
+        if ((flags & plk::kFlagTableFull) || (uint32_t)h->h_counters->num_vertices > cells / 2) {
+            if (cells >= h->max_cells) return PL_EOVERFLOW;  // cannot happen: max_cells holds every vertex
+            cells = (cells > h->max_cells / 4) ? h->max_cells : cells * 4;
+            continue;
+        }
+        break;
+    }
+    h->n_cells = cells;
+    h->M = h->h_counters->num_vertices;
+    h->last_M = h->M;
+    int rc = ensure_vertices(h, (size_t)h->M);
+    if (rc != PL_OK) return rc;
+    h->mark(EV_NBR0);
+    PL_HIP(plk::neighbours(h->pd, h->vertex_keys, h->M, h->cell_keys, h->cell_vertex, h->n_cells,
+                           h->neighbours, h->stream));
+    h->mark(EV_NBR);
+    h->replay_holds_cells = true;
+    h->built = true;
+    return PL_OK;
+}
+
+int pl_apply(pl_handle h, float *output, const float *input, int reverse) {
+    if (!h) return PL_EINVAL;
+    if (!h->built) return PL_ESTATE;
+    if (h->N == 0) return PL_OK;
+    if (!output || !input) return PL_EINVAL;
+    const int pd = h->pd, vd = h->vd, M = h->M;
+    const int in_channels = h->normalize ? vd - 1 : vd;
+
+    h->mark(EV_A0);
+    PL_HIP(plk::fill_zero(h->values[0], (size_t)M * vd, h->stream));
+    h->mark(EV_FILL);
+    PL_HIP(plk::splat(pd, vd, h->N, input, in_channels, h->replay_index, h->replay_weight,
+                      h->replay_holds_cells ? h->cell_vertex : nullptr, h->values[0], h->stream));
+    h->replay_holds_cells = false;
+    h->mark(EV_SPLAT);
+
+    int cur = 0;
+    for (int step = 0; step <= pd; ++step) {
+        const int axis = reverse ? pd - step : step;
+        PL_HIP(plk::blur_axis(vd, M, h->values[cur], h->values[1 - cur],
+                              h->neighbours + (size_t)axis * M, h->stream));
+        cur = 1 - cur;
+    }
+    h->mark(EV_BLUR);
+
+    PL_HIP(plk::slice(pd, vd, h->N, h->replay_index, h->replay_weight, h->values[cur], output,
+                      h->normalize ? 1 : 0, h->stream));
+    h->mark(EV_SLICE);
+    return PL_OK;
+}
+
+int pl_filter(pl_handle h, float *output, const float *input, const float *positions, int reverse) {
+    if (!h) return PL_EINVAL;
+    if (h->N > 0 && (!output || !input || !positions)) return PL_EINVAL;
+    int rc = pl_build(h, positions);
+    if (rc != PL_OK) return rc;
+    return pl_apply(h, output, input, reverse);
+}
+
+int pl_num_vertices(pl_handle h, int *num_vertices) {
+    if (!h || !num_vertices) return PL_EINVAL;
+    if (!h->built) return PL_ESTATE;
+    *num_vertices = h->M;
+    return PL_OK;
+}
+
+int pl_stage_ms(pl_handle h, float ms[7]) {
+    if (!h || !ms) return PL_EINVAL;
+    if (!h->profile) return PL_ESTATE;
+    PL_HIP(hipStreamSynchronize(h->stream));
+    const int pairs[7][2] = {{EV_T0, EV_CLEAR},  {EV_CLEAR, EV_BUILD}, {EV_NBR0, EV_NBR},
+                             {EV_A0, EV_FILL},   {EV_FILL, EV_SPLAT},  {EV_SPLAT, EV_BLUR},
+                             {EV_BLUR, EV_SLICE}};
+    for (int i = 0; i < 7; ++i) {
+        ms[i] = 0.0f;
+        if (h->ev_recorded[pairs[i][0]] && h->ev_recorded[pairs[i][1]])
+            PL_HIP(hipEventElapsedTime(&ms[i], h->ev[pairs[i][0]], h->ev[pairs[i][1]]));
+    }
+    return PL_OK;
+}
+
+int pl_debug_simplex(pl_handle h, const float *positions, short *rem0, short *rank, short *keys,
+                     float *barycentric) {
+    if (!h || (!positions && h->N > 0)) return PL_EINVAL;
+    PL_HIP(plk::debug_simplex(h->pd, positions, h->N, h->scale, rem0, rank, keys, barycentric,
+                              h->stream));
+    return PL_OK;
+}
+
+int pl_debug_keys(pl_handle h, short *keys) {
+    if (!h || !keys) return PL_EINVAL;
+    if (!h->built) return PL_ESTATE;
+    PL_HIP(plk::export_keys(h->pd, h->vertex_keys, h->M, keys, h->stream));
+    return PL_OK;
+}
+
+int pl_debug_replay(pl_handle h, int *vertex, float *weight) {
+    if (!h) return PL_EINVAL;
+    if (!h->built || h->replay_holds_cells) return PL_ESTATE;
+    const size_t rows = (size_t)h->N * (size_t)(h->pd + 1);
+    if (vertex)
+        PL_HIP(hipMemcpyAsync(vertex, h->replay_index, sizeof(int) * rows, hipMemcpyDeviceToDevice,
+                              h->stream));
+    if (weight)
+        PL_HIP(hipMemcpyAsync(weight, h->replay_weight, sizeof(float) * rows,
+                              hipMemcpyDeviceToDevice, h->stream));
+    return PL_OK;
+}
+
+int pl_compute_positions(const float *reference, float *positions, int num_super_pixels,
+                         int n_reference_channels, int n_spatial_dims, const int *spatial_dims,
+                         float spatial_std, float feature_std, pl_stream stream) {
+    if (num_super_pixels < 0 || n_reference_channels < 0 || n_spatial_dims < 0) return PL_EINVAL;
+    if (n_spatial_dims > plk::kMaxSpatialDims) return PL_EUNSUPPORTED;
+    if (n_spatial_dims + n_reference_channels < 1) return PL_EINVAL;
+    if (num_super_pixels == 0) return PL_OK;
+    if (!positions || (n_spatial_dims > 0 && !spatial_dims)) return PL_EINVAL;
+    if (n_reference_channels > 0 && !reference) return PL_EINVAL;
+    plk::SpatialDims dims{};
+    for (int i = 0; i < plk::kMaxSpatialDims; ++i) dims.v[i] = 1;
+    for (int i = 0; i < n_spatial_dims; ++i) {
+        if (spatial_dims[i] < 1) return PL_EINVAL;
+        dims.v[i] = spatial_dims[i];
+    }
+    PL_HIP(plk::compute_positions(reference, positions, num_super_pixels, n_reference_channels,
+                                  n_spatial_dims, dims, spatial_std, feature_std,
+                                  (hipStream_t)stream));
+    return PL_OK;
+}
+
+}  // extern "C"
+
+// ------------------------------------------------------------------------------------------------
+// Op level: shape arithmetic and per-item loop of LatticeFilterOp::Compute
+// (src/LatticeFilterKernel.cpp:111-179 of the reference tree)
+// ------------------------------------------------------------------------------------------------
+namespace {
+
+// With the default allocator the op keeps its lattice and positions buffer between calls (one
+// per device and shape), because hipMalloc/hipFree per call would serialise the device.  With a
+// caller-supplied allocator everything is taken from it and returned before the call ends, as
+// the reference does with TensorFlow temporaries (src/DeviceMemoryAllocator.h:52-71).
+struct OpCacheEntry {
+    int device, pd, vd, N;
+    hipStream_t stream;
+    pl_handle lattice;
+    float *positions;
+};
+std::mutex g_op_cache_mutex;
+std::vector<OpCacheEntry> g_op_cache;
+constexpr size_t kOpCacheMax = 8;
+
+}  // namespace
+
+extern "C" int pl_lattice_filter_op(const float *input, const float *reference, float *output,
+                                    int batch, int n_spatial_dims, const int *spatial_dims,
+                                    int n_input_channels, int n_reference_channels, int bilateral,
+                                    float theta_alpha, float theta_beta, float theta_gamma,
+                                    int reverse, pl_stream stream, const pl_alloc *alloc) {
+    if (batch < 0 || n_spatial_dims < 1 || n_input_channels < 1 || !spatial_dims) return PL_EINVAL;
+    if (n_spatial_dims > plk::kMaxSpatialDims) return PL_EUNSUPPORTED;
+    long long n = 1;
+    for (int i = 0; i < n_spatial_dims; ++i) {
+        if (spatial_dims[i] < 1) return PL_EINVAL;
+        n *= spatial_dims[i];
+        if (n > 2147483647LL) return PL_EOVERFLOW;
+    }
+    // the reference refuses tensors with more than INT32_MAX elements (LatticeFilterKernel.cpp:108)
+    if (n * (long long)batch * n_input_channels > 2147483647LL) return PL_EOVERFLOW;
+    const int N = (int)n;
+    const int vd = n_input_channels + 1;
+    const int ref_ch = bilateral ? n_reference_channels : 0;
+    if (bilateral && (n_reference_channels < 1 || (!reference && batch > 0))) return PL_EINVAL;
+    const int pd = n_spatial_dims + ref_ch;
+    // bilateral: theta_alpha / theta_beta; spatial only: theta_gamma (LatticeFilterKernel.cpp:131-142)
+    const float spatial_std = bilateral ? theta_alpha : theta_gamma;
+    const float feature_std = bilateral ? theta_beta : -1.0f;
+    if (!pl_supported(pd, vd)) return PL_EUNSUPPORTED;
+    if (batch == 0) return PL_OK;
+    if (!input || !output) return PL_EINVAL;
+
+    int device = 0;
+    PL_HIP(hipGetDevice(&device));
+
+    pl_handle lattice = nullptr;
+    float *positions = nullptr;
+    bool cached = false;
+    std::unique_lock<std::mutex> lock(g_op_cache_mutex, std::defer_lock);
+    if (!alloc) {
+        lock.lock();  // held for the whole call: a cached lattice is not re-entrant
+        for (auto &e : g_op_cache)
+            if (e.device == device && e.pd == pd && e.vd == vd && e.N == N &&
+                e.stream == (hipStream_t)stream) {
+                lattice = e.lattice;
+                positions = e.positions;
+                cached = true;
+                break;
+            }
+    }
+    int rc = PL_OK;
+    if (!lattice) {
+        rc = pl_create(pd, vd, N, stream, alloc, &lattice);
+        if (rc != PL_OK) return rc;
+        const size_t bytes = sizeof(float) * (size_t)N * (size_t)pd;
+        positions = (float *)(alloc ? alloc->alloc(alloc->ctx, bytes) : default_alloc(nullptr, bytes));
+        if (!positions) {
+            pl_destroy(lattice);
+            return PL_ENOMEM;
+        }
+        if (!alloc) {
+            if (g_op_cache.size() >= kOpCacheMax) {
+                pl_destroy(g_op_cache.front().lattice);
+                default_free(nullptr, g_op_cache.front().positions);
+                g_op_cache.erase(g_op_cache.begin());
+            }
+            g_op_cache.push_back({device, pd, vd, N, (hipStream_t)stream, lattice, positions});
+            cached = true;
+        }
+    }
+
+    for (int b = 0; b < batch && rc == PL_OK; ++b) {
+        const float *ref_b = ref_ch ? reference + (size_t)b * N * ref_ch : nullptr;
+        rc = pl_compute_positions(ref_b, positions, N, ref_ch, n_spatial_dims, spatial_dims,
+                                  spatial_std, feature_std, stream);
+        if (rc != PL_OK) break;
+        rc = pl_filter(lattice, output + (size_t)b * N * n_input_channels,
+                       input + (size_t)b * N * n_input_channels, positions, reverse);
+    }
+
+    if (!cached) {
+        pl_destroy(lattice);  // synchronises the stream first
+        alloc->free(alloc->ctx, positions);
+    }
+    return rc;
+}

@@ -1,0 +1,76 @@
+// Internal launch interface between the host-side lattice object (pl_api.cpp) and the gfx950
+// kernels (pl_kernels.hip).  Not part of the public ABI.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace plk {
+
+constexpr int kMaxPd = 8;          // feature dimensions the build/neighbour kernels are instantiated for
+constexpr int kMaxSpatialDims = 8;
+constexpr uint64_t kEmptyCell = ~0ull;
+
+// bits of Counters::flags
+enum : int {
+    kFlagTableFull = 1,   // a probe sequence wrapped, or more than cells/2 vertices were created
+    kFlagKeyRange = 2,    // a lattice coordinate does not fit its field of the packed key
+};
+
+struct Counters {
+    int num_vertices;
+    int flags;
+};
+
+struct ScaleFactor {
+    float v[kMaxPd];
+};
+
+struct SpatialDims {
+    int v[kMaxSpatialDims];
+};
+
+// Bits per lattice coordinate in the packed 64-bit key, and the coordinate range that fits.
+int key_field_bits(int pd);
+
+// Hash cells := empty, counters := 0.
+hipError_t clear_table(uint64_t *cell_keys, uint32_t n_cells, Counters *counters, hipStream_t s);
+
+// Stage 1+2: per point embed, enclosing simplex, barycentric weights, then insertion of the pd+1
+// vertex keys.  replay_index[r*N+n] := hash cell of vertex r of point n, replay_weight likewise.
+// Winners of a cell draw a dense vertex index, publish it in cell_vertex and store the packed key
+// in vertex_keys.
+hipError_t build(int pd, const float *positions, int N, const ScaleFactor &scale,
+                 uint64_t *cell_keys, int *cell_vertex, uint32_t n_cells, uint64_t *vertex_keys,
+                 Counters *counters, int *replay_index, float *replay_weight, hipStream_t s);
+
+// neighbours[a*M+v] := vertex indices of v's two neighbours along blur axis a (-1 = absent).
+hipError_t neighbours(int pd, const uint64_t *vertex_keys, int M, const uint64_t *cell_keys,
+                      const int *cell_vertex, uint32_t n_cells, int2 *neighbours, hipStream_t s);
+
+hipError_t fill_zero(float *p, size_t n, hipStream_t s);
+
+// Stage 3.  in_channels is vd-1 (the homogeneous channel is the bare weight) or vd.
+// cell_vertex != nullptr: replay_index still holds hash cells; they are translated to vertex
+// indices and written back.
+hipError_t splat(int pd, int vd, int N, const float *input, int in_channels, int *replay_index,
+                 const float *replay_weight, const int *cell_vertex, float *values, hipStream_t s);
+
+// Stage 4, one axis: dst[v] = 1/4 src[n1] + 1/2 src[v] + 1/4 src[n2].
+hipError_t blur_axis(int vd, int M, const float *src, float *dst, const int2 *neighbours_of_axis,
+                     hipStream_t s);
+
+// Stage 5.  normalize: divide by the homogeneous channel and write vd-1 channels; else write vd.
+hipError_t slice(int pd, int vd, int N, const int *replay_index, const float *replay_weight,
+                 const float *values, float *output, int normalize, hipStream_t s);
+
+hipError_t debug_simplex(int pd, const float *positions, int N, const ScaleFactor &scale,
+                         short *rem0, short *rank, short *keys, float *barycentric, hipStream_t s);
+
+hipError_t export_keys(int pd, const uint64_t *vertex_keys, int M, short *keys, hipStream_t s);
+
+hipError_t compute_positions(const float *reference, float *positions, int N, int n_ref_channels,
+                             int n_spatial_dims, const SpatialDims &dims, float spatial_std,
+                             float feature_std, hipStream_t s);
+
+}  // namespace plk

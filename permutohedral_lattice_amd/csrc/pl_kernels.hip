@@ -1,0 +1,670 @@
+// gfx950 kernels of the permutohedral-lattice filter.
+//
+// This translation unit must be compiled with -ffp-contract=off: the integer results (nearest
+// lattice point, rank permutation, vertex keys) are only equal to those of the reference CPU path
+// (src/PermutohedralLatticeCPU.h:220-304 of the reference tree) if every float operation of the
+// embedding is a single IEEE operation, and the three double-precision steps are kept in double.
+//
+// Data layout in HBM
+//   cell_keys[n_cells]     u64  open-addressed hash cells holding packed vertex keys (all-ones = empty)
+//   cell_vertex[n_cells]   i32  dense vertex index of the key in the same cell
+//   vertex_keys[M]         u64  packed key of vertex v
+//   neighbours[(pd+1)*M]   int2 per blur axis a and vertex v: indices of v's two neighbours or -1
+//   values[M*vd]           f32  vertex values, two buffers (ping-pong across blur axes)
+//   replay_index[(pd+1)*N] i32  [r][n]: vertex r of point n (hash cell until the first splat)
+//   replay_weight[(pd+1)*N] f32 [r][n]: its barycentric weight
+//
+// Packed key.  Every coordinate of lattice vertex with remainder r is (pd+1)*q_i + r, so a key is
+// (r, q_0..q_{pd-1}): r in bits 60..63, q_i biased into a field of B = min(16, 60/pd) bits.
+#include "pl_kernels.h"
+
+namespace plk {
+
+namespace {
+
+constexpr int kBlock = 256;
+
+template <int PD>
+struct KeyCodec {
+    static constexpr int kBits = (60 / PD) > 16 ? 16 : (60 / PD);
+    static constexpr int kBias = 1 << (kBits - 1);
+    // one step of margin on both sides so that a neighbour's coordinate never leaves its field
+    static constexpr int kMinQ = -kBias + 1;
+    static constexpr int kMaxQ = kBias - 2;
+    static constexpr uint64_t kFieldMask = (1ull << kBits) - 1ull;
+
+    __device__ static uint64_t pack(const int (&q)[PD], int r) {
+        uint64_t k = (uint64_t)(uint32_t)r << 60;
+#pragma unroll
+        for (int i = 0; i < PD; ++i) k |= (uint64_t)(uint32_t)(q[i] + kBias) << (i * kBits);
+        return k;
+    }
+    __device__ static void unpack(uint64_t k, int (&q)[PD], int &r) {
+        r = (int)(k >> 60);
+#pragma unroll
+        for (int i = 0; i < PD; ++i) q[i] = (int)((k >> (i * kBits)) & kFieldMask) - kBias;
+    }
+};
+
+__device__ __forceinline__ uint32_t hash_key(uint64_t k) {
+    uint32_t x = (uint32_t)k ^ ((uint32_t)(k >> 32) * 0x9E3779B1u);
+    x ^= x >> 16;
+    x *= 0x85EBCA6Bu;
+    x ^= x >> 13;
+    x *= 0xC2B2AE35u;
+    x ^= x >> 16;
+    return x;
+}
+
+// ------------------------------------------------------------------------------------------------
+// Per-point arithmetic: same operations, in the same precision and order, as
+// embed_position_vector / find_enclosing_simplex / compute_barycentric_coordinates of the
+// reference CPU path.  q[i] is rem0[i] / (pd+1).
+// ------------------------------------------------------------------------------------------------
+template <int PD>
+struct Simplex {
+    int q[PD + 1];
+    int rank[PD + 1];
+    float weight[PD + 1];
+};
+
+template <int PD>
+__device__ __forceinline__ void enclosing_simplex(const float (&pos)[PD], const ScaleFactor &scale,
+                                                  Simplex<PD> &s) {
+    constexpr int D1 = PD + 1;
+    const double inv_d1 = 1.0 / (double)D1;
+
+    // elevate onto the hyperplane sum(x) = 0 (float, unfused)
+    float el[D1];
+    float running = 0.0f;
+#pragma unroll
+    for (int i = PD; i >= 1; --i) {
+        const float c = pos[i - 1] * scale.v[i - 1];
+        const float ic = (float)i * c;
+        el[i] = running - ic;
+        running = running + c;
+    }
+    el[0] = running;
+
+    // nearest remainder-0 point: round each coordinate to a multiple of pd+1, ties go down
+    float rem[D1];
+    int qsum = 0;
+#pragma unroll
+    for (int i = 0; i < D1; ++i) {
+        const float v = (float)((double)el[i] * inv_d1);
+        const float cu = ceilf(v), fl = floorf(v);
+        const float above = cu * (float)D1, below = fl * (float)D1;
+        const bool up = (above - el[i]) < (el[i] - below);
+        rem[i] = up ? above : below;
+        s.q[i] = (int)(up ? cu : fl);
+        qsum += s.q[i];
+    }
+
+    // rank[i] = number of coordinates with a larger residual; the pairwise i<j comparison with a
+    // strict < decides ties exactly as the sequential loop does
+    float d[D1];
+#pragma unroll
+    for (int i = 0; i < D1; ++i) d[i] = el[i] - rem[i];
+#pragma unroll
+    for (int i = 0; i < D1; ++i) {
+        int rk = 0;
+#pragma unroll
+        for (int j = 0; j < D1; ++j) {
+            if (j > i) rk += (d[i] < d[j]) ? 1 : 0;
+            if (j < i) rk += (d[j] < d[i]) ? 0 : 1;
+        }
+        s.rank[i] = rk;
+    }
+
+    // the rounded point is qsum steps off the plane: rotate the ranks, wrap the coordinates
+#pragma unroll
+    for (int i = 0; i < D1; ++i) {
+        int rk = s.rank[i] + qsum;
+        if (rk < 0) {
+            rk += D1;
+            s.q[i] += 1;
+            rem[i] += (float)D1;
+        } else if (rk > PD) {
+            rk -= D1;
+            s.q[i] -= 1;
+            rem[i] -= (float)D1;
+        }
+        s.rank[i] = rk;
+    }
+
+    // barycentric weights.  by_rank[k] is the scaled residual of the coordinate of rank k; the
+    // reference's scatter b[pd-rank] += delta, b[pd-rank+1] -= delta gives
+    // b[k] = by_rank[pd-k] - by_rank[pd-k+1] with one rounding, in either order of the two updates.
+    float by_rank[D1];
+#pragma unroll
+    for (int k = 0; k < D1; ++k) by_rank[k] = 0.0f;
+#pragma unroll
+    for (int i = 0; i < D1; ++i) {
+        const float delta = (float)((double)(el[i] - rem[i]) * inv_d1);
+#pragma unroll
+        for (int k = 0; k < D1; ++k) by_rank[k] = (s.rank[i] == k) ? delta : by_rank[k];
+    }
+#pragma unroll
+    for (int k = 1; k < D1; ++k) s.weight[k] = by_rank[PD - k] - by_rank[PD - k + 1];
+    s.weight[0] = (float)((double)by_rank[PD] + (1.0 + (double)(-by_rank[0])));
+}
+
+// q-coordinates of simplex vertex r: the coordinates ranked above pd-r drop by one step
+template <int PD>
+__device__ __forceinline__ void vertex_q(const Simplex<PD> &s, int r, int (&q)[PD]) {
+#pragma unroll
+    for (int i = 0; i < PD; ++i) q[i] = s.q[i] - ((s.rank[i] > PD - r) ? 1 : 0);
+}
+
+template <int PD>
+__device__ __forceinline__ bool simplex_in_key_range(const Simplex<PD> &s) {
+    bool ok = true;
+#pragma unroll
+    for (int i = 0; i < PD; ++i)
+        ok = ok && (s.q[i] - 1 >= KeyCodec<PD>::kMinQ) && (s.q[i] <= KeyCodec<PD>::kMaxQ);
+    return ok;
+}
+
+template <int PD>
+__device__ __forceinline__ void load_position(const float *positions, int n, float (&pos)[PD]) {
+    const float *row = positions + (size_t)n * PD;
+#pragma unroll
+    for (int i = 0; i < PD; ++i) pos[i] = row[i];
+}
+
+// ------------------------------------------------------------------------------------------------
+// Hash table
+// ------------------------------------------------------------------------------------------------
+
+// Returns the cell holding `key`, inserting it if absent; -1 and kFlagTableFull when no cell is
+// free.  Cells only ever change from empty to a key, so a stale read can at worst see "empty" and
+// the compare-and-swap then returns the truth.
+__device__ __forceinline__ int table_insert(uint64_t *cell_keys, int *cell_vertex, uint32_t mask,
+                                            uint64_t *vertex_keys, Counters *counters, uint64_t key) {
+    uint32_t h = hash_key(key) & mask;
+    for (uint32_t probe = 0; probe <= mask; ++probe) {
+        uint64_t cur = cell_keys[h];
+        if (cur == kEmptyCell) {
+            cur = atomicCAS((unsigned long long *)(cell_keys + h), (unsigned long long)kEmptyCell,
+                            (unsigned long long)key);
+            if (cur == kEmptyCell) {
+                // this lane created the vertex: draw its dense index
+                const int v = atomicAdd(&counters->num_vertices, 1);
+                if ((uint32_t)v < (mask + 1u) / 2u) {
+                    vertex_keys[v] = key;
+                    cell_vertex[h] = v;
+                } else {
+                    atomicOr(&counters->flags, kFlagTableFull);
+                    cell_vertex[h] = 0;
+                }
+                return (int)h;
+            }
+        }
+        if (cur == key) return (int)h;
+        h = (h + 1u) & mask;
+    }
+    atomicOr(&counters->flags, kFlagTableFull);
+    return -1;
+}
+
+__device__ __forceinline__ int table_find(const uint64_t *cell_keys, const int *cell_vertex,
+                                          uint32_t mask, uint64_t key) {
+    uint32_t h = hash_key(key) & mask;
+    for (uint32_t probe = 0; probe <= mask; ++probe) {
+        const uint64_t cur = cell_keys[h];
+        if (cur == key) return cell_vertex[h];
+        if (cur == kEmptyCell) return -1;
+        h = (h + 1u) & mask;
+    }
+    return -1;
+}
+
+__global__ __launch_bounds__(kBlock) void k_clear_table(uint64_t *cell_keys, uint32_t n_cells,
+                                                         Counters *counters) {
+    const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
+    if (i < n_cells) cell_keys[i] = kEmptyCell;
+    if (i == 0) {
+        counters->num_vertices = 0;
+        counters->flags = 0;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Stage 1+2: embed, simplex, insert
+// ------------------------------------------------------------------------------------------------
+template <int PD>
+__global__ __launch_bounds__(kBlock) void k_build(const float *__restrict__ positions, int N,
+                                                   ScaleFactor scale, uint64_t *cell_keys,
+                                                   int *cell_vertex, uint32_t mask,
+                                                   uint64_t *vertex_keys, Counters *counters,
+                                                   int *__restrict__ replay_index,
+                                                   float *__restrict__ replay_weight) {
+    const int n = blockIdx.x * kBlock + threadIdx.x;
+    const int lane = threadIdx.x & 63;
+    const bool valid = n < N;
+
+    float pos[PD];
+#pragma unroll
+    for (int i = 0; i < PD; ++i) pos[i] = 0.0f;
+    if (valid) load_position<PD>(positions, n, pos);
+
+    Simplex<PD> s;
+    enclosing_simplex<PD>(pos, scale, s);
+
+    const bool in_range = simplex_in_key_range<PD>(s);
+    if (valid && !in_range) atomicOr(&counters->flags, kFlagKeyRange);
+    const bool active = valid && in_range;
+
+#pragma unroll 1
+    for (int r = 0; r <= PD; ++r) {
+        int q[PD];
+        vertex_q<PD>(s, r, q);
+        const uint64_t key = KeyCodec<PD>::pack(q, r);
+
+        // Wavefront-level deduplication: neighbouring points mostly share vertices, so each
+        // distinct key of the wave is inserted by one lane (the lowest that holds it) and the cell
+        // is broadcast to the others.  Only the leaders touch the table.
+        int leader = lane;
+        uint64_t remaining = __ballot(active);
+        while (remaining) {
+            const int first = __builtin_ctzll(remaining);
+            const uint64_t k = __shfl(key, first);
+            const bool same = active && key == k;
+            if (same) leader = first;
+            remaining &= ~__ballot(same);
+        }
+
+        int cell = -1;
+        if (active && leader == lane)
+            cell = table_insert(cell_keys, cell_vertex, mask, vertex_keys, counters, key);
+        cell = __shfl(cell, leader);
+
+        if (valid) {
+            replay_index[(size_t)r * N + n] = active ? cell : -1;
+            replay_weight[(size_t)r * N + n] = s.weight[r];
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Neighbour table: along axis a the neighbours of key k are k + (1,..,1) - (pd+1) e_a and its
+// mirror image (reference: src/PermutohedralLatticeCPU.h:381-388).  In (r, q) form the first is
+// r+1 with q_a-1, or, when r = pd, r = 0 with every q but q_a one higher; axis pd is the implicit
+// last coordinate, which no stored q belongs to.
+// ------------------------------------------------------------------------------------------------
+template <int PD>
+__global__ __launch_bounds__(kBlock) void k_neighbours(const uint64_t *__restrict__ vertex_keys,
+                                                        int M, const uint64_t *__restrict__ cell_keys,
+                                                        const int *__restrict__ cell_vertex,
+                                                        uint32_t mask, int2 *__restrict__ out) {
+    const size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (t >= (size_t)M * (PD + 1)) return;
+    const int a = (int)(t / (size_t)M);
+    const int v = (int)(t - (size_t)a * M);
+
+    int q[PD], r;
+    KeyCodec<PD>::unpack(vertex_keys[v], q, r);
+
+    int qp[PD], qm[PD];
+    const bool wrap_up = (r == PD), wrap_down = (r == 0);
+#pragma unroll
+    for (int i = 0; i < PD; ++i) {
+        const bool on_axis = (i == a);
+        qp[i] = q[i] + (wrap_up ? (on_axis ? 0 : 1) : (on_axis ? -1 : 0));
+        qm[i] = q[i] + (wrap_down ? (on_axis ? 0 : -1) : (on_axis ? 1 : 0));
+    }
+    const uint64_t kp = KeyCodec<PD>::pack(qp, wrap_up ? 0 : r + 1);
+    const uint64_t km = KeyCodec<PD>::pack(qm, wrap_down ? PD : r - 1);
+    out[t] = make_int2(table_find(cell_keys, cell_vertex, mask, kp),
+                       table_find(cell_keys, cell_vertex, mask, km));
+}
+
+__global__ __launch_bounds__(kBlock) void k_fill_zero(float *p, size_t n) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i < n) p[i] = 0.0f;
+}
+
+// ------------------------------------------------------------------------------------------------
+// Stage 3: splat
+// ------------------------------------------------------------------------------------------------
+
+// One thread per point, channels in registers (small vd).
+template <int VD>
+__global__ __launch_bounds__(kBlock) void k_splat_point(int d1, int N, const float *__restrict__ input,
+                                                         int in_channels, int *replay_index,
+                                                         const float *__restrict__ replay_weight,
+                                                         const int *__restrict__ cell_vertex,
+                                                         float *values) {
+    const int n = blockIdx.x * kBlock + threadIdx.x;
+    if (n >= N) return;
+    float val[VD];
+#pragma unroll
+    for (int j = 0; j < VD; ++j) val[j] = 1.0f;  // homogeneous channel when only vd-1 are given
+#pragma unroll
+    for (int j = 0; j < VD; ++j)
+        if (j < in_channels) val[j] = input[(size_t)n * in_channels + j];
+
+    for (int r = 0; r < d1; ++r) {
+        int v = replay_index[(size_t)r * N + n];
+        if (v < 0) continue;
+        if (cell_vertex) {
+            v = cell_vertex[v];
+            replay_index[(size_t)r * N + n] = v;
+        }
+        const float w = replay_weight[(size_t)r * N + n];
+        float *dst = values + (size_t)v * VD;
+#pragma unroll
+        for (int j = 0; j < VD; ++j) atomicAdd(dst + j, w * val[j]);
+    }
+}
+
+// One thread per (point, channel): consecutive lanes add to consecutive floats of one vertex.
+__global__ __launch_bounds__(kBlock) void k_splat_channel(int d1, int vd, int N,
+                                                           const float *__restrict__ input,
+                                                           int in_channels, int *replay_index,
+                                                           const float *__restrict__ replay_weight,
+                                                           const int *__restrict__ cell_vertex,
+                                                           float *values) {
+    const size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (t >= (size_t)N * vd) return;
+    const int n = (int)(t / (size_t)vd);
+    const int j = (int)(t - (size_t)n * vd);
+    const float val = (j < in_channels) ? input[(size_t)n * in_channels + j] : 1.0f;
+    for (int r = 0; r < d1; ++r) {
+        int v = replay_index[(size_t)r * N + n];
+        if (v < 0) continue;
+        if (cell_vertex) v = cell_vertex[v];
+        const float w = replay_weight[(size_t)r * N + n];
+        atomicAdd(values + (size_t)v * vd + j, w * val);
+    }
+}
+
+// cells -> vertex indices, for the per-channel splat (which cannot write back race-free itself)
+__global__ __launch_bounds__(kBlock) void k_remap_replay(size_t rows, int *replay_index,
+                                                          const int *__restrict__ cell_vertex) {
+    const size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (t >= rows) return;
+    const int c = replay_index[t];
+    if (c >= 0) replay_index[t] = cell_vertex[c];
+}
+
+// ------------------------------------------------------------------------------------------------
+// Stage 4: blur along one axis (reference: src/PermutohedralLatticeCPU.h:403-405, evaluated in
+// double and rounded once, as there)
+// ------------------------------------------------------------------------------------------------
+template <int VD>
+__global__ __launch_bounds__(kBlock) void k_blur(int vd_runtime, int M, const float *__restrict__ src,
+                                                  float *__restrict__ dst,
+                                                  const int2 *__restrict__ nbr) {
+    const int vd = VD ? VD : vd_runtime;
+    const size_t e = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (e >= (size_t)M * vd) return;
+    const int v = (int)(e / (size_t)vd);
+    const int j = (int)(e - (size_t)v * vd);
+    const int2 nb = nbr[v];
+    const double a = nb.x >= 0 ? (double)src[(size_t)nb.x * vd + j] : 0.0;
+    const double b = nb.y >= 0 ? (double)src[(size_t)nb.y * vd + j] : 0.0;
+    dst[e] = (float)(0.25 * a + 0.5 * (double)src[e] + 0.25 * b);
+}
+
+// ------------------------------------------------------------------------------------------------
+// Stage 5: slice (reference: src/PermutohedralLatticeCPU.h:333-352)
+// ------------------------------------------------------------------------------------------------
+template <int VD>
+__global__ __launch_bounds__(kBlock) void k_slice_point(int d1, int N,
+                                                         const int *__restrict__ replay_index,
+                                                         const float *__restrict__ replay_weight,
+                                                         const float *__restrict__ values,
+                                                         float *__restrict__ output, int normalize) {
+    const int n = blockIdx.x * kBlock + threadIdx.x;
+    if (n >= N) return;
+    float acc[VD];
+#pragma unroll
+    for (int j = 0; j < VD; ++j) acc[j] = 0.0f;
+    for (int r = 0; r < d1; ++r) {
+        const int v = replay_index[(size_t)r * N + n];
+        if (v < 0) continue;
+        const float w = replay_weight[(size_t)r * N + n];
+        const float *src = values + (size_t)v * VD;
+#pragma unroll
+        for (int j = 0; j < VD; ++j) acc[j] += w * src[j];
+    }
+    if (normalize) {
+        const float scale = (float)(1.0 / (double)acc[VD - 1]);
+#pragma unroll
+        for (int j = 0; j < VD - 1; ++j) output[(size_t)n * (VD - 1) + j] = acc[j] * scale;
+    } else {
+#pragma unroll
+        for (int j = 0; j < VD; ++j) output[(size_t)n * VD + j] = acc[j];
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void k_slice_channel(int d1, int vd, int N,
+                                                           const int *__restrict__ replay_index,
+                                                           const float *__restrict__ replay_weight,
+                                                           const float *__restrict__ values,
+                                                           float *__restrict__ output, int normalize) {
+    const int out_ch = normalize ? vd - 1 : vd;
+    const size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (t >= (size_t)N * out_ch) return;
+    const int n = (int)(t / (size_t)out_ch);
+    const int j = (int)(t - (size_t)n * out_ch);
+    float acc = 0.0f, hom = 0.0f;
+    for (int r = 0; r < d1; ++r) {
+        const int v = replay_index[(size_t)r * N + n];
+        if (v < 0) continue;
+        const float w = replay_weight[(size_t)r * N + n];
+        const float *src = values + (size_t)v * vd;
+        acc += w * src[j];
+        hom += w * src[vd - 1];
+    }
+    if (normalize) {
+        const float scale = (float)(1.0 / (double)hom);
+        output[t] = acc * scale;
+    } else {
+        output[t] = acc;
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Debug exports and the feature builder
+// ------------------------------------------------------------------------------------------------
+template <int PD>
+__global__ __launch_bounds__(kBlock) void k_debug_simplex(const float *__restrict__ positions, int N,
+                                                           ScaleFactor scale, short *rem0, short *rank,
+                                                           short *keys, float *barycentric) {
+    constexpr int D1 = PD + 1;
+    const int n = blockIdx.x * kBlock + threadIdx.x;
+    if (n >= N) return;
+    float pos[PD];
+    load_position<PD>(positions, n, pos);
+    Simplex<PD> s;
+    enclosing_simplex<PD>(pos, scale, s);
+#pragma unroll
+    for (int i = 0; i < D1; ++i) {
+        if (rem0) rem0[(size_t)n * D1 + i] = (short)(s.q[i] * D1);
+        if (rank) rank[(size_t)n * D1 + i] = (short)s.rank[i];
+        if (barycentric) barycentric[(size_t)n * D1 + i] = s.weight[i];
+    }
+    if (keys) {
+#pragma unroll
+        for (int r = 0; r < D1; ++r) {
+            int q[PD];
+            vertex_q<PD>(s, r, q);
+#pragma unroll
+            for (int i = 0; i < PD; ++i)
+                keys[((size_t)n * D1 + r) * PD + i] = (short)(q[i] * D1 + r);
+        }
+    }
+}
+
+template <int PD>
+__global__ __launch_bounds__(kBlock) void k_export_keys(const uint64_t *__restrict__ vertex_keys,
+                                                         int M, short *keys) {
+    const int v = blockIdx.x * kBlock + threadIdx.x;
+    if (v >= M) return;
+    int q[PD], r;
+    KeyCodec<PD>::unpack(vertex_keys[v], q, r);
+#pragma unroll
+    for (int i = 0; i < PD; ++i) keys[(size_t)v * PD + i] = (short)(q[i] * (PD + 1) + r);
+}
+
+// reference: src/PermutohedralLatticeCPU.h:464-473 (IEEE float division, int -> float exact)
+__global__ __launch_bounds__(kBlock) void k_positions(const float *__restrict__ reference,
+                                                       float *__restrict__ positions, int N, int rc,
+                                                       int nsd, SpatialDims dims, float spatial_std,
+                                                       float feature_std) {
+    const int n = blockIdx.x * kBlock + threadIdx.x;
+    if (n >= N) return;
+    const int pd = nsd + rc;
+    float *row = positions + (size_t)n * pd;
+    int stride = 1;
+    for (int s = nsd - 1; s >= 0; --s) {
+        const int coord = (n / stride) % dims.v[s];
+        row[s] = (float)coord / spatial_std;
+        stride *= dims.v[s];
+    }
+    for (int c = 0; c < rc; ++c) row[nsd + c] = reference[(size_t)n * rc + c] / feature_std;
+}
+
+inline unsigned blocks_for(size_t n) { return (unsigned)((n + kBlock - 1) / kBlock); }
+
+#define PLK_DISPATCH_PD(pd, CALL)                 \
+    switch (pd) {                                 \
+        case 1: { constexpr int PD = 1; CALL; } break; \
+        case 2: { constexpr int PD = 2; CALL; } break; \
+        case 3: { constexpr int PD = 3; CALL; } break; \
+        case 4: { constexpr int PD = 4; CALL; } break; \
+        case 5: { constexpr int PD = 5; CALL; } break; \
+        case 6: { constexpr int PD = 6; CALL; } break; \
+        case 7: { constexpr int PD = 7; CALL; } break; \
+        case 8: { constexpr int PD = 8; CALL; } break; \
+        default: return hipErrorInvalidValue;     \
+    }
+
+}  // namespace
+
+int key_field_bits(int pd) {
+    if (pd < 1 || pd > kMaxPd) return 0;
+    const int b = 60 / pd;
+    return b > 16 ? 16 : b;
+}
+
+hipError_t clear_table(uint64_t *cell_keys, uint32_t n_cells, Counters *counters, hipStream_t s) {
+    hipLaunchKernelGGL(k_clear_table, dim3(blocks_for(n_cells)), dim3(kBlock), 0, s, cell_keys,
+                       n_cells, counters);
+    return hipGetLastError();
+}
+
+hipError_t build(int pd, const float *positions, int N, const ScaleFactor &scale,
+                 uint64_t *cell_keys, int *cell_vertex, uint32_t n_cells, uint64_t *vertex_keys,
+                 Counters *counters, int *replay_index, float *replay_weight, hipStream_t s) {
+    if (N <= 0) return hipSuccess;
+    PLK_DISPATCH_PD(pd, hipLaunchKernelGGL(k_build<PD>, dim3(blocks_for((size_t)N)), dim3(kBlock), 0,
+                                           s, positions, N, scale, cell_keys, cell_vertex,
+                                           n_cells - 1u, vertex_keys, counters, replay_index,
+                                           replay_weight));
+    return hipGetLastError();
+}
+
+hipError_t neighbours(int pd, const uint64_t *vertex_keys, int M, const uint64_t *cell_keys,
+                      const int *cell_vertex, uint32_t n_cells, int2 *out, hipStream_t s) {
+    if (M <= 0) return hipSuccess;
+    PLK_DISPATCH_PD(pd, hipLaunchKernelGGL(k_neighbours<PD>, dim3(blocks_for((size_t)M * (PD + 1))),
+                                           dim3(kBlock), 0, s, vertex_keys, M, cell_keys,
+                                           cell_vertex, n_cells - 1u, out));
+    return hipGetLastError();
+}
+
+hipError_t fill_zero(float *p, size_t n, hipStream_t s) {
+    if (n == 0) return hipSuccess;
+    hipLaunchKernelGGL(k_fill_zero, dim3(blocks_for(n)), dim3(kBlock), 0, s, p, n);
+    return hipGetLastError();
+}
+
+hipError_t splat(int pd, int vd, int N, const float *input, int in_channels, int *replay_index,
+                 const float *replay_weight, const int *cell_vertex, float *values, hipStream_t s) {
+    if (N <= 0) return hipSuccess;
+    const int d1 = pd + 1;
+    const dim3 grid(blocks_for((size_t)N)), block(kBlock);
+#define PLK_SPLAT(VD)                                                                             \
+    case VD:                                                                                      \
+        hipLaunchKernelGGL(k_splat_point<VD>, grid, block, 0, s, d1, N, input, in_channels,       \
+                           replay_index, replay_weight, cell_vertex, values);                     \
+        break;
+    switch (vd) {
+        PLK_SPLAT(2) PLK_SPLAT(3) PLK_SPLAT(4) PLK_SPLAT(5) PLK_SPLAT(6) PLK_SPLAT(7) PLK_SPLAT(8)
+        default:
+            if (cell_vertex) {
+                const size_t rows = (size_t)N * d1;
+                hipLaunchKernelGGL(k_remap_replay, dim3(blocks_for(rows)), block, 0, s, rows,
+                                   replay_index, cell_vertex);
+            }
+            hipLaunchKernelGGL(k_splat_channel, dim3(blocks_for((size_t)N * vd)), block, 0, s, d1, vd,
+                               N, input, in_channels, replay_index, replay_weight,
+                               (const int *)nullptr, values);
+            break;
+    }
+#undef PLK_SPLAT
+    return hipGetLastError();
+}
+
+hipError_t blur_axis(int vd, int M, const float *src, float *dst, const int2 *nbr, hipStream_t s) {
+    if (M <= 0) return hipSuccess;
+    const dim3 grid(blocks_for((size_t)M * vd)), block(kBlock);
+    switch (vd) {
+        case 2: hipLaunchKernelGGL(k_blur<2>, grid, block, 0, s, vd, M, src, dst, nbr); break;
+        case 4: hipLaunchKernelGGL(k_blur<4>, grid, block, 0, s, vd, M, src, dst, nbr); break;
+        default: hipLaunchKernelGGL(k_blur<0>, grid, block, 0, s, vd, M, src, dst, nbr); break;
+    }
+    return hipGetLastError();
+}
+
+hipError_t slice(int pd, int vd, int N, const int *replay_index, const float *replay_weight,
+                 const float *values, float *output, int normalize, hipStream_t s) {
+    if (N <= 0) return hipSuccess;
+    const int d1 = pd + 1;
+    const dim3 grid(blocks_for((size_t)N)), block(kBlock);
+#define PLK_SLICE(VD)                                                                          \
+    case VD:                                                                                   \
+        hipLaunchKernelGGL(k_slice_point<VD>, grid, block, 0, s, d1, N, replay_index,          \
+                           replay_weight, values, output, normalize);                          \
+        break;
+    switch (vd) {
+        PLK_SLICE(2) PLK_SLICE(3) PLK_SLICE(4) PLK_SLICE(5) PLK_SLICE(6) PLK_SLICE(7) PLK_SLICE(8)
+        default: {
+            const int out_ch = normalize ? vd - 1 : vd;
+            hipLaunchKernelGGL(k_slice_channel, dim3(blocks_for((size_t)N * out_ch)), block, 0, s, d1,
+                               vd, N, replay_index, replay_weight, values, output, normalize);
+        } break;
+    }
+#undef PLK_SLICE
+    return hipGetLastError();
+}
+
+hipError_t debug_simplex(int pd, const float *positions, int N, const ScaleFactor &scale,
+                         short *rem0, short *rank, short *keys, float *barycentric, hipStream_t s) {
+    if (N <= 0) return hipSuccess;
+    PLK_DISPATCH_PD(pd, hipLaunchKernelGGL(k_debug_simplex<PD>, dim3(blocks_for((size_t)N)),
+                                           dim3(kBlock), 0, s, positions, N, scale, rem0, rank, keys,
+                                           barycentric));
+    return hipGetLastError();
+}
+
+hipError_t export_keys(int pd, const uint64_t *vertex_keys, int M, short *keys, hipStream_t s) {
+    if (M <= 0) return hipSuccess;
+    PLK_DISPATCH_PD(pd, hipLaunchKernelGGL(k_export_keys<PD>, dim3(blocks_for((size_t)M)),
+                                           dim3(kBlock), 0, s, vertex_keys, M, keys));
+    return hipGetLastError();
+}
+
+hipError_t compute_positions(const float *reference, float *positions, int N, int n_ref_channels,
+                             int n_spatial_dims, const SpatialDims &dims, float spatial_std,
+                             float feature_std, hipStream_t s) {
+    if (N <= 0) return hipSuccess;
+    hipLaunchKernelGGL(k_positions, dim3(blocks_for((size_t)N)), dim3(kBlock), 0, s, reference,
+                       positions, N, n_ref_channels, n_spatial_dims, dims, spatial_std, feature_std);
+    return hipGetLastError();
+}
+
+}  // namespace plk

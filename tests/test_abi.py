@@ -1,0 +1,91 @@
+"""Host-side checks that need no GPU: the C-ABI library loads, exports exactly what the header
+declares, and rejects bad arguments with status codes before touching the device."""
+import ctypes as C
+import os
+import re
+
+import pytest
+
+from conftest import ROOT
+
+import permutohedral_lattice_amd as pla
+
+
+def _declared_functions():
+    text = open(os.path.join(ROOT, "include", "permutohedral_lattice.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(pl_[a-z_0-9]+)\s*\(", text)))
+
+
+def test_library_is_in_tree_and_exports_every_declared_symbol():
+    assert os.path.dirname(pla.LIB_PATH) == os.path.join(ROOT, "permutohedral_lattice_amd")
+    declared = _declared_functions()
+    assert declared == sorted(pla.EXPORTS)
+    lib = C.CDLL(pla.LIB_PATH)
+    for name in declared:
+        assert getattr(lib, name) is not None
+
+
+def test_supported_dimensions():
+    for pd in range(1, 9):
+        for vd in (2, 3, 4, 5, 8, 9, 22, 64):
+            assert pla.supported(pd, vd)
+    assert not pla.supported(0, 4)
+    assert not pla.supported(9, 4)
+    assert not pla.supported(5, 1)
+
+
+def test_strerror_covers_every_status():
+    seen = set()
+    for code in range(0, -7, -1):
+        msg = pla._lib.pl_strerror(code).decode()
+        assert msg and msg != "unknown status"
+        seen.add(msg)
+    assert len(seen) == 7
+    assert pla._lib.pl_strerror(-99).decode() == "unknown status"
+
+
+@pytest.mark.parametrize("pd,vd,n,expect", [
+    (5, 4, -1, pla.PL_EINVAL),
+    (0, 4, 10, pla.PL_EINVAL),
+    (5, 1, 10, pla.PL_EINVAL),
+    (9, 4, 10, pla.PL_EUNSUPPORTED),
+    (5, 4, 2 ** 30, pla.PL_EOVERFLOW),      # N*(pd+1) replay rows beyond the supported range
+])
+def test_create_rejects_bad_arguments_without_a_device(pd, vd, n, expect):
+    h = C.c_void_p()
+    assert pla._lib.pl_create(pd, vd, n, None, None, C.byref(h)) == expect
+    assert not h.value
+    assert pla._lib.pl_create(5, 4, 10, None, None, None) == pla.PL_EINVAL
+
+
+def test_null_handles_are_rejected():
+    lib = pla._lib
+    assert lib.pl_filter(None, None, None, None, 0) == pla.PL_EINVAL
+    assert lib.pl_build(None, None) == pla.PL_EINVAL
+    assert lib.pl_apply(None, None, None, 0) == pla.PL_EINVAL
+    assert lib.pl_num_vertices(None, None) == pla.PL_EINVAL
+    assert lib.pl_set_option(None, 1, 0) == pla.PL_EINVAL
+    assert lib.pl_destroy(None) == pla.PL_OK
+
+
+def test_op_and_feature_builder_argument_checks():
+    lib = pla._lib
+    dims = (C.c_int * 2)(8, 8)
+    bad = (C.c_int * 2)(8, 0)
+    # no spatial dims / no channels / non-positive extent
+    assert lib.pl_lattice_filter_op(None, None, None, 1, 0, dims, 3, 3, 1, 1.0, 1.0, 1.0, 0, None, None) == pla.PL_EINVAL
+    assert lib.pl_lattice_filter_op(None, None, None, 1, 2, dims, 0, 3, 1, 1.0, 1.0, 1.0, 0, None, None) == pla.PL_EINVAL
+    assert lib.pl_lattice_filter_op(None, None, None, 1, 2, bad, 3, 3, 1, 1.0, 1.0, 1.0, 0, None, None) == pla.PL_EINVAL
+    # bilateral without a reference image
+    assert lib.pl_lattice_filter_op(None, None, None, 1, 2, dims, 3, 3, 1, 1.0, 1.0, 1.0, 0, None, None) == pla.PL_EINVAL
+    # pd = 2 + 7 reference channels is not instantiated
+    assert lib.pl_lattice_filter_op(None, None, None, 0, 2, dims, 3, 7, 1, 1.0, 1.0, 1.0, 0, None, None) == pla.PL_EUNSUPPORTED
+    # more than INT32_MAX tensor elements, as the reference op refuses
+    big = (C.c_int * 2)(65536, 32768)
+    assert lib.pl_lattice_filter_op(None, None, None, 1, 2, big, 3, 3, 1, 1.0, 1.0, 1.0, 0, None, None) == pla.PL_EOVERFLOW
+    # empty batch is a no-op
+    assert lib.pl_lattice_filter_op(None, None, None, 0, 2, dims, 3, 3, 1, 1.0, 1.0, 1.0, 0, None, None) == pla.PL_OK
+    assert lib.pl_compute_positions(None, None, -1, 3, 2, dims, 1.0, 1.0, None) == pla.PL_EINVAL
+    assert lib.pl_compute_positions(None, None, 0, 3, 2, dims, 1.0, 1.0, None) == pla.PL_OK
+    assert lib.pl_compute_positions(None, None, 64, 3, 2, dims, 1.0, 1.0, None) == pla.PL_EINVAL

@@ -1,0 +1,378 @@
+"""Parity of the HIP library (through its C ABI) with the CPU oracle and the golden fixtures.
+
+Integers (rem0, rank, per-point keys, vertex count, key set) must be bit-equal; filter outputs
+within max|d| <= 1e-3 (data in [0,1]) and relative L2 <= 1e-4 -- the tolerances are in conftest.
+"""
+import numpy as np
+import pytest
+import torch
+
+from conftest import (MAX_ABS_TOL, REL_L2_TOL, bits, golden_lattice_cases, load_golden, rel_l2,
+                      sorted_keys)
+from permutohedral_lattice_amd import synth
+
+import oracle
+import permutohedral_lattice_amd as pla
+
+pytestmark = pytest.mark.gpu
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    return t.detach().cpu().numpy()
+
+
+def gpu_filter(pd, vd, positions, values, reverse=False, lattice=None):
+    n = positions.shape[0]
+    lat = lattice or pla.PermutohedralLattice(pd, vd, n)
+    out = torch.empty((n, vd - 1), dtype=torch.float32, device="cuda")
+    lat.filter(out, dev(values), dev(positions), reverse)
+    torch.cuda.synchronize()
+    return host(out), lat
+
+
+def assert_float_parity(got, want, scale=1.0):
+    assert np.isfinite(got).all()
+    assert np.abs(got - want).max() <= MAX_ABS_TOL * scale
+    assert rel_l2(got, want) <= REL_L2_TOL
+
+
+def check_integers(pd, positions, lat=None):
+    n = positions.shape[0]
+    lat = lat or pla.PermutohedralLattice(pd, 2, n)
+    d = {k: host(v) for k, v in lat.debug_simplex(dev(positions)).items()}
+    o = oracle.dump_simplex(positions)
+    assert (d["rem0"] == o["rem0"]).all()
+    assert (d["rank"] == o["rank"]).all()
+    assert (d["keys"] == o["keys"]).all()
+    # the weights follow the same operations in the same order: bit-equal as well
+    assert (bits(d["barycentric"]) == bits(o["barycentric"])).all()
+    return o
+
+
+# ---------------------------------------------------------------------------------------------
+# golden fixtures (outputs of the reference's own CPU header)
+# ---------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("name", golden_lattice_cases())
+def test_golden_integers(name):
+    g = load_golden("lattice_" + name)
+    pd = int(g["pd"])
+    n = g["positions"].shape[0]
+    lat = pla.PermutohedralLattice(pd, int(g["vd"]), n)
+    d = {k: host(v) for k, v in lat.debug_simplex(dev(g["positions"])).items()}
+    assert (d["rem0"] == g["rem0"]).all()
+    assert (d["rank"] == g["rank"]).all()
+    assert (d["keys"] == g["keys"]).all()
+    if g["barycentric"].size:
+        assert (bits(d["barycentric"]) == bits(g["barycentric"])).all()
+
+
+@pytest.mark.parametrize("name", golden_lattice_cases())
+def test_golden_filter(name):
+    g = load_golden("lattice_" + name)
+    pd, vd = int(g["pd"]), int(g["vd"])
+    out_f, lat = gpu_filter(pd, vd, g["positions"], g["values"], False)
+    # vertex count and key set: one vertex per distinct key (the reference's list may repeat a
+    # key once per doubling of its index; the fixture keeps that list as the reference made it)
+    distinct = np.unique(g["vertex_keys"], axis=0)
+    assert lat.num_vertices == len(distinct)
+    assert (sorted_keys(host(lat.debug_keys()))[0] == sorted_keys(distinct)[0]).all()
+    assert_float_parity(out_f, g["output_forward"])
+    out_r, _ = gpu_filter(pd, vd, g["positions"], g["values"], True, lattice=lat)
+    assert_float_parity(out_r, g["output_reverse"])
+
+
+# ---------------------------------------------------------------------------------------------
+# the benchmark configurations at sizes the oracle finishes in seconds
+# ---------------------------------------------------------------------------------------------
+
+def _config_case(name):
+    if name == "cfg1_bilateral_rgb":
+        img = synth.blob_image(256, 256, seed=1)
+        return 5, 4, synth.bilateral_positions(img, 8.0, 0.125), img.reshape(-1, 3)
+    if name == "cfg2_spatial":
+        return 2, 2, synth.spatial_positions((512, 512), 8.0), synth.uniform_image((512 * 512, 1), 2)
+    if name == "cfg3_guided_grey":
+        guide = synth.blob_image(256, 256, seed=3)
+        return 5, 2, synth.bilateral_positions(guide, 8.0, 0.125), synth.uniform_image((256 * 256, 1), 4)
+    if name == "cfg4_volume":
+        vol = synth.ellipsoid_volume(32, 64, 64, seed=5)
+        return 4, 2, synth.bilateral_positions(vol, 5.0, 0.1), vol.reshape(-1, 1)
+    if name == "cfg5_crf_bilateral":
+        guide = synth.blob_image(128, 128, seed=6) * 255.0
+        return 5, 22, synth.bilateral_positions(guide, 80.0, 13.0), synth.softmax_logits((128 * 128, 21), 7)
+    if name == "cfg5_crf_spatial":
+        return 2, 22, synth.spatial_positions((128, 128), 3.0), synth.softmax_logits((128 * 128, 21), 7)
+    if name == "odd_size_pd3_vd5":
+        rng = np.random.default_rng(8)
+        return 3, 5, rng.uniform(0, 9, (1000 * 3 + 37, 3)).astype(np.float32), \
+            rng.uniform(0, 1, (3037, 4)).astype(np.float32)
+    if name == "wide_pd6_vd9":
+        rng = np.random.default_rng(9)
+        return 6, 9, rng.uniform(0, 3, (5000, 6)).astype(np.float32), \
+            rng.uniform(0, 1, (5000, 8)).astype(np.float32)
+    raise KeyError(name)
+
+
+CONFIG_CASES = ["cfg1_bilateral_rgb", "cfg2_spatial", "cfg3_guided_grey", "cfg4_volume",
+                "cfg5_crf_bilateral", "cfg5_crf_spatial", "odd_size_pd3_vd5", "wide_pd6_vd9"]
+
+
+@pytest.mark.parametrize("name", CONFIG_CASES)
+def test_config_parity_with_oracle(name):
+    pd, vd, pos, val = _config_case(name)
+    n = pos.shape[0]
+    lat = pla.PermutohedralLattice(pd, vd, n)
+    o = check_integers(pd, pos, lat)
+    cpu = oracle.Lattice(pd, vd, n)
+    want_f = cpu.filter(val, pos, False)
+    got_f, _ = gpu_filter(pd, vd, pos, val, False, lattice=lat)
+    assert lat.num_vertices == cpu.num_vertices == len(np.unique(o["keys"].reshape(-1, pd), axis=0))
+    assert (sorted_keys(host(lat.debug_keys()))[0] == sorted_keys(cpu.keys())[0]).all()
+    assert_float_parity(got_f, want_f)
+    want_r = oracle.Lattice(pd, vd, n).filter(val, pos, True)
+    got_r, _ = gpu_filter(pd, vd, pos, val, True, lattice=lat)
+    assert_float_parity(got_r, want_r)
+    assert np.abs(want_f - want_r).max() > 0  # the two orders are different computations
+
+
+def test_replay_matrix_matches_oracle():
+    """Vertex numbering differs (first touch on the CPU, arbitrary on the GPU), so replay rows are
+    compared through the vertex keys they point at."""
+    pd, vd, pos, val = _config_case("cfg1_bilateral_rgb")
+    n = pos.shape[0]
+    got, lat = gpu_filter(pd, vd, pos, val)
+    vertex, weight = (host(t) for t in lat.debug_replay())
+    keys = host(lat.debug_keys())
+    o = oracle.dump_simplex(pos)
+    assert vertex.min() >= 0 and vertex.max() < lat.num_vertices
+    assert (keys[vertex.T] == o["keys"]).all()          # [N, pd+1, pd]
+    assert (bits(weight.T) == bits(o["barycentric"])).all()
+
+
+def test_gradient_pass_on_normal_upstream_gradient():
+    """cfg3: the backward pass filters an N(0,1) upstream gradient with reverse=True."""
+    guide = synth.blob_image(192, 192, seed=11)
+    pos = synth.bilateral_positions(guide, 8.0, 0.125)
+    grad = synth.normal_image((192 * 192, 1), 12)
+    want = oracle.Lattice(5, 2, 192 * 192).filter(grad, pos, True)
+    got, _ = gpu_filter(5, 2, pos, grad, True)
+    assert_float_parity(got, want, scale=float(np.abs(want).max()))
+
+
+# ---------------------------------------------------------------------------------------------
+# lattice reuse, object semantics, edge cases
+# ---------------------------------------------------------------------------------------------
+
+def test_build_once_apply_many_equals_filter():
+    pd, vd, pos, val = _config_case("cfg3_guided_grey")
+    n = pos.shape[0]
+    lat = pla.PermutohedralLattice(pd, vd, n)
+    lat.build(dev(pos))
+    out = torch.empty((n, 1), dtype=torch.float32, device="cuda")
+    grad = synth.normal_image((n, 1), 13)
+    for values, reverse in ((val, False), (grad, True), (val, True), (val, False)):
+        lat.apply(out, dev(values), reverse)
+        torch.cuda.synchronize()
+        want = oracle.Lattice(pd, vd, n).filter(values, pos, reverse)
+        assert_float_parity(host(out), want, scale=max(1.0, float(np.abs(want).max())))
+
+
+def test_handle_is_reusable_and_each_filter_is_fresh():
+    """The reference object is single-shot; here every filter() behaves as on a new lattice, also
+    when the positions change between calls."""
+    rng = np.random.default_rng(14)
+    n = 5000
+    lat = pla.PermutohedralLattice(3, 3, n)
+    for trial in range(3):
+        pos = rng.uniform(0, 5 + 10 * trial, (n, 3)).astype(np.float32)
+        val = rng.uniform(0, 1, (n, 2)).astype(np.float32)
+        got, _ = gpu_filter(3, 3, pos, val, lattice=lat)
+        cpu = oracle.Lattice(3, 3, n)
+        want = cpu.filter(val, pos)
+        assert lat.num_vertices == cpu.num_vertices
+        assert_float_parity(got, want)
+
+
+def test_apply_before_build_is_an_error():
+    lat = pla.PermutohedralLattice(2, 2, 16)
+    x = torch.zeros((16, 1), device="cuda")
+    with pytest.raises(pla.PermutohedralError) as e:
+        lat.apply(x, x)
+    assert e.value.status == pla.PL_ESTATE
+
+
+@pytest.mark.parametrize("n", [0, 1, 63, 64, 65, 257])
+def test_tiny_and_ragged_sizes(n):
+    rng = np.random.default_rng(n)
+    pos = rng.uniform(0, 3, (n, 4)).astype(np.float32)
+    val = rng.uniform(0, 1, (n, 2)).astype(np.float32)
+    got, lat = gpu_filter(4, 3, pos, val)
+    if n == 0:
+        assert got.shape == (0, 2)
+        return
+    check_integers(4, pos)
+    want = oracle.Lattice(4, 3, n).filter(val, pos)
+    assert_float_parity(got, want)
+
+
+def test_isolated_points_pass_through():
+    """Features so far apart that no two points share a vertex and no vertex has a neighbour:
+    blur only halves every value, and normalisation restores it: out == in."""
+    n = 200
+    pos = (np.arange(n, dtype=np.float32)[:, None] * 50.0 + np.array([[0.3, 0.1]], np.float32))
+    val = np.random.default_rng(15).uniform(0, 1, (n, 3)).astype(np.float32)
+    got, lat = gpu_filter(2, 4, pos, val)
+    assert lat.num_vertices == 3 * n
+    assert np.abs(got - val).max() <= 1e-5
+
+
+def test_hash_table_growth_is_transparent():
+    """Force a table far too small: the build detects the overflow, regrows and reruns."""
+    pd, vd, pos, val = _config_case("cfg1_bilateral_rgb")
+    n = pos.shape[0]
+    lat = pla.PermutohedralLattice(pd, vd, n)
+    lat.set_option(pla.PL_OPT_TABLE_CELLS, 4096)
+    got, _ = gpu_filter(pd, vd, pos, val, lattice=lat)
+    cpu = oracle.Lattice(pd, vd, n)
+    want = cpu.filter(val, pos)
+    assert cpu.num_vertices > 4096 // 2
+    assert lat.num_vertices == cpu.num_vertices
+    assert_float_parity(got, want)
+
+
+def test_all_points_in_one_simplex_collide_on_every_vertex():
+    n = 4096
+    pos = np.tile(np.array([[0.31, 0.12, 0.55, 0.2, 0.4]], np.float32), (n, 1))
+    val = np.random.default_rng(16).uniform(0, 1, (n, 3)).astype(np.float32)
+    got, lat = gpu_filter(5, 4, pos, val)
+    assert lat.num_vertices == 6
+    want = oracle.Lattice(5, 4, n).filter(val, pos)
+    assert_float_parity(got, want)
+    assert np.abs(got - val.mean(axis=0)).max() <= 1e-4
+
+
+def test_coordinates_beyond_the_packed_key_range_are_reported():
+    """pd=5 packs 12 bits per coordinate; positions far outside must fail loudly, not wrap."""
+    n = 256
+    pos = np.full((n, 5), 1.0, np.float32)
+    pos[7, 0] = 30000.0
+    lat = pla.PermutohedralLattice(5, 2, n)
+    out = torch.empty((n, 1), dtype=torch.float32, device="cuda")
+    with pytest.raises(pla.PermutohedralError) as e:
+        lat.filter(out, dev(np.ones((n, 1), np.float32)), dev(pos))
+    assert e.value.status == pla.PL_EOVERFLOW
+    # pd <= 4 holds the full short range of the reference's keys
+    pos4 = np.full((n, 4), 1.0, np.float32)
+    pos4[7, 0] = 5000.0
+    val = np.random.default_rng(17).uniform(0, 1, (n, 1)).astype(np.float32)
+    got, _ = gpu_filter(4, 2, pos4, val)
+    check_integers(4, pos4)
+    assert_float_parity(got, oracle.Lattice(4, 2, n).filter(val, pos4))
+
+
+def test_large_lattice_coordinates_pd5_within_range():
+    rng = np.random.default_rng(18)
+    n = 20000
+    pos = rng.uniform(0, 1, (n, 5)).astype(np.float32) * np.array([[1900, 1400, 8, 8, 8]], np.float32)
+    val = rng.uniform(0, 1, (n, 3)).astype(np.float32)
+    o = check_integers(5, pos)
+    assert np.abs(o["keys"]).max() > 4000
+    got, lat = gpu_filter(5, 4, pos, val)
+    cpu = oracle.Lattice(5, 4, n)
+    want = cpu.filter(val, pos)
+    assert lat.num_vertices == cpu.num_vertices
+    assert_float_parity(got, want)
+
+
+# ---------------------------------------------------------------------------------------------
+# feature builder and the op
+# ---------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("name", ["2d_rgb", "3d_grey", "2d_spatial", "2d_crf"])
+def test_compute_positions_bit_exact(name):
+    g = load_golden("positions")
+    sdims, rc = [int(s) for s in g[name + "_sdims"]], int(g[name + "_rc"])
+    s_std, f_std = [float(x) for x in g[name + "_stds"]]
+    ref = dev(g[name + "_reference"]) if rc else None
+    pos = host(pla.compute_positions(ref, sdims, s_std, f_std))
+    assert (bits(pos) == bits(g[name + "_positions"])).all()
+
+
+def test_compute_positions_bit_exact_at_size_with_awkward_stds():
+    sdims, rc = (96, 80, 70), 2
+    n = int(np.prod(sdims))
+    ref = synth.uniform_image((n, rc), 19)
+    for s_std, f_std in ((5.0, 0.1), (3.0, 13.0), (7.3, 0.017)):
+        want = oracle.compute_positions(ref, sdims, s_std, f_std, rc)
+        got = host(pla.compute_positions(dev(ref), sdims, s_std, f_std))
+        assert (bits(got) == bits(want)).all()
+
+
+def test_op_bilateral_batch_and_gradient():
+    b, h, w = 2, 96, 80
+    guide = np.stack([synth.blob_image(h, w, seed=20 + i) for i in range(b)])
+    inp = synth.uniform_image((b, h, w, 2), 22)
+    want = oracle.lattice_filter(inp, guide, True, 8.0, 0.125, 1.0, False)
+    x = dev(inp).requires_grad_(True)
+    y = pla.lattice_filter(x, dev(guide), bilateral=True, theta_alpha=8.0, theta_beta=0.125)
+    assert y.shape == x.shape
+    assert_float_parity(host(y), want)
+    up = synth.normal_image(inp.shape, 23)
+    y.backward(dev(up))
+    want_grad = oracle.lattice_filter(up, guide, True, 8.0, 0.125, 1.0, True)
+    assert_float_parity(host(x.grad), want_grad, scale=float(np.abs(want_grad).max()))
+
+
+def test_op_spatial_only_uses_theta_gamma_and_ignores_the_reference():
+    inp = synth.uniform_image((1, 64, 48, 3), 24)
+    want = oracle.lattice_filter(inp, None, False, 77.0, 77.0, 3.0, False)
+    got = pla.lattice_filter(dev(inp), dev(synth.uniform_image((1, 64, 48, 5), 25)), bilateral=False,
+                             theta_alpha=77.0, theta_beta=77.0, theta_gamma=3.0)
+    assert_float_parity(host(got), want)
+    got2 = pla.lattice_filter(dev(inp), None, bilateral=False, theta_gamma=3.0)
+    assert_float_parity(host(got2), want)
+
+
+def test_op_3d_volume():
+    vol = synth.ellipsoid_volume(24, 40, 32, seed=26)[None]
+    want = oracle.lattice_filter(vol, vol, True, 5.0, 0.1, 1.0, False)
+    got = pla.lattice_filter(dev(vol), dev(vol), theta_alpha=5.0, theta_beta=0.1)
+    assert_float_parity(host(got), want, scale=max(1.0, float(np.abs(want).max())))
+
+
+def test_op_rejects_unsupported_dimensions():
+    x = torch.zeros((1, 8, 8, 2), device="cuda")
+    ref = torch.zeros((1, 8, 8, 7), device="cuda")   # pd = 9
+    with pytest.raises(pla.PermutohedralError) as e:
+        pla.lattice_filter(x, ref)
+    assert e.value.status == pla.PL_EUNSUPPORTED
+
+
+# ---------------------------------------------------------------------------------------------
+# the reference's image fixtures
+# ---------------------------------------------------------------------------------------------
+
+def test_reference_image_fixtures():
+    """input.bmp -> bilateral_out_1.bmp (batch of two, as Tests/bilateral_filter.py) and
+    gray_original.bmp -> filtered_grey.bmp under the RGB guide (Tests/greyscale_test.py), theta
+    8 / 0.125, rounded to 8 bits: no value off by more than one level, almost none off at all."""
+    im = load_golden("reference_images")
+    rgb = (im["input"] / 255.0).astype(np.float32)
+    batch = dev(np.stack([rgb, rgb]))
+    out = host(pla.lattice_filter(batch, batch, theta_alpha=8.0, theta_beta=0.125))
+    for item in out:
+        q = np.round(item.astype(np.float64) * 255).astype(np.int64)
+        diff = np.abs(q - im["bilateral_out_1"].astype(np.int64))
+        assert diff.max() <= 1
+        assert (diff != 0).mean() <= 2e-4
+    grey = (im["gray_original"] / 255.0).astype(np.float32)[None, :, :, None]
+    out = host(pla.lattice_filter(dev(grey), dev(rgb[None]), theta_alpha=8.0, theta_beta=0.125))
+    q = np.round(out[0, :, :, 0].astype(np.float64) * 255).astype(np.int64)
+    diff = np.abs(q - im["filtered_grey"].astype(np.int64))
+    assert diff.max() <= 1
+    assert (diff != 0).mean() <= 1e-3
