@@ -52,7 +52,9 @@ typedef enum pl_option {
                               does (src/PermutohedralLatticeCPU.h:347-350).  0: input and output carry all
                               vd channels and nothing is divided -- the bare linear operator, for tests. */
     PL_OPT_PROFILE = 2,    /* 1: record per-stage HIP events, read with pl_stage_ms */
-    PL_OPT_TABLE_CELLS = 3 /* force the initial number of hash cells (power of two), 0 = automatic */
+    PL_OPT_TABLE_CELLS = 3, /* force the initial number of hash cells (power of two), 0 = automatic */
+    PL_OPT_XCD_AWARE = 4    /* 1 (default): kernels with atomic updates give each XCD a contiguous range
+                               of points; 0: plain workgroup order (for measuring the difference) */
 } pl_option;
 
 /* 1 when a lattice can be built for these dimensions, else 0.
@@ -93,6 +95,15 @@ int pl_filter(pl_handle h, float *output, const float *input, const float *posit
 int pl_build(pl_handle h, const float *positions);
 int pl_apply(pl_handle h, float *output, const float *input, int reverse);
 
+/*
+ * Optional hint: the N points are a row-major grid of these extents (their product must be N),
+ * as the op's tensors are (src/LatticeFilterKernel.cpp:117-124: spatial_dims).  Workgroups then
+ * take compact tiles of the grid instead of runs of consecutive points, so more of the points
+ * that share lattice vertices meet inside one wavefront.  Results do not depend on the hint.
+ * n_dims = 0 removes it.  pl_lattice_filter_op sets it by itself.
+ */
+int pl_set_point_grid(pl_handle h, int n_dims, const int *dims);
+
 /* Number of lattice vertices of the last build (HashTableCPU::size(), src/PermutohedralLatticeCPU.h:151). */
 int pl_num_vertices(pl_handle h, int *num_vertices);
 
@@ -100,9 +111,9 @@ int pl_set_option(pl_handle h, int option, long value);
 
 /* Milliseconds of the kernels of the last pl_build and pl_apply (or pl_filter) with
  * PL_OPT_PROFILE on, from HIP events on the lattice's stream: ms[0] table clear, ms[1] build
- * (embed + simplex + hash insertion), ms[2] neighbour table, ms[3] value clear, ms[4] splat,
- * ms[5] blur (all pd+1 launches together), ms[6] slice.  Synchronises the stream. */
-int pl_stage_ms(pl_handle h, float ms[7]);
+ * (embed + simplex + hash insertion), ms[2] vertex numbering, ms[3] neighbour table, ms[4] value
+ * clear, ms[5] splat, ms[6] blur (all pd+1 launches together), ms[7] slice.  Synchronises the stream. */
+int pl_stage_ms(pl_handle h, float ms[8]);
 
 /*
  * Debug export of the per-point integer results of the last build, for parity checks; device

@@ -20,12 +20,12 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libpermutohedral_hip.so")
 
 PL_OK, PL_EINVAL, PL_EUNSUPPORTED, PL_ENOMEM, PL_EOVERFLOW, PL_EHIP, PL_ESTATE = 0, -1, -2, -3, -4, -5, -6
-PL_OPT_NORMALIZE, PL_OPT_PROFILE, PL_OPT_TABLE_CELLS = 1, 2, 3
+PL_OPT_NORMALIZE, PL_OPT_PROFILE, PL_OPT_TABLE_CELLS, PL_OPT_XCD_AWARE = 1, 2, 3, 4
 
 # every symbol include/permutohedral_lattice.h declares
 EXPORTS = (
     "pl_supported", "pl_strerror", "pl_last_hip_error", "pl_create", "pl_destroy", "pl_filter",
-    "pl_build", "pl_apply", "pl_num_vertices", "pl_set_option", "pl_stage_ms", "pl_debug_simplex",
+    "pl_build", "pl_apply", "pl_set_point_grid", "pl_num_vertices", "pl_set_option", "pl_stage_ms", "pl_debug_simplex",
     "pl_debug_keys", "pl_debug_replay", "pl_compute_positions", "pl_lattice_filter_op",
 )
 
@@ -54,6 +54,7 @@ def _load():
     lib.pl_filter.argtypes = [vp, vp, vp, vp, ci]
     lib.pl_build.argtypes = [vp, vp]
     lib.pl_apply.argtypes = [vp, vp, vp, ci]
+    lib.pl_set_point_grid.argtypes = [vp, ci, C.POINTER(ci)]
     lib.pl_num_vertices.argtypes = [vp, C.POINTER(ci)]
     lib.pl_set_option.argtypes = [vp, ci, C.c_long]
     lib.pl_stage_ms.argtypes = [vp, C.POINTER(cf)]
@@ -130,6 +131,12 @@ class PermutohedralLattice:
                              _dev_f32(input, "input", self.N * ch), int(bool(reverse))), "pl_apply")
         return output
 
+    def set_point_grid(self, dims):
+        """Hint: the N points form a row-major grid of these extents (None removes the hint)."""
+        dims = [int(d) for d in (dims or [])]
+        arr = (C.c_int * max(1, len(dims)))(*dims)
+        _check(_lib.pl_set_point_grid(self._h, len(dims), arr), "pl_set_point_grid")
+
     @property
     def num_vertices(self):
         m = C.c_int()
@@ -142,9 +149,10 @@ class PermutohedralLattice:
             self._normalize = bool(value)
 
     def stage_ms(self):
-        ms = (C.c_float * 7)()
+        ms = (C.c_float * 8)()
         _check(_lib.pl_stage_ms(self._h, ms), "pl_stage_ms")
-        return dict(zip(("clear", "build", "neighbours", "fill", "splat", "blur", "slice"), list(ms)))
+        return dict(zip(("clear", "build", "ids", "neighbours", "fill", "splat", "blur", "slice"),
+                        list(ms)))
 
     # -- parity exports ------------------------------------------------------------------------
     def debug_simplex(self, positions):

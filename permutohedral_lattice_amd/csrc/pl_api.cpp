@@ -51,7 +51,7 @@ void compute_scale_factor(int pd, plk::ScaleFactor &sf) {
         sf.v[i] = (float)(1.0 / std::sqrt((double)((i + 1) * (i + 2))) * (double)inv_std_dev);
 }
 
-enum { EV_T0, EV_CLEAR, EV_BUILD, EV_NBR0, EV_NBR, EV_A0, EV_FILL, EV_SPLAT, EV_BLUR, EV_SLICE, EV_COUNT };
+enum { EV_T0, EV_CLEAR, EV_BUILD, EV_IDS, EV_NBR0, EV_NBR, EV_A0, EV_FILL, EV_SPLAT, EV_BLUR, EV_SLICE, EV_COUNT };
 
 }  // namespace
 
@@ -76,9 +76,11 @@ struct pl_lattice {
     int2 *neighbours = nullptr;
     size_t vertex_capacity = 0;
 
-    // per-point arrays
+    // per-point arrays, (pd+1) rows of map.n_blocks*256 entries in thread order
+    plk::PointMap map{};
     int *replay_index = nullptr;
     float *replay_weight = nullptr;
+    size_t replay_capacity = 0;  // entries per array
 
     plk::Counters *d_counters = nullptr;
     plk::Counters *h_counters = nullptr;  // pinned
@@ -89,6 +91,7 @@ struct pl_lattice {
     bool replay_holds_cells = false;
     bool normalize = true;
     bool profile = false;
+    bool xcd_aware = true;
     hipEvent_t ev[EV_COUNT] = {};
     bool ev_recorded[EV_COUNT] = {};
 
@@ -137,6 +140,21 @@ int ensure_vertices(pl_lattice *h, size_t m) {
     h->neighbours = (int2 *)h->dmalloc(sizeof(int2) * cap * (size_t)(h->pd + 1));
     if (!h->values[0] || !h->values[1] || !h->neighbours) return PL_ENOMEM;
     h->vertex_capacity = cap;
+    return PL_OK;
+}
+
+int ensure_replay(pl_lattice *h) {
+    const size_t want = (size_t)h->map.n_blocks * 256 * (size_t)(h->pd + 1);
+    if (want <= h->replay_capacity && h->replay_index) return PL_OK;
+    h->dfree(h->replay_index);
+    h->dfree(h->replay_weight);
+    h->replay_index = nullptr;
+    h->replay_weight = nullptr;
+    h->replay_capacity = 0;
+    h->replay_index = (int *)h->dmalloc(sizeof(int) * (want ? want : 1));
+    h->replay_weight = (float *)h->dmalloc(sizeof(float) * (want ? want : 1));
+    if (!h->replay_index || !h->replay_weight) return PL_ENOMEM;
+    h->replay_capacity = want;
     return PL_OK;
 }
 
@@ -204,11 +222,11 @@ int pl_create(int pd, int vd, int N, pl_stream stream, const pl_alloc *alloc, pl
 
     int rc = PL_OK;
     if (hip_failed(hipGetDevice(&h->device))) rc = PL_EHIP;
+    h->map = plk::make_point_map(N, 0, nullptr);
+    if (rc == PL_OK) rc = ensure_replay(h);
     if (rc == PL_OK) {
-        h->replay_index = (int *)h->dmalloc(sizeof(int) * (size_t)(rows ? rows : 1));
-        h->replay_weight = (float *)h->dmalloc(sizeof(float) * (size_t)(rows ? rows : 1));
         h->d_counters = (plk::Counters *)h->dmalloc(sizeof(plk::Counters));
-        if (!h->replay_index || !h->replay_weight || !h->d_counters) rc = PL_ENOMEM;
+        if (!h->d_counters) rc = PL_ENOMEM;
     }
     if (rc == PL_OK && hip_failed(hipHostMalloc((void **)&h->h_counters, sizeof(plk::Counters), hipHostMallocDefault)))
         rc = PL_EHIP;
@@ -251,6 +269,9 @@ int pl_set_option(pl_handle h, int option, long value) {
                 for (int i = 0; i < EV_COUNT; ++i)
                     if (!h->ev[i]) PL_HIP(hipEventCreate(&h->ev[i]));
             return PL_OK;
+        case PL_OPT_XCD_AWARE:
+            h->xcd_aware = value != 0;
+            return PL_OK;
         case PL_OPT_TABLE_CELLS:
             if (value < 0 || (value & (value - 1)) != 0) return PL_EINVAL;
             h->forced_cells = value;
@@ -259,6 +280,22 @@ int pl_set_option(pl_handle h, int option, long value) {
         default:
             return PL_EINVAL;
     }
+}
+
+int pl_set_point_grid(pl_handle h, int n_dims, const int *dims) {
+    if (!h || n_dims < 0 || (n_dims > 0 && !dims)) return PL_EINVAL;
+    if (n_dims > 0) {
+        long long prod = 1;
+        for (int i = 0; i < n_dims; ++i) {
+            if (dims[i] < 1) return PL_EINVAL;
+            prod *= dims[i];
+            if (prod > 2147483647LL) return PL_EINVAL;
+        }
+        if (prod != (long long)h->N) return PL_EINVAL;
+    }
+    h->built = false;
+    h->map = plk::make_point_map(h->N, n_dims, dims);
+    return ensure_replay(h);
 }
 
 int pl_build(pl_handle h, const float *positions) {
@@ -277,10 +314,12 @@ int pl_build(pl_handle h, const float *positions) {
         h->mark(EV_T0);
         PL_HIP(plk::clear_table(h->cell_keys, cells, h->d_counters, h->stream));
         h->mark(EV_CLEAR);
-        PL_HIP(plk::build(h->pd, positions, h->N, h->scale, h->cell_keys, h->cell_vertex, cells,
-                          h->vertex_keys, h->d_counters, h->replay_index, h->replay_weight,
-                          h->stream));
+        PL_HIP(plk::build(h->pd, positions, h->map, h->scale, h->cell_keys, cells, h->d_counters,
+                          h->replay_index, h->replay_weight, h->xcd_aware ? 1 : 0, h->stream));
         h->mark(EV_BUILD);
+        PL_HIP(plk::assign_vertex_ids(h->cell_keys, cells, h->cell_vertex, h->vertex_keys,
+                                      h->d_counters, h->stream));
+        h->mark(EV_IDS);
         PL_HIP(hipMemcpyAsync(h->h_counters, h->d_counters, sizeof(plk::Counters),
                               hipMemcpyDeviceToHost, h->stream));
         PL_HIP(hipStreamSynchronize(h->stream));
@@ -318,8 +357,9 @@ int pl_apply(pl_handle h, float *output, const float *input, int reverse) {
     h->mark(EV_A0);
     PL_HIP(plk::fill_zero(h->values[0], (size_t)M * vd, h->stream));
     h->mark(EV_FILL);
-    PL_HIP(plk::splat(pd, vd, h->N, input, in_channels, h->replay_index, h->replay_weight,
-                      h->replay_holds_cells ? h->cell_vertex : nullptr, h->values[0], h->stream));
+    PL_HIP(plk::splat(pd, vd, h->map, input, in_channels, h->replay_index, h->replay_weight,
+                      h->replay_holds_cells ? h->cell_vertex : nullptr, h->values[0],
+                      h->xcd_aware ? 1 : 0, h->stream));
     h->replay_holds_cells = false;
     h->mark(EV_SPLAT);
 
@@ -332,7 +372,7 @@ int pl_apply(pl_handle h, float *output, const float *input, int reverse) {
     }
     h->mark(EV_BLUR);
 
-    PL_HIP(plk::slice(pd, vd, h->N, h->replay_index, h->replay_weight, h->values[cur], output,
+    PL_HIP(plk::slice(pd, vd, h->map, h->replay_index, h->replay_weight, h->values[cur], output,
                       h->normalize ? 1 : 0, h->stream));
     h->mark(EV_SLICE);
     return PL_OK;
@@ -353,14 +393,14 @@ int pl_num_vertices(pl_handle h, int *num_vertices) {
     return PL_OK;
 }
 
-int pl_stage_ms(pl_handle h, float ms[7]) {
+int pl_stage_ms(pl_handle h, float ms[8]) {
     if (!h || !ms) return PL_EINVAL;
     if (!h->profile) return PL_ESTATE;
     PL_HIP(hipStreamSynchronize(h->stream));
-    const int pairs[7][2] = {{EV_T0, EV_CLEAR},  {EV_CLEAR, EV_BUILD}, {EV_NBR0, EV_NBR},
-                             {EV_A0, EV_FILL},   {EV_FILL, EV_SPLAT},  {EV_SPLAT, EV_BLUR},
-                             {EV_BLUR, EV_SLICE}};
-    for (int i = 0; i < 7; ++i) {
+    const int pairs[8][2] = {{EV_T0, EV_CLEAR},  {EV_CLEAR, EV_BUILD}, {EV_BUILD, EV_IDS},
+                             {EV_NBR0, EV_NBR},  {EV_A0, EV_FILL},     {EV_FILL, EV_SPLAT},
+                             {EV_SPLAT, EV_BLUR}, {EV_BLUR, EV_SLICE}};
+    for (int i = 0; i < 8; ++i) {
         ms[i] = 0.0f;
         if (h->ev_recorded[pairs[i][0]] && h->ev_recorded[pairs[i][1]])
             PL_HIP(hipEventElapsedTime(&ms[i], h->ev[pairs[i][0]], h->ev[pairs[i][1]]));
@@ -386,13 +426,8 @@ int pl_debug_keys(pl_handle h, short *keys) {
 int pl_debug_replay(pl_handle h, int *vertex, float *weight) {
     if (!h) return PL_EINVAL;
     if (!h->built || h->replay_holds_cells) return PL_ESTATE;
-    const size_t rows = (size_t)h->N * (size_t)(h->pd + 1);
-    if (vertex)
-        PL_HIP(hipMemcpyAsync(vertex, h->replay_index, sizeof(int) * rows, hipMemcpyDeviceToDevice,
+    PL_HIP(plk::export_replay(h->pd, h->map, h->replay_index, h->replay_weight, vertex, weight,
                               h->stream));
-    if (weight)
-        PL_HIP(hipMemcpyAsync(weight, h->replay_weight, sizeof(float) * rows,
-                              hipMemcpyDeviceToDevice, h->stream));
     return PL_OK;
 }
 
@@ -507,6 +542,7 @@ extern "C" int pl_lattice_filter_op(const float *input, const float *reference, 
         }
     }
 
+    rc = pl_set_point_grid(lattice, n_spatial_dims, spatial_dims);
     for (int b = 0; b < batch && rc == PL_OK; ++b) {
         const float *ref_b = ref_ch ? reference + (size_t)b * N * ref_ch : nullptr;
         rc = pl_compute_positions(ref_b, positions, N, ref_ch, n_spatial_dims, spatial_dims,

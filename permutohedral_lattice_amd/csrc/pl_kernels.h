@@ -30,19 +30,36 @@ struct SpatialDims {
     int v[kMaxSpatialDims];
 };
 
+// How threads are laid over the points (see point_of_thread in pl_kernels.hip).
+struct PointMap {
+    int N;
+    int mode;        // 0: 256 consecutive points per workgroup; 2: 16x16 tiles; 3: 4x8x8 tiles
+    int dims[3];     // grid extents, slowest first (leading extents folded into dims[0])
+    int tiles[3];    // workgroup tiles along each extent
+    unsigned n_blocks;
+};
+
 // Bits per lattice coordinate in the packed 64-bit key, and the coordinate range that fits.
 int key_field_bits(int pd);
+
+// n_dims < 2 or dims == nullptr: no grid, consecutive points.
+PointMap make_point_map(int N, int n_dims, const int *dims);
 
 // Hash cells := empty, counters := 0.
 hipError_t clear_table(uint64_t *cell_keys, uint32_t n_cells, Counters *counters, hipStream_t s);
 
 // Stage 1+2: per point embed, enclosing simplex, barycentric weights, then insertion of the pd+1
-// vertex keys.  replay_index[r*N+n] := hash cell of vertex r of point n, replay_weight likewise.
-// Winners of a cell draw a dense vertex index, publish it in cell_vertex and store the packed key
-// in vertex_keys.
-hipError_t build(int pd, const float *positions, int N, const ScaleFactor &scale,
-                 uint64_t *cell_keys, int *cell_vertex, uint32_t n_cells, uint64_t *vertex_keys,
-                 Counters *counters, int *replay_index, float *replay_weight, hipStream_t s);
+// vertex keys.  The replay arrays hold (pd+1) rows of T = map.n_blocks*256 entries in thread
+// order: replay_index[r*T+t] := hash cell of vertex r of the point of thread t (-1: no point),
+// replay_weight likewise.
+hipError_t build(int pd, const float *positions, const PointMap &map, const ScaleFactor &scale,
+                 uint64_t *cell_keys, uint32_t n_cells, Counters *counters, int *replay_index,
+                 float *replay_weight, int xcd_aware, hipStream_t s);
+
+// Every occupied cell draws a dense vertex index: cell_vertex[cell] := v, vertex_keys[v] := key,
+// counters->num_vertices := M.
+hipError_t assign_vertex_ids(const uint64_t *cell_keys, uint32_t n_cells, int *cell_vertex,
+                             uint64_t *vertex_keys, Counters *counters, hipStream_t s);
 
 // neighbours[a*M+v] := vertex indices of v's two neighbours along blur axis a (-1 = absent).
 hipError_t neighbours(int pd, const uint64_t *vertex_keys, int M, const uint64_t *cell_keys,
@@ -53,21 +70,27 @@ hipError_t fill_zero(float *p, size_t n, hipStream_t s);
 // Stage 3.  in_channels is vd-1 (the homogeneous channel is the bare weight) or vd.
 // cell_vertex != nullptr: replay_index still holds hash cells; they are translated to vertex
 // indices and written back.
-hipError_t splat(int pd, int vd, int N, const float *input, int in_channels, int *replay_index,
-                 const float *replay_weight, const int *cell_vertex, float *values, hipStream_t s);
+hipError_t splat(int pd, int vd, const PointMap &map, const float *input, int in_channels,
+                 int *replay_index, const float *replay_weight, const int *cell_vertex, float *values,
+                 int xcd_aware, hipStream_t s);
 
 // Stage 4, one axis: dst[v] = 1/4 src[n1] + 1/2 src[v] + 1/4 src[n2].
 hipError_t blur_axis(int vd, int M, const float *src, float *dst, const int2 *neighbours_of_axis,
                      hipStream_t s);
 
 // Stage 5.  normalize: divide by the homogeneous channel and write vd-1 channels; else write vd.
-hipError_t slice(int pd, int vd, int N, const int *replay_index, const float *replay_weight,
-                 const float *values, float *output, int normalize, hipStream_t s);
+hipError_t slice(int pd, int vd, const PointMap &map, const int *replay_index,
+                 const float *replay_weight, const float *values, float *output, int normalize,
+                 hipStream_t s);
 
 hipError_t debug_simplex(int pd, const float *positions, int N, const ScaleFactor &scale,
                          short *rem0, short *rank, short *keys, float *barycentric, hipStream_t s);
 
 hipError_t export_keys(int pd, const uint64_t *vertex_keys, int M, short *keys, hipStream_t s);
+
+// replay arrays in point order: vertex[r*N+n], weight[r*N+n]
+hipError_t export_replay(int pd, const PointMap &map, const int *replay_index,
+                         const float *replay_weight, int *vertex, float *weight, hipStream_t s);
 
 hipError_t compute_positions(const float *reference, float *positions, int N, int n_ref_channels,
                              int n_spatial_dims, const SpatialDims &dims, float spatial_std,

@@ -23,6 +23,18 @@ namespace plk {
 namespace {
 
 constexpr int kBlock = 256;
+constexpr unsigned kXcds = 8;  // MI355X: 8 accelerator dies, each with its own L2
+
+// Workgroups are handed to the XCDs round-robin (workgroup b runs on XCD b % 8).  Points that are
+// close in memory share lattice vertices, so the kernels that update shared cells or values
+// atomically give each XCD one contiguous range of points: the contended lines then stay in
+// one L2 instead of migrating between dies.
+__device__ __forceinline__ unsigned xcd_contiguous_block(unsigned b, unsigned nb, int enabled) {
+    if (!enabled) return b;
+    const unsigned q = nb / kXcds, rem = nb % kXcds;
+    const unsigned xcd = b % kXcds, i = b / kXcds;
+    return xcd * q + (xcd < rem ? xcd : rem) + i;
+}
 
 template <int PD>
 struct KeyCodec {
@@ -173,32 +185,56 @@ __device__ __forceinline__ void load_position(const float *positions, int n, flo
 }
 
 // ------------------------------------------------------------------------------------------------
+// Which point a thread works on.  Points that are neighbours in the image share lattice vertices,
+// and every duplicate that meets inside one wavefront is merged before it reaches memory, so a
+// wavefront should cover a compact tile of the image, not a run of 64 points of one row.  With a
+// grid hint (the op knows its spatial extents) a workgroup takes a 16x16 tile of a 2-D grid
+// (wavefronts 8x8) or a 4x8x8 tile of a 3-D grid (wavefronts 4x4x4); without one it takes 256
+// consecutive points.  The mapping only changes the order of work, never a result.
+// Per-point scratch (the replay arrays) is stored in thread order, so it stays coalesced.
+// ------------------------------------------------------------------------------------------------
+__device__ __forceinline__ int point_of_thread(const PointMap &m, unsigned vblock, unsigned tid) {
+    if (m.mode == 0) {
+        const size_t n = (size_t)vblock * kBlock + tid;
+        return n < (size_t)m.N ? (int)n : -1;
+    }
+    const unsigned wave = tid >> 6, lane = tid & 63;
+    const unsigned tiles_yx = (unsigned)m.tiles[1] * (unsigned)m.tiles[2];
+    const unsigned tz = vblock / tiles_yx;
+    const unsigned rest = vblock - tz * tiles_yx;
+    const unsigned ty = rest / (unsigned)m.tiles[2];
+    const unsigned tx = rest - ty * (unsigned)m.tiles[2];
+    unsigned z, y, x;
+    if (m.mode == 2) {
+        z = tz;
+        y = ty * 16 + (wave >> 1) * 8 + (lane >> 3);
+        x = tx * 16 + (wave & 1) * 8 + (lane & 7);
+    } else {
+        z = tz * 4 + (lane >> 4);
+        y = ty * 8 + (wave >> 1) * 4 + ((lane >> 2) & 3);
+        x = tx * 8 + (wave & 1) * 4 + (lane & 3);
+    }
+    if (z >= (unsigned)m.dims[0] || y >= (unsigned)m.dims[1] || x >= (unsigned)m.dims[2]) return -1;
+    return (int)(((size_t)z * m.dims[1] + y) * m.dims[2] + x);
+}
+
+// ------------------------------------------------------------------------------------------------
 // Hash table
 // ------------------------------------------------------------------------------------------------
 
 // Returns the cell holding `key`, inserting it if absent; -1 and kFlagTableFull when no cell is
 // free.  Cells only ever change from empty to a key, so a stale read can at worst see "empty" and
 // the compare-and-swap then returns the truth.
-__device__ __forceinline__ int table_insert(uint64_t *cell_keys, int *cell_vertex, uint32_t mask,
-                                            uint64_t *vertex_keys, Counters *counters, uint64_t key) {
-    uint32_t h = hash_key(key) & mask;
+// `h` is the key's home cell and `cur` what a load of it returned (the caller issues the first
+// loads of all its keys together, so that their latencies overlap).
+__device__ __forceinline__ int table_insert(uint64_t *cell_keys, uint32_t mask, Counters *counters,
+                                            uint64_t key, uint32_t h, uint64_t cur) {
     for (uint32_t probe = 0; probe <= mask; ++probe) {
-        uint64_t cur = cell_keys[h];
+        if (probe) cur = cell_keys[h];
         if (cur == kEmptyCell) {
             cur = atomicCAS((unsigned long long *)(cell_keys + h), (unsigned long long)kEmptyCell,
                             (unsigned long long)key);
-            if (cur == kEmptyCell) {
-                // this lane created the vertex: draw its dense index
-                const int v = atomicAdd(&counters->num_vertices, 1);
-                if ((uint32_t)v < (mask + 1u) / 2u) {
-                    vertex_keys[v] = key;
-                    cell_vertex[h] = v;
-                } else {
-                    atomicOr(&counters->flags, kFlagTableFull);
-                    cell_vertex[h] = 0;
-                }
-                return (int)h;
-            }
+            if (cur == kEmptyCell) return (int)h;
         }
         if (cur == key) return (int)h;
         h = (h + 1u) & mask;
@@ -229,19 +265,44 @@ __global__ __launch_bounds__(kBlock) void k_clear_table(uint64_t *cell_keys, uin
     }
 }
 
+// Lanes that hold the same value of `x` elect the lowest of them as leader.  Returns the leader's
+// lane and, in `members`, the lanes of the caller's group; inactive lanes get their own lane and
+// an empty group.  One iteration per distinct value in the wavefront.
+template <typename T>
+__device__ __forceinline__ int wave_leader_of_equal(T x, bool active, int lane, uint64_t &members) {
+    int leader = lane;
+    members = 0;
+    uint64_t remaining = __ballot(active);
+    while (remaining) {
+        const int first = __builtin_ctzll(remaining);
+        const T k = __shfl(x, first);
+        const bool same = active && x == k;
+        const uint64_t group = __ballot(same);
+        if (same) {
+            leader = first;
+            members = group;
+        }
+        remaining &= ~group;
+    }
+    return leader;
+}
+
 // ------------------------------------------------------------------------------------------------
 // Stage 1+2: embed, simplex, insert
 // ------------------------------------------------------------------------------------------------
 template <int PD>
-__global__ __launch_bounds__(kBlock) void k_build(const float *__restrict__ positions, int N,
+__global__ __launch_bounds__(kBlock) void k_build(const float *__restrict__ positions, PointMap map,
                                                    ScaleFactor scale, uint64_t *cell_keys,
-                                                   int *cell_vertex, uint32_t mask,
-                                                   uint64_t *vertex_keys, Counters *counters,
+                                                   uint32_t mask, Counters *counters,
                                                    int *__restrict__ replay_index,
-                                                   float *__restrict__ replay_weight) {
-    const int n = blockIdx.x * kBlock + threadIdx.x;
+                                                   float *__restrict__ replay_weight,
+                                                   int xcd_aware) {
+    const unsigned vblock = xcd_contiguous_block(blockIdx.x, gridDim.x, xcd_aware);
+    const size_t t = (size_t)vblock * kBlock + threadIdx.x;   // slot in the replay arrays
+    const size_t T = (size_t)gridDim.x * kBlock;
+    const int n = point_of_thread(map, vblock, threadIdx.x);
     const int lane = threadIdx.x & 63;
-    const bool valid = n < N;
+    const bool valid = n >= 0;
 
     float pos[PD];
 #pragma unroll
@@ -255,33 +316,71 @@ __global__ __launch_bounds__(kBlock) void k_build(const float *__restrict__ posi
     if (valid && !in_range) atomicOr(&counters->flags, kFlagKeyRange);
     const bool active = valid && in_range;
 
-#pragma unroll 1
+    // Wavefront-level deduplication: each distinct key of the wavefront is inserted by one lane
+    // (the lowest that holds it) and its cell is broadcast to the others.  Only leaders touch the
+    // table, and they load the home cells of all pd+1 keys before looking at any of them.
+    uint64_t key[PD + 1], home_value[PD + 1];
+    uint32_t home[PD + 1];
+    int leader[PD + 1];
+#pragma unroll
     for (int r = 0; r <= PD; ++r) {
         int q[PD];
         vertex_q<PD>(s, r, q);
-        const uint64_t key = KeyCodec<PD>::pack(q, r);
-
-        // Wavefront-level deduplication: neighbouring points mostly share vertices, so each
-        // distinct key of the wave is inserted by one lane (the lowest that holds it) and the cell
-        // is broadcast to the others.  Only the leaders touch the table.
-        int leader = lane;
-        uint64_t remaining = __ballot(active);
-        while (remaining) {
-            const int first = __builtin_ctzll(remaining);
-            const uint64_t k = __shfl(key, first);
-            const bool same = active && key == k;
-            if (same) leader = first;
-            remaining &= ~__ballot(same);
-        }
-
+        key[r] = KeyCodec<PD>::pack(q, r);
+        uint64_t members;
+        leader[r] = wave_leader_of_equal(key[r], active, lane, members);
+        home[r] = hash_key(key[r]) & mask;
+    }
+#pragma unroll
+    for (int r = 0; r <= PD; ++r)
+        home_value[r] = (active && leader[r] == lane) ? cell_keys[home[r]] : kEmptyCell;
+#pragma unroll
+    for (int r = 0; r <= PD; ++r) {
         int cell = -1;
-        if (active && leader == lane)
-            cell = table_insert(cell_keys, cell_vertex, mask, vertex_keys, counters, key);
-        cell = __shfl(cell, leader);
+        if (active && leader[r] == lane)
+            cell = table_insert(cell_keys, mask, counters, key[r], home[r], home_value[r]);
+        cell = __shfl(cell, leader[r]);
+        replay_index[(size_t)r * T + t] = active ? cell : -1;
+        replay_weight[(size_t)r * T + t] = valid ? s.weight[r] : 0.0f;
+    }
+}
 
-        if (valid) {
-            replay_index[(size_t)r * N + n] = active ? cell : -1;
-            replay_weight[(size_t)r * N + n] = s.weight[r];
+// Dense vertex numbering: every occupied cell draws an index.  One atomic per workgroup (counts are
+// combined by ballot inside a wavefront and through LDS across the workgroup), because thousands
+// of atomics on one address would serialise in a single L2 channel.
+constexpr int kIdBlock = 1024;
+__global__ __launch_bounds__(kIdBlock) void k_assign_vertex_ids(const uint64_t *__restrict__ cell_keys,
+                                                                 uint32_t n_cells, int *cell_vertex,
+                                                                 uint64_t *vertex_keys,
+                                                                 Counters *counters) {
+    __shared__ int wave_count[kIdBlock / 64];
+    __shared__ int block_base;
+    const uint32_t cell = blockIdx.x * kIdBlock + threadIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const uint64_t key = cell < n_cells ? cell_keys[cell] : kEmptyCell;
+    const bool occupied = key != kEmptyCell;
+    const uint64_t ballot = __ballot(occupied);
+    if (lane == 0) wave_count[wave] = __builtin_popcountll(ballot);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int total = 0;
+        for (int w = 0; w < kIdBlock / 64; ++w) {
+            const int c = wave_count[w];
+            wave_count[w] = total;
+            total += c;
+        }
+        block_base = total ? atomicAdd(&counters->num_vertices, total) : 0;
+    }
+    __syncthreads();
+    if (occupied) {
+        const int v = block_base + wave_count[wave] +
+                      __builtin_popcountll(ballot & ((1ull << lane) - 1ull));
+        if ((uint32_t)v < n_cells / 2u) {
+            cell_vertex[cell] = v;
+            vertex_keys[v] = key;
+        } else {
+            cell_vertex[cell] = 0;
+            atomicOr(&counters->flags, kFlagTableFull);
         }
     }
 }
@@ -326,60 +425,103 @@ __global__ __launch_bounds__(kBlock) void k_fill_zero(float *p, size_t n) {
 
 // ------------------------------------------------------------------------------------------------
 // Stage 3: splat
+//
+// What bounds it is the L2 atomic unit, which retires about 20 G requests per second on MI355X,
+// where a request is what one instruction sends to one 64-byte line, however many lanes it
+// carries.  So (a) the contributions of a wavefront to one vertex are first summed in LDS
+// (ds_add_f32) and (b) the sums are flushed with consecutive lanes on consecutive channels of a
+// vertex, so that a vertex row costs one request and not vd.
 // ------------------------------------------------------------------------------------------------
-
-// One thread per point, channels in registers (small vd).
 template <int VD>
-__global__ __launch_bounds__(kBlock) void k_splat_point(int d1, int N, const float *__restrict__ input,
+__global__ __launch_bounds__(kBlock) void k_splat_point(int d1, PointMap map,
+                                                         const float *__restrict__ input,
                                                          int in_channels, int *replay_index,
                                                          const float *__restrict__ replay_weight,
                                                          const int *__restrict__ cell_vertex,
-                                                         float *values) {
-    const int n = blockIdx.x * kBlock + threadIdx.x;
-    if (n >= N) return;
+                                                         float *values, int xcd_aware) {
+    // per wavefront: every lane's weighted value, and per group of equal vertices its member
+    // lanes and its vertex
+    __shared__ float s_term[kBlock / 64][64 * VD];
+    __shared__ uint64_t s_members[kBlock / 64][64];
+    __shared__ int s_vertex[kBlock / 64][64];
+
+    const unsigned vblock = xcd_contiguous_block(blockIdx.x, gridDim.x, xcd_aware);
+    const size_t t = (size_t)vblock * kBlock + threadIdx.x;
+    const size_t T = (size_t)gridDim.x * kBlock;
+    const int n = point_of_thread(map, vblock, threadIdx.x);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+
     float val[VD];
 #pragma unroll
     for (int j = 0; j < VD; ++j) val[j] = 1.0f;  // homogeneous channel when only vd-1 are given
+    if (n >= 0) {
 #pragma unroll
-    for (int j = 0; j < VD; ++j)
-        if (j < in_channels) val[j] = input[(size_t)n * in_channels + j];
+        for (int j = 0; j < VD; ++j)
+            if (j < in_channels) val[j] = input[(size_t)n * in_channels + j];
+    }
 
     for (int r = 0; r < d1; ++r) {
-        int v = replay_index[(size_t)r * N + n];
-        if (v < 0) continue;
-        if (cell_vertex) {
+        int v = n >= 0 ? replay_index[(size_t)r * T + t] : -1;
+        if (cell_vertex && v >= 0) {
             v = cell_vertex[v];
-            replay_index[(size_t)r * N + n] = v;
+            replay_index[(size_t)r * T + t] = v;
         }
-        const float w = replay_weight[(size_t)r * N + n];
-        float *dst = values + (size_t)v * VD;
+        const float w = replay_weight[(size_t)r * T + t];
+        const bool active = v >= 0;
+
+        uint64_t members;
+        const int leader = wave_leader_of_equal(v, active, lane, members);
+        const bool is_leader = active && leader == lane;
+        const uint64_t leaders = __ballot(is_leader);
+        const int groups = __builtin_popcountll(leaders);
+        if (is_leader) {
+            const int slot = __builtin_popcountll(leaders & ((1ull << lane) - 1ull));
+            s_vertex[wave][slot] = v;
+            s_members[wave][slot] = members;
+        }
 #pragma unroll
-        for (int j = 0; j < VD; ++j) atomicAdd(dst + j, w * val[j]);
+        for (int j = 0; j < VD; ++j) s_term[wave][lane * VD + j] = w * val[j];
+        __syncthreads();
+        // lane e sums channel e % VD of group e / VD over the group's lanes (in lane order) and
+        // sends one atomic; the VD lanes of a group hit consecutive floats of one vertex row
+        for (int e = lane; e < groups * VD; e += 64) {
+            const int g = e / VD, j = e - g * VD;
+            uint64_t m = s_members[wave][g];
+            float sum = 0.0f;
+            while (m) {
+                const int l = __builtin_ctzll(m);
+                sum += s_term[wave][l * VD + j];
+                m &= m - 1;
+            }
+            atomicAdd(values + (size_t)s_vertex[wave][g] * VD + j, sum);
+        }
+        __syncthreads();
     }
 }
 
 // One thread per (point, channel): consecutive lanes add to consecutive floats of one vertex.
-__global__ __launch_bounds__(kBlock) void k_splat_channel(int d1, int vd, int N,
+__global__ __launch_bounds__(kBlock) void k_splat_channel(int d1, int vd, PointMap map, size_t T,
                                                            const float *__restrict__ input,
-                                                           int in_channels, int *replay_index,
+                                                           int in_channels,
+                                                           const int *__restrict__ replay_index,
                                                            const float *__restrict__ replay_weight,
-                                                           const int *__restrict__ cell_vertex,
                                                            float *values) {
-    const size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x;
-    if (t >= (size_t)N * vd) return;
-    const int n = (int)(t / (size_t)vd);
-    const int j = (int)(t - (size_t)n * vd);
+    const size_t g = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (g >= T * vd) return;
+    const size_t t = g / (size_t)vd;
+    const int j = (int)(g - t * vd);
+    const int n = point_of_thread(map, (unsigned)(t / kBlock), (unsigned)(t % kBlock));
+    if (n < 0) return;
     const float val = (j < in_channels) ? input[(size_t)n * in_channels + j] : 1.0f;
     for (int r = 0; r < d1; ++r) {
-        int v = replay_index[(size_t)r * N + n];
+        const int v = replay_index[(size_t)r * T + t];
         if (v < 0) continue;
-        if (cell_vertex) v = cell_vertex[v];
-        const float w = replay_weight[(size_t)r * N + n];
+        const float w = replay_weight[(size_t)r * T + t];
         atomicAdd(values + (size_t)v * vd + j, w * val);
     }
 }
 
-// cells -> vertex indices, for the per-channel splat (which cannot write back race-free itself)
+// cells -> vertex indices in the replay array
 __global__ __launch_bounds__(kBlock) void k_remap_replay(size_t rows, int *replay_index,
                                                           const int *__restrict__ cell_vertex) {
     const size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x;
@@ -411,20 +553,22 @@ __global__ __launch_bounds__(kBlock) void k_blur(int vd_runtime, int M, const fl
 // Stage 5: slice (reference: src/PermutohedralLatticeCPU.h:333-352)
 // ------------------------------------------------------------------------------------------------
 template <int VD>
-__global__ __launch_bounds__(kBlock) void k_slice_point(int d1, int N,
+__global__ __launch_bounds__(kBlock) void k_slice_point(int d1, PointMap map,
                                                          const int *__restrict__ replay_index,
                                                          const float *__restrict__ replay_weight,
                                                          const float *__restrict__ values,
                                                          float *__restrict__ output, int normalize) {
-    const int n = blockIdx.x * kBlock + threadIdx.x;
-    if (n >= N) return;
+    const size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    const size_t T = (size_t)gridDim.x * kBlock;
+    const int n = point_of_thread(map, blockIdx.x, threadIdx.x);
+    if (n < 0) return;
     float acc[VD];
 #pragma unroll
     for (int j = 0; j < VD; ++j) acc[j] = 0.0f;
     for (int r = 0; r < d1; ++r) {
-        const int v = replay_index[(size_t)r * N + n];
+        const int v = replay_index[(size_t)r * T + t];
         if (v < 0) continue;
-        const float w = replay_weight[(size_t)r * N + n];
+        const float w = replay_weight[(size_t)r * T + t];
         const float *src = values + (size_t)v * VD;
 #pragma unroll
         for (int j = 0; j < VD; ++j) acc[j] += w * src[j];
@@ -439,30 +583,33 @@ __global__ __launch_bounds__(kBlock) void k_slice_point(int d1, int N,
     }
 }
 
-__global__ __launch_bounds__(kBlock) void k_slice_channel(int d1, int vd, int N,
+__global__ __launch_bounds__(kBlock) void k_slice_channel(int d1, int vd, PointMap map, size_t T,
                                                            const int *__restrict__ replay_index,
                                                            const float *__restrict__ replay_weight,
                                                            const float *__restrict__ values,
                                                            float *__restrict__ output, int normalize) {
     const int out_ch = normalize ? vd - 1 : vd;
-    const size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x;
-    if (t >= (size_t)N * out_ch) return;
-    const int n = (int)(t / (size_t)out_ch);
-    const int j = (int)(t - (size_t)n * out_ch);
+    const size_t g = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (g >= T * out_ch) return;
+    const size_t t = g / (size_t)out_ch;
+    const int j = (int)(g - t * out_ch);
+    const int n = point_of_thread(map, (unsigned)(t / kBlock), (unsigned)(t % kBlock));
+    if (n < 0) return;
     float acc = 0.0f, hom = 0.0f;
     for (int r = 0; r < d1; ++r) {
-        const int v = replay_index[(size_t)r * N + n];
+        const int v = replay_index[(size_t)r * T + t];
         if (v < 0) continue;
-        const float w = replay_weight[(size_t)r * N + n];
+        const float w = replay_weight[(size_t)r * T + t];
         const float *src = values + (size_t)v * vd;
         acc += w * src[j];
         hom += w * src[vd - 1];
     }
+    const size_t o = (size_t)n * out_ch + j;
     if (normalize) {
         const float scale = (float)(1.0 / (double)hom);
-        output[t] = acc * scale;
+        output[o] = acc * scale;
     } else {
-        output[t] = acc;
+        output[o] = acc;
     }
 }
 
@@ -509,6 +656,21 @@ __global__ __launch_bounds__(kBlock) void k_export_keys(const uint64_t *__restri
     for (int i = 0; i < PD; ++i) keys[(size_t)v * PD + i] = (short)(q[i] * (PD + 1) + r);
 }
 
+// replay arrays from thread order to point order: out[r*N + n]
+__global__ __launch_bounds__(kBlock) void k_export_replay(int d1, PointMap map,
+                                                           const int *__restrict__ replay_index,
+                                                           const float *__restrict__ replay_weight,
+                                                           int *vertex, float *weight) {
+    const size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    const size_t T = (size_t)gridDim.x * kBlock;
+    const int n = point_of_thread(map, blockIdx.x, threadIdx.x);
+    if (n < 0) return;
+    for (int r = 0; r < d1; ++r) {
+        if (vertex) vertex[(size_t)r * map.N + n] = replay_index[(size_t)r * T + t];
+        if (weight) weight[(size_t)r * map.N + n] = replay_weight[(size_t)r * T + t];
+    }
+}
+
 // reference: src/PermutohedralLatticeCPU.h:464-473 (IEEE float division, int -> float exact)
 __global__ __launch_bounds__(kBlock) void k_positions(const float *__restrict__ reference,
                                                        float *__restrict__ positions, int N, int rc,
@@ -527,7 +689,7 @@ __global__ __launch_bounds__(kBlock) void k_positions(const float *__restrict__ 
     for (int c = 0; c < rc; ++c) row[nsd + c] = reference[(size_t)n * rc + c] / feature_std;
 }
 
-inline unsigned blocks_for(size_t n) { return (unsigned)((n + kBlock - 1) / kBlock); }
+inline unsigned blocks_for(size_t n, int block = kBlock) { return (unsigned)((n + block - 1) / block); }
 
 #define PLK_DISPATCH_PD(pd, CALL)                 \
     switch (pd) {                                 \
@@ -550,20 +712,54 @@ int key_field_bits(int pd) {
     return b > 16 ? 16 : b;
 }
 
+PointMap make_point_map(int N, int n_dims, const int *dims) {
+    PointMap m{};
+    m.N = N;
+    m.mode = 0;
+    m.dims[0] = m.dims[1] = 1;
+    m.dims[2] = N;
+    m.tiles[0] = m.tiles[1] = m.tiles[2] = 1;
+    m.n_blocks = (unsigned)(((size_t)N + kBlock - 1) / kBlock);
+    if (n_dims >= 2 && dims) {
+        // fold every leading extent into the slowest one: (d_0 * ... * d_{k-3}, d_{k-2}, d_{k-1})
+        long long lead = 1;
+        for (int i = 0; i < n_dims - 2; ++i) lead *= dims[i];
+        const int H = dims[n_dims - 2], W = dims[n_dims - 1];
+        if (n_dims == 2 || lead == 1) {
+            m.mode = 2;
+            m.dims[0] = 1; m.dims[1] = H; m.dims[2] = W;
+            m.tiles[0] = 1; m.tiles[1] = (H + 15) / 16; m.tiles[2] = (W + 15) / 16;
+        } else {
+            m.mode = 3;
+            m.dims[0] = (int)lead; m.dims[1] = H; m.dims[2] = W;
+            m.tiles[0] = (int)((lead + 3) / 4); m.tiles[1] = (H + 7) / 8; m.tiles[2] = (W + 7) / 8;
+        }
+        m.n_blocks = (unsigned)((size_t)m.tiles[0] * m.tiles[1] * m.tiles[2]);
+    }
+    if (N == 0) m.n_blocks = 0;
+    return m;
+}
+
 hipError_t clear_table(uint64_t *cell_keys, uint32_t n_cells, Counters *counters, hipStream_t s) {
     hipLaunchKernelGGL(k_clear_table, dim3(blocks_for(n_cells)), dim3(kBlock), 0, s, cell_keys,
                        n_cells, counters);
     return hipGetLastError();
 }
 
-hipError_t build(int pd, const float *positions, int N, const ScaleFactor &scale,
-                 uint64_t *cell_keys, int *cell_vertex, uint32_t n_cells, uint64_t *vertex_keys,
-                 Counters *counters, int *replay_index, float *replay_weight, hipStream_t s) {
-    if (N <= 0) return hipSuccess;
-    PLK_DISPATCH_PD(pd, hipLaunchKernelGGL(k_build<PD>, dim3(blocks_for((size_t)N)), dim3(kBlock), 0,
-                                           s, positions, N, scale, cell_keys, cell_vertex,
-                                           n_cells - 1u, vertex_keys, counters, replay_index,
-                                           replay_weight));
+hipError_t build(int pd, const float *positions, const PointMap &map, const ScaleFactor &scale,
+                 uint64_t *cell_keys, uint32_t n_cells, Counters *counters, int *replay_index,
+                 float *replay_weight, int xcd_aware, hipStream_t s) {
+    if (map.n_blocks == 0) return hipSuccess;
+    PLK_DISPATCH_PD(pd, hipLaunchKernelGGL(k_build<PD>, dim3(map.n_blocks), dim3(kBlock), 0, s,
+                                           positions, map, scale, cell_keys, n_cells - 1u, counters,
+                                           replay_index, replay_weight, xcd_aware));
+    return hipGetLastError();
+}
+
+hipError_t assign_vertex_ids(const uint64_t *cell_keys, uint32_t n_cells, int *cell_vertex,
+                             uint64_t *vertex_keys, Counters *counters, hipStream_t s) {
+    hipLaunchKernelGGL(k_assign_vertex_ids, dim3(blocks_for(n_cells, kIdBlock)), dim3(kIdBlock), 0, s,
+                       cell_keys, n_cells, cell_vertex, vertex_keys, counters);
     return hipGetLastError();
 }
 
@@ -582,27 +778,28 @@ hipError_t fill_zero(float *p, size_t n, hipStream_t s) {
     return hipGetLastError();
 }
 
-hipError_t splat(int pd, int vd, int N, const float *input, int in_channels, int *replay_index,
-                 const float *replay_weight, const int *cell_vertex, float *values, hipStream_t s) {
-    if (N <= 0) return hipSuccess;
+hipError_t splat(int pd, int vd, const PointMap &map, const float *input, int in_channels,
+                 int *replay_index, const float *replay_weight, const int *cell_vertex, float *values,
+                 int xcd_aware, hipStream_t s) {
+    if (map.n_blocks == 0) return hipSuccess;
     const int d1 = pd + 1;
-    const dim3 grid(blocks_for((size_t)N)), block(kBlock);
+    const dim3 grid(map.n_blocks), block(kBlock);
+    const size_t T = (size_t)map.n_blocks * kBlock;
 #define PLK_SPLAT(VD)                                                                             \
     case VD:                                                                                      \
-        hipLaunchKernelGGL(k_splat_point<VD>, grid, block, 0, s, d1, N, input, in_channels,       \
-                           replay_index, replay_weight, cell_vertex, values);                     \
+        hipLaunchKernelGGL(k_splat_point<VD>, grid, block, 0, s, d1, map, input, in_channels,     \
+                           replay_index, replay_weight, cell_vertex, values, xcd_aware);          \
         break;
     switch (vd) {
         PLK_SPLAT(2) PLK_SPLAT(3) PLK_SPLAT(4) PLK_SPLAT(5) PLK_SPLAT(6) PLK_SPLAT(7) PLK_SPLAT(8)
         default:
             if (cell_vertex) {
-                const size_t rows = (size_t)N * d1;
+                const size_t rows = T * d1;
                 hipLaunchKernelGGL(k_remap_replay, dim3(blocks_for(rows)), block, 0, s, rows,
                                    replay_index, cell_vertex);
             }
-            hipLaunchKernelGGL(k_splat_channel, dim3(blocks_for((size_t)N * vd)), block, 0, s, d1, vd,
-                               N, input, in_channels, replay_index, replay_weight,
-                               (const int *)nullptr, values);
+            hipLaunchKernelGGL(k_splat_channel, dim3(blocks_for(T * vd)), block, 0, s, d1, vd, map, T,
+                               input, in_channels, (const int *)replay_index, replay_weight, values);
             break;
     }
 #undef PLK_SPLAT
@@ -620,22 +817,24 @@ hipError_t blur_axis(int vd, int M, const float *src, float *dst, const int2 *nb
     return hipGetLastError();
 }
 
-hipError_t slice(int pd, int vd, int N, const int *replay_index, const float *replay_weight,
-                 const float *values, float *output, int normalize, hipStream_t s) {
-    if (N <= 0) return hipSuccess;
+hipError_t slice(int pd, int vd, const PointMap &map, const int *replay_index,
+                 const float *replay_weight, const float *values, float *output, int normalize,
+                 hipStream_t s) {
+    if (map.n_blocks == 0) return hipSuccess;
     const int d1 = pd + 1;
-    const dim3 grid(blocks_for((size_t)N)), block(kBlock);
+    const dim3 grid(map.n_blocks), block(kBlock);
+    const size_t T = (size_t)map.n_blocks * kBlock;
 #define PLK_SLICE(VD)                                                                          \
     case VD:                                                                                   \
-        hipLaunchKernelGGL(k_slice_point<VD>, grid, block, 0, s, d1, N, replay_index,          \
+        hipLaunchKernelGGL(k_slice_point<VD>, grid, block, 0, s, d1, map, replay_index,        \
                            replay_weight, values, output, normalize);                          \
         break;
     switch (vd) {
         PLK_SLICE(2) PLK_SLICE(3) PLK_SLICE(4) PLK_SLICE(5) PLK_SLICE(6) PLK_SLICE(7) PLK_SLICE(8)
         default: {
             const int out_ch = normalize ? vd - 1 : vd;
-            hipLaunchKernelGGL(k_slice_channel, dim3(blocks_for((size_t)N * out_ch)), block, 0, s, d1,
-                               vd, N, replay_index, replay_weight, values, output, normalize);
+            hipLaunchKernelGGL(k_slice_channel, dim3(blocks_for(T * out_ch)), block, 0, s, d1, vd, map,
+                               T, replay_index, replay_weight, values, output, normalize);
         } break;
     }
 #undef PLK_SLICE
@@ -655,6 +854,14 @@ hipError_t export_keys(int pd, const uint64_t *vertex_keys, int M, short *keys, 
     if (M <= 0) return hipSuccess;
     PLK_DISPATCH_PD(pd, hipLaunchKernelGGL(k_export_keys<PD>, dim3(blocks_for((size_t)M)),
                                            dim3(kBlock), 0, s, vertex_keys, M, keys));
+    return hipGetLastError();
+}
+
+hipError_t export_replay(int pd, const PointMap &map, const int *replay_index,
+                         const float *replay_weight, int *vertex, float *weight, hipStream_t s) {
+    if (map.n_blocks == 0) return hipSuccess;
+    hipLaunchKernelGGL(k_export_replay, dim3(map.n_blocks), dim3(kBlock), 0, s, pd + 1, map,
+                       replay_index, replay_weight, vertex, weight);
     return hipGetLastError();
 }
 

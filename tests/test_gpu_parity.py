@@ -182,6 +182,47 @@ def test_build_once_apply_many_equals_filter():
         assert_float_parity(host(out), want, scale=max(1.0, float(np.abs(want).max())))
 
 
+@pytest.mark.parametrize("dims,pd,vd", [((64, 64), 5, 4), ((37, 53), 5, 4), ((5, 300), 2, 2),
+                                         ((20, 24, 28), 4, 2), ((3, 9, 17, 21), 4, 3),
+                                         ((2, 50, 40), 5, 22), ((1, 1, 700), 3, 2)])
+def test_point_grid_hint_changes_nothing_but_the_order_of_work(dims, pd, vd):
+    """With the grid hint workgroups take 2-D / 3-D tiles (ragged at the edges here); integers,
+    vertex set, replay rows and outputs are those of the plain order and of the oracle."""
+    n = int(np.prod(dims))
+    rng = np.random.default_rng(sum(dims))
+    grids = np.meshgrid(*[np.arange(d, dtype=np.float32) for d in dims], indexing="ij")
+    spatial = np.stack([g.reshape(-1) for g in grids[-2:]], axis=1) / 4.0
+    extra = rng.uniform(0, 6, (n, pd - 2)).astype(np.float32)
+    pos = np.concatenate([spatial, extra], axis=1).astype(np.float32)
+    val = rng.uniform(0, 1, (n, vd - 1)).astype(np.float32)
+    cpu = oracle.Lattice(pd, vd, n)
+    want = cpu.filter(val, pos)
+    lat = pla.PermutohedralLattice(pd, vd, n)
+    plain, _ = gpu_filter(pd, vd, pos, val, lattice=lat)
+    lat.set_point_grid(dims)
+    tiled, _ = gpu_filter(pd, vd, pos, val, lattice=lat)
+    assert lat.num_vertices == cpu.num_vertices
+    assert (sorted_keys(host(lat.debug_keys()))[0] == sorted_keys(cpu.keys())[0]).all()
+    vertex, weight = (host(t) for t in lat.debug_replay())
+    o = oracle.dump_simplex(pos)
+    assert (host(lat.debug_keys())[vertex.T] == o["keys"]).all()
+    assert (bits(weight.T) == bits(o["barycentric"])).all()
+    assert_float_parity(tiled, want)
+    assert_float_parity(plain, want)
+    tiled_rev, _ = gpu_filter(pd, vd, pos, val, True, lattice=lat)
+    assert_float_parity(tiled_rev, oracle.Lattice(pd, vd, n).filter(val, pos, True))
+    lat.set_point_grid(None)
+    again, _ = gpu_filter(pd, vd, pos, val, lattice=lat)
+    assert_float_parity(again, want)
+
+
+def test_point_grid_must_match_the_number_of_points():
+    lat = pla.PermutohedralLattice(2, 2, 100)
+    with pytest.raises(pla.PermutohedralError) as e:
+        lat.set_point_grid((10, 11))
+    assert e.value.status == pla.PL_EINVAL
+
+
 def test_handle_is_reusable_and_each_filter_is_fresh():
     """The reference object is single-shot; here every filter() behaves as on a new lattice, also
     when the positions change between calls."""
