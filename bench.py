@@ -66,6 +66,8 @@ def main():
     out_f = torch.empty_like(d_val)
     out_r = torch.empty_like(d_val)
     lat = pla.PermutohedralLattice(pd, vd, n)
+    # what the op passes along with its tensors: the points are a side x side row-major grid
+    lat.set_point_grid((side, side))
 
     def step():
         lat.filter(out_f, d_val, d_pos, False)
@@ -83,6 +85,18 @@ def main():
     m = lat.num_vertices
     pixels_per_step = 2 * n
     value = pixels_per_step / (ms_per_step * 1e-3) / 1e6
+
+    # the same without the grid hint (a caller of filter() that only has N points)
+    lat.set_point_grid(None)
+    for _ in range(2):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    plain_ms = 1e3 * (time.perf_counter() - t0) / args.steps
+    lat.set_point_grid((side, side))
 
     # build once, apply forward and reverse (what a caller that keeps the lattice gets)
     lat.build(d_pos)
@@ -115,7 +129,8 @@ def main():
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 5),
                 "traffic": None, "algorithmic_bytes_per_launch": alg[dominant],
                 "launch_ms": round(per_launch_ms[dominant], 5)}
-    gpu_kernel_ms = sum(stages[k] for k in ("clear", "build", "neighbours", "fill", "splat", "blur", "slice"))
+    gpu_kernel_ms = sum(stages[k] for k in ("clear", "build", "ids", "neighbours", "fill", "splat",
+                                            "blur", "slice"))
     filter_gbs = 2 * alg["filter"] / (ms_per_step * 1e-3) / 1e9
 
     result = {
@@ -124,7 +139,8 @@ def main():
         "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4), "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "bilateral RGB %dx%d, pd=5 vd=4, theta 8/0.125, filter() forward + "
-                               "filter() reverse per step, positions given" % (side, side),
+                               "filter() reverse per step, positions given, grid hint set as the "
+                               "op sets it" % (side, side),
                    "pixels_per_step": pixels_per_step, "num_vertices": m},
         "roofline": roofline,
         "filter_roofline": {"algorithmic_bytes_per_step": 2 * alg["filter"],
@@ -132,6 +148,9 @@ def main():
                             "frac": round(filter_gbs / HBM_PEAK_GBS, 5)},
         "stage_ms": {k: round(v, 5) for k, v in stages.items()},
         "kernel_ms_per_filter": round(gpu_kernel_ms, 4),
+        "no_grid_hint": {"what": "same step, points treated as a plain list",
+                         "ms_per_step": round(plain_ms, 4),
+                         "value": round(pixels_per_step / (plain_ms * 1e-3) / 1e6, 3)},
         "reuse": {"what": "build once, apply forward + reverse per step",
                   "ms_per_step": round(reuse_ms, 4),
                   "value": round(pixels_per_step / (reuse_ms * 1e-3) / 1e6, 3)},

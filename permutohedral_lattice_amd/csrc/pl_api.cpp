@@ -1,5 +1,9 @@
 // Host side of the C ABI declared in include/permutohedral_lattice.h: the lattice object, its
 // scratch memory, the build/apply orchestration and the LatticeFilter op loop.
+//
+// A filter call enqueues its kernels back to back: the vertex count of the lattice stays on the
+// device (every later kernel reads it there, launched for an upper bound of vertices), so the
+// host waits once, at the end, to learn whether the hash table was large enough.
 #include "permutohedral_lattice.h"
 
 #include <hip/hip_runtime.h>
@@ -51,7 +55,7 @@ void compute_scale_factor(int pd, plk::ScaleFactor &sf) {
         sf.v[i] = (float)(1.0 / std::sqrt((double)((i + 1) * (i + 2))) * (double)inv_std_dev);
 }
 
-enum { EV_T0, EV_CLEAR, EV_BUILD, EV_IDS, EV_NBR0, EV_NBR, EV_A0, EV_FILL, EV_SPLAT, EV_BLUR, EV_SLICE, EV_COUNT };
+enum { EV_T0, EV_CLEAR, EV_BUILD, EV_IDS, EV_NBR, EV_A0, EV_FILL, EV_SPLAT, EV_BLUR, EV_SLICE, EV_COUNT };
 
 }  // namespace
 
@@ -62,33 +66,35 @@ struct pl_lattice {
     pl_alloc alloc{};
     plk::ScaleFactor scale{};
 
-    // hash table
-    uint64_t *cell_keys = nullptr;
-    int *cell_vertex = nullptr;
-    uint64_t *vertex_keys = nullptr;  // n_cells_alloc / 2 entries
-    uint32_t n_cells_alloc = 0;       // allocated
-    uint32_t n_cells = 0;             // in use by the last build
-    uint32_t max_cells = 0;           // enough for N*(pd+1) vertices at load 1/2
+    // hash table and the per-vertex arrays; a table of n_cells holds at most n_cells/2 vertices
+    uint64_t *cell_keys = nullptr;     // [n_cells_alloc]
+    int *cell_vertex = nullptr;        // [n_cells_alloc]
+    uint64_t *vertex_keys = nullptr;   // [n_cells_alloc/2]
+    int *vertex_cell = nullptr;        // [n_cells_alloc/2]
+    float *values[2] = {nullptr, nullptr};  // [n_cells_alloc/2 * vd]
+    int2 *neighbours = nullptr;        // [(pd+1) * n_cells_alloc/2]
+    uint32_t n_cells_alloc = 0;
+    uint32_t n_cells = 0;              // in use by the last build
+    uint32_t max_cells = 0;            // enough for N*(pd+1) vertices at load 1/2
     long forced_cells = 0;
-
-    // per-vertex arrays, sized after the build
-    float *values[2] = {nullptr, nullptr};
-    int2 *neighbours = nullptr;
-    size_t vertex_capacity = 0;
+    bool table_clean = false;          // every cell of [0, n_cells) is empty
 
     // per-point arrays, (pd+1) rows of map.n_blocks*256 entries in thread order
     plk::PointMap map{};
     int *replay_index = nullptr;
     float *replay_weight = nullptr;
-    size_t replay_capacity = 0;  // entries per array
+    size_t replay_capacity = 0;
 
-    plk::Counters *d_counters = nullptr;
-    plk::Counters *h_counters = nullptr;  // pinned
+    plk::Counters *d_counters = nullptr;   // two sets, used by alternate builds
+    int counter_set = 0;                   // the set of the last build
+    plk::HostStatus *h_status = nullptr;   // pinned, written by the device
 
     int M = 0;
     int last_M = -1;
-    bool built = false;
+    bool built = false;                // a build has been enqueued and, if verified, fitted
+    bool verified = false;             // its status has been read on the host
     bool replay_holds_cells = false;
+    bool values_zeroed = false;        // values[0] rows of all vertices are zero
     bool normalize = true;
     bool profile = false;
     bool xcd_aware = true;
@@ -96,60 +102,54 @@ struct pl_lattice {
     bool ev_recorded[EV_COUNT] = {};
 
     void *dmalloc(size_t bytes) { return alloc.alloc(alloc.ctx, bytes); }
-    void dfree(void *p) {
-        if (p) alloc.free(alloc.ctx, p);
+    template <typename T>
+    void dfree(T *&p) {
+        if (p) alloc.free(alloc.ctx, (void *)p);
+        p = nullptr;
     }
     void mark(int which) {
-        if (profile && ev[which]) {
-            ev_recorded[which] = hipEventRecord(ev[which], stream) == hipSuccess;
-        }
+        if (profile && ev[which]) ev_recorded[which] = hipEventRecord(ev[which], stream) == hipSuccess;
     }
+    plk::Counters *counters() { return d_counters + counter_set; }
+    int max_vertices() const { return (int)(n_cells / 2); }
 };
 
 namespace {
 
 int ensure_table(pl_lattice *h, uint32_t cells) {
     if (cells <= h->n_cells_alloc) return PL_OK;
+    // the old arrays may still be read by work in flight
+    PL_HIP(hipStreamSynchronize(h->stream));
     h->dfree(h->cell_keys);
     h->dfree(h->cell_vertex);
     h->dfree(h->vertex_keys);
-    h->cell_keys = nullptr;
-    h->cell_vertex = nullptr;
-    h->vertex_keys = nullptr;
-    h->n_cells_alloc = 0;
-    h->cell_keys = (uint64_t *)h->dmalloc(sizeof(uint64_t) * (size_t)cells);
-    h->cell_vertex = (int *)h->dmalloc(sizeof(int) * (size_t)cells);
-    h->vertex_keys = (uint64_t *)h->dmalloc(sizeof(uint64_t) * (size_t)(cells / 2));
-    if (!h->cell_keys || !h->cell_vertex || !h->vertex_keys) return PL_ENOMEM;
-    h->n_cells_alloc = cells;
-    return PL_OK;
-}
-
-int ensure_vertices(pl_lattice *h, size_t m) {
-    if (m <= h->vertex_capacity) return PL_OK;
-    size_t cap = h->vertex_capacity ? h->vertex_capacity : 1024;
-    while (cap < m) cap *= 2;
+    h->dfree(h->vertex_cell);
     h->dfree(h->values[0]);
     h->dfree(h->values[1]);
     h->dfree(h->neighbours);
-    h->values[0] = h->values[1] = nullptr;
-    h->neighbours = nullptr;
-    h->vertex_capacity = 0;
-    h->values[0] = (float *)h->dmalloc(sizeof(float) * cap * (size_t)h->vd);
-    h->values[1] = (float *)h->dmalloc(sizeof(float) * cap * (size_t)h->vd);
-    h->neighbours = (int2 *)h->dmalloc(sizeof(int2) * cap * (size_t)(h->pd + 1));
-    if (!h->values[0] || !h->values[1] || !h->neighbours) return PL_ENOMEM;
-    h->vertex_capacity = cap;
+    h->n_cells_alloc = 0;
+    h->table_clean = false;
+    const size_t mv = cells / 2;
+    h->cell_keys = (uint64_t *)h->dmalloc(sizeof(uint64_t) * (size_t)cells);
+    h->cell_vertex = (int *)h->dmalloc(sizeof(int) * (size_t)cells);
+    h->vertex_keys = (uint64_t *)h->dmalloc(sizeof(uint64_t) * mv);
+    h->vertex_cell = (int *)h->dmalloc(sizeof(int) * mv);
+    h->values[0] = (float *)h->dmalloc(sizeof(float) * mv * (size_t)h->vd);
+    h->values[1] = (float *)h->dmalloc(sizeof(float) * mv * (size_t)h->vd);
+    h->neighbours = (int2 *)h->dmalloc(sizeof(int2) * mv * (size_t)(h->pd + 1));
+    if (!h->cell_keys || !h->cell_vertex || !h->vertex_keys || !h->vertex_cell || !h->values[0] ||
+        !h->values[1] || !h->neighbours)
+        return PL_ENOMEM;
+    h->n_cells_alloc = cells;
     return PL_OK;
 }
 
 int ensure_replay(pl_lattice *h) {
     const size_t want = (size_t)h->map.n_blocks * 256 * (size_t)(h->pd + 1);
     if (want <= h->replay_capacity && h->replay_index) return PL_OK;
+    PL_HIP(hipStreamSynchronize(h->stream));
     h->dfree(h->replay_index);
     h->dfree(h->replay_weight);
-    h->replay_index = nullptr;
-    h->replay_weight = nullptr;
     h->replay_capacity = 0;
     h->replay_index = (int *)h->dmalloc(sizeof(int) * (want ? want : 1));
     h->replay_weight = (float *)h->dmalloc(sizeof(float) * (want ? want : 1));
@@ -171,6 +171,93 @@ uint32_t initial_cells(const pl_lattice *h) {
     uint32_t cells = pow2_at_least(want);
     if (cells > h->max_cells) cells = h->max_cells;
     return cells;
+}
+
+// Enqueue one build with a table of `cells` cells.  Nothing here waits for the device.
+int enqueue_build(pl_lattice *h, const float *positions, uint32_t cells) {
+    int rc = ensure_table(h, cells);
+    if (rc != PL_OK) return rc;
+    h->mark(EV_T0);
+    if (!h->table_clean || cells != h->n_cells) {
+        PL_HIP(plk::clear_table(h->cell_keys, cells, h->stream));
+    }
+    h->table_clean = false;
+    h->n_cells = cells;
+    h->mark(EV_CLEAR);
+    // the previous vertex-numbering kernel (or pl_create) left the other counter set zeroed
+    const int previous_set = h->counter_set;
+    h->counter_set = 1 - previous_set;
+    PL_HIP(plk::build(h->pd, positions, h->map, h->scale, h->cell_keys, cells, h->counters(),
+                      h->replay_index, h->replay_weight, h->xcd_aware ? 1 : 0, h->stream));
+    h->mark(EV_BUILD);
+    PL_HIP(plk::assign_vertex_ids(h->cell_keys, cells, h->cell_vertex, h->vertex_keys, h->vertex_cell,
+                                  h->values[0], h->vd, h->counters(), h->d_counters + previous_set,
+                                  h->h_status, h->stream));
+    h->mark(EV_IDS);
+    PL_HIP(plk::neighbours(h->pd, h->vertex_keys, h->counters(), h->max_vertices(), h->cell_keys,
+                           h->cell_vertex, cells, h->neighbours, h->stream));
+    h->mark(EV_NBR);
+    h->replay_holds_cells = true;
+    h->values_zeroed = true;
+    h->built = true;
+    h->verified = false;
+    return PL_OK;
+}
+
+int enqueue_apply(pl_lattice *h, float *output, const float *input, int reverse) {
+    const int pd = h->pd, vd = h->vd;
+    const int in_channels = h->normalize ? vd - 1 : vd;
+    const int mv = h->max_vertices();
+    h->mark(EV_A0);
+    if (!h->values_zeroed) PL_HIP(plk::fill_zero(h->values[0], (size_t)mv * vd, h->stream));
+    h->values_zeroed = false;
+    h->mark(EV_FILL);
+    PL_HIP(plk::splat(pd, vd, h->map, input, in_channels, h->replay_index, h->replay_weight,
+                      h->replay_holds_cells ? h->cell_vertex : nullptr, h->values[0],
+                      h->xcd_aware ? 1 : 0, h->stream));
+    h->replay_holds_cells = false;
+    h->mark(EV_SPLAT);
+    int cur = 0;
+    for (int step = 0; step <= pd; ++step) {
+        const int axis = reverse ? pd - step : step;
+        // the first blur after a build also empties the vertices' hash cells
+        const bool reset = !h->table_clean && step == 0;
+        PL_HIP(plk::blur_axis(vd, h->counters(), mv, h->values[cur], h->values[1 - cur],
+                              h->neighbours + (size_t)axis * mv, reset ? h->cell_keys : nullptr,
+                              h->vertex_cell, h->stream));
+        if (reset) h->table_clean = true;
+        cur = 1 - cur;
+    }
+    h->mark(EV_BLUR);
+    PL_HIP(plk::slice(pd, vd, h->map, h->replay_index, h->replay_weight, h->values[cur], output,
+                      h->normalize ? 1 : 0, h->stream));
+    h->mark(EV_SLICE);
+    return PL_OK;
+}
+
+// Wait for the stream and read what the last build reported.  PL_OK: it fitted, h->M is valid.
+// Otherwise *retry_cells is the table size to try next (0: give up with the returned status).
+int verify_build(pl_lattice *h, uint32_t *retry_cells) {
+    *retry_cells = 0;
+    PL_HIP(hipStreamSynchronize(h->stream));
+    const int flags = h->h_status->flags;
+    const int m = h->h_status->num_vertices;
+    if (flags & plk::kFlagKeyRange) {
+        h->built = false;
+        h->table_clean = false;
+        return PL_EOVERFLOW;
+    }
+    if ((flags & plk::kFlagTableFull) || (uint32_t)m > h->n_cells / 2) {
+        h->built = false;
+        h->table_clean = false;  // keys beyond the numbered vertices may remain
+        if (h->n_cells >= h->max_cells) return PL_EOVERFLOW;  // cannot happen: max_cells holds every vertex
+        *retry_cells = (h->n_cells > h->max_cells / 4) ? h->max_cells : h->n_cells * 4;
+        return PL_EOVERFLOW;
+    }
+    h->M = m;
+    h->last_M = m;
+    h->verified = true;
+    return PL_OK;
 }
 
 }  // namespace
@@ -219,21 +306,26 @@ int pl_create(int pd, int vd, int N, pl_stream stream, const pl_alloc *alloc, pl
     }
     compute_scale_factor(pd, h->scale);
     h->max_cells = pow2_at_least(rows * 2 < 4096 ? 4096 : rows * 2);
+    h->map = plk::make_point_map(N, 0, nullptr);
 
     int rc = PL_OK;
     if (hip_failed(hipGetDevice(&h->device))) rc = PL_EHIP;
-    h->map = plk::make_point_map(N, 0, nullptr);
     if (rc == PL_OK) rc = ensure_replay(h);
     if (rc == PL_OK) {
-        h->d_counters = (plk::Counters *)h->dmalloc(sizeof(plk::Counters));
+        h->d_counters = (plk::Counters *)h->dmalloc(2 * sizeof(plk::Counters));
         if (!h->d_counters) rc = PL_ENOMEM;
     }
-    if (rc == PL_OK && hip_failed(hipHostMalloc((void **)&h->h_counters, sizeof(plk::Counters), hipHostMallocDefault)))
+    if (rc == PL_OK && hip_failed(hipMemsetAsync(h->d_counters, 0, 2 * sizeof(plk::Counters), h->stream)))
+        rc = PL_EHIP;
+    if (rc == PL_OK &&
+        hip_failed(hipHostMalloc((void **)&h->h_status, sizeof(plk::HostStatus), hipHostMallocDefault)))
         rc = PL_EHIP;
     if (rc != PL_OK) {
         pl_destroy(h);
         return rc;
     }
+    h->h_status->num_vertices = 0;
+    h->h_status->flags = 0;
     *out = h;
     return PL_OK;
 }
@@ -244,13 +336,14 @@ int pl_destroy(pl_handle h) {
     h->dfree(h->cell_keys);
     h->dfree(h->cell_vertex);
     h->dfree(h->vertex_keys);
+    h->dfree(h->vertex_cell);
     h->dfree(h->values[0]);
     h->dfree(h->values[1]);
     h->dfree(h->neighbours);
     h->dfree(h->replay_index);
     h->dfree(h->replay_weight);
     h->dfree(h->d_counters);
-    if (h->h_counters) (void)hipHostFree(h->h_counters);
+    if (h->h_status) (void)hipHostFree(h->h_status);
     for (int i = 0; i < EV_COUNT; ++i)
         if (h->ev[i]) (void)hipEventDestroy(h->ev[i]);
     delete h;
@@ -304,91 +397,54 @@ int pl_build(pl_handle h, const float *positions) {
     h->M = 0;
     for (int i = 0; i <= EV_NBR; ++i) h->ev_recorded[i] = false;
     if (h->N == 0) {
-        h->built = true;
+        h->built = h->verified = true;
         return PL_OK;
     }
     uint32_t cells = initial_cells(h);
     for (;;) {
-        int rc = ensure_table(h, cells);
+        int rc = enqueue_build(h, positions, cells);
         if (rc != PL_OK) return rc;
-        h->mark(EV_T0);
-        PL_HIP(plk::clear_table(h->cell_keys, cells, h->d_counters, h->stream));
-        h->mark(EV_CLEAR);
-        PL_HIP(plk::build(h->pd, positions, h->map, h->scale, h->cell_keys, cells, h->d_counters,
-                          h->replay_index, h->replay_weight, h->xcd_aware ? 1 : 0, h->stream));
-        h->mark(EV_BUILD);
-        PL_HIP(plk::assign_vertex_ids(h->cell_keys, cells, h->cell_vertex, h->vertex_keys,
-                                      h->d_counters, h->stream));
-        h->mark(EV_IDS);
-        PL_HIP(hipMemcpyAsync(h->h_counters, h->d_counters, sizeof(plk::Counters),
-                              hipMemcpyDeviceToHost, h->stream));
-        PL_HIP(hipStreamSynchronize(h->stream));
-        const int flags = h->h_counters->flags;
-        if (flags & plk::kFlagKeyRange) return PL_EOVERFLOW;
-        if ((flags & plk::kFlagTableFull) || (uint32_t)h->h_counters->num_vertices > cells / 2) {
-            if (cells >= h->max_cells) return PL_EOVERFLOW;  // cannot happen: max_cells holds every vertex
-            cells = (cells > h->max_cells / 4) ? h->max_cells : cells * 4;
-            continue;
-        }
-        break;
+        rc = verify_build(h, &cells);
+        if (rc == PL_OK) return PL_OK;
+        if (!cells) return rc;
     }
-    h->n_cells = cells;
-    h->M = h->h_counters->num_vertices;
-    h->last_M = h->M;
-    int rc = ensure_vertices(h, (size_t)h->M);
-    if (rc != PL_OK) return rc;
-    h->mark(EV_NBR0);
-    PL_HIP(plk::neighbours(h->pd, h->vertex_keys, h->M, h->cell_keys, h->cell_vertex, h->n_cells,
-                           h->neighbours, h->stream));
-    h->mark(EV_NBR);
-    h->replay_holds_cells = true;
-    h->built = true;
-    return PL_OK;
 }
 
 int pl_apply(pl_handle h, float *output, const float *input, int reverse) {
     if (!h) return PL_EINVAL;
-    if (!h->built) return PL_ESTATE;
+    if (!h->built || !h->verified) return PL_ESTATE;
     if (h->N == 0) return PL_OK;
     if (!output || !input) return PL_EINVAL;
-    const int pd = h->pd, vd = h->vd, M = h->M;
-    const int in_channels = h->normalize ? vd - 1 : vd;
-
-    h->mark(EV_A0);
-    PL_HIP(plk::fill_zero(h->values[0], (size_t)M * vd, h->stream));
-    h->mark(EV_FILL);
-    PL_HIP(plk::splat(pd, vd, h->map, input, in_channels, h->replay_index, h->replay_weight,
-                      h->replay_holds_cells ? h->cell_vertex : nullptr, h->values[0],
-                      h->xcd_aware ? 1 : 0, h->stream));
-    h->replay_holds_cells = false;
-    h->mark(EV_SPLAT);
-
-    int cur = 0;
-    for (int step = 0; step <= pd; ++step) {
-        const int axis = reverse ? pd - step : step;
-        PL_HIP(plk::blur_axis(vd, M, h->values[cur], h->values[1 - cur],
-                              h->neighbours + (size_t)axis * M, h->stream));
-        cur = 1 - cur;
-    }
-    h->mark(EV_BLUR);
-
-    PL_HIP(plk::slice(pd, vd, h->map, h->replay_index, h->replay_weight, h->values[cur], output,
-                      h->normalize ? 1 : 0, h->stream));
-    h->mark(EV_SLICE);
-    return PL_OK;
+    return enqueue_apply(h, output, input, reverse);
 }
 
 int pl_filter(pl_handle h, float *output, const float *input, const float *positions, int reverse) {
     if (!h) return PL_EINVAL;
     if (h->N > 0 && (!output || !input || !positions)) return PL_EINVAL;
-    int rc = pl_build(h, positions);
-    if (rc != PL_OK) return rc;
-    return pl_apply(h, output, input, reverse);
+    h->built = false;
+    h->M = 0;
+    for (int i = 0; i < EV_COUNT; ++i) h->ev_recorded[i] = false;
+    if (h->N == 0) {
+        h->built = h->verified = true;
+        return PL_OK;
+    }
+    // build and apply are enqueued together; if the table turns out too small the whole call is
+    // repeated with a larger one (the output is simply written again)
+    uint32_t cells = initial_cells(h);
+    for (;;) {
+        int rc = enqueue_build(h, positions, cells);
+        if (rc != PL_OK) return rc;
+        rc = enqueue_apply(h, output, input, reverse);
+        if (rc != PL_OK) return rc;
+        rc = verify_build(h, &cells);
+        if (rc == PL_OK) return PL_OK;
+        if (!cells) return rc;
+    }
 }
 
 int pl_num_vertices(pl_handle h, int *num_vertices) {
     if (!h || !num_vertices) return PL_EINVAL;
-    if (!h->built) return PL_ESTATE;
+    if (!h->built || !h->verified) return PL_ESTATE;
     *num_vertices = h->M;
     return PL_OK;
 }
@@ -397,8 +453,8 @@ int pl_stage_ms(pl_handle h, float ms[8]) {
     if (!h || !ms) return PL_EINVAL;
     if (!h->profile) return PL_ESTATE;
     PL_HIP(hipStreamSynchronize(h->stream));
-    const int pairs[8][2] = {{EV_T0, EV_CLEAR},  {EV_CLEAR, EV_BUILD}, {EV_BUILD, EV_IDS},
-                             {EV_NBR0, EV_NBR},  {EV_A0, EV_FILL},     {EV_FILL, EV_SPLAT},
+    const int pairs[8][2] = {{EV_T0, EV_CLEAR},   {EV_CLEAR, EV_BUILD}, {EV_BUILD, EV_IDS},
+                             {EV_IDS, EV_NBR},    {EV_A0, EV_FILL},     {EV_FILL, EV_SPLAT},
                              {EV_SPLAT, EV_BLUR}, {EV_BLUR, EV_SLICE}};
     for (int i = 0; i < 8; ++i) {
         ms[i] = 0.0f;
@@ -418,14 +474,14 @@ int pl_debug_simplex(pl_handle h, const float *positions, short *rem0, short *ra
 
 int pl_debug_keys(pl_handle h, short *keys) {
     if (!h || !keys) return PL_EINVAL;
-    if (!h->built) return PL_ESTATE;
+    if (!h->built || !h->verified) return PL_ESTATE;
     PL_HIP(plk::export_keys(h->pd, h->vertex_keys, h->M, keys, h->stream));
     return PL_OK;
 }
 
 int pl_debug_replay(pl_handle h, int *vertex, float *weight) {
     if (!h) return PL_EINVAL;
-    if (!h->built || h->replay_holds_cells) return PL_ESTATE;
+    if (!h->built || !h->verified || h->replay_holds_cells) return PL_ESTATE;
     PL_HIP(plk::export_replay(h->pd, h->map, h->replay_index, h->replay_weight, vertex, weight,
                               h->stream));
     return PL_OK;
@@ -542,6 +598,7 @@ extern "C" int pl_lattice_filter_op(const float *input, const float *reference, 
         }
     }
 
+    // the op knows the spatial extents of its tensors: workgroups take tiles of the image
     rc = pl_set_point_grid(lattice, n_spatial_dims, spatial_dims);
     for (int b = 0; b < batch && rc == PL_OK; ++b) {
         const float *ref_b = ref_ch ? reference + (size_t)b * N * ref_ch : nullptr;

@@ -17,7 +17,17 @@ enum : int {
     kFlagKeyRange = 2,    // a lattice coordinate does not fit its field of the packed key
 };
 
+// Device-side state of one build.  Kernels after the build read the vertex count from here, so
+// the host never has to wait for it between launches.
 struct Counters {
+    unsigned long long vertices_and_blocks;  // low word: vertices numbered so far; high word:
+                                             // workgroups of the numbering kernel that are done
+    int flags;
+    int pad;
+};
+
+// What the last workgroup of the vertex-numbering kernel writes to pinned host memory.
+struct HostStatus {
     int num_vertices;
     int flags;
 };
@@ -45,8 +55,8 @@ int key_field_bits(int pd);
 // n_dims < 2 or dims == nullptr: no grid, consecutive points.
 PointMap make_point_map(int N, int n_dims, const int *dims);
 
-// Hash cells := empty, counters := 0.
-hipError_t clear_table(uint64_t *cell_keys, uint32_t n_cells, Counters *counters, hipStream_t s);
+// Hash cells := empty.
+hipError_t clear_table(uint64_t *cell_keys, uint32_t n_cells, hipStream_t s);
 
 // Stage 1+2: per point embed, enclosing simplex, barycentric weights, then insertion of the pd+1
 // vertex keys.  The replay arrays hold (pd+1) rows of T = map.n_blocks*256 entries in thread
@@ -57,13 +67,18 @@ hipError_t build(int pd, const float *positions, const PointMap &map, const Scal
                  float *replay_weight, int xcd_aware, hipStream_t s);
 
 // Every occupied cell draws a dense vertex index: cell_vertex[cell] := v, vertex_keys[v] := key,
-// counters->num_vertices := M.
+// vertex_cell[v] := cell, values[v*vd .. +vd) := 0, counters->num_vertices := M.  The last
+// workgroup copies M and the flags to *host_status and zeroes *next_counters.
 hipError_t assign_vertex_ids(const uint64_t *cell_keys, uint32_t n_cells, int *cell_vertex,
-                             uint64_t *vertex_keys, Counters *counters, hipStream_t s);
+                             uint64_t *vertex_keys, int *vertex_cell, float *values, int vd,
+                             Counters *counters, Counters *next_counters, HostStatus *host_status,
+                             hipStream_t s);
 
-// neighbours[a*M+v] := vertex indices of v's two neighbours along blur axis a (-1 = absent).
-hipError_t neighbours(int pd, const uint64_t *vertex_keys, int M, const uint64_t *cell_keys,
-                      const int *cell_vertex, uint32_t n_cells, int2 *neighbours, hipStream_t s);
+// neighbours[a*max_vertices+v] := vertex indices of v's two neighbours along blur axis a (-1 =
+// absent), for v < counters->num_vertices.
+hipError_t neighbours(int pd, const uint64_t *vertex_keys, const Counters *counters, int max_vertices,
+                      const uint64_t *cell_keys, const int *cell_vertex, uint32_t n_cells,
+                      int2 *neighbours, hipStream_t s);
 
 hipError_t fill_zero(float *p, size_t n, hipStream_t s);
 
@@ -74,9 +89,11 @@ hipError_t splat(int pd, int vd, const PointMap &map, const float *input, int in
                  int *replay_index, const float *replay_weight, const int *cell_vertex, float *values,
                  int xcd_aware, hipStream_t s);
 
-// Stage 4, one axis: dst[v] = 1/4 src[n1] + 1/2 src[v] + 1/4 src[n2].
-hipError_t blur_axis(int vd, int M, const float *src, float *dst, const int2 *neighbours_of_axis,
-                     hipStream_t s);
+// Stage 4, one axis: dst[v] = 1/4 src[n1] + 1/2 src[v] + 1/4 src[n2] for v < counters->num_vertices.
+// reset_cell_keys != nullptr: also empty the hash cell of every vertex (vertex_cell[v]).
+hipError_t blur_axis(int vd, const Counters *counters, int max_vertices, const float *src, float *dst,
+                     const int2 *neighbours_of_axis, uint64_t *reset_cell_keys,
+                     const int *vertex_cell, hipStream_t s);
 
 // Stage 5.  normalize: divide by the homogeneous channel and write vd-1 channels; else write vd.
 hipError_t slice(int pd, int vd, const PointMap &map, const int *replay_index,

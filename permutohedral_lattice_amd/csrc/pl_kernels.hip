@@ -222,32 +222,10 @@ __device__ __forceinline__ int point_of_thread(const PointMap &m, unsigned vbloc
 // Hash table
 // ------------------------------------------------------------------------------------------------
 
-// Returns the cell holding `key`, inserting it if absent; -1 and kFlagTableFull when no cell is
-// free.  Cells only ever change from empty to a key, so a stale read can at worst see "empty" and
-// the compare-and-swap then returns the truth.
-// `h` is the key's home cell and `cur` what a load of it returned (the caller issues the first
-// loads of all its keys together, so that their latencies overlap).
-__device__ __forceinline__ int table_insert(uint64_t *cell_keys, uint32_t mask, Counters *counters,
-                                            uint64_t key, uint32_t h, uint64_t cur) {
+__device__ __forceinline__ int table_find(const uint64_t *cell_keys, const int *cell_vertex,
+                                          uint32_t mask, uint64_t key, uint32_t h, uint64_t cur) {
     for (uint32_t probe = 0; probe <= mask; ++probe) {
         if (probe) cur = cell_keys[h];
-        if (cur == kEmptyCell) {
-            cur = atomicCAS((unsigned long long *)(cell_keys + h), (unsigned long long)kEmptyCell,
-                            (unsigned long long)key);
-            if (cur == kEmptyCell) return (int)h;
-        }
-        if (cur == key) return (int)h;
-        h = (h + 1u) & mask;
-    }
-    atomicOr(&counters->flags, kFlagTableFull);
-    return -1;
-}
-
-__device__ __forceinline__ int table_find(const uint64_t *cell_keys, const int *cell_vertex,
-                                          uint32_t mask, uint64_t key) {
-    uint32_t h = hash_key(key) & mask;
-    for (uint32_t probe = 0; probe <= mask; ++probe) {
-        const uint64_t cur = cell_keys[h];
         if (cur == key) return cell_vertex[h];
         if (cur == kEmptyCell) return -1;
         h = (h + 1u) & mask;
@@ -255,34 +233,31 @@ __device__ __forceinline__ int table_find(const uint64_t *cell_keys, const int *
     return -1;
 }
 
-__global__ __launch_bounds__(kBlock) void k_clear_table(uint64_t *cell_keys, uint32_t n_cells,
-                                                         Counters *counters) {
+__global__ __launch_bounds__(kBlock) void k_clear_table(uint64_t *cell_keys, uint32_t n_cells) {
     const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
     if (i < n_cells) cell_keys[i] = kEmptyCell;
-    if (i == 0) {
-        counters->num_vertices = 0;
-        counters->flags = 0;
-    }
+}
+
+__device__ __forceinline__ int lane_value(int x, int lane) { return __builtin_amdgcn_readlane(x, lane); }
+__device__ __forceinline__ uint64_t lane_value(uint64_t x, int lane) {
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)x, lane);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(x >> 32), lane);
+    return ((uint64_t)hi << 32) | lo;
 }
 
 // Lanes that hold the same value of `x` elect the lowest of them as leader.  Returns the leader's
-// lane and, in `members`, the lanes of the caller's group; inactive lanes get their own lane and
-// an empty group.  One iteration per distinct value in the wavefront.
+// lane; inactive lanes get their own.  One iteration per distinct value in the wavefront, each a
+// v_readlane of the first unassigned lane's value, a compare and a ballot.
 template <typename T>
-__device__ __forceinline__ int wave_leader_of_equal(T x, bool active, int lane, uint64_t &members) {
+__device__ __forceinline__ int wave_leader_of_equal(T x, bool active, int lane) {
     int leader = lane;
-    members = 0;
     uint64_t remaining = __ballot(active);
     while (remaining) {
         const int first = __builtin_ctzll(remaining);
-        const T k = __shfl(x, first);
+        const T k = lane_value(x, first);
         const bool same = active && x == k;
-        const uint64_t group = __ballot(same);
-        if (same) {
-            leader = first;
-            members = group;
-        }
-        remaining &= ~group;
+        if (same) leader = first;
+        remaining &= ~__ballot(same);
     }
     return leader;
 }
@@ -297,6 +272,7 @@ __global__ __launch_bounds__(kBlock) void k_build(const float *__restrict__ posi
                                                    int *__restrict__ replay_index,
                                                    float *__restrict__ replay_weight,
                                                    int xcd_aware) {
+    constexpr int D1 = PD + 1;
     const unsigned vblock = xcd_contiguous_block(blockIdx.x, gridDim.x, xcd_aware);
     const size_t t = (size_t)vblock * kBlock + threadIdx.x;   // slot in the replay arrays
     const size_t T = (size_t)gridDim.x * kBlock;
@@ -318,41 +294,76 @@ __global__ __launch_bounds__(kBlock) void k_build(const float *__restrict__ posi
 
     // Wavefront-level deduplication: each distinct key of the wavefront is inserted by one lane
     // (the lowest that holds it) and its cell is broadcast to the others.  Only leaders touch the
-    // table, and they load the home cells of all pd+1 keys before looking at any of them.
-    uint64_t key[PD + 1], home_value[PD + 1];
-    uint32_t home[PD + 1];
-    int leader[PD + 1];
+    // table.
+    uint64_t key[D1];
+    int leader[D1];
 #pragma unroll
-    for (int r = 0; r <= PD; ++r) {
+    for (int r = 0; r < D1; ++r) {
         int q[PD];
         vertex_q<PD>(s, r, q);
         key[r] = KeyCodec<PD>::pack(q, r);
-        uint64_t members;
-        leader[r] = wave_leader_of_equal(key[r], active, lane, members);
-        home[r] = hash_key(key[r]) & mask;
+        leader[r] = wave_leader_of_equal(key[r], active, lane);
     }
+
+    // Insertion of a lane's pd+1 keys proceeds in rounds over all of them at once, so that the
+    // loads and compare-and-swaps of one round are in flight together: a round loads the current
+    // cell of every unresolved key, swaps the key into the cells seen empty, and steps the
+    // keys that met another key to their next cell.  Cells only ever change from empty to a key,
+    // so a stale load can at worst report "empty" and the compare-and-swap returns the truth.
+    uint32_t cell[D1];
+    uint64_t seen[D1];
+    bool open[D1];
+    bool any_open = false;
 #pragma unroll
-    for (int r = 0; r <= PD; ++r)
-        home_value[r] = (active && leader[r] == lane) ? cell_keys[home[r]] : kEmptyCell;
+    for (int r = 0; r < D1; ++r) {
+        open[r] = active && leader[r] == lane;
+        cell[r] = hash_key(key[r]) & mask;
+        any_open = any_open || open[r];
+    }
+    for (uint32_t probe = 0; any_open && probe <= mask; ++probe) {
 #pragma unroll
-    for (int r = 0; r <= PD; ++r) {
-        int cell = -1;
-        if (active && leader[r] == lane)
-            cell = table_insert(cell_keys, mask, counters, key[r], home[r], home_value[r]);
-        cell = __shfl(cell, leader[r]);
-        replay_index[(size_t)r * T + t] = active ? cell : -1;
+        for (int r = 0; r < D1; ++r) seen[r] = open[r] ? cell_keys[cell[r]] : key[r];
+#pragma unroll
+        for (int r = 0; r < D1; ++r)
+            if (open[r] && seen[r] == kEmptyCell)
+                seen[r] = atomicCAS((unsigned long long *)(cell_keys + cell[r]),
+                                    (unsigned long long)kEmptyCell, (unsigned long long)key[r]);
+        any_open = false;
+#pragma unroll
+        for (int r = 0; r < D1; ++r) {
+            if (open[r]) {
+                if (seen[r] == kEmptyCell || seen[r] == key[r]) {
+                    open[r] = false;              // swapped in, or already there
+                } else {
+                    cell[r] = (cell[r] + 1u) & mask;
+                    any_open = true;
+                }
+            }
+        }
+    }
+    if (any_open) atomicOr(&counters->flags, kFlagTableFull);
+
+#pragma unroll
+    for (int r = 0; r < D1; ++r) {
+        int c = open[r] ? -1 : (int)cell[r];
+        c = __shfl(c, leader[r]);
+        replay_index[(size_t)r * T + t] = active ? c : -1;
         replay_weight[(size_t)r * T + t] = valid ? s.weight[r] : 0.0f;
     }
 }
 
 // Dense vertex numbering: every occupied cell draws an index.  One atomic per workgroup (counts are
 // combined by ballot inside a wavefront and through LDS across the workgroup), because thousands
-// of atomics on one address would serialise in a single L2 channel.
+// of atomics on one address would serialise in a single L2 channel.  That one 64-bit atomic adds
+// the workgroup's vertices to the low word and 1 to the high word, so the workgroup that reads
+// gridDim-1 in the high word knows it is the last and what the final count is, without a fence:
+// it publishes count and flags to host-visible memory and clears the counters the next build
+// will use.  The same pass zeroes each vertex's row of the value table.
 constexpr int kIdBlock = 1024;
-__global__ __launch_bounds__(kIdBlock) void k_assign_vertex_ids(const uint64_t *__restrict__ cell_keys,
-                                                                 uint32_t n_cells, int *cell_vertex,
-                                                                 uint64_t *vertex_keys,
-                                                                 Counters *counters) {
+__global__ __launch_bounds__(kIdBlock) void k_assign_vertex_ids(
+    const uint64_t *__restrict__ cell_keys, uint32_t n_cells, int *cell_vertex,
+    uint64_t *vertex_keys, int *vertex_cell, float *values, int vd, Counters *counters,
+    Counters *next_counters, HostStatus *host_status) {
     __shared__ int wave_count[kIdBlock / 64];
     __shared__ int block_base;
     const uint32_t cell = blockIdx.x * kIdBlock + threadIdx.x;
@@ -369,7 +380,17 @@ __global__ __launch_bounds__(kIdBlock) void k_assign_vertex_ids(const uint64_t *
             wave_count[w] = total;
             total += c;
         }
-        block_base = total ? atomicAdd(&counters->num_vertices, total) : 0;
+        const unsigned long long before = atomicAdd(
+            (unsigned long long *)&counters->vertices_and_blocks, (1ull << 32) | (unsigned)total);
+        block_base = (int)(uint32_t)before;
+        if ((uint32_t)(before >> 32) == gridDim.x - 1) {
+            const uint32_t m = (uint32_t)before + (uint32_t)total;
+            const int flags = atomicOr(&counters->flags, 0);
+            host_status->num_vertices = (int)m;
+            host_status->flags = flags | (m > n_cells / 2u ? kFlagTableFull : 0);
+            next_counters->vertices_and_blocks = 0;
+            next_counters->flags = 0;
+        }
     }
     __syncthreads();
     if (occupied) {
@@ -378,28 +399,36 @@ __global__ __launch_bounds__(kIdBlock) void k_assign_vertex_ids(const uint64_t *
         if ((uint32_t)v < n_cells / 2u) {
             cell_vertex[cell] = v;
             vertex_keys[v] = key;
+            vertex_cell[v] = (int)cell;
+            for (int j = 0; j < vd; ++j) values[(size_t)v * vd + j] = 0.0f;
         } else {
-            cell_vertex[cell] = 0;
-            atomicOr(&counters->flags, kFlagTableFull);
+            cell_vertex[cell] = 0;   // the host sees count > n_cells/2 and repeats with a larger table
         }
     }
+}
+
+__device__ __forceinline__ int vertex_count(const Counters *counters, int max_vertices) {
+    const uint32_t m = (uint32_t)counters->vertices_and_blocks;
+    return m < (uint32_t)max_vertices ? (int)m : max_vertices;
 }
 
 // ------------------------------------------------------------------------------------------------
 // Neighbour table: along axis a the neighbours of key k are k + (1,..,1) - (pd+1) e_a and its
 // mirror image (reference: src/PermutohedralLatticeCPU.h:381-388).  In (r, q) form the first is
 // r+1 with q_a-1, or, when r = pd, r = 0 with every q but q_a one higher; axis pd is the implicit
-// last coordinate, which no stored q belongs to.
+// last coordinate, which no stored q belongs to.  out[a*max_vertices + v].
 // ------------------------------------------------------------------------------------------------
 template <int PD>
 __global__ __launch_bounds__(kBlock) void k_neighbours(const uint64_t *__restrict__ vertex_keys,
-                                                        int M, const uint64_t *__restrict__ cell_keys,
+                                                        const Counters *counters, int max_vertices,
+                                                        const uint64_t *__restrict__ cell_keys,
                                                         const int *__restrict__ cell_vertex,
                                                         uint32_t mask, int2 *__restrict__ out) {
+    const int M = vertex_count(counters, max_vertices);
     const size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x;
-    if (t >= (size_t)M * (PD + 1)) return;
-    const int a = (int)(t / (size_t)M);
-    const int v = (int)(t - (size_t)a * M);
+    const int a = (int)(t / (size_t)max_vertices);
+    const int v = (int)(t - (size_t)a * max_vertices);
+    if (a > PD || v >= M) return;
 
     int q[PD], r;
     KeyCodec<PD>::unpack(vertex_keys[v], q, r);
@@ -414,8 +443,10 @@ __global__ __launch_bounds__(kBlock) void k_neighbours(const uint64_t *__restric
     }
     const uint64_t kp = KeyCodec<PD>::pack(qp, wrap_up ? 0 : r + 1);
     const uint64_t km = KeyCodec<PD>::pack(qm, wrap_down ? PD : r - 1);
-    out[t] = make_int2(table_find(cell_keys, cell_vertex, mask, kp),
-                       table_find(cell_keys, cell_vertex, mask, km));
+    const uint32_t hp = hash_key(kp) & mask, hm = hash_key(km) & mask;
+    const uint64_t cp = cell_keys[hp], cm = cell_keys[hm];   // both home cells in flight together
+    out[t] = make_int2(table_find(cell_keys, cell_vertex, mask, kp, hp, cp),
+                       table_find(cell_keys, cell_vertex, mask, km, hm, cm));
 }
 
 __global__ __launch_bounds__(kBlock) void k_fill_zero(float *p, size_t n) {
@@ -428,10 +459,144 @@ __global__ __launch_bounds__(kBlock) void k_fill_zero(float *p, size_t n) {
 //
 // What bounds it is the L2 atomic unit, which retires about 20 G requests per second on MI355X,
 // where a request is what one instruction sends to one 64-byte line, however many lanes it
-// carries.  So (a) the contributions of a wavefront to one vertex are first summed in LDS
-// (ds_add_f32) and (b) the sums are flushed with consecutive lanes on consecutive channels of a
+// carries.  So (a) the contributions of a wavefront to one vertex are summed before they leave
+// the wavefront and (b) the sums go out with consecutive lanes on consecutive channels of the
 // vertex, so that a vertex row costs one request and not vd.
 // ------------------------------------------------------------------------------------------------
+
+// x + (x of another lane, by DPP control), zero where the source lane does not exist or the row is
+// masked out
+template <int CTRL, int ROW_MASK = 0xf>
+__device__ __forceinline__ float add_from_lane(float x) {
+    const int other = __builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, ROW_MASK, 0xf, true);
+    return x + __int_as_float(other);
+}
+constexpr int kDppQuadSwap1 = 0xB1;   // quad_perm:[1,0,3,2]
+constexpr int kDppQuadSwap2 = 0x4E;   // quad_perm:[2,3,0,1]
+constexpr int kDppRowShr2 = 0x112, kDppRowShr4 = 0x114, kDppRowShr8 = 0x118;
+
+// Adds to the lanes of rows 1 and 3 (of 16 lanes) what the same lanes of rows 0 and 2 hold, then to
+// rows 2 and 3 what rows 0 and 1 hold: afterwards row 3 has the sum over the four rows, lane by
+// lane.  v_permlane16_swap / v_permlane32_swap are gfx950 instructions.
+__device__ __forceinline__ float add_rows_into_last(float x, int lane) {
+    const unsigned u = __float_as_uint(x);
+    const float from_even_row = __uint_as_float(__builtin_amdgcn_permlane16_swap(u, u, false, false)[0]);
+    if (lane & 16) x += from_even_row;
+    const unsigned w = __float_as_uint(x);
+    const float from_low_half = __uint_as_float(__builtin_amdgcn_permlane32_swap(w, w, false, false)[0]);
+    if (lane & 32) x += from_low_half;
+    return x;
+}
+
+// vd <= 4: all in registers.  The group loop of the deduplication doubles as the reduction loop:
+// for each distinct vertex of the wavefront the members' terms are reduce-scattered inside each
+// quad of lanes (lane keeps one channel), summed across the quads of a row and across the four rows,
+// and lanes 60..63 send the four channel sums of the vertex as one atomic instruction.
+template <int VD, int D1>
+__global__ __launch_bounds__(kBlock) void k_splat_dpp(PointMap map,
+                                                       const float *__restrict__ input,
+                                                       int in_channels, int *replay_index,
+                                                       const float *__restrict__ replay_weight,
+                                                       const int *__restrict__ cell_vertex,
+                                                       float *values, int xcd_aware) {
+    static_assert(VD >= 2 && VD <= 4, "register splat handles 2..4 channels");
+    constexpr int P = VD == 2 ? 2 : 4;   // lanes per vertex row in the final atomic
+    const unsigned vblock = xcd_contiguous_block(blockIdx.x, gridDim.x, xcd_aware);
+    const size_t t = (size_t)vblock * kBlock + threadIdx.x;
+    const size_t T = (size_t)gridDim.x * kBlock;
+    const int n = point_of_thread(map, vblock, threadIdx.x);
+    const int lane = threadIdx.x & 63;
+    const bool bit0 = lane & 1, bit1 = lane & 2;
+    // channel a lane ends up holding: quads keep (c0,c1 | c2,c3) by bit0, then first/second by bit1
+    const int my_channel = P == 2 ? (lane & 1) : (((lane & 1) << 1) | ((lane >> 1) & 1));
+
+    float val[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (int j = 0; j < VD; ++j) val[j] = 1.0f;  // homogeneous channel when only vd-1 are given
+    if (n >= 0) {
+#pragma unroll
+        for (int j = 0; j < VD; ++j)
+            if (j < in_channels) val[j] = input[(size_t)n * in_channels + j];
+    }
+
+    // all rows of the point at once, so that their latencies overlap
+    int vertex[D1];
+    float weight[D1];
+#pragma unroll
+    for (int r = 0; r < D1; ++r) {
+        vertex[r] = n >= 0 ? replay_index[(size_t)r * T + t] : -1;
+        weight[r] = replay_weight[(size_t)r * T + t];
+    }
+    if (cell_vertex) {
+#pragma unroll
+        for (int r = 0; r < D1; ++r)
+            if (vertex[r] >= 0) vertex[r] = cell_vertex[vertex[r]];
+#pragma unroll
+        for (int r = 0; r < D1; ++r)
+            if (n >= 0) replay_index[(size_t)r * T + t] = vertex[r];
+    }
+
+#pragma unroll
+    for (int r = 0; r < D1; ++r) {
+        const int v = vertex[r];
+        const float w = weight[r];
+        uint64_t remaining = __ballot(v >= 0);
+        while (remaining) {
+            const int first = __builtin_ctzll(remaining);
+            const int k = lane_value(v, first);
+            const bool same = v == k;
+            remaining &= ~__ballot(same);
+            float x0 = same ? w * val[0] : 0.0f, x1 = same ? w * val[1] : 0.0f;
+            float sum;
+            if (P == 2) {
+                const float keep = bit0 ? x1 : x0, send = bit0 ? x0 : x1;
+                sum = keep + __int_as_float(__builtin_amdgcn_update_dpp(
+                                 0, __float_as_int(send), kDppQuadSwap1, 0xf, 0xf, true));
+                sum = add_from_lane<kDppRowShr2>(sum);
+            } else {
+                float x2 = same ? w * val[2] : 0.0f, x3 = same ? w * val[3] : 0.0f;
+                const float keep_a = bit0 ? x2 : x0, keep_b = bit0 ? x3 : x1;
+                const float send_a = bit0 ? x0 : x2, send_b = bit0 ? x1 : x3;
+                const float ya = keep_a + __int_as_float(__builtin_amdgcn_update_dpp(
+                                              0, __float_as_int(send_a), kDppQuadSwap1, 0xf, 0xf, true));
+                const float yb = keep_b + __int_as_float(__builtin_amdgcn_update_dpp(
+                                              0, __float_as_int(send_b), kDppQuadSwap1, 0xf, 0xf, true));
+                const float keep = bit1 ? yb : ya, send = bit1 ? ya : yb;
+                sum = keep + __int_as_float(__builtin_amdgcn_update_dpp(
+                                 0, __float_as_int(send), kDppQuadSwap2, 0xf, 0xf, true));
+            }
+            sum = add_from_lane<kDppRowShr4>(sum);
+            sum = add_from_lane<kDppRowShr8>(sum);
+            sum = add_rows_into_last(sum, lane);
+            if (lane >= 64 - P && my_channel < VD)
+                atomicAdd(values + (size_t)k * VD + my_channel, sum);
+        }
+    }
+}
+
+// As wave_leader_of_equal, and also the lanes of the caller's group.
+template <typename T>
+__device__ __forceinline__ int wave_group_of_equal(T x, bool active, int lane, uint64_t &members) {
+    int leader = lane;
+    members = 0;
+    uint64_t remaining = __ballot(active);
+    while (remaining) {
+        const int first = __builtin_ctzll(remaining);
+        const T k = lane_value(x, first);
+        const bool same = active && x == k;
+        const uint64_t group = __ballot(same);
+        if (same) {
+            leader = first;
+            members = group;
+        }
+        remaining &= ~group;
+    }
+    return leader;
+}
+
+// vd 5..8: the terms of a wavefront go through LDS; lane e of the flush sums channel e % vd of
+// group e / vd over the group's lanes and sends one atomic, so the vd lanes of a group again hit
+// consecutive floats of one vertex row.
 template <int VD>
 __global__ __launch_bounds__(kBlock) void k_splat_point(int d1, PointMap map,
                                                          const float *__restrict__ input,
@@ -470,7 +635,7 @@ __global__ __launch_bounds__(kBlock) void k_splat_point(int d1, PointMap map,
         const bool active = v >= 0;
 
         uint64_t members;
-        const int leader = wave_leader_of_equal(v, active, lane, members);
+        const int leader = wave_group_of_equal(v, active, lane, members);
         const bool is_leader = active && leader == lane;
         const uint64_t leaders = __ballot(is_leader);
         const int groups = __builtin_popcountll(leaders);
@@ -532,21 +697,61 @@ __global__ __launch_bounds__(kBlock) void k_remap_replay(size_t rows, int *repla
 
 // ------------------------------------------------------------------------------------------------
 // Stage 4: blur along one axis (reference: src/PermutohedralLatticeCPU.h:403-405, evaluated in
-// double and rounded once, as there)
+// double and rounded once, as there).  The vertex count is read on the device.  The first blur
+// after a build also empties the hash cells of its vertices (reset_cell_keys != nullptr), which
+// leaves the table clean for the next build without a pass over all cells.
 // ------------------------------------------------------------------------------------------------
-template <int VD>
-__global__ __launch_bounds__(kBlock) void k_blur(int vd_runtime, int M, const float *__restrict__ src,
-                                                  float *__restrict__ dst,
-                                                  const int2 *__restrict__ nbr) {
-    const int vd = VD ? VD : vd_runtime;
+__device__ __forceinline__ float blur_tap(float a, float self, float b) {
+    return (float)(0.25 * (double)a + 0.5 * (double)self + 0.25 * (double)b);
+}
+
+// one thread per vertex, the row as one vector
+template <typename Vec, int VD>
+__global__ __launch_bounds__(kBlock) void k_blur_vertex(const Counters *counters, int max_vertices,
+                                                         const float *__restrict__ src,
+                                                         float *__restrict__ dst,
+                                                         const int2 *__restrict__ nbr,
+                                                         uint64_t *reset_cell_keys,
+                                                         const int *__restrict__ vertex_cell) {
+    const int M = vertex_count(counters, max_vertices);
+    const int v = blockIdx.x * kBlock + threadIdx.x;
+    if (v >= M) return;
+    const Vec *in = reinterpret_cast<const Vec *>(src);
+    const int2 nb = nbr[v];
+    Vec zero;
+    float *zf = reinterpret_cast<float *>(&zero);
+#pragma unroll
+    for (int j = 0; j < VD; ++j) zf[j] = 0.0f;
+    const Vec self = in[v];
+    const Vec a = nb.x >= 0 ? in[nb.x] : zero;
+    const Vec b = nb.y >= 0 ? in[nb.y] : zero;
+    Vec out;
+    const float *af = reinterpret_cast<const float *>(&a), *bf = reinterpret_cast<const float *>(&b),
+                *sf = reinterpret_cast<const float *>(&self);
+    float *of = reinterpret_cast<float *>(&out);
+#pragma unroll
+    for (int j = 0; j < VD; ++j) of[j] = blur_tap(af[j], sf[j], bf[j]);
+    reinterpret_cast<Vec *>(dst)[v] = out;
+    if (reset_cell_keys) reset_cell_keys[vertex_cell[v]] = kEmptyCell;
+}
+
+// one thread per (vertex, channel), any vd
+__global__ __launch_bounds__(kBlock) void k_blur_element(const Counters *counters, int max_vertices,
+                                                          int vd, const float *__restrict__ src,
+                                                          float *__restrict__ dst,
+                                                          const int2 *__restrict__ nbr,
+                                                          uint64_t *reset_cell_keys,
+                                                          const int *__restrict__ vertex_cell) {
+    const int M = vertex_count(counters, max_vertices);
     const size_t e = (size_t)blockIdx.x * kBlock + threadIdx.x;
     if (e >= (size_t)M * vd) return;
     const int v = (int)(e / (size_t)vd);
     const int j = (int)(e - (size_t)v * vd);
     const int2 nb = nbr[v];
-    const double a = nb.x >= 0 ? (double)src[(size_t)nb.x * vd + j] : 0.0;
-    const double b = nb.y >= 0 ? (double)src[(size_t)nb.y * vd + j] : 0.0;
-    dst[e] = (float)(0.25 * a + 0.5 * (double)src[e] + 0.25 * b);
+    const float a = nb.x >= 0 ? src[(size_t)nb.x * vd + j] : 0.0f;
+    const float b = nb.y >= 0 ? src[(size_t)nb.y * vd + j] : 0.0f;
+    dst[e] = blur_tap(a, src[e], b);
+    if (reset_cell_keys && j == 0) reset_cell_keys[vertex_cell[v]] = kEmptyCell;
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -740,9 +945,8 @@ PointMap make_point_map(int N, int n_dims, const int *dims) {
     return m;
 }
 
-hipError_t clear_table(uint64_t *cell_keys, uint32_t n_cells, Counters *counters, hipStream_t s) {
-    hipLaunchKernelGGL(k_clear_table, dim3(blocks_for(n_cells)), dim3(kBlock), 0, s, cell_keys,
-                       n_cells, counters);
+hipError_t clear_table(uint64_t *cell_keys, uint32_t n_cells, hipStream_t s) {
+    hipLaunchKernelGGL(k_clear_table, dim3(blocks_for(n_cells)), dim3(kBlock), 0, s, cell_keys, n_cells);
     return hipGetLastError();
 }
 
@@ -757,18 +961,23 @@ hipError_t build(int pd, const float *positions, const PointMap &map, const Scal
 }
 
 hipError_t assign_vertex_ids(const uint64_t *cell_keys, uint32_t n_cells, int *cell_vertex,
-                             uint64_t *vertex_keys, Counters *counters, hipStream_t s) {
+                             uint64_t *vertex_keys, int *vertex_cell, float *values, int vd,
+                             Counters *counters, Counters *next_counters, HostStatus *host_status,
+                             hipStream_t s) {
     hipLaunchKernelGGL(k_assign_vertex_ids, dim3(blocks_for(n_cells, kIdBlock)), dim3(kIdBlock), 0, s,
-                       cell_keys, n_cells, cell_vertex, vertex_keys, counters);
+                       cell_keys, n_cells, cell_vertex, vertex_keys, vertex_cell, values, vd, counters,
+                       next_counters, host_status);
     return hipGetLastError();
 }
 
-hipError_t neighbours(int pd, const uint64_t *vertex_keys, int M, const uint64_t *cell_keys,
-                      const int *cell_vertex, uint32_t n_cells, int2 *out, hipStream_t s) {
-    if (M <= 0) return hipSuccess;
-    PLK_DISPATCH_PD(pd, hipLaunchKernelGGL(k_neighbours<PD>, dim3(blocks_for((size_t)M * (PD + 1))),
-                                           dim3(kBlock), 0, s, vertex_keys, M, cell_keys,
-                                           cell_vertex, n_cells - 1u, out));
+hipError_t neighbours(int pd, const uint64_t *vertex_keys, const Counters *counters, int max_vertices,
+                      const uint64_t *cell_keys, const int *cell_vertex, uint32_t n_cells, int2 *out,
+                      hipStream_t s) {
+    if (max_vertices <= 0) return hipSuccess;
+    PLK_DISPATCH_PD(pd, hipLaunchKernelGGL(k_neighbours<PD>,
+                                           dim3(blocks_for((size_t)max_vertices * (PD + 1))),
+                                           dim3(kBlock), 0, s, vertex_keys, counters, max_vertices,
+                                           cell_keys, cell_vertex, n_cells - 1u, out));
     return hipGetLastError();
 }
 
@@ -785,13 +994,21 @@ hipError_t splat(int pd, int vd, const PointMap &map, const float *input, int in
     const int d1 = pd + 1;
     const dim3 grid(map.n_blocks), block(kBlock);
     const size_t T = (size_t)map.n_blocks * kBlock;
-#define PLK_SPLAT(VD)                                                                             \
+#define PLK_SPLAT(KERNEL, VD)                                                                    \
     case VD:                                                                                      \
-        hipLaunchKernelGGL(k_splat_point<VD>, grid, block, 0, s, d1, map, input, in_channels,     \
+        hipLaunchKernelGGL(KERNEL<VD>, grid, block, 0, s, d1, map, input, in_channels,            \
                            replay_index, replay_weight, cell_vertex, values, xcd_aware);          \
         break;
+#define PLK_SPLAT_DPP(VD)                                                                         \
+    case VD:                                                                                      \
+        PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_splat_dpp<VD, PD + 1>), grid, block, 0, s, map, \
+                                               input, in_channels, replay_index, replay_weight,   \
+                                               cell_vertex, values, xcd_aware));                  \
+        break;
     switch (vd) {
-        PLK_SPLAT(2) PLK_SPLAT(3) PLK_SPLAT(4) PLK_SPLAT(5) PLK_SPLAT(6) PLK_SPLAT(7) PLK_SPLAT(8)
+        PLK_SPLAT_DPP(2) PLK_SPLAT_DPP(3) PLK_SPLAT_DPP(4)
+        PLK_SPLAT(k_splat_point, 5) PLK_SPLAT(k_splat_point, 6) PLK_SPLAT(k_splat_point, 7)
+        PLK_SPLAT(k_splat_point, 8)
         default:
             if (cell_vertex) {
                 const size_t rows = T * d1;
@@ -803,16 +1020,24 @@ hipError_t splat(int pd, int vd, const PointMap &map, const float *input, int in
             break;
     }
 #undef PLK_SPLAT
+#undef PLK_SPLAT_DPP
     return hipGetLastError();
 }
 
-hipError_t blur_axis(int vd, int M, const float *src, float *dst, const int2 *nbr, hipStream_t s) {
-    if (M <= 0) return hipSuccess;
-    const dim3 grid(blocks_for((size_t)M * vd)), block(kBlock);
-    switch (vd) {
-        case 2: hipLaunchKernelGGL(k_blur<2>, grid, block, 0, s, vd, M, src, dst, nbr); break;
-        case 4: hipLaunchKernelGGL(k_blur<4>, grid, block, 0, s, vd, M, src, dst, nbr); break;
-        default: hipLaunchKernelGGL(k_blur<0>, grid, block, 0, s, vd, M, src, dst, nbr); break;
+hipError_t blur_axis(int vd, const Counters *counters, int max_vertices, const float *src, float *dst,
+                     const int2 *nbr, uint64_t *reset_cell_keys, const int *vertex_cell,
+                     hipStream_t s) {
+    if (max_vertices <= 0) return hipSuccess;
+    const dim3 block(kBlock);
+    if (vd == 2) {
+        hipLaunchKernelGGL((k_blur_vertex<float2, 2>), dim3(blocks_for((size_t)max_vertices)), block, 0,
+                           s, counters, max_vertices, src, dst, nbr, reset_cell_keys, vertex_cell);
+    } else if (vd == 4) {
+        hipLaunchKernelGGL((k_blur_vertex<float4, 4>), dim3(blocks_for((size_t)max_vertices)), block, 0,
+                           s, counters, max_vertices, src, dst, nbr, reset_cell_keys, vertex_cell);
+    } else {
+        hipLaunchKernelGGL(k_blur_element, dim3(blocks_for((size_t)max_vertices * vd)), block, 0, s,
+                           counters, max_vertices, vd, src, dst, nbr, reset_cell_keys, vertex_cell);
     }
     return hipGetLastError();
 }
