@@ -41,6 +41,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--size", type=int, default=1024, help="image side (default 1024)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and parity legs")
+    ap.add_argument("--calibrate-copy-mib", type=int, default=0,
+                    help="only run device-to-device copies of this many MiB (a kernel of known "
+                         "traffic, for scaling rocprofv3's FETCH_SIZE / WRITE_SIZE) and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on exactly one GPU (got --gpus %d); there is no "
@@ -53,6 +56,16 @@ def main():
     from permutohedral_lattice_amd import synth
 
     torch.cuda.set_device(0)
+    if args.calibrate_copy_mib:
+        nbytes = args.calibrate_copy_mib << 20
+        src = torch.arange(nbytes // 4, dtype=torch.float32, device="cuda")
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibration": "5 x dst.copy_(src), float32", "bytes_read_per_copy": nbytes,
+                          "bytes_written_per_copy": nbytes}))
+        return
     side = args.size
     n, pd, vd = side * side, 5, 4
     img = synth.blob_image(side, side, seed=0xC0FFEE)

@@ -129,8 +129,7 @@ int pl_debug_simplex(pl_handle h, const float *positions, short *rem0, short *ra
  * (HashTableCPU::getKeys(), src/PermutohedralLatticeCPU.h:154; the order is not the reference's). */
 int pl_debug_keys(pl_handle h, short *keys);
 
-/* Vertex index (0..M-1) and weight of each point's simplex vertices after the last pl_apply or
- * pl_filter: vertex[(pd+1)*N], weight[(pd+1)*N], laid out [r][n]; device pointers.  The replay
+/* Vertex index (0..M-1) and weight of each point's simplex vertices of the last build: vertex[(pd+1)*N], weight[(pd+1)*N], laid out [r][n]; device pointers.  The replay
  * matrix of src/PermutohedralLatticeCPU.h:187-191, 314-317. */
 int pl_debug_replay(pl_handle h, int *vertex, float *weight);
 

@@ -73,6 +73,8 @@ struct pl_lattice {
     int *vertex_cell = nullptr;        // [n_cells_alloc/2]
     float *values[2] = {nullptr, nullptr};  // [n_cells_alloc/2 * vd]
     int2 *neighbours = nullptr;        // [(pd+1) * n_cells_alloc/2]
+    float *cell_values = nullptr;      // [n_cells_alloc * vd], rows by hash cell (fused build+splat)
+    bool cell_values_clean = false;    // all zero
     uint32_t n_cells_alloc = 0;
     uint32_t n_cells = 0;              // in use by the last build
     uint32_t max_cells = 0;            // enough for N*(pd+1) vertices at load 1/2
@@ -95,6 +97,7 @@ struct pl_lattice {
     bool verified = false;             // its status has been read on the host
     bool replay_holds_cells = false;
     bool values_zeroed = false;        // values[0] rows of all vertices are zero
+    bool values_splatted = false;      // values[0] already holds the splat of the pending apply
     bool normalize = true;
     bool profile = false;
     bool xcd_aware = true;
@@ -127,8 +130,10 @@ int ensure_table(pl_lattice *h, uint32_t cells) {
     h->dfree(h->values[0]);
     h->dfree(h->values[1]);
     h->dfree(h->neighbours);
+    h->dfree(h->cell_values);
     h->n_cells_alloc = 0;
     h->table_clean = false;
+    h->cell_values_clean = false;
     const size_t mv = cells / 2;
     h->cell_keys = (uint64_t *)h->dmalloc(sizeof(uint64_t) * (size_t)cells);
     h->cell_vertex = (int *)h->dmalloc(sizeof(int) * (size_t)cells);
@@ -137,8 +142,10 @@ int ensure_table(pl_lattice *h, uint32_t cells) {
     h->values[0] = (float *)h->dmalloc(sizeof(float) * mv * (size_t)h->vd);
     h->values[1] = (float *)h->dmalloc(sizeof(float) * mv * (size_t)h->vd);
     h->neighbours = (int2 *)h->dmalloc(sizeof(int2) * mv * (size_t)(h->pd + 1));
+    if (plk::build_can_splat(h->vd))
+        h->cell_values = (float *)h->dmalloc(sizeof(float) * (size_t)cells * (size_t)h->vd);
     if (!h->cell_keys || !h->cell_vertex || !h->vertex_keys || !h->vertex_cell || !h->values[0] ||
-        !h->values[1] || !h->neighbours)
+        !h->values[1] || !h->neighbours || (plk::build_can_splat(h->vd) && !h->cell_values))
         return PL_ENOMEM;
     h->n_cells_alloc = cells;
     return PL_OK;
@@ -174,9 +181,16 @@ uint32_t initial_cells(const pl_lattice *h) {
 }
 
 // Enqueue one build with a table of `cells` cells.  Nothing here waits for the device.
-int enqueue_build(pl_lattice *h, const float *positions, uint32_t cells) {
+// splat_input != nullptr: the build kernel also splats these values (when it can for this vd),
+// and the value table holds them when the build is done.
+int enqueue_build(pl_lattice *h, const float *positions, uint32_t cells, const float *splat_input) {
     int rc = ensure_table(h, cells);
     if (rc != PL_OK) return rc;
+    const bool fused = splat_input && plk::build_can_splat(h->vd);
+    if (fused && !h->cell_values_clean) {
+        PL_HIP(plk::fill_zero(h->cell_values, (size_t)h->n_cells_alloc * h->vd, h->stream));
+        h->cell_values_clean = true;
+    }
     h->mark(EV_T0);
     if (!h->table_clean || cells != h->n_cells) {
         PL_HIP(plk::clear_table(h->cell_keys, cells, h->stream));
@@ -188,17 +202,20 @@ int enqueue_build(pl_lattice *h, const float *positions, uint32_t cells) {
     const int previous_set = h->counter_set;
     h->counter_set = 1 - previous_set;
     PL_HIP(plk::build(h->pd, positions, h->map, h->scale, h->cell_keys, cells, h->counters(),
-                      h->replay_index, h->replay_weight, h->xcd_aware ? 1 : 0, h->stream));
+                      h->replay_index, h->replay_weight, h->xcd_aware ? 1 : 0, fused ? h->vd : 0,
+                      splat_input, h->normalize ? h->vd - 1 : h->vd, h->cell_values, h->stream));
     h->mark(EV_BUILD);
     PL_HIP(plk::assign_vertex_ids(h->cell_keys, cells, h->cell_vertex, h->vertex_keys, h->vertex_cell,
-                                  h->values[0], h->vd, h->counters(), h->d_counters + previous_set,
-                                  h->h_status, h->stream));
+                                  h->values[0], h->vd, fused ? h->cell_values : nullptr,
+                                  h->counters(), h->d_counters + previous_set, h->h_status,
+                                  h->stream));
     h->mark(EV_IDS);
     PL_HIP(plk::neighbours(h->pd, h->vertex_keys, h->counters(), h->max_vertices(), h->cell_keys,
                            h->cell_vertex, cells, h->neighbours, h->stream));
     h->mark(EV_NBR);
     h->replay_holds_cells = true;
-    h->values_zeroed = true;
+    h->values_zeroed = !fused;
+    h->values_splatted = fused;
     h->built = true;
     h->verified = false;
     return PL_OK;
@@ -209,13 +226,18 @@ int enqueue_apply(pl_lattice *h, float *output, const float *input, int reverse)
     const int in_channels = h->normalize ? vd - 1 : vd;
     const int mv = h->max_vertices();
     h->mark(EV_A0);
-    if (!h->values_zeroed) PL_HIP(plk::fill_zero(h->values[0], (size_t)mv * vd, h->stream));
+    if (!h->values_splatted) {
+        if (!h->values_zeroed) PL_HIP(plk::fill_zero(h->values[0], (size_t)mv * vd, h->stream));
+        h->mark(EV_FILL);
+        PL_HIP(plk::splat(pd, vd, h->map, input, in_channels, h->replay_index, h->replay_weight,
+                          h->replay_holds_cells ? h->cell_vertex : nullptr, h->values[0],
+                          h->xcd_aware ? 1 : 0, h->stream));
+        h->replay_holds_cells = false;
+    } else {
+        h->mark(EV_FILL);
+    }
     h->values_zeroed = false;
-    h->mark(EV_FILL);
-    PL_HIP(plk::splat(pd, vd, h->map, input, in_channels, h->replay_index, h->replay_weight,
-                      h->replay_holds_cells ? h->cell_vertex : nullptr, h->values[0],
-                      h->xcd_aware ? 1 : 0, h->stream));
-    h->replay_holds_cells = false;
+    h->values_splatted = false;
     h->mark(EV_SPLAT);
     int cur = 0;
     for (int step = 0; step <= pd; ++step) {
@@ -229,7 +251,8 @@ int enqueue_apply(pl_lattice *h, float *output, const float *input, int reverse)
         cur = 1 - cur;
     }
     h->mark(EV_BLUR);
-    PL_HIP(plk::slice(pd, vd, h->map, h->replay_index, h->replay_weight, h->values[cur], output,
+    PL_HIP(plk::slice(pd, vd, h->map, h->replay_index, h->replay_weight,
+                      h->replay_holds_cells ? h->cell_vertex : nullptr, h->values[cur], output,
                       h->normalize ? 1 : 0, h->stream));
     h->mark(EV_SLICE);
     return PL_OK;
@@ -250,6 +273,7 @@ int verify_build(pl_lattice *h, uint32_t *retry_cells) {
     if ((flags & plk::kFlagTableFull) || (uint32_t)m > h->n_cells / 2) {
         h->built = false;
         h->table_clean = false;  // keys beyond the numbered vertices may remain
+        h->cell_values_clean = false;
         if (h->n_cells >= h->max_cells) return PL_EOVERFLOW;  // cannot happen: max_cells holds every vertex
         *retry_cells = (h->n_cells > h->max_cells / 4) ? h->max_cells : h->n_cells * 4;
         return PL_EOVERFLOW;
@@ -340,6 +364,7 @@ int pl_destroy(pl_handle h) {
     h->dfree(h->values[0]);
     h->dfree(h->values[1]);
     h->dfree(h->neighbours);
+    h->dfree(h->cell_values);
     h->dfree(h->replay_index);
     h->dfree(h->replay_weight);
     h->dfree(h->d_counters);
@@ -402,7 +427,7 @@ int pl_build(pl_handle h, const float *positions) {
     }
     uint32_t cells = initial_cells(h);
     for (;;) {
-        int rc = enqueue_build(h, positions, cells);
+        int rc = enqueue_build(h, positions, cells, nullptr);
         if (rc != PL_OK) return rc;
         rc = verify_build(h, &cells);
         if (rc == PL_OK) return PL_OK;
@@ -432,7 +457,7 @@ int pl_filter(pl_handle h, float *output, const float *input, const float *posit
     // repeated with a larger one (the output is simply written again)
     uint32_t cells = initial_cells(h);
     for (;;) {
-        int rc = enqueue_build(h, positions, cells);
+        int rc = enqueue_build(h, positions, cells, input);
         if (rc != PL_OK) return rc;
         rc = enqueue_apply(h, output, input, reverse);
         if (rc != PL_OK) return rc;
@@ -481,8 +506,9 @@ int pl_debug_keys(pl_handle h, short *keys) {
 
 int pl_debug_replay(pl_handle h, int *vertex, float *weight) {
     if (!h) return PL_EINVAL;
-    if (!h->built || !h->verified || h->replay_holds_cells) return PL_ESTATE;
-    PL_HIP(plk::export_replay(h->pd, h->map, h->replay_index, h->replay_weight, vertex, weight,
+    if (!h->built || !h->verified) return PL_ESTATE;
+    PL_HIP(plk::export_replay(h->pd, h->map, h->replay_index, h->replay_weight,
+                              h->replay_holds_cells ? h->cell_vertex : nullptr, vertex, weight,
                               h->stream));
     return PL_OK;
 }

@@ -62,17 +62,23 @@ hipError_t clear_table(uint64_t *cell_keys, uint32_t n_cells, hipStream_t s);
 // vertex keys.  The replay arrays hold (pd+1) rows of T = map.n_blocks*256 entries in thread
 // order: replay_index[r*T+t] := hash cell of vertex r of the point of thread t (-1: no point),
 // replay_weight likewise.
+// splat_vd != 0 (allowed when build_can_splat(vd)): the kernel also splats `input`
+// (in_channels per point) into cell_values[cell*vd ..], rows addressed by hash cell;
+// assign_vertex_ids then moves them into the dense value table.
+bool build_can_splat(int vd);
 hipError_t build(int pd, const float *positions, const PointMap &map, const ScaleFactor &scale,
                  uint64_t *cell_keys, uint32_t n_cells, Counters *counters, int *replay_index,
-                 float *replay_weight, int xcd_aware, hipStream_t s);
+                 float *replay_weight, int xcd_aware, int splat_vd, const float *input,
+                 int in_channels, float *cell_values, hipStream_t s);
 
 // Every occupied cell draws a dense vertex index: cell_vertex[cell] := v, vertex_keys[v] := key,
-// vertex_cell[v] := cell, values[v*vd .. +vd) := 0, counters->num_vertices := M.  The last
-// workgroup copies M and the flags to *host_status and zeroes *next_counters.
+// vertex_cell[v] := cell, the vertex count in *counters := M, and the vertex's row of `values` :=
+// 0, or, with cell_values != nullptr, := the row cell_values[cell*vd ..], which is zeroed.  The
+// last workgroup copies M and the flags to *host_status and zeroes *next_counters.
 hipError_t assign_vertex_ids(const uint64_t *cell_keys, uint32_t n_cells, int *cell_vertex,
                              uint64_t *vertex_keys, int *vertex_cell, float *values, int vd,
-                             Counters *counters, Counters *next_counters, HostStatus *host_status,
-                             hipStream_t s);
+                             float *cell_values, Counters *counters, Counters *next_counters,
+                             HostStatus *host_status, hipStream_t s);
 
 // neighbours[a*max_vertices+v] := vertex indices of v's two neighbours along blur axis a (-1 =
 // absent), for v < counters->num_vertices.
@@ -96,18 +102,21 @@ hipError_t blur_axis(int vd, const Counters *counters, int max_vertices, const f
                      const int *vertex_cell, hipStream_t s);
 
 // Stage 5.  normalize: divide by the homogeneous channel and write vd-1 channels; else write vd.
+// cell_vertex != nullptr: replay_index still holds hash cells (vd <= 8 only).
 hipError_t slice(int pd, int vd, const PointMap &map, const int *replay_index,
-                 const float *replay_weight, const float *values, float *output, int normalize,
-                 hipStream_t s);
+                 const float *replay_weight, const int *cell_vertex, const float *values,
+                 float *output, int normalize, hipStream_t s);
 
 hipError_t debug_simplex(int pd, const float *positions, int N, const ScaleFactor &scale,
                          short *rem0, short *rank, short *keys, float *barycentric, hipStream_t s);
 
 hipError_t export_keys(int pd, const uint64_t *vertex_keys, int M, short *keys, hipStream_t s);
 
-// replay arrays in point order: vertex[r*N+n], weight[r*N+n]
+// replay arrays in point order: vertex[r*N+n], weight[r*N+n]; cell_vertex != nullptr when
+// replay_index still holds hash cells
 hipError_t export_replay(int pd, const PointMap &map, const int *replay_index,
-                         const float *replay_weight, int *vertex, float *weight, hipStream_t s);
+                         const float *replay_weight, const int *cell_vertex, int *vertex,
+                         float *weight, hipStream_t s);
 
 hipError_t compute_positions(const float *reference, float *positions, int N, int n_ref_channels,
                              int n_spatial_dims, const SpatialDims &dims, float spatial_std,

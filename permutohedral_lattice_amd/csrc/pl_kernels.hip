@@ -263,15 +263,83 @@ __device__ __forceinline__ int wave_leader_of_equal(T x, bool active, int lane) 
 }
 
 // ------------------------------------------------------------------------------------------------
+// Wavefront reduction used by the splat
+// ------------------------------------------------------------------------------------------------
+// x + (x of another lane, by DPP control), zero where the source lane does not exist or the row is
+// masked out
+template <int CTRL, int ROW_MASK = 0xf>
+__device__ __forceinline__ float add_from_lane(float x) {
+    const int other = __builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, ROW_MASK, 0xf, true);
+    return x + __int_as_float(other);
+}
+constexpr int kDppQuadSwap1 = 0xB1;   // quad_perm:[1,0,3,2]
+constexpr int kDppQuadSwap2 = 0x4E;   // quad_perm:[2,3,0,1]
+constexpr int kDppRowShr2 = 0x112, kDppRowShr4 = 0x114, kDppRowShr8 = 0x118;
+
+// Adds to the lanes of rows 1 and 3 (of 16 lanes) what the same lanes of rows 0 and 2 hold, then to
+// rows 2 and 3 what rows 0 and 1 hold: afterwards row 3 has the sum over the four rows, lane by
+// lane.  v_permlane16_swap / v_permlane32_swap are gfx950 instructions.
+__device__ __forceinline__ float add_rows_into_last(float x, int lane) {
+    const unsigned u = __float_as_uint(x);
+    const float from_even_row = __uint_as_float(__builtin_amdgcn_permlane16_swap(u, u, false, false)[0]);
+    if (lane & 16) x += from_even_row;
+    const unsigned w = __float_as_uint(x);
+    const float from_low_half = __uint_as_float(__builtin_amdgcn_permlane32_swap(w, w, false, false)[0]);
+    if (lane & 32) x += from_low_half;
+    return x;
+}
+
+// Sum over the lanes with `member` set of term[0..VD) (VD <= 4), delivered channel-wise to the
+// last lanes of the wavefront: lane 64-P+i (P = 2 for VD == 2, else 4) returns the sum of channel
+// channel_of_lane(i).  The terms are reduce-scattered inside each quad of lanes (a lane keeps one
+// channel), then summed across the quads of a row and across the four rows.  All 64 lanes must
+// call it.
+template <int VD>
+__device__ __forceinline__ int channel_of_lane(int lane) {
+    return VD == 2 ? (lane & 1) : (((lane & 1) << 1) | ((lane >> 1) & 1));
+}
+template <int VD>
+__device__ __forceinline__ float wave_sum_to_last_lanes(bool member, const float (&term)[4], int lane) {
+    const bool bit0 = lane & 1, bit1 = lane & 2;
+    const float x0 = member ? term[0] : 0.0f, x1 = member ? term[1] : 0.0f;
+    float sum;
+    if (VD == 2) {
+        const float keep = bit0 ? x1 : x0, send = bit0 ? x0 : x1;
+        sum = keep + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(send),
+                                                                 kDppQuadSwap1, 0xf, 0xf, true));
+        sum = add_from_lane<kDppRowShr2>(sum);
+    } else {
+        const float x2 = member ? term[2] : 0.0f, x3 = member ? term[3] : 0.0f;
+        const float keep_a = bit0 ? x2 : x0, keep_b = bit0 ? x3 : x1;
+        const float send_a = bit0 ? x0 : x2, send_b = bit0 ? x1 : x3;
+        const float ya = keep_a + __int_as_float(__builtin_amdgcn_update_dpp(
+                                      0, __float_as_int(send_a), kDppQuadSwap1, 0xf, 0xf, true));
+        const float yb = keep_b + __int_as_float(__builtin_amdgcn_update_dpp(
+                                      0, __float_as_int(send_b), kDppQuadSwap1, 0xf, 0xf, true));
+        const float keep = bit1 ? yb : ya, send = bit1 ? ya : yb;
+        sum = keep + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(send),
+                                                                 kDppQuadSwap2, 0xf, 0xf, true));
+    }
+    sum = add_from_lane<kDppRowShr4>(sum);
+    sum = add_from_lane<kDppRowShr8>(sum);
+    return add_rows_into_last(sum, lane);
+}
+
+// ------------------------------------------------------------------------------------------------
 // Stage 1+2: embed, simplex, insert
 // ------------------------------------------------------------------------------------------------
-template <int PD>
+// SPLAT_VD != 0 (2..4): the kernel also splats.  The sums of each group of equal keys go, by one
+// atomic instruction per group, to the row of the key's CELL in cell_values (the vertices are not
+// numbered yet); the numbering pass moves the rows into the dense value table.  One kernel then
+// does the work of two, shares the deduplication between them and never reads the replay arrays.
+template <int PD, int SPLAT_VD>
 __global__ __launch_bounds__(kBlock) void k_build(const float *__restrict__ positions, PointMap map,
                                                    ScaleFactor scale, uint64_t *cell_keys,
                                                    uint32_t mask, Counters *counters,
                                                    int *__restrict__ replay_index,
                                                    float *__restrict__ replay_weight,
-                                                   int xcd_aware) {
+                                                   int xcd_aware, const float *__restrict__ input,
+                                                   int in_channels, float *cell_values) {
     constexpr int D1 = PD + 1;
     const unsigned vblock = xcd_contiguous_block(blockIdx.x, gridDim.x, xcd_aware);
     const size_t t = (size_t)vblock * kBlock + threadIdx.x;   // slot in the replay arrays
@@ -343,12 +411,39 @@ __global__ __launch_bounds__(kBlock) void k_build(const float *__restrict__ posi
     }
     if (any_open) atomicOr(&counters->flags, kFlagTableFull);
 
+    float val[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (SPLAT_VD) {
+#pragma unroll
+        for (int j = 0; j < SPLAT_VD; ++j) val[j] = 1.0f;  // homogeneous channel when vd-1 are given
+        if (valid) {
+#pragma unroll
+            for (int j = 0; j < SPLAT_VD; ++j)
+                if (j < in_channels) val[j] = input[(size_t)n * in_channels + j];
+        }
+    }
+
 #pragma unroll
     for (int r = 0; r < D1; ++r) {
-        int c = open[r] ? -1 : (int)cell[r];
-        c = __shfl(c, leader[r]);
+        const int own = open[r] ? -1 : (int)cell[r];
+        const int c = __shfl(own, leader[r]);
         replay_index[(size_t)r * T + t] = active ? c : -1;
         replay_weight[(size_t)r * T + t] = valid ? s.weight[r] : 0.0f;
+        if (SPLAT_VD) {
+            constexpr int VD = SPLAT_VD ? SPLAT_VD : 2;
+            constexpr int P = VD == 2 ? 2 : 4;
+            const float w = s.weight[r];
+            const float term[4] = {w * val[0], w * val[1], w * val[2], w * val[3]};
+            uint64_t remaining = __ballot(active);
+            while (remaining) {
+                const int first = __builtin_ctzll(remaining);
+                const bool same = active && leader[r] == first;
+                remaining &= ~__ballot(same);
+                const int group_cell = lane_value(own, first);
+                const float sum = wave_sum_to_last_lanes<VD>(same, term, lane);
+                if (group_cell >= 0 && lane >= 64 - P && channel_of_lane<VD>(lane) < VD)
+                    atomicAdd(cell_values + (size_t)group_cell * VD + channel_of_lane<VD>(lane), sum);
+            }
+        }
     }
 }
 
@@ -362,8 +457,8 @@ __global__ __launch_bounds__(kBlock) void k_build(const float *__restrict__ posi
 constexpr int kIdBlock = 1024;
 __global__ __launch_bounds__(kIdBlock) void k_assign_vertex_ids(
     const uint64_t *__restrict__ cell_keys, uint32_t n_cells, int *cell_vertex,
-    uint64_t *vertex_keys, int *vertex_cell, float *values, int vd, Counters *counters,
-    Counters *next_counters, HostStatus *host_status) {
+    uint64_t *vertex_keys, int *vertex_cell, float *values, int vd, float *cell_values,
+    Counters *counters, Counters *next_counters, HostStatus *host_status) {
     __shared__ int wave_count[kIdBlock / 64];
     __shared__ int block_base;
     const uint32_t cell = blockIdx.x * kIdBlock + threadIdx.x;
@@ -400,7 +495,15 @@ __global__ __launch_bounds__(kIdBlock) void k_assign_vertex_ids(
             cell_vertex[cell] = v;
             vertex_keys[v] = key;
             vertex_cell[v] = (int)cell;
-            for (int j = 0; j < vd; ++j) values[(size_t)v * vd + j] = 0.0f;
+            if (cell_values) {
+                // the fused build+splat accumulated by cell: move the row, leave zeros behind
+                for (int j = 0; j < vd; ++j) {
+                    values[(size_t)v * vd + j] = cell_values[(size_t)cell * vd + j];
+                    cell_values[(size_t)cell * vd + j] = 0.0f;
+                }
+            } else {
+                for (int j = 0; j < vd; ++j) values[(size_t)v * vd + j] = 0.0f;
+            }
         } else {
             cell_vertex[cell] = 0;   // the host sees count > n_cells/2 and repeats with a larger table
         }
@@ -464,30 +567,6 @@ __global__ __launch_bounds__(kBlock) void k_fill_zero(float *p, size_t n) {
 // vertex, so that a vertex row costs one request and not vd.
 // ------------------------------------------------------------------------------------------------
 
-// x + (x of another lane, by DPP control), zero where the source lane does not exist or the row is
-// masked out
-template <int CTRL, int ROW_MASK = 0xf>
-__device__ __forceinline__ float add_from_lane(float x) {
-    const int other = __builtin_amdgcn_update_dpp(0, __float_as_int(x), CTRL, ROW_MASK, 0xf, true);
-    return x + __int_as_float(other);
-}
-constexpr int kDppQuadSwap1 = 0xB1;   // quad_perm:[1,0,3,2]
-constexpr int kDppQuadSwap2 = 0x4E;   // quad_perm:[2,3,0,1]
-constexpr int kDppRowShr2 = 0x112, kDppRowShr4 = 0x114, kDppRowShr8 = 0x118;
-
-// Adds to the lanes of rows 1 and 3 (of 16 lanes) what the same lanes of rows 0 and 2 hold, then to
-// rows 2 and 3 what rows 0 and 1 hold: afterwards row 3 has the sum over the four rows, lane by
-// lane.  v_permlane16_swap / v_permlane32_swap are gfx950 instructions.
-__device__ __forceinline__ float add_rows_into_last(float x, int lane) {
-    const unsigned u = __float_as_uint(x);
-    const float from_even_row = __uint_as_float(__builtin_amdgcn_permlane16_swap(u, u, false, false)[0]);
-    if (lane & 16) x += from_even_row;
-    const unsigned w = __float_as_uint(x);
-    const float from_low_half = __uint_as_float(__builtin_amdgcn_permlane32_swap(w, w, false, false)[0]);
-    if (lane & 32) x += from_low_half;
-    return x;
-}
-
 // vd <= 4: all in registers.  The group loop of the deduplication doubles as the reduction loop:
 // for each distinct vertex of the wavefront the members' terms are reduce-scattered inside each
 // quad of lanes (lane keeps one channel), summed across the quads of a row and across the four rows,
@@ -506,9 +585,7 @@ __global__ __launch_bounds__(kBlock) void k_splat_dpp(PointMap map,
     const size_t T = (size_t)gridDim.x * kBlock;
     const int n = point_of_thread(map, vblock, threadIdx.x);
     const int lane = threadIdx.x & 63;
-    const bool bit0 = lane & 1, bit1 = lane & 2;
-    // channel a lane ends up holding: quads keep (c0,c1 | c2,c3) by bit0, then first/second by bit1
-    const int my_channel = P == 2 ? (lane & 1) : (((lane & 1) << 1) | ((lane >> 1) & 1));
+    const int my_channel = channel_of_lane<VD>(lane);
 
     float val[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
@@ -546,28 +623,8 @@ __global__ __launch_bounds__(kBlock) void k_splat_dpp(PointMap map,
             const int k = lane_value(v, first);
             const bool same = v == k;
             remaining &= ~__ballot(same);
-            float x0 = same ? w * val[0] : 0.0f, x1 = same ? w * val[1] : 0.0f;
-            float sum;
-            if (P == 2) {
-                const float keep = bit0 ? x1 : x0, send = bit0 ? x0 : x1;
-                sum = keep + __int_as_float(__builtin_amdgcn_update_dpp(
-                                 0, __float_as_int(send), kDppQuadSwap1, 0xf, 0xf, true));
-                sum = add_from_lane<kDppRowShr2>(sum);
-            } else {
-                float x2 = same ? w * val[2] : 0.0f, x3 = same ? w * val[3] : 0.0f;
-                const float keep_a = bit0 ? x2 : x0, keep_b = bit0 ? x3 : x1;
-                const float send_a = bit0 ? x0 : x2, send_b = bit0 ? x1 : x3;
-                const float ya = keep_a + __int_as_float(__builtin_amdgcn_update_dpp(
-                                              0, __float_as_int(send_a), kDppQuadSwap1, 0xf, 0xf, true));
-                const float yb = keep_b + __int_as_float(__builtin_amdgcn_update_dpp(
-                                              0, __float_as_int(send_b), kDppQuadSwap1, 0xf, 0xf, true));
-                const float keep = bit1 ? yb : ya, send = bit1 ? ya : yb;
-                sum = keep + __int_as_float(__builtin_amdgcn_update_dpp(
-                                 0, __float_as_int(send), kDppQuadSwap2, 0xf, 0xf, true));
-            }
-            sum = add_from_lane<kDppRowShr4>(sum);
-            sum = add_from_lane<kDppRowShr8>(sum);
-            sum = add_rows_into_last(sum, lane);
+            const float term[4] = {w * val[0], w * val[1], w * val[2], w * val[3]};
+            const float sum = wave_sum_to_last_lanes<VD>(same, term, lane);
             if (lane >= 64 - P && my_channel < VD)
                 atomicAdd(values + (size_t)k * VD + my_channel, sum);
         }
@@ -757,10 +814,12 @@ __global__ __launch_bounds__(kBlock) void k_blur_element(const Counters *counter
 // ------------------------------------------------------------------------------------------------
 // Stage 5: slice (reference: src/PermutohedralLatticeCPU.h:333-352)
 // ------------------------------------------------------------------------------------------------
+// cell_vertex != nullptr: the replay rows still hold hash cells (nothing has translated them yet)
 template <int VD>
 __global__ __launch_bounds__(kBlock) void k_slice_point(int d1, PointMap map,
                                                          const int *__restrict__ replay_index,
                                                          const float *__restrict__ replay_weight,
+                                                         const int *__restrict__ cell_vertex,
                                                          const float *__restrict__ values,
                                                          float *__restrict__ output, int normalize) {
     const size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x;
@@ -771,8 +830,9 @@ __global__ __launch_bounds__(kBlock) void k_slice_point(int d1, PointMap map,
 #pragma unroll
     for (int j = 0; j < VD; ++j) acc[j] = 0.0f;
     for (int r = 0; r < d1; ++r) {
-        const int v = replay_index[(size_t)r * T + t];
+        int v = replay_index[(size_t)r * T + t];
         if (v < 0) continue;
+        if (cell_vertex) v = cell_vertex[v];
         const float w = replay_weight[(size_t)r * T + t];
         const float *src = values + (size_t)v * VD;
 #pragma unroll
@@ -861,17 +921,23 @@ __global__ __launch_bounds__(kBlock) void k_export_keys(const uint64_t *__restri
     for (int i = 0; i < PD; ++i) keys[(size_t)v * PD + i] = (short)(q[i] * (PD + 1) + r);
 }
 
-// replay arrays from thread order to point order: out[r*N + n]
+// replay arrays from thread order to point order: out[r*N + n]; cells are translated to vertex
+// indices when cell_vertex != nullptr
 __global__ __launch_bounds__(kBlock) void k_export_replay(int d1, PointMap map,
                                                            const int *__restrict__ replay_index,
                                                            const float *__restrict__ replay_weight,
+                                                           const int *__restrict__ cell_vertex,
                                                            int *vertex, float *weight) {
     const size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x;
     const size_t T = (size_t)gridDim.x * kBlock;
     const int n = point_of_thread(map, blockIdx.x, threadIdx.x);
     if (n < 0) return;
     for (int r = 0; r < d1; ++r) {
-        if (vertex) vertex[(size_t)r * map.N + n] = replay_index[(size_t)r * T + t];
+        if (vertex) {
+            int v = replay_index[(size_t)r * T + t];
+            if (cell_vertex && v >= 0) v = cell_vertex[v];
+            vertex[(size_t)r * map.N + n] = v;
+        }
         if (weight) weight[(size_t)r * map.N + n] = replay_weight[(size_t)r * T + t];
     }
 }
@@ -950,23 +1016,36 @@ hipError_t clear_table(uint64_t *cell_keys, uint32_t n_cells, hipStream_t s) {
     return hipGetLastError();
 }
 
+bool build_can_splat(int vd) { return vd >= 2 && vd <= 4; }
+
 hipError_t build(int pd, const float *positions, const PointMap &map, const ScaleFactor &scale,
                  uint64_t *cell_keys, uint32_t n_cells, Counters *counters, int *replay_index,
-                 float *replay_weight, int xcd_aware, hipStream_t s) {
+                 float *replay_weight, int xcd_aware, int splat_vd, const float *input,
+                 int in_channels, float *cell_values, hipStream_t s) {
     if (map.n_blocks == 0) return hipSuccess;
-    PLK_DISPATCH_PD(pd, hipLaunchKernelGGL(k_build<PD>, dim3(map.n_blocks), dim3(kBlock), 0, s,
-                                           positions, map, scale, cell_keys, n_cells - 1u, counters,
-                                           replay_index, replay_weight, xcd_aware));
+#define PLK_BUILD(SPLAT_VD)                                                                        \
+    PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_build<PD, SPLAT_VD>), dim3(map.n_blocks),            \
+                                           dim3(kBlock), 0, s, positions, map, scale, cell_keys,   \
+                                           n_cells - 1u, counters, replay_index, replay_weight,    \
+                                           xcd_aware, input, in_channels, cell_values))
+    switch (splat_vd) {
+        case 0: PLK_BUILD(0); break;
+        case 2: PLK_BUILD(2); break;
+        case 3: PLK_BUILD(3); break;
+        case 4: PLK_BUILD(4); break;
+        default: return hipErrorInvalidValue;
+    }
+#undef PLK_BUILD
     return hipGetLastError();
 }
 
 hipError_t assign_vertex_ids(const uint64_t *cell_keys, uint32_t n_cells, int *cell_vertex,
                              uint64_t *vertex_keys, int *vertex_cell, float *values, int vd,
-                             Counters *counters, Counters *next_counters, HostStatus *host_status,
-                             hipStream_t s) {
+                             float *cell_values, Counters *counters, Counters *next_counters,
+                             HostStatus *host_status, hipStream_t s) {
     hipLaunchKernelGGL(k_assign_vertex_ids, dim3(blocks_for(n_cells, kIdBlock)), dim3(kIdBlock), 0, s,
-                       cell_keys, n_cells, cell_vertex, vertex_keys, vertex_cell, values, vd, counters,
-                       next_counters, host_status);
+                       cell_keys, n_cells, cell_vertex, vertex_keys, vertex_cell, values, vd,
+                       cell_values, counters, next_counters, host_status);
     return hipGetLastError();
 }
 
@@ -1043,8 +1122,8 @@ hipError_t blur_axis(int vd, const Counters *counters, int max_vertices, const f
 }
 
 hipError_t slice(int pd, int vd, const PointMap &map, const int *replay_index,
-                 const float *replay_weight, const float *values, float *output, int normalize,
-                 hipStream_t s) {
+                 const float *replay_weight, const int *cell_vertex, const float *values,
+                 float *output, int normalize, hipStream_t s) {
     if (map.n_blocks == 0) return hipSuccess;
     const int d1 = pd + 1;
     const dim3 grid(map.n_blocks), block(kBlock);
@@ -1052,7 +1131,7 @@ hipError_t slice(int pd, int vd, const PointMap &map, const int *replay_index,
 #define PLK_SLICE(VD)                                                                          \
     case VD:                                                                                   \
         hipLaunchKernelGGL(k_slice_point<VD>, grid, block, 0, s, d1, map, replay_index,        \
-                           replay_weight, values, output, normalize);                          \
+                           replay_weight, cell_vertex, values, output, normalize);             \
         break;
     switch (vd) {
         PLK_SLICE(2) PLK_SLICE(3) PLK_SLICE(4) PLK_SLICE(5) PLK_SLICE(6) PLK_SLICE(7) PLK_SLICE(8)
@@ -1083,10 +1162,11 @@ hipError_t export_keys(int pd, const uint64_t *vertex_keys, int M, short *keys, 
 }
 
 hipError_t export_replay(int pd, const PointMap &map, const int *replay_index,
-                         const float *replay_weight, int *vertex, float *weight, hipStream_t s) {
+                         const float *replay_weight, const int *cell_vertex, int *vertex,
+                         float *weight, hipStream_t s) {
     if (map.n_blocks == 0) return hipSuccess;
     hipLaunchKernelGGL(k_export_replay, dim3(map.n_blocks), dim3(kBlock), 0, s, pd + 1, map,
-                       replay_index, replay_weight, vertex, weight);
+                       replay_index, replay_weight, cell_vertex, vertex, weight);
     return hipGetLastError();
 }
 
