@@ -47,6 +47,27 @@ def build(verbose=False):
     return LIB_PATH
 
 
+CPP_DRIVER_SRC = os.path.join(_ROOT, "tests", "cpp", "compare_cpu_and_gpu.cpp")
+CPP_DRIVER_BIN = os.path.join(_ROOT, "tests", "cpp", "compare_cpu_and_gpu.bin")
+
+
+def build_cpp_driver(verbose=False):
+    """The C++ CPU-vs-GPU comparison driver (tests/cpp), linked against the HIP library and the
+    CPU oracle; both are found through rpath entries relative to the binary."""
+    oracle_dir = os.path.join(_ROOT, "oracle")
+    cmd = [hipcc(), "-O2", "-std=c++17", "-Wno-unused-command-line-argument",
+           "-I" + os.path.join(_ROOT, "include"), "-I" + oracle_dir, CPP_DRIVER_SRC,
+           "-L" + _HERE, "-lpermutohedral_hip", "-L" + oracle_dir, "-loracle",
+           "-Wl,-rpath,$ORIGIN/../../permutohedral_lattice_amd", "-Wl,-rpath,$ORIGIN/../../oracle",
+           "-o", CPP_DRIVER_BIN]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + res.stdout)
+    return CPP_DRIVER_BIN
+
+
 if __name__ == "__main__":
     print(build(verbose=True))
     sys.exit(0)
