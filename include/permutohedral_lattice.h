@@ -53,8 +53,10 @@ typedef enum pl_option {
                               vd channels and nothing is divided -- the bare linear operator, for tests. */
     PL_OPT_PROFILE = 2,    /* 1: record per-stage HIP events, read with pl_stage_ms */
     PL_OPT_TABLE_CELLS = 3, /* force the initial number of hash cells (power of two), 0 = automatic */
-    PL_OPT_XCD_AWARE = 4    /* 1 (default): kernels with atomic updates give each XCD a contiguous range
+    PL_OPT_XCD_AWARE = 4,   /* 1 (default): kernels with atomic updates give each XCD a contiguous range
                                of points; 0: plain workgroup order (for measuring the difference) */
+    PL_OPT_PAIR_BLUR = 5    /* 1 (default): two blur axes per kernel launch; 0: one launch per axis
+                               (same results bit for bit; for measuring the difference) */
 } pl_option;
 
 /* 1 when a lattice can be built for these dimensions, else 0.

@@ -101,6 +101,7 @@ struct pl_lattice {
     bool normalize = true;
     bool profile = false;
     bool xcd_aware = true;
+    bool pair_blur = true;
     hipEvent_t ev[EV_COUNT] = {};
     bool ev_recorded[EV_COUNT] = {};
 
@@ -240,13 +241,23 @@ int enqueue_apply(pl_lattice *h, float *output, const float *input, int reverse)
     h->values_splatted = false;
     h->mark(EV_SPLAT);
     int cur = 0;
-    for (int step = 0; step <= pd; ++step) {
+    for (int step = 0; step <= pd;) {
+        // axes 0..pd, or pd..0 for the reverse pass; two per launch while two are left
         const int axis = reverse ? pd - step : step;
         // the first blur after a build also empties the vertices' hash cells
-        const bool reset = !h->table_clean && step == 0;
-        PL_HIP(plk::blur_axis(vd, h->counters(), mv, h->values[cur], h->values[1 - cur],
-                              h->neighbours + (size_t)axis * mv, reset ? h->cell_keys : nullptr,
-                              h->vertex_cell, h->stream));
+        uint64_t *reset = (!h->table_clean && step == 0) ? h->cell_keys : nullptr;
+        if (h->pair_blur && step + 1 <= pd) {
+            const int next_axis = reverse ? axis - 1 : axis + 1;
+            PL_HIP(plk::blur_two_axes(vd, h->counters(), mv, h->values[cur], h->values[1 - cur],
+                                      h->neighbours + (size_t)axis * mv,
+                                      h->neighbours + (size_t)next_axis * mv, reset, h->vertex_cell,
+                                      h->stream));
+            step += 2;
+        } else {
+            PL_HIP(plk::blur_axis(vd, h->counters(), mv, h->values[cur], h->values[1 - cur],
+                                  h->neighbours + (size_t)axis * mv, reset, h->vertex_cell, h->stream));
+            step += 1;
+        }
         if (reset) h->table_clean = true;
         cur = 1 - cur;
     }
@@ -389,6 +400,9 @@ int pl_set_option(pl_handle h, int option, long value) {
             return PL_OK;
         case PL_OPT_XCD_AWARE:
             h->xcd_aware = value != 0;
+            return PL_OK;
+        case PL_OPT_PAIR_BLUR:
+            h->pair_blur = value != 0;
             return PL_OK;
         case PL_OPT_TABLE_CELLS:
             if (value < 0 || (value & (value - 1)) != 0) return PL_EINVAL;

@@ -101,6 +101,12 @@ hipError_t blur_axis(int vd, const Counters *counters, int max_vertices, const f
                      const int2 *neighbours_of_axis, uint64_t *reset_cell_keys,
                      const int *vertex_cell, hipStream_t s);
 
+// Two axes in one launch: the result of blur_axis with nbr_first followed by blur_axis with
+// nbr_second, bit for bit.
+hipError_t blur_two_axes(int vd, const Counters *counters, int max_vertices, const float *src,
+                         float *dst, const int2 *nbr_first, const int2 *nbr_second,
+                         uint64_t *reset_cell_keys, const int *vertex_cell, hipStream_t s);
+
 // Stage 5.  normalize: divide by the homogeneous channel and write vd-1 channels; else write vd.
 // cell_vertex != nullptr: replay_index still holds hash cells (vd <= 8 only).
 hipError_t slice(int pd, int vd, const PointMap &map, const int *replay_index,

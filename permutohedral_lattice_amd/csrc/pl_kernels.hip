@@ -811,6 +811,85 @@ __global__ __launch_bounds__(kBlock) void k_blur_element(const Counters *counter
     if (reset_cell_keys && j == 0) reset_cell_keys[vertex_cell[v]] = kEmptyCell;
 }
 
+// Two axes in one launch.  Every kernel boundary costs a cold L2 and a round of dependent loads,
+// and a blur pass has almost no work, so axis a and then axis b are applied together: the value
+// after axis a is evaluated (and rounded to float, as the separate pass would store it) at the
+// vertex and at its two b-neighbours, then the b tap combines the three.  An absent b-neighbour
+// contributes zero, whatever its own a-neighbours hold.  Same arithmetic, same results.
+template <typename Vec, int VD>
+__device__ __forceinline__ void blur_row(const Vec *in, const int2 *__restrict__ nbr_a, int u,
+                                         float (&out)[VD]) {
+    if (u < 0) {
+#pragma unroll
+        for (int j = 0; j < VD; ++j) out[j] = 0.0f;
+        return;
+    }
+    const int2 nb = nbr_a[u];
+    Vec zero;
+    float *zf = reinterpret_cast<float *>(&zero);
+#pragma unroll
+    for (int j = 0; j < VD; ++j) zf[j] = 0.0f;
+    const Vec self = in[u];
+    const Vec a = nb.x >= 0 ? in[nb.x] : zero;
+    const Vec b = nb.y >= 0 ? in[nb.y] : zero;
+    const float *af = reinterpret_cast<const float *>(&a), *bf = reinterpret_cast<const float *>(&b),
+                *sf = reinterpret_cast<const float *>(&self);
+#pragma unroll
+    for (int j = 0; j < VD; ++j) out[j] = blur_tap(af[j], sf[j], bf[j]);
+}
+
+template <typename Vec, int VD>
+__global__ __launch_bounds__(kBlock) void k_blur2_vertex(const Counters *counters, int max_vertices,
+                                                          const float *__restrict__ src,
+                                                          float *__restrict__ dst,
+                                                          const int2 *__restrict__ nbr_a,
+                                                          const int2 *__restrict__ nbr_b,
+                                                          uint64_t *reset_cell_keys,
+                                                          const int *__restrict__ vertex_cell) {
+    const int M = vertex_count(counters, max_vertices);
+    const int v = blockIdx.x * kBlock + threadIdx.x;
+    if (v >= M) return;
+    const Vec *in = reinterpret_cast<const Vec *>(src);
+    const int2 nb = nbr_b[v];
+    float plus[VD], self[VD], minus[VD];
+    blur_row<Vec, VD>(in, nbr_a, nb.x, plus);
+    blur_row<Vec, VD>(in, nbr_a, v, self);
+    blur_row<Vec, VD>(in, nbr_a, nb.y, minus);
+    Vec out;
+    float *of = reinterpret_cast<float *>(&out);
+#pragma unroll
+    for (int j = 0; j < VD; ++j) of[j] = blur_tap(plus[j], self[j], minus[j]);
+    reinterpret_cast<Vec *>(dst)[v] = out;
+    if (reset_cell_keys) reset_cell_keys[vertex_cell[v]] = kEmptyCell;
+}
+
+__device__ __forceinline__ float blur_element_of(const float *__restrict__ src,
+                                                 const int2 *__restrict__ nbr_a, int u, int vd, int j) {
+    if (u < 0) return 0.0f;
+    const int2 nb = nbr_a[u];
+    const float a = nb.x >= 0 ? src[(size_t)nb.x * vd + j] : 0.0f;
+    const float b = nb.y >= 0 ? src[(size_t)nb.y * vd + j] : 0.0f;
+    return blur_tap(a, src[(size_t)u * vd + j], b);
+}
+
+__global__ __launch_bounds__(kBlock) void k_blur2_element(const Counters *counters, int max_vertices,
+                                                           int vd, const float *__restrict__ src,
+                                                           float *__restrict__ dst,
+                                                           const int2 *__restrict__ nbr_a,
+                                                           const int2 *__restrict__ nbr_b,
+                                                           uint64_t *reset_cell_keys,
+                                                           const int *__restrict__ vertex_cell) {
+    const int M = vertex_count(counters, max_vertices);
+    const size_t e = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (e >= (size_t)M * vd) return;
+    const int v = (int)(e / (size_t)vd);
+    const int j = (int)(e - (size_t)v * vd);
+    const int2 nb = nbr_b[v];
+    dst[e] = blur_tap(blur_element_of(src, nbr_a, nb.x, vd, j), blur_element_of(src, nbr_a, v, vd, j),
+                      blur_element_of(src, nbr_a, nb.y, vd, j));
+    if (reset_cell_keys && j == 0) reset_cell_keys[vertex_cell[v]] = kEmptyCell;
+}
+
 // ------------------------------------------------------------------------------------------------
 // Stage 5: slice (reference: src/PermutohedralLatticeCPU.h:333-352)
 // ------------------------------------------------------------------------------------------------
@@ -1117,6 +1196,27 @@ hipError_t blur_axis(int vd, const Counters *counters, int max_vertices, const f
     } else {
         hipLaunchKernelGGL(k_blur_element, dim3(blocks_for((size_t)max_vertices * vd)), block, 0, s,
                            counters, max_vertices, vd, src, dst, nbr, reset_cell_keys, vertex_cell);
+    }
+    return hipGetLastError();
+}
+
+hipError_t blur_two_axes(int vd, const Counters *counters, int max_vertices, const float *src,
+                         float *dst, const int2 *nbr_first, const int2 *nbr_second,
+                         uint64_t *reset_cell_keys, const int *vertex_cell, hipStream_t s) {
+    if (max_vertices <= 0) return hipSuccess;
+    const dim3 block(kBlock);
+    if (vd == 2) {
+        hipLaunchKernelGGL((k_blur2_vertex<float2, 2>), dim3(blocks_for((size_t)max_vertices)), block, 0,
+                           s, counters, max_vertices, src, dst, nbr_first, nbr_second, reset_cell_keys,
+                           vertex_cell);
+    } else if (vd == 4) {
+        hipLaunchKernelGGL((k_blur2_vertex<float4, 4>), dim3(blocks_for((size_t)max_vertices)), block, 0,
+                           s, counters, max_vertices, src, dst, nbr_first, nbr_second, reset_cell_keys,
+                           vertex_cell);
+    } else {
+        hipLaunchKernelGGL(k_blur2_element, dim3(blocks_for((size_t)max_vertices * vd)), block, 0, s,
+                           counters, max_vertices, vd, src, dst, nbr_first, nbr_second, reset_cell_keys,
+                           vertex_cell);
     }
     return hipGetLastError();
 }
