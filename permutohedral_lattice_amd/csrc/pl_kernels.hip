@@ -631,125 +631,65 @@ __global__ __launch_bounds__(kBlock) void k_splat_dpp(PointMap map,
     }
 }
 
-// As wave_leader_of_equal, and also the lanes of the caller's group.
-template <typename T>
-__device__ __forceinline__ int wave_group_of_equal(T x, bool active, int lane, uint64_t &members) {
-    int leader = lane;
-    members = 0;
-    uint64_t remaining = __ballot(active);
-    while (remaining) {
-        const int first = __builtin_ctzll(remaining);
-        const T k = lane_value(x, first);
-        const bool same = active && x == k;
-        const uint64_t group = __ballot(same);
-        if (same) {
-            leader = first;
-            members = group;
-        }
-        remaining &= ~group;
-    }
-    return leader;
-}
-
-// vd 5..8: the terms of a wavefront go through LDS; lane e of the flush sums channel e % vd of
-// group e / vd over the group's lanes and sends one atomic, so the vd lanes of a group again hit
-// consecutive floats of one vertex row.
-template <int VD>
-__global__ __launch_bounds__(kBlock) void k_splat_point(int d1, PointMap map,
-                                                         const float *__restrict__ input,
-                                                         int in_channels, int *replay_index,
-                                                         const float *__restrict__ replay_weight,
-                                                         const int *__restrict__ cell_vertex,
-                                                         float *values, int xcd_aware) {
-    // per wavefront: every lane's weighted value, and per group of equal vertices its member
-    // lanes and its vertex
-    __shared__ float s_term[kBlock / 64][64 * VD];
-    __shared__ uint64_t s_members[kBlock / 64][64];
-    __shared__ int s_vertex[kBlock / 64][64];
-
+// Any vd: the same, four channels at a time.  The deduplication loop runs once per block of four
+// channels (it is cheap next to the reduction), the replay rows stay in registers.
+template <int D1>
+__global__ __launch_bounds__(kBlock) void k_splat_dpp_blocks(int vd, PointMap map,
+                                                              const float *__restrict__ input,
+                                                              int in_channels, int *replay_index,
+                                                              const float *__restrict__ replay_weight,
+                                                              const int *__restrict__ cell_vertex,
+                                                              float *values, int xcd_aware) {
     const unsigned vblock = xcd_contiguous_block(blockIdx.x, gridDim.x, xcd_aware);
     const size_t t = (size_t)vblock * kBlock + threadIdx.x;
     const size_t T = (size_t)gridDim.x * kBlock;
     const int n = point_of_thread(map, vblock, threadIdx.x);
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
+    const int my_channel = channel_of_lane<4>(lane);
 
-    float val[VD];
+    int vertex[D1];
+    float weight[D1];
 #pragma unroll
-    for (int j = 0; j < VD; ++j) val[j] = 1.0f;  // homogeneous channel when only vd-1 are given
-    if (n >= 0) {
+    for (int r = 0; r < D1; ++r) {
+        vertex[r] = n >= 0 ? replay_index[(size_t)r * T + t] : -1;
+        weight[r] = replay_weight[(size_t)r * T + t];
+    }
+    if (cell_vertex) {
 #pragma unroll
-        for (int j = 0; j < VD; ++j)
-            if (j < in_channels) val[j] = input[(size_t)n * in_channels + j];
+        for (int r = 0; r < D1; ++r)
+            if (vertex[r] >= 0) vertex[r] = cell_vertex[vertex[r]];
+#pragma unroll
+        for (int r = 0; r < D1; ++r)
+            if (n >= 0) replay_index[(size_t)r * T + t] = vertex[r];
     }
 
-    for (int r = 0; r < d1; ++r) {
-        int v = n >= 0 ? replay_index[(size_t)r * T + t] : -1;
-        if (cell_vertex && v >= 0) {
-            v = cell_vertex[v];
-            replay_index[(size_t)r * T + t] = v;
-        }
-        const float w = replay_weight[(size_t)r * T + t];
-        const bool active = v >= 0;
-
-        uint64_t members;
-        const int leader = wave_group_of_equal(v, active, lane, members);
-        const bool is_leader = active && leader == lane;
-        const uint64_t leaders = __ballot(is_leader);
-        const int groups = __builtin_popcountll(leaders);
-        if (is_leader) {
-            const int slot = __builtin_popcountll(leaders & ((1ull << lane) - 1ull));
-            s_vertex[wave][slot] = v;
-            s_members[wave][slot] = members;
+    for (int first_channel = 0; first_channel < vd; first_channel += 4) {
+        float val[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int c = first_channel + j;
+            // channels past the input are the homogeneous one (1), past vd nothing
+            val[j] = c >= vd ? 0.0f
+                             : (c < in_channels ? (n >= 0 ? input[(size_t)n * in_channels + c] : 0.0f)
+                                                : 1.0f);
         }
 #pragma unroll
-        for (int j = 0; j < VD; ++j) s_term[wave][lane * VD + j] = w * val[j];
-        __syncthreads();
-        // lane e sums channel e % VD of group e / VD over the group's lanes (in lane order) and
-        // sends one atomic; the VD lanes of a group hit consecutive floats of one vertex row
-        for (int e = lane; e < groups * VD; e += 64) {
-            const int g = e / VD, j = e - g * VD;
-            uint64_t m = s_members[wave][g];
-            float sum = 0.0f;
-            while (m) {
-                const int l = __builtin_ctzll(m);
-                sum += s_term[wave][l * VD + j];
-                m &= m - 1;
+        for (int r = 0; r < D1; ++r) {
+            const int v = vertex[r];
+            const float w = weight[r];
+            const float term[4] = {w * val[0], w * val[1], w * val[2], w * val[3]};
+            uint64_t remaining = __ballot(v >= 0);
+            while (remaining) {
+                const int first = __builtin_ctzll(remaining);
+                const int k = lane_value(v, first);
+                const bool same = v == k;
+                remaining &= ~__ballot(same);
+                const float sum = wave_sum_to_last_lanes<4>(same, term, lane);
+                if (lane >= 60 && first_channel + my_channel < vd)
+                    atomicAdd(values + (size_t)k * vd + first_channel + my_channel, sum);
             }
-            atomicAdd(values + (size_t)s_vertex[wave][g] * VD + j, sum);
         }
-        __syncthreads();
     }
-}
-
-// One thread per (point, channel): consecutive lanes add to consecutive floats of one vertex.
-__global__ __launch_bounds__(kBlock) void k_splat_channel(int d1, int vd, PointMap map, size_t T,
-                                                           const float *__restrict__ input,
-                                                           int in_channels,
-                                                           const int *__restrict__ replay_index,
-                                                           const float *__restrict__ replay_weight,
-                                                           float *values) {
-    const size_t g = (size_t)blockIdx.x * kBlock + threadIdx.x;
-    if (g >= T * vd) return;
-    const size_t t = g / (size_t)vd;
-    const int j = (int)(g - t * vd);
-    const int n = point_of_thread(map, (unsigned)(t / kBlock), (unsigned)(t % kBlock));
-    if (n < 0) return;
-    const float val = (j < in_channels) ? input[(size_t)n * in_channels + j] : 1.0f;
-    for (int r = 0; r < d1; ++r) {
-        const int v = replay_index[(size_t)r * T + t];
-        if (v < 0) continue;
-        const float w = replay_weight[(size_t)r * T + t];
-        atomicAdd(values + (size_t)v * vd + j, w * val);
-    }
-}
-
-// cells -> vertex indices in the replay array
-__global__ __launch_bounds__(kBlock) void k_remap_replay(size_t rows, int *replay_index,
-                                                          const int *__restrict__ cell_vertex) {
-    const size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x;
-    if (t >= rows) return;
-    const int c = replay_index[t];
-    if (c >= 0) replay_index[t] = cell_vertex[c];
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -1149,14 +1089,7 @@ hipError_t splat(int pd, int vd, const PointMap &map, const float *input, int in
                  int *replay_index, const float *replay_weight, const int *cell_vertex, float *values,
                  int xcd_aware, hipStream_t s) {
     if (map.n_blocks == 0) return hipSuccess;
-    const int d1 = pd + 1;
     const dim3 grid(map.n_blocks), block(kBlock);
-    const size_t T = (size_t)map.n_blocks * kBlock;
-#define PLK_SPLAT(KERNEL, VD)                                                                    \
-    case VD:                                                                                      \
-        hipLaunchKernelGGL(KERNEL<VD>, grid, block, 0, s, d1, map, input, in_channels,            \
-                           replay_index, replay_weight, cell_vertex, values, xcd_aware);          \
-        break;
 #define PLK_SPLAT_DPP(VD)                                                                         \
     case VD:                                                                                      \
         PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_splat_dpp<VD, PD + 1>), grid, block, 0, s, map, \
@@ -1165,19 +1098,12 @@ hipError_t splat(int pd, int vd, const PointMap &map, const float *input, int in
         break;
     switch (vd) {
         PLK_SPLAT_DPP(2) PLK_SPLAT_DPP(3) PLK_SPLAT_DPP(4)
-        PLK_SPLAT(k_splat_point, 5) PLK_SPLAT(k_splat_point, 6) PLK_SPLAT(k_splat_point, 7)
-        PLK_SPLAT(k_splat_point, 8)
         default:
-            if (cell_vertex) {
-                const size_t rows = T * d1;
-                hipLaunchKernelGGL(k_remap_replay, dim3(blocks_for(rows)), block, 0, s, rows,
-                                   replay_index, cell_vertex);
-            }
-            hipLaunchKernelGGL(k_splat_channel, dim3(blocks_for(T * vd)), block, 0, s, d1, vd, map, T,
-                               input, in_channels, (const int *)replay_index, replay_weight, values);
+            PLK_DISPATCH_PD(pd, hipLaunchKernelGGL(k_splat_dpp_blocks<PD + 1>, grid, block, 0, s, vd,
+                                                   map, input, in_channels, replay_index,
+                                                   replay_weight, cell_vertex, values, xcd_aware));
             break;
     }
-#undef PLK_SPLAT
 #undef PLK_SPLAT_DPP
     return hipGetLastError();
 }
