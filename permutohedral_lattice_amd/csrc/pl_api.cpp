@@ -66,13 +66,13 @@ struct pl_lattice {
     pl_alloc alloc{};
     plk::ScaleFactor scale{};
 
-    // hash table and the per-vertex arrays; a table of n_cells holds at most n_cells/2 vertices
+    // hash table and the per-vertex arrays; a table of n_cells holds at most 3/4 n_cells vertices
     uint64_t *cell_keys = nullptr;     // [n_cells_alloc]
     int *cell_vertex = nullptr;        // [n_cells_alloc]
-    uint64_t *vertex_keys = nullptr;   // [n_cells_alloc/2]
-    int *vertex_cell = nullptr;        // [n_cells_alloc/2]
-    float *values[2] = {nullptr, nullptr};  // [n_cells_alloc/2 * vd]
-    int2 *neighbours = nullptr;        // [(pd+1) * n_cells_alloc/2]
+    uint64_t *vertex_keys = nullptr;   // [3/4 n_cells_alloc]
+    int *vertex_cell = nullptr;        // [3/4 n_cells_alloc]
+    float *values[2] = {nullptr, nullptr};  // [3/4 n_cells_alloc * vd]
+    int2 *neighbours = nullptr;        // [(pd+1) * 3/4 n_cells_alloc]
     float *cell_values = nullptr;      // [n_cells_alloc * vd], rows by hash cell (fused build+splat)
     bool cell_values_clean = false;    // all zero
     uint32_t n_cells_alloc = 0;
@@ -115,7 +115,7 @@ struct pl_lattice {
         if (profile && ev[which]) ev_recorded[which] = hipEventRecord(ev[which], stream) == hipSuccess;
     }
     plk::Counters *counters() { return d_counters + counter_set; }
-    int max_vertices() const { return (int)(n_cells / 2); }
+    int max_vertices() const { return (int)plk::max_vertices_for(n_cells); }
 };
 
 namespace {
@@ -135,7 +135,7 @@ int ensure_table(pl_lattice *h, uint32_t cells) {
     h->n_cells_alloc = 0;
     h->table_clean = false;
     h->cell_values_clean = false;
-    const size_t mv = cells / 2;
+    const size_t mv = plk::max_vertices_for(cells);
     h->cell_keys = (uint64_t *)h->dmalloc(sizeof(uint64_t) * (size_t)cells);
     h->cell_vertex = (int *)h->dmalloc(sizeof(int) * (size_t)cells);
     h->vertex_keys = (uint64_t *)h->dmalloc(sizeof(uint64_t) * mv);
@@ -171,7 +171,7 @@ uint32_t initial_cells(const pl_lattice *h) {
     if (h->forced_cells > 0) {
         want = (uint64_t)h->forced_cells;
     } else if (h->last_M > 0) {
-        want = (uint64_t)h->last_M * 5 / 2;  // load factor 0.4 if the next input resembles the last
+        want = (uint64_t)h->last_M * 5 / 2;  // load factor 0.2..0.4 if the next input resembles the last (measured best)
     } else {
         want = (uint64_t)h->N * (uint64_t)(h->pd + 1) / 8;
     }
@@ -281,7 +281,7 @@ int verify_build(pl_lattice *h, uint32_t *retry_cells) {
         h->table_clean = false;
         return PL_EOVERFLOW;
     }
-    if ((flags & plk::kFlagTableFull) || (uint32_t)m > h->n_cells / 2) {
+    if ((flags & plk::kFlagTableFull) || (uint32_t)m > plk::max_vertices_for(h->n_cells)) {
         h->built = false;
         h->table_clean = false;  // keys beyond the numbered vertices may remain
         h->cell_values_clean = false;
@@ -340,7 +340,7 @@ int pl_create(int pd, int vd, int N, pl_stream stream, const pl_alloc *alloc, pl
         h->alloc.ctx = nullptr;
     }
     compute_scale_factor(pd, h->scale);
-    h->max_cells = pow2_at_least(rows * 2 < 4096 ? 4096 : rows * 2);
+    h->max_cells = pow2_at_least(rows * 2 < 4096 ? 4096 : rows * 2);  // holds N*(pd+1) vertices
     h->map = plk::make_point_map(N, 0, nullptr);
 
     int rc = PL_OK;

@@ -32,6 +32,10 @@ struct HostStatus {
     int flags;
 };
 
+// Vertices a table of n_cells may hold (load factor 3/4): beyond that probe sequences get long,
+// below 1/3 the table no longer fits the L2 next to everything else.
+__host__ __device__ inline uint32_t max_vertices_for(uint32_t n_cells) { return n_cells / 4u * 3u; }
+
 struct ScaleFactor {
     float v[kMaxPd];
 };

@@ -482,7 +482,7 @@ __global__ __launch_bounds__(kIdBlock) void k_assign_vertex_ids(
             const uint32_t m = (uint32_t)before + (uint32_t)total;
             const int flags = atomicOr(&counters->flags, 0);
             host_status->num_vertices = (int)m;
-            host_status->flags = flags | (m > n_cells / 2u ? kFlagTableFull : 0);
+            host_status->flags = flags | (m > max_vertices_for(n_cells) ? kFlagTableFull : 0);
             next_counters->vertices_and_blocks = 0;
             next_counters->flags = 0;
         }
@@ -491,7 +491,7 @@ __global__ __launch_bounds__(kIdBlock) void k_assign_vertex_ids(
     if (occupied) {
         const int v = block_base + wave_count[wave] +
                       __builtin_popcountll(ballot & ((1ull << lane) - 1ull));
-        if ((uint32_t)v < n_cells / 2u) {
+        if ((uint32_t)v < max_vertices_for(n_cells)) {
             cell_vertex[cell] = v;
             vertex_keys[v] = key;
             vertex_cell[v] = (int)cell;
@@ -505,7 +505,7 @@ __global__ __launch_bounds__(kIdBlock) void k_assign_vertex_ids(
                 for (int j = 0; j < vd; ++j) values[(size_t)v * vd + j] = 0.0f;
             }
         } else {
-            cell_vertex[cell] = 0;   // the host sees count > n_cells/2 and repeats with a larger table
+            cell_vertex[cell] = 0;   // the host sees the count and repeats with a larger table
         }
     }
 }
