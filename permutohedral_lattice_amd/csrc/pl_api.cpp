@@ -208,8 +208,8 @@ int enqueue_build(pl_lattice *h, const float *positions, uint32_t cells, const f
     h->mark(EV_BUILD);
     PL_HIP(plk::assign_vertex_ids(h->cell_keys, cells, h->cell_vertex, h->vertex_keys, h->vertex_cell,
                                   h->values[0], h->vd, fused ? h->cell_values : nullptr,
-                                  h->counters(), h->d_counters + previous_set, h->h_status,
-                                  h->stream));
+                                  h->neighbours, h->pd + 1, h->counters(),
+                                  h->d_counters + previous_set, h->h_status, h->stream));
     h->mark(EV_IDS);
     PL_HIP(plk::neighbours(h->pd, h->vertex_keys, h->counters(), h->max_vertices(), h->cell_keys,
                            h->cell_vertex, cells, h->neighbours, h->stream));

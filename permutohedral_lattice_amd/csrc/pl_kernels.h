@@ -78,14 +78,15 @@ hipError_t build(int pd, const float *positions, const PointMap &map, const Scal
 // Every occupied cell draws a dense vertex index: cell_vertex[cell] := v, vertex_keys[v] := key,
 // vertex_cell[v] := cell, the vertex count in *counters := M, and the vertex's row of `values` :=
 // 0, or, with cell_values != nullptr, := the row cell_values[cell*vd ..], which is zeroed.  The
-// last workgroup copies M and the flags to *host_status and zeroes *next_counters.
+// last workgroup copies M and the flags to *host_status and zeroes *next_counters.  The d1 = pd+1
+// neighbour entries of every vertex are set to (-1, -1).
 hipError_t assign_vertex_ids(const uint64_t *cell_keys, uint32_t n_cells, int *cell_vertex,
                              uint64_t *vertex_keys, int *vertex_cell, float *values, int vd,
-                             float *cell_values, Counters *counters, Counters *next_counters,
-                             HostStatus *host_status, hipStream_t s);
+                             float *cell_values, int2 *neighbours, int d1, Counters *counters,
+                             Counters *next_counters, HostStatus *host_status, hipStream_t s);
 
-// neighbours[a*max_vertices+v] := vertex indices of v's two neighbours along blur axis a (-1 =
-// absent), for v < counters->num_vertices.
+// neighbours[a*max_vertices+v] := vertex indices of v's two neighbours along blur axis a, for v
+// below the vertex count; entries of absent neighbours keep the -1 assign_vertex_ids gave them.
 hipError_t neighbours(int pd, const uint64_t *vertex_keys, const Counters *counters, int max_vertices,
                       const uint64_t *cell_keys, const int *cell_vertex, uint32_t n_cells,
                       int2 *neighbours, hipStream_t s);

@@ -458,7 +458,8 @@ constexpr int kIdBlock = 1024;
 __global__ __launch_bounds__(kIdBlock) void k_assign_vertex_ids(
     const uint64_t *__restrict__ cell_keys, uint32_t n_cells, int *cell_vertex,
     uint64_t *vertex_keys, int *vertex_cell, float *values, int vd, float *cell_values,
-    Counters *counters, Counters *next_counters, HostStatus *host_status) {
+    int2 *neighbours, int d1, Counters *counters, Counters *next_counters,
+    HostStatus *host_status) {
     __shared__ int wave_count[kIdBlock / 64];
     __shared__ int block_base;
     const uint32_t cell = blockIdx.x * kIdBlock + threadIdx.x;
@@ -495,6 +496,9 @@ __global__ __launch_bounds__(kIdBlock) void k_assign_vertex_ids(
             cell_vertex[cell] = v;
             vertex_keys[v] = key;
             vertex_cell[v] = (int)cell;
+            // "no neighbour" everywhere; the neighbour pass fills in the ones that exist
+            for (int a = 0; a < d1; ++a)
+                neighbours[(size_t)a * max_vertices_for(n_cells) + v] = make_int2(-1, -1);
             if (cell_values) {
                 // the fused build+splat accumulated by cell: move the row, leave zeros behind
                 for (int j = 0; j < vd; ++j) {
@@ -536,20 +540,23 @@ __global__ __launch_bounds__(kBlock) void k_neighbours(const uint64_t *__restric
     int q[PD], r;
     KeyCodec<PD>::unpack(vertex_keys[v], q, r);
 
-    int qp[PD], qm[PD];
-    const bool wrap_up = (r == PD), wrap_down = (r == 0);
+    int qp[PD];
+    const bool wrap_up = (r == PD);
 #pragma unroll
     for (int i = 0; i < PD; ++i) {
         const bool on_axis = (i == a);
         qp[i] = q[i] + (wrap_up ? (on_axis ? 0 : 1) : (on_axis ? -1 : 0));
-        qm[i] = q[i] + (wrap_down ? (on_axis ? 0 : -1) : (on_axis ? 1 : 0));
     }
+    // u is the + neighbour of v exactly when v is the - neighbour of u: one lookup fills both
+    // entries (all entries start as -1)
     const uint64_t kp = KeyCodec<PD>::pack(qp, wrap_up ? 0 : r + 1);
-    const uint64_t km = KeyCodec<PD>::pack(qm, wrap_down ? PD : r - 1);
-    const uint32_t hp = hash_key(kp) & mask, hm = hash_key(km) & mask;
-    const uint64_t cp = cell_keys[hp], cm = cell_keys[hm];   // both home cells in flight together
-    out[t] = make_int2(table_find(cell_keys, cell_vertex, mask, kp, hp, cp),
-                       table_find(cell_keys, cell_vertex, mask, km, hm, cm));
+    const uint32_t hp = hash_key(kp) & mask;
+    const int u = table_find(cell_keys, cell_vertex, mask, kp, hp, cell_keys[hp]);
+    if (u >= 0) {
+        int *entries = reinterpret_cast<int *>(out);
+        entries[2 * t] = u;                                        // out[a][v].x
+        entries[2 * ((size_t)a * max_vertices + u) + 1] = v;       // out[a][u].y
+    }
 }
 
 __global__ __launch_bounds__(kBlock) void k_fill_zero(float *p, size_t n) {
@@ -702,36 +709,6 @@ __device__ __forceinline__ float blur_tap(float a, float self, float b) {
     return (float)(0.25 * (double)a + 0.5 * (double)self + 0.25 * (double)b);
 }
 
-// one thread per vertex, the row as one vector
-template <typename Vec, int VD>
-__global__ __launch_bounds__(kBlock) void k_blur_vertex(const Counters *counters, int max_vertices,
-                                                         const float *__restrict__ src,
-                                                         float *__restrict__ dst,
-                                                         const int2 *__restrict__ nbr,
-                                                         uint64_t *reset_cell_keys,
-                                                         const int *__restrict__ vertex_cell) {
-    const int M = vertex_count(counters, max_vertices);
-    const int v = blockIdx.x * kBlock + threadIdx.x;
-    if (v >= M) return;
-    const Vec *in = reinterpret_cast<const Vec *>(src);
-    const int2 nb = nbr[v];
-    Vec zero;
-    float *zf = reinterpret_cast<float *>(&zero);
-#pragma unroll
-    for (int j = 0; j < VD; ++j) zf[j] = 0.0f;
-    const Vec self = in[v];
-    const Vec a = nb.x >= 0 ? in[nb.x] : zero;
-    const Vec b = nb.y >= 0 ? in[nb.y] : zero;
-    Vec out;
-    const float *af = reinterpret_cast<const float *>(&a), *bf = reinterpret_cast<const float *>(&b),
-                *sf = reinterpret_cast<const float *>(&self);
-    float *of = reinterpret_cast<float *>(&out);
-#pragma unroll
-    for (int j = 0; j < VD; ++j) of[j] = blur_tap(af[j], sf[j], bf[j]);
-    reinterpret_cast<Vec *>(dst)[v] = out;
-    if (reset_cell_keys) reset_cell_keys[vertex_cell[v]] = kEmptyCell;
-}
-
 // one thread per (vertex, channel), any vd
 __global__ __launch_bounds__(kBlock) void k_blur_element(const Counters *counters, int max_vertices,
                                                           int vd, const float *__restrict__ src,
@@ -756,53 +733,8 @@ __global__ __launch_bounds__(kBlock) void k_blur_element(const Counters *counter
 // after axis a is evaluated (and rounded to float, as the separate pass would store it) at the
 // vertex and at its two b-neighbours, then the b tap combines the three.  An absent b-neighbour
 // contributes zero, whatever its own a-neighbours hold.  Same arithmetic, same results.
-template <typename Vec, int VD>
-__device__ __forceinline__ void blur_row(const Vec *in, const int2 *__restrict__ nbr_a, int u,
-                                         float (&out)[VD]) {
-    if (u < 0) {
-#pragma unroll
-        for (int j = 0; j < VD; ++j) out[j] = 0.0f;
-        return;
-    }
-    const int2 nb = nbr_a[u];
-    Vec zero;
-    float *zf = reinterpret_cast<float *>(&zero);
-#pragma unroll
-    for (int j = 0; j < VD; ++j) zf[j] = 0.0f;
-    const Vec self = in[u];
-    const Vec a = nb.x >= 0 ? in[nb.x] : zero;
-    const Vec b = nb.y >= 0 ? in[nb.y] : zero;
-    const float *af = reinterpret_cast<const float *>(&a), *bf = reinterpret_cast<const float *>(&b),
-                *sf = reinterpret_cast<const float *>(&self);
-#pragma unroll
-    for (int j = 0; j < VD; ++j) out[j] = blur_tap(af[j], sf[j], bf[j]);
-}
-
-template <typename Vec, int VD>
-__global__ __launch_bounds__(kBlock) void k_blur2_vertex(const Counters *counters, int max_vertices,
-                                                          const float *__restrict__ src,
-                                                          float *__restrict__ dst,
-                                                          const int2 *__restrict__ nbr_a,
-                                                          const int2 *__restrict__ nbr_b,
-                                                          uint64_t *reset_cell_keys,
-                                                          const int *__restrict__ vertex_cell) {
-    const int M = vertex_count(counters, max_vertices);
-    const int v = blockIdx.x * kBlock + threadIdx.x;
-    if (v >= M) return;
-    const Vec *in = reinterpret_cast<const Vec *>(src);
-    const int2 nb = nbr_b[v];
-    float plus[VD], self[VD], minus[VD];
-    blur_row<Vec, VD>(in, nbr_a, nb.x, plus);
-    blur_row<Vec, VD>(in, nbr_a, v, self);
-    blur_row<Vec, VD>(in, nbr_a, nb.y, minus);
-    Vec out;
-    float *of = reinterpret_cast<float *>(&out);
-#pragma unroll
-    for (int j = 0; j < VD; ++j) of[j] = blur_tap(plus[j], self[j], minus[j]);
-    reinterpret_cast<Vec *>(dst)[v] = out;
-    if (reset_cell_keys) reset_cell_keys[vertex_cell[v]] = kEmptyCell;
-}
-
+// One thread per (vertex, channel): with a few hundred thousand vertices the passes are bound by
+// latency, and more threads hide more of it (41 us against 48 us for one thread per vertex row).
 __device__ __forceinline__ float blur_element_of(const float *__restrict__ src,
                                                  const int2 *__restrict__ nbr_a, int u, int vd, int j) {
     if (u < 0) return 0.0f;
@@ -1060,11 +992,11 @@ hipError_t build(int pd, const float *positions, const PointMap &map, const Scal
 
 hipError_t assign_vertex_ids(const uint64_t *cell_keys, uint32_t n_cells, int *cell_vertex,
                              uint64_t *vertex_keys, int *vertex_cell, float *values, int vd,
-                             float *cell_values, Counters *counters, Counters *next_counters,
-                             HostStatus *host_status, hipStream_t s) {
+                             float *cell_values, int2 *neighbours, int d1, Counters *counters,
+                             Counters *next_counters, HostStatus *host_status, hipStream_t s) {
     hipLaunchKernelGGL(k_assign_vertex_ids, dim3(blocks_for(n_cells, kIdBlock)), dim3(kIdBlock), 0, s,
                        cell_keys, n_cells, cell_vertex, vertex_keys, vertex_cell, values, vd,
-                       cell_values, counters, next_counters, host_status);
+                       cell_values, neighbours, d1, counters, next_counters, host_status);
     return hipGetLastError();
 }
 
@@ -1112,17 +1044,8 @@ hipError_t blur_axis(int vd, const Counters *counters, int max_vertices, const f
                      const int2 *nbr, uint64_t *reset_cell_keys, const int *vertex_cell,
                      hipStream_t s) {
     if (max_vertices <= 0) return hipSuccess;
-    const dim3 block(kBlock);
-    if (vd == 2) {
-        hipLaunchKernelGGL((k_blur_vertex<float2, 2>), dim3(blocks_for((size_t)max_vertices)), block, 0,
-                           s, counters, max_vertices, src, dst, nbr, reset_cell_keys, vertex_cell);
-    } else if (vd == 4) {
-        hipLaunchKernelGGL((k_blur_vertex<float4, 4>), dim3(blocks_for((size_t)max_vertices)), block, 0,
-                           s, counters, max_vertices, src, dst, nbr, reset_cell_keys, vertex_cell);
-    } else {
-        hipLaunchKernelGGL(k_blur_element, dim3(blocks_for((size_t)max_vertices * vd)), block, 0, s,
-                           counters, max_vertices, vd, src, dst, nbr, reset_cell_keys, vertex_cell);
-    }
+    hipLaunchKernelGGL(k_blur_element, dim3(blocks_for((size_t)max_vertices * vd)), dim3(kBlock), 0, s,
+                       counters, max_vertices, vd, src, dst, nbr, reset_cell_keys, vertex_cell);
     return hipGetLastError();
 }
 
@@ -1130,20 +1053,9 @@ hipError_t blur_two_axes(int vd, const Counters *counters, int max_vertices, con
                          float *dst, const int2 *nbr_first, const int2 *nbr_second,
                          uint64_t *reset_cell_keys, const int *vertex_cell, hipStream_t s) {
     if (max_vertices <= 0) return hipSuccess;
-    const dim3 block(kBlock);
-    if (vd == 2) {
-        hipLaunchKernelGGL((k_blur2_vertex<float2, 2>), dim3(blocks_for((size_t)max_vertices)), block, 0,
-                           s, counters, max_vertices, src, dst, nbr_first, nbr_second, reset_cell_keys,
-                           vertex_cell);
-    } else if (vd == 4) {
-        hipLaunchKernelGGL((k_blur2_vertex<float4, 4>), dim3(blocks_for((size_t)max_vertices)), block, 0,
-                           s, counters, max_vertices, src, dst, nbr_first, nbr_second, reset_cell_keys,
-                           vertex_cell);
-    } else {
-        hipLaunchKernelGGL(k_blur2_element, dim3(blocks_for((size_t)max_vertices * vd)), block, 0, s,
-                           counters, max_vertices, vd, src, dst, nbr_first, nbr_second, reset_cell_keys,
-                           vertex_cell);
-    }
+    hipLaunchKernelGGL(k_blur2_element, dim3(blocks_for((size_t)max_vertices * vd)), dim3(kBlock), 0, s,
+                       counters, max_vertices, vd, src, dst, nbr_first, nbr_second, reset_cell_keys,
+                       vertex_cell);
     return hipGetLastError();
 }
 
