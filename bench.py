@@ -34,6 +34,21 @@ def algorithmic_bytes(n, m, pd, vd):
     }
 
 
+def measured_traffic(kernel_name, side):
+    """HBM bytes per launch of a kernel (read + written) as rocprofv3's FETCH_SIZE / WRITE_SIZE gave
+    them for this workload, scaled by the copy calibration; the summary under profiles/ holds the
+    commands.  None when there is no measurement for this kernel and size."""
+    path = os.path.join(ROOT, "profiles", "bench_bilateral_%d_pd5_vd4_hbm_traffic.json" % side)
+    try:
+        table = json.load(open(path))["per_kernel_bytes"]
+    except (OSError, ValueError, KeyError):
+        return None
+    key = "%s@%d" % (kernel_name, side * side)
+    if key not in table:
+        return None
+    return int(sum(table[key]))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -133,14 +148,22 @@ def main():
     stages["blur_axis"] = stages["blur"] / (pd + 1)
 
     alg = algorithmic_bytes(n, m, pd, vd)
+    # for vd <= 4 filter() splats inside the build kernel: that launch then carries both shares
+    fused = vd <= 4
+    if fused:
+        alg["build"] += alg["splat"]
     per_launch_ms = {k: stages[k] for k in ("build", "splat", "blur_axis", "slice")}
-    dominant = max(("build", "splat", "slice"), key=lambda k: stages[k])
+    candidates = ("build", "slice") if fused else ("build", "splat", "slice")
+    dominant = max(candidates, key=lambda k: stages[k])
     if stages["blur"] > stages[dominant]:
         dominant = "blur_axis"
     achieved = alg[dominant] / (per_launch_ms[dominant] * 1e-3) / 1e9
-    roofline = {"bound": "hbm", "kernel": dominant, "achieved": round(achieved, 2),
+    kernel_name = {"build": "k_build<5, 4>" if fused else "k_build<5, 0>", "splat": "k_splat_dpp<4, 6>",
+                   "blur_axis": "k_blur2_element", "slice": "k_slice_point<4>"}[dominant]
+    roofline = {"bound": "hbm", "kernel": kernel_name, "achieved": round(achieved, 2),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 5),
-                "traffic": None, "algorithmic_bytes_per_launch": alg[dominant],
+                "traffic": measured_traffic(kernel_name, side),
+                "algorithmic_bytes_per_launch": alg[dominant],
                 "launch_ms": round(per_launch_ms[dominant], 5)}
     gpu_kernel_ms = sum(stages[k] for k in ("clear", "build", "ids", "neighbours", "fill", "splat",
                                             "blur", "slice"))
