@@ -136,6 +136,31 @@ def main():
     torch.cuda.synchronize()
     reuse_ms = 1e3 * (time.perf_counter() - t0) / args.steps
 
+    # the op's boundary: the reference image comes in, not a positions array.  First as the
+    # reference does it (feature kernel, then filter), then with the features built on the fly.
+    d_img = torch.from_numpy(np.ascontiguousarray(img.reshape(-1, 3))).cuda()
+    d_pos2 = torch.empty_like(d_pos)
+
+    def op_step_two_kernels():
+        for o, v, rev in ((out_f, d_val, False), (out_r, d_grad, True)):
+            pla.compute_positions(d_img, (side, side), 8.0, 0.125, out=d_pos2)
+            lat.filter(o, v, d_pos2, rev)
+
+    def op_step_fused():
+        for o, v, rev in ((out_f, d_val, False), (out_r, d_grad, True)):
+            lat.filter_image(o, v, d_img, (side, side), 8.0, 0.125, rev)
+
+    op_ms = {}
+    for name, fn in (("positions_then_filter", op_step_two_kernels), ("features_on_the_fly", op_step_fused)):
+        for _ in range(2):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            fn()
+        torch.cuda.synchronize()
+        op_ms[name] = 1e3 * (time.perf_counter() - t0) / args.steps
+
     # per-kernel durations from HIP events on the lattice's stream
     lat.set_option(pla.PL_OPT_PROFILE, 1)
     stage_samples = []
@@ -190,6 +215,11 @@ def main():
         "reuse": {"what": "build once, apply forward + reverse per step",
                   "ms_per_step": round(reuse_ms, 4),
                   "value": round(pixels_per_step / (reuse_ms * 1e-3) / 1e6, 3)},
+        "op_level": {"what": "reference image in, forward + reverse per step: feature kernel + "
+                             "filter(), and filter_image() (features built inside the first kernel)",
+                     "ms_per_step": {k: round(v, 4) for k, v in op_ms.items()},
+                     "value": {k: round(pixels_per_step / (v * 1e-3) / 1e6, 3)
+                               for k, v in op_ms.items()}},
     }
 
     if not args.no_cpu:

@@ -66,6 +66,23 @@ public:
         check(pl_apply(handle_, output, input, reverse ? 1 : 0), "pl_apply");
     }
 
+    // filter / build under the features ComputeKernel would write for this reference image
+    // (grid coordinates / spatial_std, reference channels / feature_std), built on the fly
+    void filter_image(float *output, const float *input, const float *reference,
+                      int n_reference_channels, int n_spatial_dims, const int *spatial_dims,
+                      float spatial_std, float feature_std, bool reverse) {
+        check(pl_filter_image(handle_, output, input, reference, n_reference_channels,
+                              n_spatial_dims, spatial_dims, spatial_std, feature_std,
+                              reverse ? 1 : 0),
+              "pl_filter_image");
+    }
+    void build_image(const float *reference, int n_reference_channels, int n_spatial_dims,
+                     const int *spatial_dims, float spatial_std, float feature_std) {
+        check(pl_build_image(handle_, reference, n_reference_channels, n_spatial_dims,
+                             spatial_dims, spatial_std, feature_std),
+              "pl_build_image");
+    }
+
     // the N points form a row-major grid of these extents (performance hint only)
     void set_point_grid(int n_dims, const int *dims) {
         check(pl_set_point_grid(handle_, n_dims, dims), "pl_set_point_grid");

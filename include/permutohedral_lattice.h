@@ -148,6 +148,24 @@ int pl_compute_positions(const float *reference, float *positions, int num_super
                          float spatial_std, float feature_std, pl_stream stream);
 
 /*
+ * pl_filter / pl_build with the feature vectors built on the fly: the result of
+ * pl_compute_positions(reference, positions, N, ...) followed by pl_filter(h, output, input,
+ * positions, reverse) (or pl_build(h, positions)), without a positions array ever being written
+ * or read.  The lattice must have pd = n_spatial_dims + n_reference_channels and N = the product
+ * of spatial_dims (a HOST array); the grid hint of pl_set_point_grid is set from them.
+ * n_reference_channels = 0: spatial features only, reference may be NULL.
+ * Stands in for the pair of functor calls of the op's per-item loop
+ * (src/LatticeFilterKernel.cpp:160-178: ComputeKernel, then LatticeFilter), i.e. compute_kernel
+ * (src/PermutohedralLatticeGPU.cuh:482-506) fused into the splat stage of filter (:454-479).
+ */
+int pl_filter_image(pl_handle h, float *output, const float *input, const float *reference,
+                    int n_reference_channels, int n_spatial_dims, const int *spatial_dims,
+                    float spatial_std, float feature_std, int reverse);
+int pl_build_image(pl_handle h, const float *reference, int n_reference_channels,
+                   int n_spatial_dims, const int *spatial_dims, float spatial_std,
+                   float feature_std);
+
+/*
  * The LatticeFilter op on channels-last device tensors input[B, s_1..s_k, C_in],
  * reference[B, s_1..s_k, C_ref] -> output (shape of input).  bilateral: features are
  * (coords/theta_alpha, reference/theta_beta); otherwise coords/theta_gamma and the reference is

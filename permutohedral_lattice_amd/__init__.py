@@ -26,7 +26,8 @@ PL_OPT_NORMALIZE, PL_OPT_PROFILE, PL_OPT_TABLE_CELLS, PL_OPT_XCD_AWARE, PL_OPT_P
 EXPORTS = (
     "pl_supported", "pl_strerror", "pl_last_hip_error", "pl_create", "pl_destroy", "pl_filter",
     "pl_build", "pl_apply", "pl_set_point_grid", "pl_num_vertices", "pl_set_option", "pl_stage_ms", "pl_debug_simplex",
-    "pl_debug_keys", "pl_debug_replay", "pl_compute_positions", "pl_lattice_filter_op",
+    "pl_debug_keys", "pl_debug_replay", "pl_compute_positions", "pl_filter_image", "pl_build_image",
+    "pl_lattice_filter_op",
 )
 
 
@@ -42,9 +43,13 @@ class PermutohedralError(RuntimeError):
 def _load():
     if not os.path.exists(LIB_PATH):
         raise ImportError(
-            "%s is missing: build it with `python -m permutohedral_lattice_amd.build` "
+            "%s is missing: build it with `python permutohedral_lattice_amd/build.py` "
             "(there is no CPU fallback)" % LIB_PATH)
     lib = C.CDLL(LIB_PATH)
+    stale = [name for name in EXPORTS if not hasattr(lib, name)]
+    if stale:
+        raise ImportError("%s lacks %s: rebuild it with `python permutohedral_lattice_amd/build.py`"
+                          % (LIB_PATH, ", ".join(stale)))
     vp, ci, cf = C.c_void_p, C.c_int, C.c_float
     lib.pl_supported.argtypes = [ci, ci]
     lib.pl_strerror.argtypes = [ci]
@@ -62,6 +67,8 @@ def _load():
     lib.pl_debug_keys.argtypes = [vp, vp]
     lib.pl_debug_replay.argtypes = [vp, vp, vp]
     lib.pl_compute_positions.argtypes = [vp, vp, ci, ci, ci, C.POINTER(ci), cf, cf, vp]
+    lib.pl_filter_image.argtypes = [vp, vp, vp, vp, ci, ci, C.POINTER(ci), cf, cf, ci]
+    lib.pl_build_image.argtypes = [vp, vp, ci, ci, C.POINTER(ci), cf, cf]
     lib.pl_lattice_filter_op.argtypes = [vp, vp, vp, ci, ci, C.POINTER(ci), ci, ci, ci, cf, cf, cf,
                                          ci, vp, vp]
     return lib
@@ -130,6 +137,32 @@ class PermutohedralLattice:
         _check(_lib.pl_apply(self._h, _dev_f32(output, "output", self.N * ch),
                              _dev_f32(input, "input", self.N * ch), int(bool(reverse))), "pl_apply")
         return output
+
+    # -- features built on the fly from the reference image and the grid coordinates ------------
+    def _image_args(self, reference, spatial_dims):
+        dims = [int(d) for d in spatial_dims]
+        rc = self.pd - len(dims)
+        if rc < 0:
+            raise ValueError("more spatial dimensions than pd")
+        ref = _dev_f32(reference, "reference", self.N * rc) if rc > 0 else None
+        return ref, rc, len(dims), (C.c_int * max(1, len(dims)))(*dims)
+
+    def filter_image(self, output, input, reference, spatial_dims, spatial_std, feature_std=1.0,
+                     reverse=False):
+        """``filter`` under the features ``compute_positions(reference, spatial_dims, spatial_std,
+        feature_std)`` would give, without building that array."""
+        ch = self.vd - 1 if self._normalize else self.vd
+        ref, rc, k, dims = self._image_args(reference, spatial_dims)
+        _check(_lib.pl_filter_image(self._h, _dev_f32(output, "output", self.N * ch),
+                                    _dev_f32(input, "input", self.N * ch), ref, rc, k, dims,
+                                    float(spatial_std), float(feature_std), int(bool(reverse))),
+               "pl_filter_image")
+        return output
+
+    def build_image(self, reference, spatial_dims, spatial_std, feature_std=1.0):
+        ref, rc, k, dims = self._image_args(reference, spatial_dims)
+        _check(_lib.pl_build_image(self._h, ref, rc, k, dims, float(spatial_std), float(feature_std)),
+               "pl_build_image")
 
     def set_point_grid(self, dims):
         """Hint: the N points form a row-major grid of these extents (None removes the hint)."""

@@ -1,6 +1,8 @@
 """Compile the HIP library for gfx950, in-tree.
 
-    python -m permutohedral_lattice_amd.build
+    python permutohedral_lattice_amd/build.py
+
+(run as a script: importing the package needs the library this file builds)
 
 Produces ``permutohedral_lattice_amd/libpermutohedral_hip.so`` (cross-compiles without a GPU).
 """

@@ -184,7 +184,8 @@ uint32_t initial_cells(const pl_lattice *h) {
 // Enqueue one build with a table of `cells` cells.  Nothing here waits for the device.
 // splat_input != nullptr: the build kernel also splats these values (when it can for this vd),
 // and the value table holds them when the build is done.
-int enqueue_build(pl_lattice *h, const float *positions, uint32_t cells, const float *splat_input) {
+int enqueue_build(pl_lattice *h, const plk::PointFeatures &features, uint32_t cells,
+                  const float *splat_input) {
     int rc = ensure_table(h, cells);
     if (rc != PL_OK) return rc;
     const bool fused = splat_input && plk::build_can_splat(h->vd);
@@ -202,7 +203,7 @@ int enqueue_build(pl_lattice *h, const float *positions, uint32_t cells, const f
     // the previous vertex-numbering kernel (or pl_create) left the other counter set zeroed
     const int previous_set = h->counter_set;
     h->counter_set = 1 - previous_set;
-    PL_HIP(plk::build(h->pd, positions, h->map, h->scale, h->cell_keys, cells, h->counters(),
+    PL_HIP(plk::build(h->pd, features, h->map, h->scale, h->cell_keys, cells, h->counters(),
                       h->replay_index, h->replay_weight, h->xcd_aware ? 1 : 0, fused ? h->vd : 0,
                       splat_input, h->normalize ? h->vd - 1 : h->vd, h->cell_values, h->stream));
     h->mark(EV_BUILD);
@@ -430,8 +431,41 @@ int pl_set_point_grid(pl_handle h, int n_dims, const int *dims) {
     return ensure_replay(h);
 }
 
-int pl_build(pl_handle h, const float *positions) {
-    if (!h || (!positions && h->N > 0)) return PL_EINVAL;
+namespace {
+
+plk::PointFeatures features_from_positions(const float *positions) {
+    plk::PointFeatures f{};
+    f.positions = positions;
+    return f;
+}
+
+// Checks the arguments of the *_image entry points, sets the grid hint and describes the features.
+int features_from_image(pl_lattice *h, const float *reference, int n_reference_channels,
+                        int n_spatial_dims, const int *spatial_dims, float spatial_std,
+                        float feature_std, plk::PointFeatures *out) {
+    if (n_reference_channels < 0 || n_spatial_dims < 0) return PL_EINVAL;
+    if (n_spatial_dims > plk::kMaxSpatialDims) return PL_EUNSUPPORTED;
+    if (n_spatial_dims + n_reference_channels != h->pd) return PL_EINVAL;
+    if (n_spatial_dims > 0 && !spatial_dims) return PL_EINVAL;
+    if (n_reference_channels > 0 && !reference && h->N > 0) return PL_EINVAL;
+    plk::PointFeatures f{};
+    f.reference = reference;
+    f.n_spatial_dims = n_spatial_dims;
+    f.n_reference_channels = n_reference_channels;
+    f.spatial_std = spatial_std;
+    f.feature_std = feature_std;
+    for (int i = 0; i < plk::kMaxSpatialDims; ++i) f.dims.v[i] = 1;
+    for (int i = 0; i < n_spatial_dims; ++i) f.dims.v[i] = spatial_dims[i];
+    if (n_spatial_dims > 0) {
+        // also checks that the extents are positive and that their product is N
+        const int rc = pl_set_point_grid(h, n_spatial_dims, spatial_dims);
+        if (rc != PL_OK) return rc;
+    }
+    *out = f;
+    return PL_OK;
+}
+
+int build_lattice(pl_lattice *h, const plk::PointFeatures &features) {
     h->built = false;
     h->M = 0;
     for (int i = 0; i <= EV_NBR; ++i) h->ev_recorded[i] = false;
@@ -441,12 +475,52 @@ int pl_build(pl_handle h, const float *positions) {
     }
     uint32_t cells = initial_cells(h);
     for (;;) {
-        int rc = enqueue_build(h, positions, cells, nullptr);
+        int rc = enqueue_build(h, features, cells, nullptr);
         if (rc != PL_OK) return rc;
         rc = verify_build(h, &cells);
         if (rc == PL_OK) return PL_OK;
         if (!cells) return rc;
     }
+}
+
+int filter_lattice(pl_lattice *h, float *output, const float *input,
+                   const plk::PointFeatures &features, int reverse) {
+    h->built = false;
+    h->M = 0;
+    for (int i = 0; i < EV_COUNT; ++i) h->ev_recorded[i] = false;
+    if (h->N == 0) {
+        h->built = h->verified = true;
+        return PL_OK;
+    }
+    // build and apply are enqueued together; if the table turns out too small the whole call is
+    // repeated with a larger one (the output is simply written again)
+    uint32_t cells = initial_cells(h);
+    for (;;) {
+        int rc = enqueue_build(h, features, cells, input);
+        if (rc != PL_OK) return rc;
+        rc = enqueue_apply(h, output, input, reverse);
+        if (rc != PL_OK) return rc;
+        rc = verify_build(h, &cells);
+        if (rc == PL_OK) return PL_OK;
+        if (!cells) return rc;
+    }
+}
+
+}  // namespace
+
+int pl_build(pl_handle h, const float *positions) {
+    if (!h || (!positions && h->N > 0)) return PL_EINVAL;
+    return build_lattice(h, features_from_positions(positions));
+}
+
+int pl_build_image(pl_handle h, const float *reference, int n_reference_channels,
+                   int n_spatial_dims, const int *spatial_dims, float spatial_std,
+                   float feature_std) {
+    if (!h) return PL_EINVAL;
+    plk::PointFeatures features;
+    const int rc = features_from_image(h, reference, n_reference_channels, n_spatial_dims,
+                                       spatial_dims, spatial_std, feature_std, &features);
+    return rc == PL_OK ? build_lattice(h, features) : rc;
 }
 
 int pl_apply(pl_handle h, float *output, const float *input, int reverse) {
@@ -460,25 +534,18 @@ int pl_apply(pl_handle h, float *output, const float *input, int reverse) {
 int pl_filter(pl_handle h, float *output, const float *input, const float *positions, int reverse) {
     if (!h) return PL_EINVAL;
     if (h->N > 0 && (!output || !input || !positions)) return PL_EINVAL;
-    h->built = false;
-    h->M = 0;
-    for (int i = 0; i < EV_COUNT; ++i) h->ev_recorded[i] = false;
-    if (h->N == 0) {
-        h->built = h->verified = true;
-        return PL_OK;
-    }
-    // build and apply are enqueued together; if the table turns out too small the whole call is
-    // repeated with a larger one (the output is simply written again)
-    uint32_t cells = initial_cells(h);
-    for (;;) {
-        int rc = enqueue_build(h, positions, cells, input);
-        if (rc != PL_OK) return rc;
-        rc = enqueue_apply(h, output, input, reverse);
-        if (rc != PL_OK) return rc;
-        rc = verify_build(h, &cells);
-        if (rc == PL_OK) return PL_OK;
-        if (!cells) return rc;
-    }
+    return filter_lattice(h, output, input, features_from_positions(positions), reverse);
+}
+
+int pl_filter_image(pl_handle h, float *output, const float *input, const float *reference,
+                    int n_reference_channels, int n_spatial_dims, const int *spatial_dims,
+                    float spatial_std, float feature_std, int reverse) {
+    if (!h) return PL_EINVAL;
+    if (h->N > 0 && (!output || !input)) return PL_EINVAL;
+    plk::PointFeatures features;
+    const int rc = features_from_image(h, reference, n_reference_channels, n_spatial_dims,
+                                       spatial_dims, spatial_std, feature_std, &features);
+    return rc == PL_OK ? filter_lattice(h, output, input, features, reverse) : rc;
 }
 
 int pl_num_vertices(pl_handle h, int *num_vertices) {
@@ -556,15 +623,14 @@ int pl_compute_positions(const float *reference, float *positions, int num_super
 // ------------------------------------------------------------------------------------------------
 namespace {
 
-// With the default allocator the op keeps its lattice and positions buffer between calls (one
-// per device and shape), because hipMalloc/hipFree per call would serialise the device.  With a
+// With the default allocator the op keeps its lattice between calls (one per device, shape and
+// stream), because hipMalloc/hipFree per call would serialise the device.  With a
 // caller-supplied allocator everything is taken from it and returned before the call ends, as
 // the reference does with TensorFlow temporaries (src/DeviceMemoryAllocator.h:52-71).
 struct OpCacheEntry {
     int device, pd, vd, N;
     hipStream_t stream;
     pl_handle lattice;
-    float *positions;
 };
 std::mutex g_op_cache_mutex;
 std::vector<OpCacheEntry> g_op_cache;
@@ -603,7 +669,6 @@ extern "C" int pl_lattice_filter_op(const float *input, const float *reference, 
     PL_HIP(hipGetDevice(&device));
 
     pl_handle lattice = nullptr;
-    float *positions = nullptr;
     bool cached = false;
     std::unique_lock<std::mutex> lock(g_op_cache_mutex, std::defer_lock);
     if (!alloc) {
@@ -612,7 +677,6 @@ extern "C" int pl_lattice_filter_op(const float *input, const float *reference, 
             if (e.device == device && e.pd == pd && e.vd == vd && e.N == N &&
                 e.stream == (hipStream_t)stream) {
                 lattice = e.lattice;
-                positions = e.positions;
                 cached = true;
                 break;
             }
@@ -621,37 +685,25 @@ extern "C" int pl_lattice_filter_op(const float *input, const float *reference, 
     if (!lattice) {
         rc = pl_create(pd, vd, N, stream, alloc, &lattice);
         if (rc != PL_OK) return rc;
-        const size_t bytes = sizeof(float) * (size_t)N * (size_t)pd;
-        positions = (float *)(alloc ? alloc->alloc(alloc->ctx, bytes) : default_alloc(nullptr, bytes));
-        if (!positions) {
-            pl_destroy(lattice);
-            return PL_ENOMEM;
-        }
         if (!alloc) {
             if (g_op_cache.size() >= kOpCacheMax) {
                 pl_destroy(g_op_cache.front().lattice);
-                default_free(nullptr, g_op_cache.front().positions);
                 g_op_cache.erase(g_op_cache.begin());
             }
-            g_op_cache.push_back({device, pd, vd, N, (hipStream_t)stream, lattice, positions});
+            g_op_cache.push_back({device, pd, vd, N, (hipStream_t)stream, lattice});
             cached = true;
         }
     }
 
-    // the op knows the spatial extents of its tensors: workgroups take tiles of the image
-    rc = pl_set_point_grid(lattice, n_spatial_dims, spatial_dims);
+    // One lattice per batch item (LatticeFilterKernel.cpp:152-179).  The feature vectors are built
+    // inside the lattice's first kernel, from the item's reference image and the grid coordinates.
     for (int b = 0; b < batch && rc == PL_OK; ++b) {
         const float *ref_b = ref_ch ? reference + (size_t)b * N * ref_ch : nullptr;
-        rc = pl_compute_positions(ref_b, positions, N, ref_ch, n_spatial_dims, spatial_dims,
-                                  spatial_std, feature_std, stream);
-        if (rc != PL_OK) break;
-        rc = pl_filter(lattice, output + (size_t)b * N * n_input_channels,
-                       input + (size_t)b * N * n_input_channels, positions, reverse);
+        rc = pl_filter_image(lattice, output + (size_t)b * N * n_input_channels,
+                             input + (size_t)b * N * n_input_channels, ref_b, ref_ch,
+                             n_spatial_dims, spatial_dims, spatial_std, feature_std, reverse);
     }
 
-    if (!cached) {
-        pl_destroy(lattice);  // synchronises the stream first
-        alloc->free(alloc->ctx, positions);
-    }
+    if (!cached) pl_destroy(lattice);  // synchronises the stream first
     return rc;
 }

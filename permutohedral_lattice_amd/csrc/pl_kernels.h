@@ -44,6 +44,17 @@ struct SpatialDims {
     int v[kMaxSpatialDims];
 };
 
+// Where the feature vector of a point comes from: the row of a positions array, or, with
+// positions == nullptr, the point's grid coordinates divided by spatial_std followed by its
+// reference channels divided by feature_std (what compute_positions would have written).
+struct PointFeatures {
+    const float *positions;   // N x pd
+    const float *reference;   // N x n_reference_channels
+    int n_spatial_dims, n_reference_channels;
+    SpatialDims dims;         // slowest first, the last runs fastest
+    float spatial_std, feature_std;
+};
+
 // How threads are laid over the points (see point_of_thread in pl_kernels.hip).
 struct PointMap {
     int N;
@@ -70,7 +81,7 @@ hipError_t clear_table(uint64_t *cell_keys, uint32_t n_cells, hipStream_t s);
 // (in_channels per point) into cell_values[cell*vd ..], rows addressed by hash cell;
 // assign_vertex_ids then moves them into the dense value table.
 bool build_can_splat(int vd);
-hipError_t build(int pd, const float *positions, const PointMap &map, const ScaleFactor &scale,
+hipError_t build(int pd, const PointFeatures &features, const PointMap &map, const ScaleFactor &scale,
                  uint64_t *cell_keys, uint32_t n_cells, Counters *counters, int *replay_index,
                  float *replay_weight, int xcd_aware, int splat_vd, const float *input,
                  int in_channels, float *cell_values, hipStream_t s);

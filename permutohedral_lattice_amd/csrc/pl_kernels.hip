@@ -184,6 +184,32 @@ __device__ __forceinline__ void load_position(const float *positions, int n, flo
     for (int i = 0; i < PD; ++i) pos[i] = row[i];
 }
 
+// The feature vector from a positions array, or built on the fly exactly as k_positions builds it
+// (reference: src/PermutohedralLatticeCPU.h:464-473): IEEE float division of the grid coordinate
+// and of the reference channels.
+template <int PD>
+__device__ __forceinline__ void load_features(const PointFeatures &f, int n, float (&pos)[PD]) {
+    if (f.positions) {
+        load_position<PD>(f.positions, n, pos);
+        return;
+    }
+    int rest = n;
+#pragma unroll
+    for (int i = PD - 1; i >= 0; --i) {
+        if (i < f.n_spatial_dims) {
+            const int next = rest / f.dims.v[i];
+            pos[i] = (float)(rest - next * f.dims.v[i]) / f.spatial_std;
+            rest = next;
+        }
+    }
+    if (f.n_reference_channels > 0) {
+        const float *row = f.reference + (size_t)n * f.n_reference_channels;
+#pragma unroll
+        for (int i = 0; i < PD; ++i)
+            if (i >= f.n_spatial_dims) pos[i] = row[i - f.n_spatial_dims] / f.feature_std;
+    }
+}
+
 // ------------------------------------------------------------------------------------------------
 // Which point a thread works on.  Points that are neighbours in the image share lattice vertices,
 // and every duplicate that meets inside one wavefront is merged before it reaches memory, so a
@@ -333,7 +359,7 @@ __device__ __forceinline__ float wave_sum_to_last_lanes(bool member, const float
 // numbered yet); the numbering pass moves the rows into the dense value table.  One kernel then
 // does the work of two, shares the deduplication between them and never reads the replay arrays.
 template <int PD, int SPLAT_VD>
-__global__ __launch_bounds__(kBlock) void k_build(const float *__restrict__ positions, PointMap map,
+__global__ __launch_bounds__(kBlock) void k_build(PointFeatures features, PointMap map,
                                                    ScaleFactor scale, uint64_t *cell_keys,
                                                    uint32_t mask, Counters *counters,
                                                    int *__restrict__ replay_index,
@@ -351,7 +377,7 @@ __global__ __launch_bounds__(kBlock) void k_build(const float *__restrict__ posi
     float pos[PD];
 #pragma unroll
     for (int i = 0; i < PD; ++i) pos[i] = 0.0f;
-    if (valid) load_position<PD>(positions, n, pos);
+    if (valid) load_features<PD>(features, n, pos);
 
     Simplex<PD> s;
     enclosing_simplex<PD>(pos, scale, s);
@@ -969,14 +995,14 @@ hipError_t clear_table(uint64_t *cell_keys, uint32_t n_cells, hipStream_t s) {
 
 bool build_can_splat(int vd) { return vd >= 2 && vd <= 4; }
 
-hipError_t build(int pd, const float *positions, const PointMap &map, const ScaleFactor &scale,
+hipError_t build(int pd, const PointFeatures &features, const PointMap &map, const ScaleFactor &scale,
                  uint64_t *cell_keys, uint32_t n_cells, Counters *counters, int *replay_index,
                  float *replay_weight, int xcd_aware, int splat_vd, const float *input,
                  int in_channels, float *cell_values, hipStream_t s) {
     if (map.n_blocks == 0) return hipSuccess;
 #define PLK_BUILD(SPLAT_VD)                                                                        \
     PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_build<PD, SPLAT_VD>), dim3(map.n_blocks),            \
-                                           dim3(kBlock), 0, s, positions, map, scale, cell_keys,   \
+                                           dim3(kBlock), 0, s, features, map, scale, cell_keys,    \
                                            n_cells - 1u, counters, replay_index, replay_weight,    \
                                            xcd_aware, input, in_channels, cell_values))
     switch (splat_vd) {

@@ -64,6 +64,9 @@ def test_null_handles_are_rejected():
     assert lib.pl_filter(None, None, None, None, 0) == pla.PL_EINVAL
     assert lib.pl_build(None, None) == pla.PL_EINVAL
     assert lib.pl_apply(None, None, None, 0) == pla.PL_EINVAL
+    dims = (C.c_int * 2)(8, 8)
+    assert lib.pl_filter_image(None, None, None, None, 3, 2, dims, 1.0, 1.0, 0) == pla.PL_EINVAL
+    assert lib.pl_build_image(None, None, 3, 2, dims, 1.0, 1.0) == pla.PL_EINVAL
     assert lib.pl_num_vertices(None, None) == pla.PL_EINVAL
     assert lib.pl_set_option(None, 1, 0) == pla.PL_EINVAL
     assert lib.pl_destroy(None) == pla.PL_OK

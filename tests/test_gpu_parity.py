@@ -409,6 +409,54 @@ def test_op_3d_volume():
     assert_float_parity(host(got), want, scale=max(1.0, float(np.abs(want).max())))
 
 
+@pytest.mark.parametrize("sdims,rc,vd,stds", [((96, 80), 3, 4, (8.0, 0.125)),
+                                               ((37, 53), 3, 4, (7.3, 0.017)),
+                                               ((20, 24, 28), 1, 2, (5.0, 0.1)),
+                                               ((64, 48), 0, 3, (3.0, 1.0)),
+                                               ((300,), 2, 3, (3.0, 13.0)),
+                                               ((6, 5, 4, 7), 1, 2, (1.5, 0.3))])
+def test_features_built_on_the_fly_give_the_lattice_of_the_positions_array(sdims, rc, vd, stds):
+    """pl_filter_image / pl_build_image against compute_positions + filter: same vertex count and
+    key set as the oracle gets from the oracle's positions (so every division rounded alike),
+    outputs within tolerance, forward and reverse."""
+    n, pd = int(np.prod(sdims)), len(sdims) + rc
+    ref = synth.uniform_image((n, rc), 41) if rc else None
+    val = synth.uniform_image((n, vd - 1), 42)
+    pos = oracle.compute_positions(ref, sdims, stds[0], stds[1], rc)
+    d_ref = dev(ref) if rc else None
+    lat = pla.PermutohedralLattice(pd, vd, n)
+    out = torch.empty((n, vd - 1), dtype=torch.float32, device="cuda")
+    for reverse in (False, True):
+        cpu = oracle.Lattice(pd, vd, n)
+        want = cpu.filter(val, pos, reverse)
+        lat.filter_image(out, dev(val), d_ref, sdims, stds[0], stds[1], reverse)
+        torch.cuda.synchronize()
+        assert lat.num_vertices == cpu.num_vertices
+        assert (sorted_keys(host(lat.debug_keys()))[0] == sorted_keys(cpu.keys())[0]).all()
+        assert_float_parity(host(out), want)
+    # build once from the image, apply many
+    lat2 = pla.PermutohedralLattice(pd, vd, n)
+    lat2.build_image(d_ref, sdims, stds[0], stds[1])
+    assert lat2.num_vertices == lat.num_vertices
+    out2 = torch.empty_like(out)
+    lat2.apply(out2, dev(val), True)
+    torch.cuda.synchronize()
+    assert_float_parity(host(out2), host(out))
+
+
+def test_image_entry_points_check_their_shapes():
+    lat = pla.PermutohedralLattice(5, 4, 64 * 64)
+    x = torch.zeros((64 * 64, 3), device="cuda")
+    ref = torch.zeros((64 * 64, 3), device="cuda")
+    with pytest.raises(pla.PermutohedralError) as e:       # extents do not multiply to N
+        lat.filter_image(torch.empty_like(x), x, ref, (64, 63), 8.0, 0.125)
+    assert e.value.status == pla.PL_EINVAL
+    lat3 = pla.PermutohedralLattice(4, 4, 64 * 64)          # pd != spatial dims + channels
+    status = pla._lib.pl_filter_image(lat3._h, x.data_ptr(), x.data_ptr(), ref.data_ptr(), 3, 2,
+                                      (pla.C.c_int * 2)(64, 64), 8.0, 0.125, 0)
+    assert status == pla.PL_EINVAL
+
+
 def test_op_rejects_unsupported_dimensions():
     x = torch.zeros((1, 8, 8, 2), device="cuda")
     ref = torch.zeros((1, 8, 8, 7), device="cuda")   # pd = 9
