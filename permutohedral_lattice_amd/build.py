@@ -70,6 +70,24 @@ def build_cpp_driver(verbose=False):
     return CPP_DRIVER_BIN
 
 
+CLI_SRC = os.path.join(_HERE, "csrc", "bilateral_filter_cli.cpp")
+CLI_BIN = os.path.join(_HERE, "bilateral_filter_hip.bin")
+
+
+def build_cli(verbose=False):
+    """The command-line bilateral filter for BMP images (the reference's test_bilateral_gpu)."""
+    cmd = [hipcc(), "-O2", "-std=c++17", "-Wno-unused-command-line-argument",
+           "-I" + os.path.join(_ROOT, "include"), CLI_SRC, "-L" + _HERE, "-lpermutohedral_hip",
+           "-Wl,-rpath,$ORIGIN", "-o", CLI_BIN]
+    if verbose:
+        print(" ".join(cmd), flush=True)
+    res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("hipcc failed:\n" + res.stdout)
+    return CLI_BIN
+
+
 if __name__ == "__main__":
     print(build(verbose=True))
+    print(build_cli(verbose=True))
     sys.exit(0)
