@@ -264,6 +264,23 @@ __global__ __launch_bounds__(kBlock) void k_clear_table(uint64_t *cell_keys, uin
     if (i < n_cells) cell_keys[i] = kEmptyCell;
 }
 
+// Mask of the lanes whose predicate holds (the compare result itself, no detour through 0/1)
+__device__ __forceinline__ uint64_t wave_ballot(bool predicate) {
+    return __builtin_amdgcn_ballot_w64(predicate);
+}
+
+// Mask of the (executing) lanes whose x equals the wavefront-uniform k, straight from the compare
+__device__ __forceinline__ uint64_t lanes_equal(uint64_t x, uint64_t k) {
+    return __builtin_amdgcn_uicmpl(x, k, 32 /* ICMP_EQ */);
+}
+__device__ __forceinline__ uint64_t lanes_equal(int x, int k) {
+    return __builtin_amdgcn_uicmp((unsigned)x, (unsigned)k, 32 /* ICMP_EQ */);
+}
+// A lane mask as a per-lane predicate
+__device__ __forceinline__ bool lane_in(uint64_t mask) {
+    return __builtin_amdgcn_inverse_ballot_w64(mask);
+}
+
 __device__ __forceinline__ int lane_value(int x, int lane) { return __builtin_amdgcn_readlane(x, lane); }
 __device__ __forceinline__ uint64_t lane_value(uint64_t x, int lane) {
     const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)x, lane);
@@ -277,13 +294,13 @@ __device__ __forceinline__ uint64_t lane_value(uint64_t x, int lane) {
 template <typename T>
 __device__ __forceinline__ int wave_leader_of_equal(T x, bool active, int lane) {
     int leader = lane;
-    uint64_t remaining = __ballot(active);
+    const uint64_t among = wave_ballot(active);
+    uint64_t remaining = among;
     while (remaining) {
         const int first = __builtin_ctzll(remaining);
-        const T k = lane_value(x, first);
-        const bool same = active && x == k;
-        if (same) leader = first;
-        remaining &= ~__ballot(same);
+        const uint64_t same = lanes_equal(x, lane_value(x, first)) & among;
+        if (lane_in(same)) leader = first;
+        remaining &= ~same;
     }
     return leader;
 }
@@ -324,20 +341,39 @@ template <int VD>
 __device__ __forceinline__ int channel_of_lane(int lane) {
     return VD == 2 ? (lane & 1) : (((lane & 1) << 1) | ((lane >> 1) & 1));
 }
+// Which of its terms a lane keeps and which it hands to its neighbour in the first exchange
+// depends only on the lane, not on the group being summed: sorted once per point.
+struct QuadTerms {
+    float keep_a, keep_b, send_a, send_b;
+};
 template <int VD>
-__device__ __forceinline__ float wave_sum_to_last_lanes(bool member, const float (&term)[4], int lane) {
-    const bool bit0 = lane & 1, bit1 = lane & 2;
-    const float x0 = member ? term[0] : 0.0f, x1 = member ? term[1] : 0.0f;
+__device__ __forceinline__ QuadTerms quad_terms(const float (&term)[4], int lane) {
+    const bool bit0 = lane & 1;
+    QuadTerms q;
+    if (VD == 2) {
+        q.keep_a = bit0 ? term[1] : term[0];
+        q.send_a = bit0 ? term[0] : term[1];
+        q.keep_b = q.send_b = 0.0f;
+    } else {
+        q.keep_a = bit0 ? term[2] : term[0];
+        q.keep_b = bit0 ? term[3] : term[1];
+        q.send_a = bit0 ? term[0] : term[2];
+        q.send_b = bit0 ? term[1] : term[3];
+    }
+    return q;
+}
+template <int VD>
+__device__ __forceinline__ float wave_sum_to_last_lanes(bool member, const QuadTerms &q, int lane) {
     float sum;
     if (VD == 2) {
-        const float keep = bit0 ? x1 : x0, send = bit0 ? x0 : x1;
+        const float keep = member ? q.keep_a : 0.0f, send = member ? q.send_a : 0.0f;
         sum = keep + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(send),
                                                                  kDppQuadSwap1, 0xf, 0xf, true));
         sum = add_from_lane<kDppRowShr2>(sum);
     } else {
-        const float x2 = member ? term[2] : 0.0f, x3 = member ? term[3] : 0.0f;
-        const float keep_a = bit0 ? x2 : x0, keep_b = bit0 ? x3 : x1;
-        const float send_a = bit0 ? x0 : x2, send_b = bit0 ? x1 : x3;
+        const bool bit1 = lane & 2;
+        const float keep_a = member ? q.keep_a : 0.0f, keep_b = member ? q.keep_b : 0.0f;
+        const float send_a = member ? q.send_a : 0.0f, send_b = member ? q.send_b : 0.0f;
         const float ya = keep_a + __int_as_float(__builtin_amdgcn_update_dpp(
                                       0, __float_as_int(send_a), kDppQuadSwap1, 0xf, 0xf, true));
         const float yb = keep_b + __int_as_float(__builtin_amdgcn_update_dpp(
@@ -459,13 +495,16 @@ __global__ __launch_bounds__(kBlock) void k_build(PointFeatures features, PointM
             constexpr int P = VD == 2 ? 2 : 4;
             const float w = s.weight[r];
             const float term[4] = {w * val[0], w * val[1], w * val[2], w * val[3]};
-            uint64_t remaining = __ballot(active);
+            const QuadTerms quad = quad_terms<VD>(term, lane);
+            const uint64_t among = wave_ballot(active);
+            uint64_t remaining = among;
             while (remaining) {
                 const int first = __builtin_ctzll(remaining);
-                const bool same = active && leader[r] == first;
-                remaining &= ~__ballot(same);
+                const uint64_t group = lanes_equal(leader[r], first) & among;
+                remaining &= ~group;
+                const bool same = lane_in(group);
                 const int group_cell = lane_value(own, first);
-                const float sum = wave_sum_to_last_lanes<VD>(same, term, lane);
+                const float sum = wave_sum_to_last_lanes<VD>(same, quad, lane);
                 if (group_cell >= 0 && lane >= 64 - P && channel_of_lane<VD>(lane) < VD)
                     atomicAdd(cell_values + (size_t)group_cell * VD + channel_of_lane<VD>(lane), sum);
             }
@@ -492,7 +531,7 @@ __global__ __launch_bounds__(kIdBlock) void k_assign_vertex_ids(
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const uint64_t key = cell < n_cells ? cell_keys[cell] : kEmptyCell;
     const bool occupied = key != kEmptyCell;
-    const uint64_t ballot = __ballot(occupied);
+    const uint64_t ballot = wave_ballot(occupied);
     if (lane == 0) wave_count[wave] = __builtin_popcountll(ballot);
     __syncthreads();
     if (threadIdx.x == 0) {
@@ -650,14 +689,16 @@ __global__ __launch_bounds__(kBlock) void k_splat_dpp(PointMap map,
     for (int r = 0; r < D1; ++r) {
         const int v = vertex[r];
         const float w = weight[r];
-        uint64_t remaining = __ballot(v >= 0);
+        const float term[4] = {w * val[0], w * val[1], w * val[2], w * val[3]};
+        const QuadTerms quad = quad_terms<VD>(term, lane);
+        uint64_t remaining = wave_ballot(v >= 0);
         while (remaining) {
             const int first = __builtin_ctzll(remaining);
             const int k = lane_value(v, first);
-            const bool same = v == k;
-            remaining &= ~__ballot(same);
-            const float term[4] = {w * val[0], w * val[1], w * val[2], w * val[3]};
-            const float sum = wave_sum_to_last_lanes<VD>(same, term, lane);
+            const uint64_t group = lanes_equal(v, k);
+            remaining &= ~group;
+            const bool same = lane_in(group);
+            const float sum = wave_sum_to_last_lanes<VD>(same, quad, lane);
             if (lane >= 64 - P && my_channel < VD)
                 atomicAdd(values + (size_t)k * VD + my_channel, sum);
         }
@@ -711,13 +752,15 @@ __global__ __launch_bounds__(kBlock) void k_splat_dpp_blocks(int vd, PointMap ma
             const int v = vertex[r];
             const float w = weight[r];
             const float term[4] = {w * val[0], w * val[1], w * val[2], w * val[3]};
-            uint64_t remaining = __ballot(v >= 0);
+            const QuadTerms quad = quad_terms<4>(term, lane);
+            uint64_t remaining = wave_ballot(v >= 0);
             while (remaining) {
                 const int first = __builtin_ctzll(remaining);
                 const int k = lane_value(v, first);
-                const bool same = v == k;
-                remaining &= ~__ballot(same);
-                const float sum = wave_sum_to_last_lanes<4>(same, term, lane);
+                const uint64_t group = lanes_equal(v, k);
+                remaining &= ~group;
+                const bool same = lane_in(group);
+                const float sum = wave_sum_to_last_lanes<4>(same, quad, lane);
                 if (lane >= 60 && first_channel + my_channel < vd)
                     atomicAdd(values + (size_t)k * vd + first_channel + my_channel, sum);
             }
