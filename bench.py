@@ -161,6 +161,28 @@ def main():
         torch.cuda.synchronize()
         op_ms[name] = 1e3 * (time.perf_counter() - t0) / args.steps
 
+    # a batch through the op: four images, forward then reverse, one item at a time as the
+    # reference's loop runs them, and with the items spread over concurrent lattices
+    batch = 4
+    b_img = torch.from_numpy(np.stack([synth.blob_image(side, side, seed=0xC0FFEE + 10 + i)
+                                       for i in range(batch)])).cuda()
+    b_grad = torch.from_numpy(synth.normal_image((batch, side, side, 3), 0xC0FFEE + 20)).cuda()
+    batch_ms = {}
+    for lanes in (1, 4):
+        pla.set_op_concurrency(lanes)
+        for _ in range(2):
+            pla._lattice_filter_raw(b_img, b_img, True, 8.0, 0.125, 1.0, False)
+        torch.cuda.synchronize()
+        reps = max(3, args.steps // 5)
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            pla._lattice_filter_raw(b_img, b_img, True, 8.0, 0.125, 1.0, False)
+            pla._lattice_filter_raw(b_grad, b_img, True, 8.0, 0.125, 1.0, True)
+        torch.cuda.synchronize()
+        batch_ms["%d_at_a_time" % lanes] = 1e3 * (time.perf_counter() - t0) / reps
+    pla.set_op_concurrency(4)
+    del b_img, b_grad
+
     # per-kernel durations from HIP events on the lattice's stream
     lat.set_option(pla.PL_OPT_PROFILE, 1)
     stage_samples = []
@@ -220,6 +242,11 @@ def main():
                      "ms_per_step": {k: round(v, 4) for k, v in op_ms.items()},
                      "value": {k: round(pixels_per_step / (v * 1e-3) / 1e6, 3)
                                for k, v in op_ms.items()}},
+        "op_batch": {"what": "the op on a batch of %d such images, forward + reverse per step, "
+                             "items one at a time and four at a time" % batch,
+                     "ms_per_step": {k: round(v, 4) for k, v in batch_ms.items()},
+                     "value": {k: round(batch * pixels_per_step / (v * 1e-3) / 1e6, 3)
+                               for k, v in batch_ms.items()}},
     }
 
     if not args.no_cpu:

@@ -166,18 +166,44 @@ int pl_build_image(pl_handle h, const float *reference, int n_reference_channels
                    float feature_std);
 
 /*
+ * pl_filter / pl_filter_image in two halves, for callers that keep several lattices (each on a
+ * stream of its own) in flight: *_begin enqueues the whole call on the lattice's stream and
+ * returns at once; pl_filter_end waits for that stream and, should the hash table have turned
+ * out too small, repeats the call with a larger one before it returns.  The arguments of *_begin
+ * must stay valid until pl_filter_end; between the two only pl_filter_end and pl_destroy may be
+ * called on the handle (anything else returns PL_ESTATE).  pl_filter_end with nothing in flight
+ * returns PL_OK.  The reference's filter (src/PermutohedralLatticeGPU.cuh:454-479) enqueues on
+ * its stream without waiting as well; what the second half adds is the check of the table size.
+ */
+int pl_filter_begin(pl_handle h, float *output, const float *input, const float *positions,
+                    int reverse);
+int pl_filter_image_begin(pl_handle h, float *output, const float *input, const float *reference,
+                          int n_reference_channels, int n_spatial_dims, const int *spatial_dims,
+                          float spatial_std, float feature_std, int reverse);
+int pl_filter_end(pl_handle h);
+
+/*
  * The LatticeFilter op on channels-last device tensors input[B, s_1..s_k, C_in],
  * reference[B, s_1..s_k, C_ref] -> output (shape of input).  bilateral: features are
  * (coords/theta_alpha, reference/theta_beta); otherwise coords/theta_gamma and the reference is
  * ignored (may be NULL).  One lattice per batch item.  Stands in for LatticeFilterOp::Compute
  * (src/LatticeFilterKernel.cpp:98-181); its gradient is the same call on the upstream gradient
- * with reverse = 1 (lattice_filter_op_loader.py:32-54).  Scratch comes from alloc (NULL = hipMalloc).
+ * with reverse = 1 (lattice_filter_op_loader.py:32-54).  Scratch comes from alloc; with NULL the
+ * library keeps lattices of its own between calls and runs several batch items at a time (see
+ * pl_set_op_concurrency).  Returns when the results are complete.
  */
 int pl_lattice_filter_op(const float *input, const float *reference, float *output, int batch,
                          int n_spatial_dims, const int *spatial_dims, int n_input_channels,
                          int n_reference_channels, int bilateral, float theta_alpha,
                          float theta_beta, float theta_gamma, int reverse, pl_stream stream,
                          const pl_alloc *alloc);
+
+/*
+ * How many batch items pl_lattice_filter_op (with alloc = NULL) keeps in flight at once, each on a
+ * lattice and a stream of its own (1..8, default 4; 1 = one after the other as the reference's
+ * loop, src/LatticeFilterKernel.cpp:152-179).  Process-wide.
+ */
+int pl_set_op_concurrency(int lanes);
 
 #ifdef __cplusplus
 }

@@ -27,7 +27,8 @@ EXPORTS = (
     "pl_supported", "pl_strerror", "pl_last_hip_error", "pl_create", "pl_destroy", "pl_filter",
     "pl_build", "pl_apply", "pl_set_point_grid", "pl_num_vertices", "pl_set_option", "pl_stage_ms", "pl_debug_simplex",
     "pl_debug_keys", "pl_debug_replay", "pl_compute_positions", "pl_filter_image", "pl_build_image",
-    "pl_lattice_filter_op",
+    "pl_filter_begin", "pl_filter_image_begin", "pl_filter_end", "pl_lattice_filter_op",
+    "pl_set_op_concurrency",
 )
 
 
@@ -69,6 +70,10 @@ def _load():
     lib.pl_compute_positions.argtypes = [vp, vp, ci, ci, ci, C.POINTER(ci), cf, cf, vp]
     lib.pl_filter_image.argtypes = [vp, vp, vp, vp, ci, ci, C.POINTER(ci), cf, cf, ci]
     lib.pl_build_image.argtypes = [vp, vp, ci, ci, C.POINTER(ci), cf, cf]
+    lib.pl_filter_begin.argtypes = [vp, vp, vp, vp, ci]
+    lib.pl_filter_image_begin.argtypes = [vp, vp, vp, vp, ci, ci, C.POINTER(ci), cf, cf, ci]
+    lib.pl_filter_end.argtypes = [vp]
+    lib.pl_set_op_concurrency.argtypes = [ci]
     lib.pl_lattice_filter_op.argtypes = [vp, vp, vp, ci, ci, C.POINTER(ci), ci, ci, ci, cf, cf, cf,
                                          ci, vp, vp]
     return lib
@@ -127,6 +132,19 @@ class PermutohedralLattice:
                               _dev_f32(positions, "positions", self.N * self.pd), int(bool(reverse))),
                "pl_filter")
         return output
+
+    # -- the same in two halves: enqueue, and later wait and check ---------------------------------
+    def filter_begin(self, output, input, positions, reverse=False):
+        ch = self.vd - 1 if self._normalize else self.vd
+        self._in_flight = (output, input, positions)   # keep the tensors alive until filter_end
+        _check(_lib.pl_filter_begin(self._h, _dev_f32(output, "output", self.N * ch),
+                                    _dev_f32(input, "input", self.N * ch),
+                                    _dev_f32(positions, "positions", self.N * self.pd),
+                                    int(bool(reverse))), "pl_filter_begin")
+
+    def filter_end(self):
+        _check(_lib.pl_filter_end(self._h), "pl_filter_end")
+        self._in_flight = None
 
     # -- build once, apply many ----------------------------------------------------------------
     def build(self, positions):
@@ -215,6 +233,11 @@ class PermutohedralLattice:
         _check(_lib.pl_debug_replay(self._h, C.c_void_p(v.data_ptr()), C.c_void_p(w.data_ptr())),
                "pl_debug_replay")
         return v, w
+
+
+def set_op_concurrency(lanes):
+    """Batch items :func:`lattice_filter` keeps in flight at once (1..8, default 4)."""
+    _check(_lib.pl_set_op_concurrency(int(lanes)), "pl_set_op_concurrency")
 
 
 def compute_positions(reference, spatial_dims, spatial_std, feature_std=1.0, out=None):

@@ -105,6 +105,16 @@ struct pl_lattice {
     hipEvent_t ev[EV_COUNT] = {};
     bool ev_recorded[EV_COUNT] = {};
 
+    // a filter call that has been enqueued but not yet checked on the host (pl_filter_*_begin)
+    struct Pending {
+        bool active = false;
+        plk::PointFeatures features{};
+        float *output = nullptr;
+        const float *input = nullptr;
+        int reverse = 0;
+        uint32_t cells = 0;
+    } pending;
+
     void *dmalloc(size_t bytes) { return alloc.alloc(alloc.ctx, bytes); }
     template <typename T>
     void dfree(T *&p) {
@@ -417,6 +427,7 @@ int pl_set_option(pl_handle h, int option, long value) {
 
 int pl_set_point_grid(pl_handle h, int n_dims, const int *dims) {
     if (!h || n_dims < 0 || (n_dims > 0 && !dims)) return PL_EINVAL;
+    if (h->pending.active) return PL_ESTATE;
     if (n_dims > 0) {
         long long prod = 1;
         for (int i = 0; i < n_dims; ++i) {
@@ -483,8 +494,12 @@ int build_lattice(pl_lattice *h, const plk::PointFeatures &features) {
     }
 }
 
-int filter_lattice(pl_lattice *h, float *output, const float *input,
-                   const plk::PointFeatures &features, int reverse) {
+// pl_filter in two halves.  begin: build and apply are enqueued together and the call returns.
+// end: waits for the lattice's stream; if the table turned out too small the whole call is
+// repeated with a larger one (the output is simply written again).
+int filter_begin(pl_lattice *h, float *output, const float *input,
+                 const plk::PointFeatures &features, int reverse) {
+    if (h->pending.active) return PL_ESTATE;
     h->built = false;
     h->M = 0;
     for (int i = 0; i < EV_COUNT; ++i) h->ev_recorded[i] = false;
@@ -492,24 +507,48 @@ int filter_lattice(pl_lattice *h, float *output, const float *input,
         h->built = h->verified = true;
         return PL_OK;
     }
-    // build and apply are enqueued together; if the table turns out too small the whole call is
-    // repeated with a larger one (the output is simply written again)
-    uint32_t cells = initial_cells(h);
+    const uint32_t cells = initial_cells(h);
+    int rc = enqueue_build(h, features, cells, input);
+    if (rc != PL_OK) return rc;
+    rc = enqueue_apply(h, output, input, reverse);
+    if (rc != PL_OK) return rc;
+    h->pending.active = true;
+    h->pending.features = features;
+    h->pending.output = output;
+    h->pending.input = input;
+    h->pending.reverse = reverse;
+    return PL_OK;
+}
+
+int filter_end(pl_lattice *h) {
+    if (!h->pending.active) return PL_OK;   // nothing in flight (or an empty lattice)
     for (;;) {
-        int rc = enqueue_build(h, features, cells, input);
-        if (rc != PL_OK) return rc;
-        rc = enqueue_apply(h, output, input, reverse);
-        if (rc != PL_OK) return rc;
-        rc = verify_build(h, &cells);
-        if (rc == PL_OK) return PL_OK;
-        if (!cells) return rc;
+        uint32_t cells = 0;
+        int rc = verify_build(h, &cells);
+        if (rc == PL_OK || !cells) {
+            h->pending.active = false;
+            return rc;
+        }
+        rc = enqueue_build(h, h->pending.features, cells, h->pending.input);
+        if (rc == PL_OK) rc = enqueue_apply(h, h->pending.output, h->pending.input, h->pending.reverse);
+        if (rc != PL_OK) {
+            h->pending.active = false;
+            return rc;
+        }
     }
+}
+
+int filter_lattice(pl_lattice *h, float *output, const float *input,
+                   const plk::PointFeatures &features, int reverse) {
+    const int rc = filter_begin(h, output, input, features, reverse);
+    return rc == PL_OK ? filter_end(h) : rc;
 }
 
 }  // namespace
 
 int pl_build(pl_handle h, const float *positions) {
     if (!h || (!positions && h->N > 0)) return PL_EINVAL;
+    if (h->pending.active) return PL_ESTATE;
     return build_lattice(h, features_from_positions(positions));
 }
 
@@ -517,6 +556,7 @@ int pl_build_image(pl_handle h, const float *reference, int n_reference_channels
                    int n_spatial_dims, const int *spatial_dims, float spatial_std,
                    float feature_std) {
     if (!h) return PL_EINVAL;
+    if (h->pending.active) return PL_ESTATE;
     plk::PointFeatures features;
     const int rc = features_from_image(h, reference, n_reference_channels, n_spatial_dims,
                                        spatial_dims, spatial_std, feature_std, &features);
@@ -525,7 +565,7 @@ int pl_build_image(pl_handle h, const float *reference, int n_reference_channels
 
 int pl_apply(pl_handle h, float *output, const float *input, int reverse) {
     if (!h) return PL_EINVAL;
-    if (!h->built || !h->verified) return PL_ESTATE;
+    if (!h->built || !h->verified || h->pending.active) return PL_ESTATE;
     if (h->N == 0) return PL_OK;
     if (!output || !input) return PL_EINVAL;
     return enqueue_apply(h, output, input, reverse);
@@ -541,11 +581,36 @@ int pl_filter_image(pl_handle h, float *output, const float *input, const float 
                     int n_reference_channels, int n_spatial_dims, const int *spatial_dims,
                     float spatial_std, float feature_std, int reverse) {
     if (!h) return PL_EINVAL;
+    if (h->pending.active) return PL_ESTATE;
     if (h->N > 0 && (!output || !input)) return PL_EINVAL;
     plk::PointFeatures features;
     const int rc = features_from_image(h, reference, n_reference_channels, n_spatial_dims,
                                        spatial_dims, spatial_std, feature_std, &features);
     return rc == PL_OK ? filter_lattice(h, output, input, features, reverse) : rc;
+}
+
+int pl_filter_begin(pl_handle h, float *output, const float *input, const float *positions,
+                    int reverse) {
+    if (!h) return PL_EINVAL;
+    if (h->N > 0 && (!output || !input || !positions)) return PL_EINVAL;
+    return filter_begin(h, output, input, features_from_positions(positions), reverse);
+}
+
+int pl_filter_image_begin(pl_handle h, float *output, const float *input, const float *reference,
+                          int n_reference_channels, int n_spatial_dims, const int *spatial_dims,
+                          float spatial_std, float feature_std, int reverse) {
+    if (!h) return PL_EINVAL;
+    if (h->pending.active) return PL_ESTATE;
+    if (h->N > 0 && (!output || !input)) return PL_EINVAL;
+    plk::PointFeatures features;
+    const int rc = features_from_image(h, reference, n_reference_channels, n_spatial_dims,
+                                       spatial_dims, spatial_std, feature_std, &features);
+    return rc == PL_OK ? filter_begin(h, output, input, features, reverse) : rc;
+}
+
+int pl_filter_end(pl_handle h) {
+    if (!h) return PL_EINVAL;
+    return filter_end(h);
 }
 
 int pl_num_vertices(pl_handle h, int *num_vertices) {
@@ -623,18 +688,65 @@ int pl_compute_positions(const float *reference, float *positions, int num_super
 // ------------------------------------------------------------------------------------------------
 namespace {
 
-// With the default allocator the op keeps its lattice between calls (one per device, shape and
-// stream), because hipMalloc/hipFree per call would serialise the device.  With a
-// caller-supplied allocator everything is taken from it and returned before the call ends, as
-// the reference does with TensorFlow temporaries (src/DeviceMemoryAllocator.h:52-71).
+// With the default allocator the op keeps its lattices between calls (per device, shape and
+// stream), because hipMalloc/hipFree per call would serialise the device.  A batch is spread
+// over up to g_op_lanes lattices, the first on the caller's stream, the others on streams of
+// their own: the items are independent lattices (LatticeFilterKernel.cpp:152-179), and the
+// kernels over the few hundred thousand vertices of one item leave most of the GPU idle.
+// With a caller-supplied allocator everything is taken from it and returned before the call
+// ends, as the reference does with TensorFlow temporaries (src/DeviceMemoryAllocator.h:52-71),
+// and the items run one after the other.
+struct OpLane {
+    pl_handle lattice = nullptr;
+    hipStream_t stream = nullptr;   // owned unless it is the caller's (lane 0)
+    bool owns_stream = false;
+    hipEvent_t done = nullptr;
+};
 struct OpCacheEntry {
     int device, pd, vd, N;
     hipStream_t stream;
-    pl_handle lattice;
+    std::vector<OpLane> lanes;
+    hipEvent_t fork = nullptr;
 };
 std::mutex g_op_cache_mutex;
 std::vector<OpCacheEntry> g_op_cache;
 constexpr size_t kOpCacheMax = 8;
+constexpr int kOpLanesMax = 8;
+int g_op_lanes = 4;
+
+void destroy_entry(OpCacheEntry &e) {
+    for (auto &lane : e.lanes) {
+        pl_destroy(lane.lattice);   // waits for the lane's stream
+        if (lane.done) (void)hipEventDestroy(lane.done);
+        if (lane.owns_stream && lane.stream) (void)hipStreamDestroy(lane.stream);
+    }
+    if (e.fork) (void)hipEventDestroy(e.fork);
+    e.lanes.clear();
+}
+
+// Lattices and streams for `want` concurrent items.
+int ensure_lanes(OpCacheEntry &e, int want) {
+    while ((int)e.lanes.size() < want) {
+        OpLane lane;
+        if (e.lanes.empty()) {
+            lane.stream = e.stream;
+        } else {
+            PL_HIP(hipStreamCreateWithFlags(&lane.stream, hipStreamNonBlocking));
+            lane.owns_stream = true;
+        }
+        int rc = pl_create(e.pd, e.vd, e.N, (pl_stream)lane.stream, nullptr, &lane.lattice);
+        if (rc == PL_OK && hipEventCreateWithFlags(&lane.done, hipEventDisableTiming) != hipSuccess)
+            rc = PL_EHIP;
+        if (rc != PL_OK) {
+            pl_destroy(lane.lattice);
+            if (lane.owns_stream) (void)hipStreamDestroy(lane.stream);
+            return rc;
+        }
+        e.lanes.push_back(lane);
+    }
+    if (want > 1 && !e.fork) PL_HIP(hipEventCreateWithFlags(&e.fork, hipEventDisableTiming));
+    return PL_OK;
+}
 
 }  // namespace
 
@@ -668,42 +780,75 @@ extern "C" int pl_lattice_filter_op(const float *input, const float *reference, 
     int device = 0;
     PL_HIP(hipGetDevice(&device));
 
-    pl_handle lattice = nullptr;
-    bool cached = false;
-    std::unique_lock<std::mutex> lock(g_op_cache_mutex, std::defer_lock);
-    if (!alloc) {
-        lock.lock();  // held for the whole call: a cached lattice is not re-entrant
-        for (auto &e : g_op_cache)
-            if (e.device == device && e.pd == pd && e.vd == vd && e.N == N &&
-                e.stream == (hipStream_t)stream) {
-                lattice = e.lattice;
-                cached = true;
-                break;
-            }
-    }
-    int rc = PL_OK;
-    if (!lattice) {
-        rc = pl_create(pd, vd, N, stream, alloc, &lattice);
-        if (rc != PL_OK) return rc;
-        if (!alloc) {
-            if (g_op_cache.size() >= kOpCacheMax) {
-                pl_destroy(g_op_cache.front().lattice);
-                g_op_cache.erase(g_op_cache.begin());
-            }
-            g_op_cache.push_back({device, pd, vd, N, (hipStream_t)stream, lattice});
-            cached = true;
+    if (alloc) {
+        // caller's scratch: one lattice, items one after the other, everything returned at the end
+        pl_handle lattice = nullptr;
+        int rc = pl_create(pd, vd, N, stream, alloc, &lattice);
+        for (int b = 0; b < batch && rc == PL_OK; ++b) {
+            const float *ref_b = ref_ch ? reference + (size_t)b * N * ref_ch : nullptr;
+            rc = pl_filter_image(lattice, output + (size_t)b * N * n_input_channels,
+                                 input + (size_t)b * N * n_input_channels, ref_b, ref_ch,
+                                 n_spatial_dims, spatial_dims, spatial_std, feature_std, reverse);
         }
+        pl_destroy(lattice);  // synchronises the stream first
+        return rc;
     }
 
+    // held for the whole call: cached lattices are not re-entrant
+    std::lock_guard<std::mutex> lock(g_op_cache_mutex);
+    OpCacheEntry *entry = nullptr;
+    for (auto &e : g_op_cache)
+        if (e.device == device && e.pd == pd && e.vd == vd && e.N == N &&
+            e.stream == (hipStream_t)stream) {
+            entry = &e;
+            break;
+        }
+    if (!entry) {
+        if (g_op_cache.size() >= kOpCacheMax) {
+            destroy_entry(g_op_cache.front());
+            g_op_cache.erase(g_op_cache.begin());
+        }
+        g_op_cache.push_back(OpCacheEntry{device, pd, vd, N, (hipStream_t)stream, {}, nullptr});
+        entry = &g_op_cache.back();
+    }
+    const int n_lanes = batch < g_op_lanes ? batch : g_op_lanes;
+    int rc = ensure_lanes(*entry, n_lanes);
+    if (rc != PL_OK) return rc;
+
+    // the other lanes start after whatever the caller's stream holds so far
+    if (n_lanes > 1) {
+        PL_HIP(hipEventRecord(entry->fork, (hipStream_t)stream));
+        for (int l = 1; l < n_lanes; ++l)
+            PL_HIP(hipStreamWaitEvent(entry->lanes[l].stream, entry->fork, 0));
+    }
     // One lattice per batch item (LatticeFilterKernel.cpp:152-179).  The feature vectors are built
     // inside the lattice's first kernel, from the item's reference image and the grid coordinates.
     for (int b = 0; b < batch && rc == PL_OK; ++b) {
+        pl_handle lattice = entry->lanes[b % n_lanes].lattice;
+        rc = pl_filter_end(lattice);   // the item this lane took before
+        if (rc != PL_OK) break;
         const float *ref_b = ref_ch ? reference + (size_t)b * N * ref_ch : nullptr;
-        rc = pl_filter_image(lattice, output + (size_t)b * N * n_input_channels,
-                             input + (size_t)b * N * n_input_channels, ref_b, ref_ch,
-                             n_spatial_dims, spatial_dims, spatial_std, feature_std, reverse);
+        rc = pl_filter_image_begin(lattice, output + (size_t)b * N * n_input_channels,
+                                   input + (size_t)b * N * n_input_channels, ref_b, ref_ch,
+                                   n_spatial_dims, spatial_dims, spatial_std, feature_std, reverse);
     }
-
-    if (!cached) pl_destroy(lattice);  // synchronises the stream first
+    // every lane is drained, also after an error; the caller's stream continues after all of them
+    for (int l = 0; l < n_lanes; ++l) {
+        const int rc_end = pl_filter_end(entry->lanes[l].lattice);
+        if (rc == PL_OK) rc = rc_end;
+    }
+    for (int l = 1; l < n_lanes; ++l) {
+        if (hipEventRecord(entry->lanes[l].done, entry->lanes[l].stream) != hipSuccess ||
+            hipStreamWaitEvent((hipStream_t)stream, entry->lanes[l].done, 0) != hipSuccess) {
+            if (rc == PL_OK) rc = PL_EHIP;
+        }
+    }
     return rc;
+}
+
+extern "C" int pl_set_op_concurrency(int lanes) {
+    if (lanes < 1 || lanes > kOpLanesMax) return PL_EINVAL;
+    std::lock_guard<std::mutex> lock(g_op_cache_mutex);
+    g_op_lanes = lanes;
+    return PL_OK;
 }

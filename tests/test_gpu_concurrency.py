@@ -1,0 +1,121 @@
+"""Several lattices in flight: the two halves of filter (pl_filter_begin / pl_filter_end) on
+lattices with streams of their own, and the op spreading a batch over concurrent lattices.
+Results must not depend on how many items run at a time; parity is against the CPU oracle."""
+import numpy as np
+import pytest
+import torch
+
+from conftest import MAX_ABS_TOL, REL_L2_TOL, rel_l2
+from permutohedral_lattice_amd import synth
+
+import oracle
+import permutohedral_lattice_amd as pla
+
+pytestmark = pytest.mark.gpu
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def close(got, want, scale=1.0):
+    assert np.isfinite(got).all()
+    assert np.abs(got - want).max() <= MAX_ABS_TOL * scale
+    assert rel_l2(got, want) <= REL_L2_TOL
+
+
+def test_two_lattices_in_flight_on_two_streams():
+    h = w = 160
+    cases = []
+    for seed, reverse in ((31, False), (32, True), (33, False)):
+        img = synth.blob_image(h, w, seed=seed)
+        pos = synth.bilateral_positions(img, 8.0, 0.125)
+        val = synth.uniform_image((h * w, 3), seed + 100)
+        cases.append((pos, val, reverse, oracle.Lattice(5, 4, h * w).filter(val, pos, reverse)))
+    streams = [torch.cuda.Stream() for _ in cases]
+    lattices, outs = [], []
+    torch.cuda.synchronize()
+    for (pos, val, reverse, _), s in zip(cases, streams):
+        d_pos, d_val = dev(pos), dev(val)
+        out = torch.empty((h * w, 3), dtype=torch.float32, device="cuda")
+        torch.cuda.synchronize()          # the uploads ran on the current stream
+        lat = pla.PermutohedralLattice(5, 4, h * w, stream=s)
+        lat.filter_begin(out, d_val, d_pos, reverse)
+        lattices.append(lat)
+        outs.append(out)
+    for lat in lattices:
+        lat.filter_end()
+    for lat, out, (_, _, _, want) in zip(lattices, outs, cases):
+        close(out.cpu().numpy(), want)
+        assert lat.num_vertices > 0
+    lattices[0].filter_end()               # nothing in flight: fine
+
+
+def test_only_end_may_follow_begin():
+    n = 64 * 64
+    img = synth.blob_image(64, 64, seed=35)
+    d_pos = dev(synth.bilateral_positions(img, 8.0, 0.125))
+    d_val = dev(img.reshape(-1, 3))
+    out = torch.empty_like(d_val)
+    lat = pla.PermutohedralLattice(5, 4, n)
+    lat.filter_begin(out, d_val, d_pos)
+    for call in (lambda: lat.apply(out, d_val), lambda: lat.build(d_pos),
+                 lambda: lat.filter(out, d_val, d_pos), lambda: lat.set_point_grid((64, 64)),
+                 lambda: lat.filter_begin(out, d_val, d_pos), lambda: lat.num_vertices):
+        with pytest.raises(pla.PermutohedralError) as e:
+            call()
+        assert e.value.status == pla.PL_ESTATE
+    lat.filter_end()
+    want = oracle.Lattice(5, 4, n).filter(img.reshape(-1, 3), synth.bilateral_positions(img, 8.0, 0.125))
+    close(out.cpu().numpy(), want)
+    lat.apply(out, d_val)                  # usable again
+
+
+def test_end_repeats_the_call_when_the_table_was_too_small():
+    rng = np.random.default_rng(36)
+    n = 20000
+    pos = rng.uniform(0, 40, (n, 3)).astype(np.float32)    # scattered: about 4 vertices per point
+    val = rng.uniform(0, 1, (n, 2)).astype(np.float32)
+    cpu = oracle.Lattice(3, 3, n)
+    want = cpu.filter(val, pos, False)
+    lat = pla.PermutohedralLattice(3, 3, n)
+    lat.set_option(pla.PL_OPT_TABLE_CELLS, 4096)
+    out = torch.empty((n, 2), dtype=torch.float32, device="cuda")
+    lat.filter_begin(out, dev(val), dev(pos))
+    lat.filter_end()
+    assert lat.num_vertices == cpu.num_vertices > 4096
+    close(out.cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("batch", [1, 3, 6])
+def test_op_results_do_not_depend_on_the_number_of_items_in_flight(batch):
+    h, w = 72, 88
+    guide = np.stack([synth.blob_image(h, w, seed=40 + i) for i in range(batch)])
+    inp = synth.uniform_image((batch, h, w, 2), 47)
+    want = oracle.lattice_filter(inp, guide, True, 8.0, 0.125, 1.0, False)
+    try:
+        for lanes in (1, 2, 4):
+            pla.set_op_concurrency(lanes)
+            got = pla.lattice_filter(dev(inp), dev(guide), theta_alpha=8.0, theta_beta=0.125)
+            torch.cuda.synchronize()
+            close(got.cpu().numpy(), want)
+    finally:
+        pla.set_op_concurrency(4)
+    with pytest.raises(pla.PermutohedralError):
+        pla.set_op_concurrency(0)
+
+
+def test_op_on_a_side_stream_is_ordered_with_that_stream():
+    h, w = 64, 64
+    guide = np.stack([synth.blob_image(h, w, seed=50 + i) for i in range(3)])
+    inp = synth.uniform_image((3, h, w, 1), 53)
+    want = oracle.lattice_filter(inp, guide, True, 8.0, 0.125, 1.0, True)
+    s = torch.cuda.Stream()
+    d_inp, d_guide = dev(inp), dev(guide)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(s):
+        x = d_inp * 2.0                     # producer on the side stream
+        y = pla._lattice_filter_raw(x, d_guide, True, 8.0, 0.125, 1.0, True)
+        z = y * 0.5                         # consumer on the side stream
+    s.synchronize()
+    close(z.cpu().numpy(), want)
