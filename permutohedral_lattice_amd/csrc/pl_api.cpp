@@ -85,6 +85,13 @@ struct pl_lattice {
     plk::PointMap map{};
     int *replay_index = nullptr;
     float *replay_weight = nullptr;
+    // what each workgroup of the build created (see plk::CreatedLists); the chunk counts exist
+    // twice and alternate between builds like the counters
+    int *created_cells = nullptr;          // [n_blocks*256*(pd+1)]
+    uint64_t *created_keys = nullptr;      // [n_blocks*256*(pd+1)]
+    int *block_count = nullptr;            // [n_blocks]
+    int *chunk_count = nullptr;            // [2][n_chunks]
+    size_t n_chunks = 0;
     size_t replay_capacity = 0;
 
     plk::Counters *d_counters = nullptr;   // two sets, used by alternate builds
@@ -168,10 +175,22 @@ int ensure_replay(pl_lattice *h) {
     PL_HIP(hipStreamSynchronize(h->stream));
     h->dfree(h->replay_index);
     h->dfree(h->replay_weight);
+    h->dfree(h->created_cells);
+    h->dfree(h->created_keys);
+    h->dfree(h->block_count);
+    h->dfree(h->chunk_count);
     h->replay_capacity = 0;
+    h->n_chunks = (h->map.n_blocks + plk::kBlocksPerChunk - 1) / plk::kBlocksPerChunk + 1;
     h->replay_index = (int *)h->dmalloc(sizeof(int) * (want ? want : 1));
     h->replay_weight = (float *)h->dmalloc(sizeof(float) * (want ? want : 1));
-    if (!h->replay_index || !h->replay_weight) return PL_ENOMEM;
+    h->created_cells = (int *)h->dmalloc(sizeof(int) * (want ? want : 1));
+    h->created_keys = (uint64_t *)h->dmalloc(sizeof(uint64_t) * (want ? want : 1));
+    h->block_count = (int *)h->dmalloc(sizeof(int) * (h->map.n_blocks ? h->map.n_blocks : 1));
+    h->chunk_count = (int *)h->dmalloc(sizeof(int) * 2 * h->n_chunks);
+    if (!h->replay_index || !h->replay_weight || !h->created_cells || !h->created_keys ||
+        !h->block_count || !h->chunk_count)
+        return PL_ENOMEM;
+    PL_HIP(hipMemsetAsync(h->chunk_count, 0, sizeof(int) * 2 * h->n_chunks, h->stream));
     h->replay_capacity = want;
     return PL_OK;
 }
@@ -213,17 +232,22 @@ int enqueue_build(pl_lattice *h, const plk::PointFeatures &features, uint32_t ce
     // the previous vertex-numbering kernel (or pl_create) left the other counter set zeroed
     const int previous_set = h->counter_set;
     h->counter_set = 1 - previous_set;
+    const plk::VertexTables vertices{h->cell_vertex, h->vertex_keys, h->vertex_cell, h->neighbours,
+                                     h->max_vertices()};
+    const plk::CreatedLists lists{h->created_cells, h->created_keys, h->block_count,
+                                  h->chunk_count + (size_t)h->counter_set * h->n_chunks};
     PL_HIP(plk::build(h->pd, features, h->map, h->scale, h->cell_keys, cells, h->counters(),
                       h->replay_index, h->replay_weight, h->xcd_aware ? 1 : 0, fused ? h->vd : 0,
-                      splat_input, h->normalize ? h->vd - 1 : h->vd, h->cell_values, h->stream));
+                      splat_input, h->normalize ? h->vd - 1 : h->vd, h->cell_values, lists,
+                      h->stream));
     h->mark(EV_BUILD);
-    PL_HIP(plk::assign_vertex_ids(h->cell_keys, cells, h->cell_vertex, h->vertex_keys, h->vertex_cell,
-                                  h->values[0], h->vd, fused ? h->cell_values : nullptr,
-                                  h->neighbours, h->pd + 1, h->counters(),
-                                  h->d_counters + previous_set, h->h_status, h->stream));
+    PL_HIP(plk::number_vertices(h->pd, h->map, lists,
+                                h->chunk_count + (size_t)previous_set * h->n_chunks,
+                                (unsigned)h->n_chunks, vertices,
+                                h->values[0], h->vd, fused ? h->cell_values : nullptr, h->counters(),
+                                h->d_counters + previous_set, h->h_status, h->stream));
     h->mark(EV_IDS);
-    PL_HIP(plk::neighbours(h->pd, h->vertex_keys, h->counters(), h->max_vertices(), h->cell_keys,
-                           h->cell_vertex, cells, h->neighbours, h->stream));
+    PL_HIP(plk::neighbours(h->pd, vertices, h->counters(), h->cell_keys, cells, h->stream));
     h->mark(EV_NBR);
     h->replay_holds_cells = true;
     h->values_zeroed = !fused;
@@ -389,6 +413,10 @@ int pl_destroy(pl_handle h) {
     h->dfree(h->cell_values);
     h->dfree(h->replay_index);
     h->dfree(h->replay_weight);
+    h->dfree(h->created_cells);
+    h->dfree(h->created_keys);
+    h->dfree(h->block_count);
+    h->dfree(h->chunk_count);
     h->dfree(h->d_counters);
     if (h->h_status) (void)hipHostFree(h->h_status);
     for (int i = 0; i < EV_COUNT; ++i)

@@ -17,19 +17,28 @@ enum : int {
     kFlagKeyRange = 2,    // a lattice coordinate does not fit its field of the packed key
 };
 
-// Device-side state of one build.  Kernels after the build read the vertex count from here, so
-// the host never has to wait for it between launches.
+// Device-side state of one build.  Kernels after the numbering pass read the vertex count from
+// here, so the host never has to wait for it between launches.
 struct Counters {
-    unsigned long long vertices_and_blocks;  // low word: vertices numbered so far; high word:
-                                             // workgroups of the numbering kernel that are done
+    unsigned int vertices;   // set by the numbering pass (may exceed what the table can hold)
     int flags;
-    int pad;
 };
 
-// What the last workgroup of the vertex-numbering kernel writes to pinned host memory.
+// What the numbering pass writes to pinned host memory about the build.
 struct HostStatus {
     int num_vertices;
     int flags;
+};
+
+// Per-vertex and per-cell tables of a lattice (all sized by the hash table): vertex v has key
+// vertex_keys[v] and sits in hash cell vertex_cell[v]; cell_vertex[cell] is the inverse;
+// neighbours[a*max_vertices + v] holds v's two neighbours along blur axis a (-1: none).
+struct VertexTables {
+    int *cell_vertex;
+    uint64_t *vertex_keys;
+    int *vertex_cell;
+    int2 *neighbours;
+    int max_vertices;
 };
 
 // Vertices a table of n_cells may hold (load factor 3/4): beyond that probe sequences get long,
@@ -42,6 +51,18 @@ struct ScaleFactor {
 
 struct SpatialDims {
     int v[kMaxSpatialDims];
+};
+
+// What the build's workgroups created, for the numbering pass: workgroup b (in the build's
+// virtual order) lists the hash cells and keys of its block_count[b] new vertices from entry
+// b*256*(pd+1) on; chunk_count[c] is the sum over the kBlocksPerChunk workgroups of chunk c and
+// must be zero before the build.
+constexpr int kBlocksPerChunk = 64;
+struct CreatedLists {
+    int *cells;
+    uint64_t *keys;
+    int *block_count;
+    int *chunk_count;
 };
 
 // Where the feature vector of a point comes from: the row of a positions array, or, with
@@ -76,31 +97,33 @@ hipError_t clear_table(uint64_t *cell_keys, uint32_t n_cells, hipStream_t s);
 // Stage 1+2: per point embed, enclosing simplex, barycentric weights, then insertion of the pd+1
 // vertex keys.  The replay arrays hold (pd+1) rows of T = map.n_blocks*256 entries in thread
 // order: replay_index[r*T+t] := hash cell of vertex r of the point of thread t (-1: no point),
-// replay_weight likewise.
+// replay_weight likewise.  The lane whose insertion created a vertex appends its cell and key to
+// its workgroup's list in created_lists.
 // splat_vd != 0 (allowed when build_can_splat(vd)): the kernel also splats `input`
 // (in_channels per point) into cell_values[cell*vd ..], rows addressed by hash cell;
-// assign_vertex_ids then moves them into the dense value table.
+// number_vertices then moves them into the dense value table.
 bool build_can_splat(int vd);
 hipError_t build(int pd, const PointFeatures &features, const PointMap &map, const ScaleFactor &scale,
                  uint64_t *cell_keys, uint32_t n_cells, Counters *counters, int *replay_index,
                  float *replay_weight, int xcd_aware, int splat_vd, const float *input,
-                 int in_channels, float *cell_values, hipStream_t s);
+                 int in_channels, float *cell_values, const CreatedLists &created_lists,
+                 hipStream_t s);
 
-// Every occupied cell draws a dense vertex index: cell_vertex[cell] := v, vertex_keys[v] := key,
-// vertex_cell[v] := cell, the vertex count in *counters := M, and the vertex's row of `values` :=
-// 0, or, with cell_values != nullptr, := the row cell_values[cell*vd ..], which is zeroed.  The
-// last workgroup copies M and the flags to *host_status and zeroes *next_counters.  The d1 = pd+1
-// neighbour entries of every vertex are set to (-1, -1).
-hipError_t assign_vertex_ids(const uint64_t *cell_keys, uint32_t n_cells, int *cell_vertex,
-                             uint64_t *vertex_keys, int *vertex_cell, float *values, int vd,
-                             float *cell_values, int2 *neighbours, int d1, Counters *counters,
-                             Counters *next_counters, HostStatus *host_status, hipStream_t s);
+// Dense vertex numbers in the order of the build's workgroups (same map as the build):
+// cell_vertex[cell] := v, vertex_keys[v] := key, vertex_cell[v] := cell,
+// neighbours[a][v] := (-1, -1) for a <= pd, counters->vertices := M, and the vertex's row of
+// `values` := 0, or, with cell_values != nullptr, := the row cell_values[cell*vd ..], which is
+// zeroed.  Copies M and the flags to *host_status, zeroes *next_counters and
+// next_chunk_count[0 .. n_chunks).
+hipError_t number_vertices(int pd, const PointMap &map, const CreatedLists &lists,
+                           int *next_chunk_count, unsigned n_chunks, const VertexTables &vertices,
+                           float *values, int vd, float *cell_values, Counters *counters, Counters *next_counters,
+                           HostStatus *host_status, hipStream_t s);
 
 // neighbours[a*max_vertices+v] := vertex indices of v's two neighbours along blur axis a, for v
-// below the vertex count; entries of absent neighbours keep the -1 assign_vertex_ids gave them.
-hipError_t neighbours(int pd, const uint64_t *vertex_keys, const Counters *counters, int max_vertices,
-                      const uint64_t *cell_keys, const int *cell_vertex, uint32_t n_cells,
-                      int2 *neighbours, hipStream_t s);
+// below the vertex count; entries of absent neighbours keep their -1.
+hipError_t neighbours(int pd, const VertexTables &vertices, const Counters *counters,
+                      const uint64_t *cell_keys, uint32_t n_cells, hipStream_t s);
 
 hipError_t fill_zero(float *p, size_t n, hipStream_t s);
 

@@ -248,17 +248,6 @@ __device__ __forceinline__ int point_of_thread(const PointMap &m, unsigned vbloc
 // Hash table
 // ------------------------------------------------------------------------------------------------
 
-__device__ __forceinline__ int table_find(const uint64_t *cell_keys, const int *cell_vertex,
-                                          uint32_t mask, uint64_t key, uint32_t h, uint64_t cur) {
-    for (uint32_t probe = 0; probe <= mask; ++probe) {
-        if (probe) cur = cell_keys[h];
-        if (cur == key) return cell_vertex[h];
-        if (cur == kEmptyCell) return -1;
-        h = (h + 1u) & mask;
-    }
-    return -1;
-}
-
 __global__ __launch_bounds__(kBlock) void k_clear_table(uint64_t *cell_keys, uint32_t n_cells) {
     const uint32_t i = blockIdx.x * kBlock + threadIdx.x;
     if (i < n_cells) cell_keys[i] = kEmptyCell;
@@ -401,7 +390,8 @@ __global__ __launch_bounds__(kBlock) void k_build(PointFeatures features, PointM
                                                    int *__restrict__ replay_index,
                                                    float *__restrict__ replay_weight,
                                                    int xcd_aware, const float *__restrict__ input,
-                                                   int in_channels, float *cell_values) {
+                                                   int in_channels, float *cell_values,
+                                                   CreatedLists created_lists) {
     constexpr int D1 = PD + 1;
     const unsigned vblock = xcd_contiguous_block(blockIdx.x, gridDim.x, xcd_aware);
     const size_t t = (size_t)vblock * kBlock + threadIdx.x;   // slot in the replay arrays
@@ -443,6 +433,7 @@ __global__ __launch_bounds__(kBlock) void k_build(PointFeatures features, PointM
     uint32_t cell[D1];
     uint64_t seen[D1];
     bool open[D1];
+    unsigned created = 0;   // bit r: this lane's swap made the vertex of rank r
     bool any_open = false;
 #pragma unroll
     for (int r = 0; r < D1; ++r) {
@@ -463,6 +454,7 @@ __global__ __launch_bounds__(kBlock) void k_build(PointFeatures features, PointM
         for (int r = 0; r < D1; ++r) {
             if (open[r]) {
                 if (seen[r] == kEmptyCell || seen[r] == key[r]) {
+                    if (seen[r] == kEmptyCell) created |= 1u << r;
                     open[r] = false;              // swapped in, or already there
                 } else {
                     cell[r] = (cell[r] + 1u) & mask;
@@ -472,6 +464,42 @@ __global__ __launch_bounds__(kBlock) void k_build(PointFeatures features, PointM
         }
     }
     if (any_open) atomicOr(&counters->flags, kFlagTableFull);
+
+    // The vertices this workgroup created (cell and key), as a list of its own, and how many:
+    // the numbering pass gives the vertices dense numbers in the order of the workgroups, that
+    // is, of the image tiles.
+    {
+        __shared__ int wave_created[kBlock / 64];
+        const int wave = threadIdx.x >> 6;
+        int offset[D1];
+        int total = 0;
+#pragma unroll
+        for (int r = 0; r < D1; ++r) {
+            const uint64_t b = wave_ballot((created >> r) & 1u);
+            offset[r] = total + (int)__builtin_amdgcn_mbcnt_hi(
+                                    (uint32_t)(b >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)b, 0u));
+            total += __builtin_popcountll(b);
+        }
+        if (lane == 0) wave_created[wave] = total;
+        __syncthreads();
+        int base = 0, sum = 0;
+        for (int w = 0; w < kBlock / 64; ++w) {
+            if (w < wave) base += wave_created[w];
+            sum += wave_created[w];
+        }
+        if (threadIdx.x == 0) {
+            created_lists.block_count[vblock] = sum;
+            if (sum) atomicAdd(&created_lists.chunk_count[vblock / kBlocksPerChunk], sum);
+        }
+        const size_t list = (size_t)vblock * (kBlock * D1);
+#pragma unroll
+        for (int r = 0; r < D1; ++r) {
+            if ((created >> r) & 1u) {
+                created_lists.cells[list + base + offset[r]] = (int)cell[r];
+                created_lists.keys[list + base + offset[r]] = key[r];
+            }
+        }
+    }
 
     float val[4] = {0.0f, 0.0f, 0.0f, 0.0f};
     if (SPLAT_VD) {
@@ -512,60 +540,56 @@ __global__ __launch_bounds__(kBlock) void k_build(PointFeatures features, PointM
     }
 }
 
-// Dense vertex numbering: every occupied cell draws an index.  One atomic per workgroup (counts are
-// combined by ballot inside a wavefront and through LDS across the workgroup), because thousands
-// of atomics on one address would serialise in a single L2 channel.  That one 64-bit atomic adds
-// the workgroup's vertices to the low word and 1 to the high word, so the workgroup that reads
-// gridDim-1 in the high word knows it is the last and what the final count is, without a fence:
-// it publishes count and flags to host-visible memory and clears the counters the next build
-// will use.  The same pass zeroes each vertex's row of the value table.
-constexpr int kIdBlock = 1024;
-__global__ __launch_bounds__(kIdBlock) void k_assign_vertex_ids(
-    const uint64_t *__restrict__ cell_keys, uint32_t n_cells, int *cell_vertex,
-    uint64_t *vertex_keys, int *vertex_cell, float *values, int vd, float *cell_values,
-    int2 *neighbours, int d1, Counters *counters, Counters *next_counters,
-    HostStatus *host_status) {
-    __shared__ int wave_count[kIdBlock / 64];
-    __shared__ int block_base;
-    const uint32_t cell = blockIdx.x * kIdBlock + threadIdx.x;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const uint64_t key = cell < n_cells ? cell_keys[cell] : kEmptyCell;
-    const bool occupied = key != kEmptyCell;
-    const uint64_t ballot = wave_ballot(occupied);
-    if (lane == 0) wave_count[wave] = __builtin_popcountll(ballot);
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        int total = 0;
-        for (int w = 0; w < kIdBlock / 64; ++w) {
-            const int c = wave_count[w];
-            wave_count[w] = total;
-            total += c;
-        }
-        const unsigned long long before = atomicAdd(
-            (unsigned long long *)&counters->vertices_and_blocks, (1ull << 32) | (unsigned)total);
-        block_base = (int)(uint32_t)before;
-        if ((uint32_t)(before >> 32) == gridDim.x - 1) {
-            const uint32_t m = (uint32_t)before + (uint32_t)total;
-            const int flags = atomicOr(&counters->flags, 0);
+// Dense vertex numbering in the order of the build's workgroups, i.e. of the image tiles: the
+// vertices a workgroup created follow those of the workgroups before it.  Vertices that are close
+// in the lattice were created by the same or a neighbouring tile, so their numbers are close, and
+// what the neighbour, blur and slice passes gather falls into few cache lines instead of one line
+// per access.  One wavefront per workgroup of the build walks that workgroup's list.  Per vertex
+// v: cell_vertex[cell] := v, vertex_keys[v], vertex_cell[v], the row of the value table (moved
+// from cell_values, which the fused build+splat filled, or zeroed), and (-1, -1) for all its
+// neighbour entries.  The last wavefront knows the total: it publishes it to the device counters
+// and to host-visible memory and clears what the next build will count in.
+template <int D1>
+__global__ __launch_bounds__(64) void k_number_vertices(CreatedLists lists, int *next_chunk_count,
+                                                        unsigned n_chunks,
+                                                        VertexTables vertices, float *values, int vd,
+                                                        float *cell_values, Counters *counters,
+                                                        Counters *next_counters,
+                                                        HostStatus *host_status) {
+    const unsigned b = blockIdx.x;
+    const int lane = threadIdx.x;
+    const unsigned chunk = b / kBlocksPerChunk;
+    // vertices of the workgroups before this one: whole chunks, then the rest one by one
+    int before = 0;
+    for (unsigned i = lane; i < chunk; i += 64) before += lists.chunk_count[i];
+    static_assert(kBlocksPerChunk == 64, "one lane per workgroup of the chunk");
+    if (chunk * kBlocksPerChunk + lane < b) before += lists.block_count[chunk * kBlocksPerChunk + lane];
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) before += __shfl_xor(before, off);
+    const int count = lists.block_count[b];
+    const int max_vertices = vertices.max_vertices;
+
+    if (b == gridDim.x - 1) {
+        if (lane == 0) {
+            const uint32_t m = (uint32_t)(before + count);
+            counters->vertices = m;
             host_status->num_vertices = (int)m;
-            host_status->flags = flags | (m > max_vertices_for(n_cells) ? kFlagTableFull : 0);
-            next_counters->vertices_and_blocks = 0;
+            host_status->flags = counters->flags | (m > (uint32_t)max_vertices ? kFlagTableFull : 0);
+            next_counters->vertices = 0;
             next_counters->flags = 0;
         }
+        for (unsigned i = lane; i < n_chunks; i += 64) next_chunk_count[i] = 0;
     }
-    __syncthreads();
-    if (occupied) {
-        const int v = block_base + wave_count[wave] +
-                      __builtin_popcountll(ballot & ((1ull << lane) - 1ull));
-        if ((uint32_t)v < max_vertices_for(n_cells)) {
-            cell_vertex[cell] = v;
-            vertex_keys[v] = key;
-            vertex_cell[v] = (int)cell;
-            // "no neighbour" everywhere; the neighbour pass fills in the ones that exist
-            for (int a = 0; a < d1; ++a)
-                neighbours[(size_t)a * max_vertices_for(n_cells) + v] = make_int2(-1, -1);
+
+    const size_t list = (size_t)b * (kBlock * D1);
+    for (int i = lane; i < count; i += 64) {
+        const int cell = lists.cells[list + i];
+        const int v = before + i;
+        if (v < max_vertices) {
+            vertices.cell_vertex[cell] = v;
+            vertices.vertex_keys[v] = lists.keys[list + i];
+            vertices.vertex_cell[v] = cell;
             if (cell_values) {
-                // the fused build+splat accumulated by cell: move the row, leave zeros behind
                 for (int j = 0; j < vd; ++j) {
                     values[(size_t)v * vd + j] = cell_values[(size_t)cell * vd + j];
                     cell_values[(size_t)cell * vd + j] = 0.0f;
@@ -573,15 +597,32 @@ __global__ __launch_bounds__(kIdBlock) void k_assign_vertex_ids(
             } else {
                 for (int j = 0; j < vd; ++j) values[(size_t)v * vd + j] = 0.0f;
             }
+            // "no neighbour" everywhere; the neighbour pass fills in the ones that exist
+            for (int a = 0; a < D1; ++a)
+                vertices.neighbours[(size_t)a * max_vertices + v] = make_int2(-1, -1);
         } else {
-            cell_vertex[cell] = 0;   // the host sees the count and repeats with a larger table
+            vertices.cell_vertex[cell] = 0;   // the host sees the count and repeats with a larger table
         }
     }
 }
 
 __device__ __forceinline__ int vertex_count(const Counters *counters, int max_vertices) {
-    const uint32_t m = (uint32_t)counters->vertices_and_blocks;
+    const uint32_t m = counters->vertices;
     return m < (uint32_t)max_vertices ? (int)m : max_vertices;
+}
+
+// Kernels over the vertices are launched for the most vertices the table can hold, because the
+// count is only known on the device.  Workgroup b runs on XCD b % 8 and each XCD has its own L2,
+// so the workgroups that have work are dealt out such that every XCD gets one contiguous eighth
+// of the items: with vertex numbers that follow the image, the vertices a workgroup gathers from
+// are then mostly ones its own XCD works on.  Returns the block of items for this workgroup or
+// -1 if it has none.
+__device__ __forceinline__ int contiguous_item_block(unsigned b, size_t n_items) {
+    const unsigned n_active = (unsigned)((n_items + kBlock - 1) / kBlock);
+    const unsigned chunk = (n_active + 7u) / 8u;
+    const unsigned i = b >> 3;
+    const unsigned vb = (b & 7u) * chunk + i;
+    return (i < chunk && vb < n_active) ? (int)vb : -1;
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -589,22 +630,27 @@ __device__ __forceinline__ int vertex_count(const Counters *counters, int max_ve
 // mirror image (reference: src/PermutohedralLatticeCPU.h:381-388).  In (r, q) form the first is
 // r+1 with q_a-1, or, when r = pd, r = 0 with every q but q_a one higher; axis pd is the implicit
 // last coordinate, which no stored q belongs to.  out[a*max_vertices + v].
+// A workgroup takes 256 consecutive vertices along one axis; the pd+1 workgroups of a run of
+// vertices follow each other.  u is the + neighbour of v exactly when v is the - neighbour of u:
+// one lookup fills out[a][v].x and out[a][u].y (all entries start as -1).
 // ------------------------------------------------------------------------------------------------
 template <int PD>
-__global__ __launch_bounds__(kBlock) void k_neighbours(const uint64_t *__restrict__ vertex_keys,
-                                                        const Counters *counters, int max_vertices,
+__global__ __launch_bounds__(kBlock) void k_neighbours(VertexTables vertices,
+                                                        const Counters *counters,
                                                         const uint64_t *__restrict__ cell_keys,
-                                                        const int *__restrict__ cell_vertex,
-                                                        uint32_t mask, int2 *__restrict__ out) {
+                                                        uint32_t mask) {
+    constexpr int D1 = PD + 1;
+    const int max_vertices = vertices.max_vertices;
     const int M = vertex_count(counters, max_vertices);
-    const size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x;
-    const int a = (int)(t / (size_t)max_vertices);
-    const int v = (int)(t - (size_t)a * max_vertices);
-    if (a > PD || v >= M) return;
+    const unsigned runs = (unsigned)((M + kBlock - 1) / kBlock);
+    const int ib = contiguous_item_block(blockIdx.x, (size_t)runs * D1 * kBlock);
+    if (ib < 0) return;
+    const int a = ib % D1;
+    const int v = (ib / D1) * kBlock + (int)threadIdx.x;
+    if (v >= M) return;
 
     int q[PD], r;
-    KeyCodec<PD>::unpack(vertex_keys[v], q, r);
-
+    KeyCodec<PD>::unpack(vertices.vertex_keys[v], q, r);
     int qp[PD];
     const bool wrap_up = (r == PD);
 #pragma unroll
@@ -612,15 +658,22 @@ __global__ __launch_bounds__(kBlock) void k_neighbours(const uint64_t *__restric
         const bool on_axis = (i == a);
         qp[i] = q[i] + (wrap_up ? (on_axis ? 0 : 1) : (on_axis ? -1 : 0));
     }
-    // u is the + neighbour of v exactly when v is the - neighbour of u: one lookup fills both
-    // entries (all entries start as -1)
-    const uint64_t kp = KeyCodec<PD>::pack(qp, wrap_up ? 0 : r + 1);
-    const uint32_t hp = hash_key(kp) & mask;
-    const int u = table_find(cell_keys, cell_vertex, mask, kp, hp, cell_keys[hp]);
+    const uint64_t want = KeyCodec<PD>::pack(qp, wrap_up ? 0 : r + 1);
+    uint32_t h = hash_key(want) & mask;
+    int u = -1;
+    for (uint32_t probe = 0; probe <= mask; ++probe) {
+        const uint64_t cur = cell_keys[h];
+        if (cur == want) {
+            u = vertices.cell_vertex[h];
+            break;
+        }
+        if (cur == kEmptyCell) break;
+        h = (h + 1u) & mask;
+    }
     if (u >= 0) {
-        int *entries = reinterpret_cast<int *>(out);
-        entries[2 * t] = u;                                        // out[a][v].x
-        entries[2 * ((size_t)a * max_vertices + u) + 1] = v;       // out[a][u].y
+        int *entries = reinterpret_cast<int *>(vertices.neighbours);
+        entries[2 * ((size_t)a * max_vertices + v)] = u;          // out[a][v].x
+        entries[2 * ((size_t)a * max_vertices + u) + 1] = v;      // out[a][u].y
     }
 }
 
@@ -786,7 +839,9 @@ __global__ __launch_bounds__(kBlock) void k_blur_element(const Counters *counter
                                                           uint64_t *reset_cell_keys,
                                                           const int *__restrict__ vertex_cell) {
     const int M = vertex_count(counters, max_vertices);
-    const size_t e = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    const int eb = contiguous_item_block(blockIdx.x, (size_t)M * vd);
+    if (eb < 0) return;
+    const size_t e = (size_t)eb * kBlock + threadIdx.x;
     if (e >= (size_t)M * vd) return;
     const int v = (int)(e / (size_t)vd);
     const int j = (int)(e - (size_t)v * vd);
@@ -821,7 +876,9 @@ __global__ __launch_bounds__(kBlock) void k_blur2_element(const Counters *counte
                                                            uint64_t *reset_cell_keys,
                                                            const int *__restrict__ vertex_cell) {
     const int M = vertex_count(counters, max_vertices);
-    const size_t e = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    const int eb = contiguous_item_block(blockIdx.x, (size_t)M * vd);
+    if (eb < 0) return;
+    const size_t e = (size_t)eb * kBlock + threadIdx.x;
     if (e >= (size_t)M * vd) return;
     const int v = (int)(e / (size_t)vd);
     const int j = (int)(e - (size_t)v * vd);
@@ -981,6 +1038,8 @@ __global__ __launch_bounds__(kBlock) void k_positions(const float *__restrict__ 
 }
 
 inline unsigned blocks_for(size_t n, int block = kBlock) { return (unsigned)((n + block - 1) / block); }
+// grids of the kernels that deal their workgroups out with contiguous_item_block: a multiple of 8
+inline unsigned vertex_blocks(size_t n_items) { return (blocks_for(n_items) + 7u) & ~7u; }
 
 #define PLK_DISPATCH_PD(pd, CALL)                 \
     switch (pd) {                                 \
@@ -1041,13 +1100,15 @@ bool build_can_splat(int vd) { return vd >= 2 && vd <= 4; }
 hipError_t build(int pd, const PointFeatures &features, const PointMap &map, const ScaleFactor &scale,
                  uint64_t *cell_keys, uint32_t n_cells, Counters *counters, int *replay_index,
                  float *replay_weight, int xcd_aware, int splat_vd, const float *input,
-                 int in_channels, float *cell_values, hipStream_t s) {
+                 int in_channels, float *cell_values, const CreatedLists &created_lists,
+                 hipStream_t s) {
     if (map.n_blocks == 0) return hipSuccess;
 #define PLK_BUILD(SPLAT_VD)                                                                        \
     PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_build<PD, SPLAT_VD>), dim3(map.n_blocks),            \
                                            dim3(kBlock), 0, s, features, map, scale, cell_keys,    \
                                            n_cells - 1u, counters, replay_index, replay_weight,    \
-                                           xcd_aware, input, in_channels, cell_values))
+                                           xcd_aware, input, in_channels, cell_values,             \
+                                           created_lists))
     switch (splat_vd) {
         case 0: PLK_BUILD(0); break;
         case 2: PLK_BUILD(2); break;
@@ -1059,24 +1120,25 @@ hipError_t build(int pd, const PointFeatures &features, const PointMap &map, con
     return hipGetLastError();
 }
 
-hipError_t assign_vertex_ids(const uint64_t *cell_keys, uint32_t n_cells, int *cell_vertex,
-                             uint64_t *vertex_keys, int *vertex_cell, float *values, int vd,
-                             float *cell_values, int2 *neighbours, int d1, Counters *counters,
-                             Counters *next_counters, HostStatus *host_status, hipStream_t s) {
-    hipLaunchKernelGGL(k_assign_vertex_ids, dim3(blocks_for(n_cells, kIdBlock)), dim3(kIdBlock), 0, s,
-                       cell_keys, n_cells, cell_vertex, vertex_keys, vertex_cell, values, vd,
-                       cell_values, neighbours, d1, counters, next_counters, host_status);
+hipError_t number_vertices(int pd, const PointMap &map, const CreatedLists &lists,
+                           int *next_chunk_count, unsigned n_chunks, const VertexTables &vertices,
+                           float *values,
+                           int vd, float *cell_values, Counters *counters, Counters *next_counters,
+                           HostStatus *host_status, hipStream_t s) {
+    if (map.n_blocks == 0) return hipErrorInvalidValue;
+    PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_number_vertices<PD + 1>), dim3(map.n_blocks), dim3(64),
+                                           0, s, lists, next_chunk_count, n_chunks, vertices, values, vd,
+                                           cell_values, counters, next_counters, host_status));
     return hipGetLastError();
 }
 
-hipError_t neighbours(int pd, const uint64_t *vertex_keys, const Counters *counters, int max_vertices,
-                      const uint64_t *cell_keys, const int *cell_vertex, uint32_t n_cells, int2 *out,
-                      hipStream_t s) {
-    if (max_vertices <= 0) return hipSuccess;
-    PLK_DISPATCH_PD(pd, hipLaunchKernelGGL(k_neighbours<PD>,
-                                           dim3(blocks_for((size_t)max_vertices * (PD + 1))),
-                                           dim3(kBlock), 0, s, vertex_keys, counters, max_vertices,
-                                           cell_keys, cell_vertex, n_cells - 1u, out));
+hipError_t neighbours(int pd, const VertexTables &vertices, const Counters *counters,
+                      const uint64_t *cell_keys, uint32_t n_cells, hipStream_t s) {
+    if (vertices.max_vertices <= 0) return hipErrorInvalidValue;
+    const size_t items = (size_t)(pd + 1) * ((size_t)vertices.max_vertices + kBlock);
+    PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_neighbours<PD>), dim3(vertex_blocks(items)),
+                                           dim3(kBlock), 0, s, vertices, counters, cell_keys,
+                                           n_cells - 1u));
     return hipGetLastError();
 }
 
@@ -1113,7 +1175,7 @@ hipError_t blur_axis(int vd, const Counters *counters, int max_vertices, const f
                      const int2 *nbr, uint64_t *reset_cell_keys, const int *vertex_cell,
                      hipStream_t s) {
     if (max_vertices <= 0) return hipSuccess;
-    hipLaunchKernelGGL(k_blur_element, dim3(blocks_for((size_t)max_vertices * vd)), dim3(kBlock), 0, s,
+    hipLaunchKernelGGL(k_blur_element, dim3(vertex_blocks((size_t)max_vertices * vd)), dim3(kBlock), 0, s,
                        counters, max_vertices, vd, src, dst, nbr, reset_cell_keys, vertex_cell);
     return hipGetLastError();
 }
@@ -1122,7 +1184,7 @@ hipError_t blur_two_axes(int vd, const Counters *counters, int max_vertices, con
                          float *dst, const int2 *nbr_first, const int2 *nbr_second,
                          uint64_t *reset_cell_keys, const int *vertex_cell, hipStream_t s) {
     if (max_vertices <= 0) return hipSuccess;
-    hipLaunchKernelGGL(k_blur2_element, dim3(blocks_for((size_t)max_vertices * vd)), dim3(kBlock), 0, s,
+    hipLaunchKernelGGL(k_blur2_element, dim3(vertex_blocks((size_t)max_vertices * vd)), dim3(kBlock), 0, s,
                        counters, max_vertices, vd, src, dst, nbr_first, nbr_second, reset_cell_keys,
                        vertex_cell);
     return hipGetLastError();
