@@ -133,6 +133,15 @@ struct pl_lattice {
     }
     plk::Counters *counters() { return d_counters + counter_set; }
     int max_vertices() const { return (int)plk::max_vertices_for(n_cells); }
+    // what the grids of the kernels over the vertices are sized for: the count when the host
+    // knows it, else the previous build's with a margin (the kernels cover any count)
+    int launch_vertices() const {
+        const int mv = max_vertices();
+        if (built && verified) return M < mv ? M : mv;
+        if (last_M <= 0) return mv;
+        const long long guess = (long long)last_M + last_M / 8 + 1024;
+        return guess < mv ? (int)guess : mv;
+    }
 };
 
 namespace {
@@ -247,7 +256,8 @@ int enqueue_build(pl_lattice *h, const plk::PointFeatures &features, uint32_t ce
                                 h->values[0], h->vd, fused ? h->cell_values : nullptr, h->counters(),
                                 h->d_counters + previous_set, h->h_status, h->stream));
     h->mark(EV_IDS);
-    PL_HIP(plk::neighbours(h->pd, vertices, h->counters(), h->cell_keys, cells, h->stream));
+    PL_HIP(plk::neighbours(h->pd, vertices, h->counters(), h->cell_keys, cells,
+                           h->launch_vertices(), h->stream));
     h->mark(EV_NBR);
     h->replay_holds_cells = true;
     h->values_zeroed = !fused;
@@ -286,11 +296,12 @@ int enqueue_apply(pl_lattice *h, float *output, const float *input, int reverse)
             PL_HIP(plk::blur_two_axes(vd, h->counters(), mv, h->values[cur], h->values[1 - cur],
                                       h->neighbours + (size_t)axis * mv,
                                       h->neighbours + (size_t)next_axis * mv, reset, h->vertex_cell,
-                                      h->stream));
+                                      h->launch_vertices(), h->stream));
             step += 2;
         } else {
             PL_HIP(plk::blur_axis(vd, h->counters(), mv, h->values[cur], h->values[1 - cur],
-                                  h->neighbours + (size_t)axis * mv, reset, h->vertex_cell, h->stream));
+                                  h->neighbours + (size_t)axis * mv, reset, h->vertex_cell,
+                                  h->launch_vertices(), h->stream));
             step += 1;
         }
         if (reset) h->table_clean = true;

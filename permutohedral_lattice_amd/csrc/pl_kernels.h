@@ -122,8 +122,11 @@ hipError_t number_vertices(int pd, const PointMap &map, const CreatedLists &list
 
 // neighbours[a*max_vertices+v] := vertex indices of v's two neighbours along blur axis a, for v
 // below the vertex count; entries of absent neighbours keep their -1.
+// launch_vertices (here and below): the vertex count the grid is sized for; any count is
+// covered, a wrong estimate only costs time.
 hipError_t neighbours(int pd, const VertexTables &vertices, const Counters *counters,
-                      const uint64_t *cell_keys, uint32_t n_cells, hipStream_t s);
+                      const uint64_t *cell_keys, uint32_t n_cells, int launch_vertices,
+                      hipStream_t s);
 
 hipError_t fill_zero(float *p, size_t n, hipStream_t s);
 
@@ -138,13 +141,14 @@ hipError_t splat(int pd, int vd, const PointMap &map, const float *input, int in
 // reset_cell_keys != nullptr: also empty the hash cell of every vertex (vertex_cell[v]).
 hipError_t blur_axis(int vd, const Counters *counters, int max_vertices, const float *src, float *dst,
                      const int2 *neighbours_of_axis, uint64_t *reset_cell_keys,
-                     const int *vertex_cell, hipStream_t s);
+                     const int *vertex_cell, int launch_vertices, hipStream_t s);
 
 // Two axes in one launch: the result of blur_axis with nbr_first followed by blur_axis with
 // nbr_second, bit for bit.
 hipError_t blur_two_axes(int vd, const Counters *counters, int max_vertices, const float *src,
                          float *dst, const int2 *nbr_first, const int2 *nbr_second,
-                         uint64_t *reset_cell_keys, const int *vertex_cell, hipStream_t s);
+                         uint64_t *reset_cell_keys, const int *vertex_cell, int launch_vertices,
+                         hipStream_t s);
 
 // Stage 5.  normalize: divide by the homogeneous channel and write vd-1 channels; else write vd.
 // cell_vertex != nullptr: replay_index still holds hash cells (vd <= 8 only).

@@ -393,6 +393,12 @@ __global__ __launch_bounds__(kBlock) void k_build(PointFeatures features, PointM
                                                    int in_channels, float *cell_values,
                                                    CreatedLists created_lists) {
     constexpr int D1 = PD + 1;
+    __shared__ int group_created, waves_done;
+    if (threadIdx.x == 0) {
+        group_created = 0;
+        waves_done = 0;
+    }
+    __syncthreads();
     const unsigned vblock = xcd_contiguous_block(blockIdx.x, gridDim.x, xcd_aware);
     const size_t t = (size_t)vblock * kBlock + threadIdx.x;   // slot in the replay arrays
     const size_t T = (size_t)gridDim.x * kBlock;
@@ -467,10 +473,10 @@ __global__ __launch_bounds__(kBlock) void k_build(PointFeatures features, PointM
 
     // The vertices this workgroup created (cell and key), as a list of its own, and how many:
     // the numbering pass gives the vertices dense numbers in the order of the workgroups, that
-    // is, of the image tiles.
+    // is, of the image tiles.  A wavefront draws its run of list entries with one LDS atomic; the
+    // wavefront that finishes last knows the workgroup's total.  No barrier: the wavefronts of a
+    // workgroup leave the insertion at very different times.
     {
-        __shared__ int wave_created[kBlock / 64];
-        const int wave = threadIdx.x >> 6;
         int offset[D1];
         int total = 0;
 #pragma unroll
@@ -480,17 +486,9 @@ __global__ __launch_bounds__(kBlock) void k_build(PointFeatures features, PointM
                                     (uint32_t)(b >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)b, 0u));
             total += __builtin_popcountll(b);
         }
-        if (lane == 0) wave_created[wave] = total;
-        __syncthreads();
-        int base = 0, sum = 0;
-        for (int w = 0; w < kBlock / 64; ++w) {
-            if (w < wave) base += wave_created[w];
-            sum += wave_created[w];
-        }
-        if (threadIdx.x == 0) {
-            created_lists.block_count[vblock] = sum;
-            if (sum) atomicAdd(&created_lists.chunk_count[vblock / kBlocksPerChunk], sum);
-        }
+        int base = 0;
+        if (lane == 0 && total) base = atomicAdd(&group_created, total);
+        base = __builtin_amdgcn_readfirstlane(base);
         const size_t list = (size_t)vblock * (kBlock * D1);
 #pragma unroll
         for (int r = 0; r < D1; ++r) {
@@ -498,6 +496,11 @@ __global__ __launch_bounds__(kBlock) void k_build(PointFeatures features, PointM
                 created_lists.cells[list + base + offset[r]] = (int)cell[r];
                 created_lists.keys[list + base + offset[r]] = key[r];
             }
+        }
+        if (lane == 0 && atomicAdd(&waves_done, 1) == kBlock / 64 - 1) {
+            const int sum = atomicAdd(&group_created, 0);
+            created_lists.block_count[vblock] = sum;
+            if (sum) atomicAdd(&created_lists.chunk_count[vblock / kBlocksPerChunk], sum);
         }
     }
 
@@ -611,19 +614,28 @@ __device__ __forceinline__ int vertex_count(const Counters *counters, int max_ve
     return m < (uint32_t)max_vertices ? (int)m : max_vertices;
 }
 
-// Kernels over the vertices are launched for the most vertices the table can hold, because the
-// count is only known on the device.  Workgroup b runs on XCD b % 8 and each XCD has its own L2,
-// so the workgroups that have work are dealt out such that every XCD gets one contiguous eighth
-// of the items: with vertex numbers that follow the image, the vertices a workgroup gathers from
-// are then mostly ones its own XCD works on.  Returns the block of items for this workgroup or
-// -1 if it has none.
-__device__ __forceinline__ int contiguous_item_block(unsigned b, size_t n_items) {
-    const unsigned n_active = (unsigned)((n_items + kBlock - 1) / kBlock);
-    const unsigned chunk = (n_active + 7u) / 8u;
-    const unsigned i = b >> 3;
-    const unsigned vb = (b & 7u) * chunk + i;
-    return (i < chunk && vb < n_active) ? (int)vb : -1;
-}
+// The vertex count is only known on the device, so kernels over the vertices are launched for an
+// estimate (the count of the lattice's previous build, with a margin) and every workgroup walks
+// the blocks of 256 items in strides of the grid: a launch for the most vertices the table can
+// hold would spend more time dispatching empty workgroups than the passes spend working.
+// Workgroup b runs on XCD b % 8 and each XCD has its own L2, so the blocks are dealt out such
+// that every XCD gets one contiguous eighth of the items (the grid is a multiple of 8): with
+// vertex numbers that follow the image, the vertices a workgroup gathers from are then mostly
+// ones its own XCD works on.
+struct ItemBlocks {
+    unsigned n_active, chunk, k;
+    __device__ explicit ItemBlocks(size_t n_items)
+        : n_active((unsigned)((n_items + kBlock - 1) / kBlock)), chunk((n_active + 7u) / 8u),
+          k(blockIdx.x) {}
+    __device__ bool next(unsigned &block) {
+        while (k < 8u * chunk) {
+            block = (k & 7u) * chunk + (k >> 3);
+            k += gridDim.x;
+            if (block < n_active) return true;
+        }
+        return false;
+    }
+};
 
 // ------------------------------------------------------------------------------------------------
 // Neighbour table: along axis a the neighbours of key k are k + (1,..,1) - (pd+1) e_a and its
@@ -643,11 +655,12 @@ __global__ __launch_bounds__(kBlock) void k_neighbours(VertexTables vertices,
     const int max_vertices = vertices.max_vertices;
     const int M = vertex_count(counters, max_vertices);
     const unsigned runs = (unsigned)((M + kBlock - 1) / kBlock);
-    const int ib = contiguous_item_block(blockIdx.x, (size_t)runs * D1 * kBlock);
-    if (ib < 0) return;
-    const int a = ib % D1;
-    const int v = (ib / D1) * kBlock + (int)threadIdx.x;
-    if (v >= M) return;
+    ItemBlocks blocks((size_t)runs * D1 * kBlock);
+    unsigned ib;
+    while (blocks.next(ib)) {
+    const int a = (int)(ib % D1);
+    const int v = (int)(ib / D1) * kBlock + (int)threadIdx.x;
+    if (v >= M) continue;
 
     int q[PD], r;
     KeyCodec<PD>::unpack(vertices.vertex_keys[v], q, r);
@@ -674,6 +687,7 @@ __global__ __launch_bounds__(kBlock) void k_neighbours(VertexTables vertices,
         int *entries = reinterpret_cast<int *>(vertices.neighbours);
         entries[2 * ((size_t)a * max_vertices + v)] = u;          // out[a][v].x
         entries[2 * ((size_t)a * max_vertices + u) + 1] = v;      // out[a][u].y
+    }
     }
 }
 
@@ -839,17 +853,19 @@ __global__ __launch_bounds__(kBlock) void k_blur_element(const Counters *counter
                                                           uint64_t *reset_cell_keys,
                                                           const int *__restrict__ vertex_cell) {
     const int M = vertex_count(counters, max_vertices);
-    const int eb = contiguous_item_block(blockIdx.x, (size_t)M * vd);
-    if (eb < 0) return;
-    const size_t e = (size_t)eb * kBlock + threadIdx.x;
-    if (e >= (size_t)M * vd) return;
-    const int v = (int)(e / (size_t)vd);
-    const int j = (int)(e - (size_t)v * vd);
-    const int2 nb = nbr[v];
-    const float a = nb.x >= 0 ? src[(size_t)nb.x * vd + j] : 0.0f;
-    const float b = nb.y >= 0 ? src[(size_t)nb.y * vd + j] : 0.0f;
-    dst[e] = blur_tap(a, src[e], b);
-    if (reset_cell_keys && j == 0) reset_cell_keys[vertex_cell[v]] = kEmptyCell;
+    ItemBlocks blocks((size_t)M * vd);
+    unsigned eb;
+    while (blocks.next(eb)) {
+        const size_t e = (size_t)eb * kBlock + threadIdx.x;
+        if (e >= (size_t)M * vd) continue;
+        const int v = (int)(e / (size_t)vd);
+        const int j = (int)(e - (size_t)v * vd);
+        const int2 nb = nbr[v];
+        const float a = nb.x >= 0 ? src[(size_t)nb.x * vd + j] : 0.0f;
+        const float b = nb.y >= 0 ? src[(size_t)nb.y * vd + j] : 0.0f;
+        dst[e] = blur_tap(a, src[e], b);
+        if (reset_cell_keys && j == 0) reset_cell_keys[vertex_cell[v]] = kEmptyCell;
+    }
 }
 
 // Two axes in one launch.  Every kernel boundary costs a cold L2 and a round of dependent loads,
@@ -876,16 +892,19 @@ __global__ __launch_bounds__(kBlock) void k_blur2_element(const Counters *counte
                                                            uint64_t *reset_cell_keys,
                                                            const int *__restrict__ vertex_cell) {
     const int M = vertex_count(counters, max_vertices);
-    const int eb = contiguous_item_block(blockIdx.x, (size_t)M * vd);
-    if (eb < 0) return;
-    const size_t e = (size_t)eb * kBlock + threadIdx.x;
-    if (e >= (size_t)M * vd) return;
-    const int v = (int)(e / (size_t)vd);
-    const int j = (int)(e - (size_t)v * vd);
-    const int2 nb = nbr_b[v];
-    dst[e] = blur_tap(blur_element_of(src, nbr_a, nb.x, vd, j), blur_element_of(src, nbr_a, v, vd, j),
-                      blur_element_of(src, nbr_a, nb.y, vd, j));
-    if (reset_cell_keys && j == 0) reset_cell_keys[vertex_cell[v]] = kEmptyCell;
+    ItemBlocks blocks((size_t)M * vd);
+    unsigned eb;
+    while (blocks.next(eb)) {
+        const size_t e = (size_t)eb * kBlock + threadIdx.x;
+        if (e >= (size_t)M * vd) continue;
+        const int v = (int)(e / (size_t)vd);
+        const int j = (int)(e - (size_t)v * vd);
+        const int2 nb = nbr_b[v];
+        dst[e] = blur_tap(blur_element_of(src, nbr_a, nb.x, vd, j),
+                          blur_element_of(src, nbr_a, v, vd, j),
+                          blur_element_of(src, nbr_a, nb.y, vd, j));
+        if (reset_cell_keys && j == 0) reset_cell_keys[vertex_cell[v]] = kEmptyCell;
+    }
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -1038,8 +1057,11 @@ __global__ __launch_bounds__(kBlock) void k_positions(const float *__restrict__ 
 }
 
 inline unsigned blocks_for(size_t n, int block = kBlock) { return (unsigned)((n + block - 1) / block); }
-// grids of the kernels that deal their workgroups out with contiguous_item_block: a multiple of 8
-inline unsigned vertex_blocks(size_t n_items) { return (blocks_for(n_items) + 7u) & ~7u; }
+// grids of the kernels that walk their items with ItemBlocks: a multiple of 8
+inline unsigned vertex_blocks(size_t n_items) {
+    const unsigned b = (blocks_for(n_items) + 7u) & ~7u;
+    return b ? b : 8u;
+}
 
 #define PLK_DISPATCH_PD(pd, CALL)                 \
     switch (pd) {                                 \
@@ -1133,9 +1155,10 @@ hipError_t number_vertices(int pd, const PointMap &map, const CreatedLists &list
 }
 
 hipError_t neighbours(int pd, const VertexTables &vertices, const Counters *counters,
-                      const uint64_t *cell_keys, uint32_t n_cells, hipStream_t s) {
+                      const uint64_t *cell_keys, uint32_t n_cells, int launch_vertices,
+                      hipStream_t s) {
     if (vertices.max_vertices <= 0) return hipErrorInvalidValue;
-    const size_t items = (size_t)(pd + 1) * ((size_t)vertices.max_vertices + kBlock);
+    const size_t items = (size_t)(pd + 1) * ((size_t)launch_vertices + kBlock);
     PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_neighbours<PD>), dim3(vertex_blocks(items)),
                                            dim3(kBlock), 0, s, vertices, counters, cell_keys,
                                            n_cells - 1u));
@@ -1173,18 +1196,19 @@ hipError_t splat(int pd, int vd, const PointMap &map, const float *input, int in
 
 hipError_t blur_axis(int vd, const Counters *counters, int max_vertices, const float *src, float *dst,
                      const int2 *nbr, uint64_t *reset_cell_keys, const int *vertex_cell,
-                     hipStream_t s) {
+                     int launch_vertices, hipStream_t s) {
     if (max_vertices <= 0) return hipSuccess;
-    hipLaunchKernelGGL(k_blur_element, dim3(vertex_blocks((size_t)max_vertices * vd)), dim3(kBlock), 0, s,
+    hipLaunchKernelGGL(k_blur_element, dim3(vertex_blocks((size_t)launch_vertices * vd)), dim3(kBlock), 0, s,
                        counters, max_vertices, vd, src, dst, nbr, reset_cell_keys, vertex_cell);
     return hipGetLastError();
 }
 
 hipError_t blur_two_axes(int vd, const Counters *counters, int max_vertices, const float *src,
                          float *dst, const int2 *nbr_first, const int2 *nbr_second,
-                         uint64_t *reset_cell_keys, const int *vertex_cell, hipStream_t s) {
+                         uint64_t *reset_cell_keys, const int *vertex_cell, int launch_vertices,
+                         hipStream_t s) {
     if (max_vertices <= 0) return hipSuccess;
-    hipLaunchKernelGGL(k_blur2_element, dim3(vertex_blocks((size_t)max_vertices * vd)), dim3(kBlock), 0, s,
+    hipLaunchKernelGGL(k_blur2_element, dim3(vertex_blocks((size_t)launch_vertices * vd)), dim3(kBlock), 0, s,
                        counters, max_vertices, vd, src, dst, nbr_first, nbr_second, reset_cell_keys,
                        vertex_cell);
     return hipGetLastError();
