@@ -87,8 +87,7 @@ struct pl_lattice {
     float *replay_weight = nullptr;
     // what each workgroup of the build created (see plk::CreatedLists); the chunk counts exist
     // twice and alternate between builds like the counters
-    int *created_cells = nullptr;          // [n_blocks*256*(pd+1)]
-    uint64_t *created_keys = nullptr;      // [n_blocks*256*(pd+1)]
+    uint4 *created_entries = nullptr;      // [n_blocks*256*(pd+1)]
     int *block_count = nullptr;            // [n_blocks]
     int *chunk_count = nullptr;            // [2][n_chunks]
     size_t n_chunks = 0;
@@ -184,19 +183,17 @@ int ensure_replay(pl_lattice *h) {
     PL_HIP(hipStreamSynchronize(h->stream));
     h->dfree(h->replay_index);
     h->dfree(h->replay_weight);
-    h->dfree(h->created_cells);
-    h->dfree(h->created_keys);
+    h->dfree(h->created_entries);
     h->dfree(h->block_count);
     h->dfree(h->chunk_count);
     h->replay_capacity = 0;
     h->n_chunks = (h->map.n_blocks + plk::kBlocksPerChunk - 1) / plk::kBlocksPerChunk + 1;
     h->replay_index = (int *)h->dmalloc(sizeof(int) * (want ? want : 1));
     h->replay_weight = (float *)h->dmalloc(sizeof(float) * (want ? want : 1));
-    h->created_cells = (int *)h->dmalloc(sizeof(int) * (want ? want : 1));
-    h->created_keys = (uint64_t *)h->dmalloc(sizeof(uint64_t) * (want ? want : 1));
+    h->created_entries = (uint4 *)h->dmalloc(sizeof(uint4) * (want ? want : 1));
     h->block_count = (int *)h->dmalloc(sizeof(int) * (h->map.n_blocks ? h->map.n_blocks : 1));
     h->chunk_count = (int *)h->dmalloc(sizeof(int) * 2 * h->n_chunks);
-    if (!h->replay_index || !h->replay_weight || !h->created_cells || !h->created_keys ||
+    if (!h->replay_index || !h->replay_weight || !h->created_entries ||
         !h->block_count || !h->chunk_count)
         return PL_ENOMEM;
     PL_HIP(hipMemsetAsync(h->chunk_count, 0, sizeof(int) * 2 * h->n_chunks, h->stream));
@@ -243,7 +240,7 @@ int enqueue_build(pl_lattice *h, const plk::PointFeatures &features, uint32_t ce
     h->counter_set = 1 - previous_set;
     const plk::VertexTables vertices{h->cell_vertex, h->vertex_keys, h->vertex_cell, h->neighbours,
                                      h->max_vertices()};
-    const plk::CreatedLists lists{h->created_cells, h->created_keys, h->block_count,
+    const plk::CreatedLists lists{h->created_entries, h->block_count,
                                   h->chunk_count + (size_t)h->counter_set * h->n_chunks};
     PL_HIP(plk::build(h->pd, features, h->map, h->scale, h->cell_keys, cells, h->counters(),
                       h->replay_index, h->replay_weight, h->xcd_aware ? 1 : 0, fused ? h->vd : 0,
@@ -424,8 +421,7 @@ int pl_destroy(pl_handle h) {
     h->dfree(h->cell_values);
     h->dfree(h->replay_index);
     h->dfree(h->replay_weight);
-    h->dfree(h->created_cells);
-    h->dfree(h->created_keys);
+    h->dfree(h->created_entries);
     h->dfree(h->block_count);
     h->dfree(h->chunk_count);
     h->dfree(h->d_counters);

@@ -54,13 +54,12 @@ struct SpatialDims {
 };
 
 // What the build's workgroups created, for the numbering pass: workgroup b (in the build's
-// virtual order) lists the hash cells and keys of its block_count[b] new vertices from entry
-// b*256*(pd+1) on; chunk_count[c] is the sum over the kBlocksPerChunk workgroups of chunk c and
-// must be zero before the build.
+// virtual order) lists its block_count[b] new vertices from entry b*256*(pd+1) on, one uint4
+// each: (key low word, key high word, hash cell, 0).  chunk_count[c] is the sum over the
+// kBlocksPerChunk workgroups of chunk c and must be zero before the build.
 constexpr int kBlocksPerChunk = 64;
 struct CreatedLists {
-    int *cells;
-    uint64_t *keys;
+    uint4 *entries;
     int *block_count;
     int *chunk_count;
 };

@@ -493,8 +493,8 @@ __global__ __launch_bounds__(kBlock) void k_build(PointFeatures features, PointM
 #pragma unroll
         for (int r = 0; r < D1; ++r) {
             if ((created >> r) & 1u) {
-                created_lists.cells[list + base + offset[r]] = (int)cell[r];
-                created_lists.keys[list + base + offset[r]] = key[r];
+                created_lists.entries[list + base + offset[r]] =
+                    make_uint4((uint32_t)key[r], (uint32_t)(key[r] >> 32), cell[r], 0u);
             }
         }
         if (lane == 0 && atomicAdd(&waves_done, 1) == kBlock / 64 - 1) {
@@ -586,13 +586,22 @@ __global__ __launch_bounds__(64) void k_number_vertices(CreatedLists lists, int 
 
     const size_t list = (size_t)b * (kBlock * D1);
     for (int i = lane; i < count; i += 64) {
-        const int cell = lists.cells[list + i];
+        const uint4 entry = lists.entries[list + i];
+        const int cell = (int)entry.z;
         const int v = before + i;
         if (v < max_vertices) {
             vertices.cell_vertex[cell] = v;
-            vertices.vertex_keys[v] = lists.keys[list + i];
+            vertices.vertex_keys[v] = ((uint64_t)entry.y << 32) | entry.x;
             vertices.vertex_cell[v] = cell;
-            if (cell_values) {
+            if (cell_values && vd == 4) {
+                float4 *from = reinterpret_cast<float4 *>(cell_values) + cell;
+                reinterpret_cast<float4 *>(values)[v] = *from;
+                *from = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            } else if (cell_values && vd == 2) {
+                float2 *from = reinterpret_cast<float2 *>(cell_values) + cell;
+                reinterpret_cast<float2 *>(values)[v] = *from;
+                *from = make_float2(0.0f, 0.0f);
+            } else if (cell_values) {
                 for (int j = 0; j < vd; ++j) {
                     values[(size_t)v * vd + j] = cell_values[(size_t)cell * vd + j];
                     cell_values[(size_t)cell * vd + j] = 0.0f;
