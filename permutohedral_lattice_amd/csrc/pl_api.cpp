@@ -83,8 +83,7 @@ struct pl_lattice {
 
     // per-point arrays, (pd+1) rows of map.n_blocks*256 entries in thread order
     plk::PointMap map{};
-    int *replay_index = nullptr;
-    float *replay_weight = nullptr;
+    plk::ReplayEntry *replay = nullptr;
     // what each workgroup of the build created (see plk::CreatedLists); the chunk counts exist
     // twice and alternate between builds like the counters
     uint4 *created_entries = nullptr;      // [n_blocks*256*(pd+1)]
@@ -179,21 +178,19 @@ int ensure_table(pl_lattice *h, uint32_t cells) {
 
 int ensure_replay(pl_lattice *h) {
     const size_t want = (size_t)h->map.n_blocks * 256 * (size_t)(h->pd + 1);
-    if (want <= h->replay_capacity && h->replay_index) return PL_OK;
+    if (want <= h->replay_capacity && h->replay) return PL_OK;
     PL_HIP(hipStreamSynchronize(h->stream));
-    h->dfree(h->replay_index);
-    h->dfree(h->replay_weight);
+    h->dfree(h->replay);
     h->dfree(h->created_entries);
     h->dfree(h->block_count);
     h->dfree(h->chunk_count);
     h->replay_capacity = 0;
     h->n_chunks = (h->map.n_blocks + plk::kBlocksPerChunk - 1) / plk::kBlocksPerChunk + 1;
-    h->replay_index = (int *)h->dmalloc(sizeof(int) * (want ? want : 1));
-    h->replay_weight = (float *)h->dmalloc(sizeof(float) * (want ? want : 1));
+    h->replay = (plk::ReplayEntry *)h->dmalloc(sizeof(plk::ReplayEntry) * (want ? want : 1));
     h->created_entries = (uint4 *)h->dmalloc(sizeof(uint4) * (want ? want : 1));
     h->block_count = (int *)h->dmalloc(sizeof(int) * (h->map.n_blocks ? h->map.n_blocks : 1));
     h->chunk_count = (int *)h->dmalloc(sizeof(int) * 2 * h->n_chunks);
-    if (!h->replay_index || !h->replay_weight || !h->created_entries ||
+    if (!h->replay || !h->created_entries ||
         !h->block_count || !h->chunk_count)
         return PL_ENOMEM;
     PL_HIP(hipMemsetAsync(h->chunk_count, 0, sizeof(int) * 2 * h->n_chunks, h->stream));
@@ -243,7 +240,7 @@ int enqueue_build(pl_lattice *h, const plk::PointFeatures &features, uint32_t ce
     const plk::CreatedLists lists{h->created_entries, h->block_count,
                                   h->chunk_count + (size_t)h->counter_set * h->n_chunks};
     PL_HIP(plk::build(h->pd, features, h->map, h->scale, h->cell_keys, cells, h->counters(),
-                      h->replay_index, h->replay_weight, h->xcd_aware ? 1 : 0, fused ? h->vd : 0,
+                      h->replay, h->xcd_aware ? 1 : 0, fused ? h->vd : 0,
                       splat_input, h->normalize ? h->vd - 1 : h->vd, h->cell_values, lists,
                       h->stream));
     h->mark(EV_BUILD);
@@ -272,7 +269,7 @@ int enqueue_apply(pl_lattice *h, float *output, const float *input, int reverse)
     if (!h->values_splatted) {
         if (!h->values_zeroed) PL_HIP(plk::fill_zero(h->values[0], (size_t)mv * vd, h->stream));
         h->mark(EV_FILL);
-        PL_HIP(plk::splat(pd, vd, h->map, input, in_channels, h->replay_index, h->replay_weight,
+        PL_HIP(plk::splat(pd, vd, h->map, input, in_channels, h->replay,
                           h->replay_holds_cells ? h->cell_vertex : nullptr, h->values[0],
                           h->xcd_aware ? 1 : 0, h->stream));
         h->replay_holds_cells = false;
@@ -305,7 +302,7 @@ int enqueue_apply(pl_lattice *h, float *output, const float *input, int reverse)
         cur = 1 - cur;
     }
     h->mark(EV_BLUR);
-    PL_HIP(plk::slice(pd, vd, h->map, h->replay_index, h->replay_weight,
+    PL_HIP(plk::slice(pd, vd, h->map, h->replay,
                       h->replay_holds_cells ? h->cell_vertex : nullptr, h->values[cur], output,
                       h->normalize ? 1 : 0, h->stream));
     h->mark(EV_SLICE);
@@ -419,8 +416,7 @@ int pl_destroy(pl_handle h) {
     h->dfree(h->values[1]);
     h->dfree(h->neighbours);
     h->dfree(h->cell_values);
-    h->dfree(h->replay_index);
-    h->dfree(h->replay_weight);
+    h->dfree(h->replay);
     h->dfree(h->created_entries);
     h->dfree(h->block_count);
     h->dfree(h->chunk_count);
@@ -688,7 +684,7 @@ int pl_debug_keys(pl_handle h, short *keys) {
 int pl_debug_replay(pl_handle h, int *vertex, float *weight) {
     if (!h) return PL_EINVAL;
     if (!h->built || !h->verified) return PL_ESTATE;
-    PL_HIP(plk::export_replay(h->pd, h->map, h->replay_index, h->replay_weight,
+    PL_HIP(plk::export_replay(h->pd, h->map, h->replay,
                               h->replay_holds_cells ? h->cell_vertex : nullptr, vertex, weight,
                               h->stream));
     return PL_OK;

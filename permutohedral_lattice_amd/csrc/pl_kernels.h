@@ -45,6 +45,13 @@ struct VertexTables {
 // below 1/3 the table no longer fits the L2 next to everything else.
 __host__ __device__ inline uint32_t max_vertices_for(uint32_t n_cells) { return n_cells / 4u * 3u; }
 
+// One row of the replay matrix (reference: MatrixEntry, src/PermutohedralLatticeCPU.h:187-190):
+// which vertex a point's simplex corner is (hash cell until the first splat) and its weight.
+struct ReplayEntry {
+    int index;
+    float weight;
+};
+
 struct ScaleFactor {
     float v[kMaxPd];
 };
@@ -95,16 +102,16 @@ hipError_t clear_table(uint64_t *cell_keys, uint32_t n_cells, hipStream_t s);
 
 // Stage 1+2: per point embed, enclosing simplex, barycentric weights, then insertion of the pd+1
 // vertex keys.  The replay arrays hold (pd+1) rows of T = map.n_blocks*256 entries in thread
-// order: replay_index[r*T+t] := hash cell of vertex r of the point of thread t (-1: no point),
-// replay_weight likewise.  The lane whose insertion created a vertex appends its cell and key to
+// order: replay[r*T+t] := hash cell of vertex r of the point of thread t (-1: no point) and its
+// barycentric weight.  The lane whose insertion created a vertex appends its cell and key to
 // its workgroup's list in created_lists.
 // splat_vd != 0 (allowed when build_can_splat(vd)): the kernel also splats `input`
 // (in_channels per point) into cell_values[cell*vd ..], rows addressed by hash cell;
 // number_vertices then moves them into the dense value table.
 bool build_can_splat(int vd);
 hipError_t build(int pd, const PointFeatures &features, const PointMap &map, const ScaleFactor &scale,
-                 uint64_t *cell_keys, uint32_t n_cells, Counters *counters, int *replay_index,
-                 float *replay_weight, int xcd_aware, int splat_vd, const float *input,
+                 uint64_t *cell_keys, uint32_t n_cells, Counters *counters, ReplayEntry *replay,
+                 int xcd_aware, int splat_vd, const float *input,
                  int in_channels, float *cell_values, const CreatedLists &created_lists,
                  hipStream_t s);
 
@@ -130,10 +137,10 @@ hipError_t neighbours(int pd, const VertexTables &vertices, const Counters *coun
 hipError_t fill_zero(float *p, size_t n, hipStream_t s);
 
 // Stage 3.  in_channels is vd-1 (the homogeneous channel is the bare weight) or vd.
-// cell_vertex != nullptr: replay_index still holds hash cells; they are translated to vertex
+// cell_vertex != nullptr: the replay rows still hold hash cells; they are translated to vertex
 // indices and written back.
 hipError_t splat(int pd, int vd, const PointMap &map, const float *input, int in_channels,
-                 int *replay_index, const float *replay_weight, const int *cell_vertex, float *values,
+                 ReplayEntry *replay, const int *cell_vertex, float *values,
                  int xcd_aware, hipStream_t s);
 
 // Stage 4, one axis: dst[v] = 1/4 src[n1] + 1/2 src[v] + 1/4 src[n2] for v < counters->num_vertices.
@@ -150,9 +157,9 @@ hipError_t blur_two_axes(int vd, const Counters *counters, int max_vertices, con
                          hipStream_t s);
 
 // Stage 5.  normalize: divide by the homogeneous channel and write vd-1 channels; else write vd.
-// cell_vertex != nullptr: replay_index still holds hash cells (vd <= 8 only).
-hipError_t slice(int pd, int vd, const PointMap &map, const int *replay_index,
-                 const float *replay_weight, const int *cell_vertex, const float *values,
+// cell_vertex != nullptr: the replay rows still hold hash cells (vd <= 8 only).
+hipError_t slice(int pd, int vd, const PointMap &map, const ReplayEntry *replay,
+                 const int *cell_vertex, const float *values,
                  float *output, int normalize, hipStream_t s);
 
 hipError_t debug_simplex(int pd, const float *positions, int N, const ScaleFactor &scale,
@@ -161,9 +168,9 @@ hipError_t debug_simplex(int pd, const float *positions, int N, const ScaleFacto
 hipError_t export_keys(int pd, const uint64_t *vertex_keys, int M, short *keys, hipStream_t s);
 
 // replay arrays in point order: vertex[r*N+n], weight[r*N+n]; cell_vertex != nullptr when
-// replay_index still holds hash cells
-hipError_t export_replay(int pd, const PointMap &map, const int *replay_index,
-                         const float *replay_weight, const int *cell_vertex, int *vertex,
+// the replay rows still hold hash cells
+hipError_t export_replay(int pd, const PointMap &map, const ReplayEntry *replay,
+                         const int *cell_vertex, int *vertex,
                          float *weight, hipStream_t s);
 
 hipError_t compute_positions(const float *reference, float *positions, int N, int n_ref_channels,

@@ -11,8 +11,8 @@
 //   vertex_keys[M]         u64  packed key of vertex v
 //   neighbours[(pd+1)*M]   int2 per blur axis a and vertex v: indices of v's two neighbours or -1
 //   values[M*vd]           f32  vertex values, two buffers (ping-pong across blur axes)
-//   replay_index[(pd+1)*N] i32  [r][n]: vertex r of point n (hash cell until the first splat)
-//   replay_weight[(pd+1)*N] f32 [r][n]: its barycentric weight
+//   replay[(pd+1)*T] {i32, f32} [r][t]: vertex r of the point of thread t (hash cell until the
+//                                first splat) and its barycentric weight
 //
 // Packed key.  Every coordinate of lattice vertex with remainder r is (pd+1)*q_i + r, so a key is
 // (r, q_0..q_{pd-1}): r in bits 60..63, q_i biased into a field of B = min(16, 60/pd) bits.
@@ -387,8 +387,7 @@ template <int PD, int SPLAT_VD>
 __global__ __launch_bounds__(kBlock) void k_build(PointFeatures features, PointMap map,
                                                    ScaleFactor scale, uint64_t *cell_keys,
                                                    uint32_t mask, Counters *counters,
-                                                   int *__restrict__ replay_index,
-                                                   float *__restrict__ replay_weight,
+                                                   ReplayEntry *__restrict__ replay,
                                                    int xcd_aware, const float *__restrict__ input,
                                                    int in_channels, float *cell_values,
                                                    CreatedLists created_lists) {
@@ -519,8 +518,7 @@ __global__ __launch_bounds__(kBlock) void k_build(PointFeatures features, PointM
     for (int r = 0; r < D1; ++r) {
         const int own = open[r] ? -1 : (int)cell[r];
         const int c = __shfl(own, leader[r]);
-        replay_index[(size_t)r * T + t] = active ? c : -1;
-        replay_weight[(size_t)r * T + t] = valid ? s.weight[r] : 0.0f;
+        replay[(size_t)r * T + t] = ReplayEntry{active ? c : -1, valid ? s.weight[r] : 0.0f};
         if (SPLAT_VD) {
             constexpr int VD = SPLAT_VD ? SPLAT_VD : 2;
             constexpr int P = VD == 2 ? 2 : 4;
@@ -722,8 +720,7 @@ __global__ __launch_bounds__(kBlock) void k_fill_zero(float *p, size_t n) {
 template <int VD, int D1>
 __global__ __launch_bounds__(kBlock) void k_splat_dpp(PointMap map,
                                                        const float *__restrict__ input,
-                                                       int in_channels, int *replay_index,
-                                                       const float *__restrict__ replay_weight,
+                                                       int in_channels, ReplayEntry *replay,
                                                        const int *__restrict__ cell_vertex,
                                                        float *values, int xcd_aware) {
     static_assert(VD >= 2 && VD <= 4, "register splat handles 2..4 channels");
@@ -749,8 +746,9 @@ __global__ __launch_bounds__(kBlock) void k_splat_dpp(PointMap map,
     float weight[D1];
 #pragma unroll
     for (int r = 0; r < D1; ++r) {
-        vertex[r] = n >= 0 ? replay_index[(size_t)r * T + t] : -1;
-        weight[r] = replay_weight[(size_t)r * T + t];
+        const ReplayEntry e = replay[(size_t)r * T + t];
+        vertex[r] = n >= 0 ? e.index : -1;
+        weight[r] = e.weight;
     }
     if (cell_vertex) {
 #pragma unroll
@@ -758,7 +756,7 @@ __global__ __launch_bounds__(kBlock) void k_splat_dpp(PointMap map,
             if (vertex[r] >= 0) vertex[r] = cell_vertex[vertex[r]];
 #pragma unroll
         for (int r = 0; r < D1; ++r)
-            if (n >= 0) replay_index[(size_t)r * T + t] = vertex[r];
+            if (n >= 0) replay[(size_t)r * T + t].index = vertex[r];
     }
 
 #pragma unroll
@@ -786,8 +784,7 @@ __global__ __launch_bounds__(kBlock) void k_splat_dpp(PointMap map,
 template <int D1>
 __global__ __launch_bounds__(kBlock) void k_splat_dpp_blocks(int vd, PointMap map,
                                                               const float *__restrict__ input,
-                                                              int in_channels, int *replay_index,
-                                                              const float *__restrict__ replay_weight,
+                                                              int in_channels, ReplayEntry *replay,
                                                               const int *__restrict__ cell_vertex,
                                                               float *values, int xcd_aware) {
     const unsigned vblock = xcd_contiguous_block(blockIdx.x, gridDim.x, xcd_aware);
@@ -801,8 +798,9 @@ __global__ __launch_bounds__(kBlock) void k_splat_dpp_blocks(int vd, PointMap ma
     float weight[D1];
 #pragma unroll
     for (int r = 0; r < D1; ++r) {
-        vertex[r] = n >= 0 ? replay_index[(size_t)r * T + t] : -1;
-        weight[r] = replay_weight[(size_t)r * T + t];
+        const ReplayEntry e = replay[(size_t)r * T + t];
+        vertex[r] = n >= 0 ? e.index : -1;
+        weight[r] = e.weight;
     }
     if (cell_vertex) {
 #pragma unroll
@@ -810,7 +808,7 @@ __global__ __launch_bounds__(kBlock) void k_splat_dpp_blocks(int vd, PointMap ma
             if (vertex[r] >= 0) vertex[r] = cell_vertex[vertex[r]];
 #pragma unroll
         for (int r = 0; r < D1; ++r)
-            if (n >= 0) replay_index[(size_t)r * T + t] = vertex[r];
+            if (n >= 0) replay[(size_t)r * T + t].index = vertex[r];
     }
 
     for (int first_channel = 0; first_channel < vd; first_channel += 4) {
@@ -922,8 +920,7 @@ __global__ __launch_bounds__(kBlock) void k_blur2_element(const Counters *counte
 // cell_vertex != nullptr: the replay rows still hold hash cells (nothing has translated them yet)
 template <int VD>
 __global__ __launch_bounds__(kBlock) void k_slice_point(int d1, PointMap map,
-                                                         const int *__restrict__ replay_index,
-                                                         const float *__restrict__ replay_weight,
+                                                         const ReplayEntry *__restrict__ replay,
                                                          const int *__restrict__ cell_vertex,
                                                          const float *__restrict__ values,
                                                          float *__restrict__ output, int normalize) {
@@ -935,10 +932,11 @@ __global__ __launch_bounds__(kBlock) void k_slice_point(int d1, PointMap map,
 #pragma unroll
     for (int j = 0; j < VD; ++j) acc[j] = 0.0f;
     for (int r = 0; r < d1; ++r) {
-        int v = replay_index[(size_t)r * T + t];
+        const ReplayEntry e = replay[(size_t)r * T + t];
+        int v = e.index;
         if (v < 0) continue;
         if (cell_vertex) v = cell_vertex[v];
-        const float w = replay_weight[(size_t)r * T + t];
+        const float w = e.weight;
         const float *src = values + (size_t)v * VD;
 #pragma unroll
         for (int j = 0; j < VD; ++j) acc[j] += w * src[j];
@@ -954,8 +952,7 @@ __global__ __launch_bounds__(kBlock) void k_slice_point(int d1, PointMap map,
 }
 
 __global__ __launch_bounds__(kBlock) void k_slice_channel(int d1, int vd, PointMap map, size_t T,
-                                                           const int *__restrict__ replay_index,
-                                                           const float *__restrict__ replay_weight,
+                                                           const ReplayEntry *__restrict__ replay,
                                                            const float *__restrict__ values,
                                                            float *__restrict__ output, int normalize) {
     const int out_ch = normalize ? vd - 1 : vd;
@@ -967,9 +964,10 @@ __global__ __launch_bounds__(kBlock) void k_slice_channel(int d1, int vd, PointM
     if (n < 0) return;
     float acc = 0.0f, hom = 0.0f;
     for (int r = 0; r < d1; ++r) {
-        const int v = replay_index[(size_t)r * T + t];
+        const ReplayEntry e = replay[(size_t)r * T + t];
+        const int v = e.index;
         if (v < 0) continue;
-        const float w = replay_weight[(size_t)r * T + t];
+        const float w = e.weight;
         const float *src = values + (size_t)v * vd;
         acc += w * src[j];
         hom += w * src[vd - 1];
@@ -1029,8 +1027,7 @@ __global__ __launch_bounds__(kBlock) void k_export_keys(const uint64_t *__restri
 // replay arrays from thread order to point order: out[r*N + n]; cells are translated to vertex
 // indices when cell_vertex != nullptr
 __global__ __launch_bounds__(kBlock) void k_export_replay(int d1, PointMap map,
-                                                           const int *__restrict__ replay_index,
-                                                           const float *__restrict__ replay_weight,
+                                                           const ReplayEntry *__restrict__ replay,
                                                            const int *__restrict__ cell_vertex,
                                                            int *vertex, float *weight) {
     const size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x;
@@ -1038,12 +1035,13 @@ __global__ __launch_bounds__(kBlock) void k_export_replay(int d1, PointMap map,
     const int n = point_of_thread(map, blockIdx.x, threadIdx.x);
     if (n < 0) return;
     for (int r = 0; r < d1; ++r) {
+        const ReplayEntry e = replay[(size_t)r * T + t];
         if (vertex) {
-            int v = replay_index[(size_t)r * T + t];
+            int v = e.index;
             if (cell_vertex && v >= 0) v = cell_vertex[v];
             vertex[(size_t)r * map.N + n] = v;
         }
-        if (weight) weight[(size_t)r * map.N + n] = replay_weight[(size_t)r * T + t];
+        if (weight) weight[(size_t)r * map.N + n] = e.weight;
     }
 }
 
@@ -1129,15 +1127,15 @@ hipError_t clear_table(uint64_t *cell_keys, uint32_t n_cells, hipStream_t s) {
 bool build_can_splat(int vd) { return vd >= 2 && vd <= 4; }
 
 hipError_t build(int pd, const PointFeatures &features, const PointMap &map, const ScaleFactor &scale,
-                 uint64_t *cell_keys, uint32_t n_cells, Counters *counters, int *replay_index,
-                 float *replay_weight, int xcd_aware, int splat_vd, const float *input,
+                 uint64_t *cell_keys, uint32_t n_cells, Counters *counters, ReplayEntry *replay,
+                 int xcd_aware, int splat_vd, const float *input,
                  int in_channels, float *cell_values, const CreatedLists &created_lists,
                  hipStream_t s) {
     if (map.n_blocks == 0) return hipSuccess;
 #define PLK_BUILD(SPLAT_VD)                                                                        \
     PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_build<PD, SPLAT_VD>), dim3(map.n_blocks),            \
                                            dim3(kBlock), 0, s, features, map, scale, cell_keys,    \
-                                           n_cells - 1u, counters, replay_index, replay_weight,    \
+                                           n_cells - 1u, counters, replay,                         \
                                            xcd_aware, input, in_channels, cell_values,             \
                                            created_lists))
     switch (splat_vd) {
@@ -1181,22 +1179,22 @@ hipError_t fill_zero(float *p, size_t n, hipStream_t s) {
 }
 
 hipError_t splat(int pd, int vd, const PointMap &map, const float *input, int in_channels,
-                 int *replay_index, const float *replay_weight, const int *cell_vertex, float *values,
+                 ReplayEntry *replay, const int *cell_vertex, float *values,
                  int xcd_aware, hipStream_t s) {
     if (map.n_blocks == 0) return hipSuccess;
     const dim3 grid(map.n_blocks), block(kBlock);
 #define PLK_SPLAT_DPP(VD)                                                                         \
     case VD:                                                                                      \
         PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_splat_dpp<VD, PD + 1>), grid, block, 0, s, map, \
-                                               input, in_channels, replay_index, replay_weight,   \
+                                               input, in_channels, replay,                        \
                                                cell_vertex, values, xcd_aware));                  \
         break;
     switch (vd) {
         PLK_SPLAT_DPP(2) PLK_SPLAT_DPP(3) PLK_SPLAT_DPP(4)
         default:
             PLK_DISPATCH_PD(pd, hipLaunchKernelGGL(k_splat_dpp_blocks<PD + 1>, grid, block, 0, s, vd,
-                                                   map, input, in_channels, replay_index,
-                                                   replay_weight, cell_vertex, values, xcd_aware));
+                                                   map, input, in_channels, replay,
+                                                   cell_vertex, values, xcd_aware));
             break;
     }
 #undef PLK_SPLAT_DPP
@@ -1223,8 +1221,8 @@ hipError_t blur_two_axes(int vd, const Counters *counters, int max_vertices, con
     return hipGetLastError();
 }
 
-hipError_t slice(int pd, int vd, const PointMap &map, const int *replay_index,
-                 const float *replay_weight, const int *cell_vertex, const float *values,
+hipError_t slice(int pd, int vd, const PointMap &map, const ReplayEntry *replay,
+                 const int *cell_vertex, const float *values,
                  float *output, int normalize, hipStream_t s) {
     if (map.n_blocks == 0) return hipSuccess;
     const int d1 = pd + 1;
@@ -1232,15 +1230,15 @@ hipError_t slice(int pd, int vd, const PointMap &map, const int *replay_index,
     const size_t T = (size_t)map.n_blocks * kBlock;
 #define PLK_SLICE(VD)                                                                          \
     case VD:                                                                                   \
-        hipLaunchKernelGGL(k_slice_point<VD>, grid, block, 0, s, d1, map, replay_index,        \
-                           replay_weight, cell_vertex, values, output, normalize);             \
+        hipLaunchKernelGGL(k_slice_point<VD>, grid, block, 0, s, d1, map, replay,              \
+                           cell_vertex, values, output, normalize);                            \
         break;
     switch (vd) {
         PLK_SLICE(2) PLK_SLICE(3) PLK_SLICE(4) PLK_SLICE(5) PLK_SLICE(6) PLK_SLICE(7) PLK_SLICE(8)
         default: {
             const int out_ch = normalize ? vd - 1 : vd;
             hipLaunchKernelGGL(k_slice_channel, dim3(blocks_for(T * out_ch)), block, 0, s, d1, vd, map,
-                               T, replay_index, replay_weight, values, output, normalize);
+                               T, replay, values, output, normalize);
         } break;
     }
 #undef PLK_SLICE
@@ -1263,12 +1261,12 @@ hipError_t export_keys(int pd, const uint64_t *vertex_keys, int M, short *keys, 
     return hipGetLastError();
 }
 
-hipError_t export_replay(int pd, const PointMap &map, const int *replay_index,
-                         const float *replay_weight, const int *cell_vertex, int *vertex,
+hipError_t export_replay(int pd, const PointMap &map, const ReplayEntry *replay,
+                         const int *cell_vertex, int *vertex,
                          float *weight, hipStream_t s) {
     if (map.n_blocks == 0) return hipSuccess;
     hipLaunchKernelGGL(k_export_replay, dim3(map.n_blocks), dim3(kBlock), 0, s, pd + 1, map,
-                       replay_index, replay_weight, cell_vertex, vertex, weight);
+                       replay, cell_vertex, vertex, weight);
     return hipGetLastError();
 }
 
