@@ -914,6 +914,80 @@ __global__ __launch_bounds__(kBlock) void k_blur2_element(const Counters *counte
     }
 }
 
+// For up to four channels: one thread per vertex, the whole row in one vector access.  With
+// vertex numbers that follow the image the rows a thread gathers are near each other, and a
+// quarter of the memory instructions moves the same bytes (34 -> 25 us for the three launches
+// of pd = 5, vd = 4).  Same arithmetic per channel, same results.
+template <int VD>
+struct alignas(VD == 3 ? 4 : 4 * VD) ValueRow {
+    float c[VD];
+};
+
+template <int VD>
+__device__ __forceinline__ ValueRow<VD> blur_rows(const ValueRow<VD> &a, const ValueRow<VD> &self,
+                                                  const ValueRow<VD> &b) {
+    ValueRow<VD> out;
+#pragma unroll
+    for (int j = 0; j < VD; ++j) out.c[j] = blur_tap(a.c[j], self.c[j], b.c[j]);
+    return out;
+}
+
+template <int VD>
+__device__ __forceinline__ ValueRow<VD> row_or_zero(const ValueRow<VD> *__restrict__ src, int u) {
+    if (u >= 0) return src[u];
+    ValueRow<VD> zero;
+#pragma unroll
+    for (int j = 0; j < VD; ++j) zero.c[j] = 0.0f;
+    return zero;
+}
+
+template <int VD>
+__device__ __forceinline__ ValueRow<VD> blur_row_of(const ValueRow<VD> *__restrict__ src,
+                                                    const int2 *__restrict__ nbr_a, int u) {
+    if (u < 0) return row_or_zero<VD>(src, -1);
+    const int2 nb = nbr_a[u];
+    return blur_rows<VD>(row_or_zero<VD>(src, nb.x), src[u], row_or_zero<VD>(src, nb.y));
+}
+
+template <int VD>
+__global__ __launch_bounds__(kBlock) void k_blur_row(const Counters *counters, int max_vertices,
+                                                      const ValueRow<VD> *__restrict__ src,
+                                                      ValueRow<VD> *__restrict__ dst,
+                                                      const int2 *__restrict__ nbr,
+                                                      uint64_t *reset_cell_keys,
+                                                      const int *__restrict__ vertex_cell) {
+    const int M = vertex_count(counters, max_vertices);
+    ItemBlocks blocks((size_t)M);
+    unsigned vb;
+    while (blocks.next(vb)) {
+        const int v = (int)(vb * kBlock + threadIdx.x);
+        if (v >= M) continue;
+        dst[v] = blur_row_of<VD>(src, nbr, v);
+        if (reset_cell_keys) reset_cell_keys[vertex_cell[v]] = kEmptyCell;
+    }
+}
+
+template <int VD>
+__global__ __launch_bounds__(kBlock) void k_blur2_row(const Counters *counters, int max_vertices,
+                                                       const ValueRow<VD> *__restrict__ src,
+                                                       ValueRow<VD> *__restrict__ dst,
+                                                       const int2 *__restrict__ nbr_a,
+                                                       const int2 *__restrict__ nbr_b,
+                                                       uint64_t *reset_cell_keys,
+                                                       const int *__restrict__ vertex_cell) {
+    const int M = vertex_count(counters, max_vertices);
+    ItemBlocks blocks((size_t)M);
+    unsigned vb;
+    while (blocks.next(vb)) {
+        const int v = (int)(vb * kBlock + threadIdx.x);
+        if (v >= M) continue;
+        const int2 nb = nbr_b[v];
+        dst[v] = blur_rows<VD>(blur_row_of<VD>(src, nbr_a, nb.x), blur_row_of<VD>(src, nbr_a, v),
+                               blur_row_of<VD>(src, nbr_a, nb.y));
+        if (reset_cell_keys) reset_cell_keys[vertex_cell[v]] = kEmptyCell;
+    }
+}
+
 // ------------------------------------------------------------------------------------------------
 // Stage 5: slice (reference: src/PermutohedralLatticeCPU.h:333-352)
 // ------------------------------------------------------------------------------------------------
@@ -1205,6 +1279,19 @@ hipError_t blur_axis(int vd, const Counters *counters, int max_vertices, const f
                      const int2 *nbr, uint64_t *reset_cell_keys, const int *vertex_cell,
                      int launch_vertices, hipStream_t s) {
     if (max_vertices <= 0) return hipSuccess;
+#define PLK_BLUR_ROW(VD)                                                                          \
+    case VD:                                                                                      \
+        hipLaunchKernelGGL(k_blur_row<VD>, dim3(vertex_blocks((size_t)launch_vertices)),          \
+                           dim3(kBlock), 0, s, counters, max_vertices,                            \
+                           reinterpret_cast<const ValueRow<VD> *>(src),                           \
+                           reinterpret_cast<ValueRow<VD> *>(dst), nbr, reset_cell_keys,           \
+                           vertex_cell);                                                          \
+        return hipGetLastError();
+    switch (vd) {
+        PLK_BLUR_ROW(2) PLK_BLUR_ROW(3) PLK_BLUR_ROW(4)
+        default: break;
+    }
+#undef PLK_BLUR_ROW
     hipLaunchKernelGGL(k_blur_element, dim3(vertex_blocks((size_t)launch_vertices * vd)), dim3(kBlock), 0, s,
                        counters, max_vertices, vd, src, dst, nbr, reset_cell_keys, vertex_cell);
     return hipGetLastError();
@@ -1215,6 +1302,19 @@ hipError_t blur_two_axes(int vd, const Counters *counters, int max_vertices, con
                          uint64_t *reset_cell_keys, const int *vertex_cell, int launch_vertices,
                          hipStream_t s) {
     if (max_vertices <= 0) return hipSuccess;
+#define PLK_BLUR2_ROW(VD)                                                                         \
+    case VD:                                                                                      \
+        hipLaunchKernelGGL(k_blur2_row<VD>, dim3(vertex_blocks((size_t)launch_vertices)),         \
+                           dim3(kBlock), 0, s, counters, max_vertices,                            \
+                           reinterpret_cast<const ValueRow<VD> *>(src),                           \
+                           reinterpret_cast<ValueRow<VD> *>(dst), nbr_first, nbr_second,          \
+                           reset_cell_keys, vertex_cell);                                         \
+        return hipGetLastError();
+    switch (vd) {
+        PLK_BLUR2_ROW(2) PLK_BLUR2_ROW(3) PLK_BLUR2_ROW(4)
+        default: break;
+    }
+#undef PLK_BLUR2_ROW
     hipLaunchKernelGGL(k_blur2_element, dim3(vertex_blocks((size_t)launch_vertices * vd)), dim3(kBlock), 0, s,
                        counters, max_vertices, vd, src, dst, nbr_first, nbr_second, reset_cell_keys,
                        vertex_cell);
