@@ -49,6 +49,82 @@ def measured_traffic(kernel_name, side):
     return int(sum(table[key]))
 
 
+def run_side_legs(args, pla, synth, lat, step, img, d_pos, d_val, d_grad, out_f, out_r, side, batch):
+    """The legs beside the headline: no grid hint, lattice reuse, the op's boundary, a batch."""
+    import numpy as np
+    import torch
+
+    # the same without the grid hint (a caller of filter() that only has N points)
+    lat.set_point_grid(None)
+    for _ in range(2):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        step()
+    torch.cuda.synchronize()
+    plain_ms = 1e3 * (time.perf_counter() - t0) / args.steps
+    lat.set_point_grid((side, side))
+
+    # build once, apply forward and reverse (what a caller that keeps the lattice gets)
+    lat.build(d_pos)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        lat.apply(out_f, d_val, False)
+        lat.apply(out_r, d_grad, True)
+    torch.cuda.synchronize()
+    reuse_ms = 1e3 * (time.perf_counter() - t0) / args.steps
+
+    # the op's boundary: the reference image comes in, not a positions array.  First as the
+    # reference does it (feature kernel, then filter), then with the features built on the fly.
+    d_img = torch.from_numpy(np.ascontiguousarray(img.reshape(-1, 3))).cuda()
+    d_pos2 = torch.empty_like(d_pos)
+
+    def op_step_two_kernels():
+        for o, v, rev in ((out_f, d_val, False), (out_r, d_grad, True)):
+            pla.compute_positions(d_img, (side, side), 8.0, 0.125, out=d_pos2)
+            lat.filter(o, v, d_pos2, rev)
+
+    def op_step_fused():
+        for o, v, rev in ((out_f, d_val, False), (out_r, d_grad, True)):
+            lat.filter_image(o, v, d_img, (side, side), 8.0, 0.125, rev)
+
+    op_ms = {}
+    for name, fn in (("positions_then_filter", op_step_two_kernels), ("features_on_the_fly", op_step_fused)):
+        for _ in range(2):
+            fn()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            fn()
+        torch.cuda.synchronize()
+        op_ms[name] = 1e3 * (time.perf_counter() - t0) / args.steps
+
+    # a batch through the op: four images, forward then reverse, one item at a time as the
+    # reference's loop runs them, and with the items spread over concurrent lattices
+    b_img = torch.from_numpy(np.stack([synth.blob_image(side, side, seed=0xC0FFEE + 10 + i)
+                                       for i in range(batch)])).cuda()
+    b_grad = torch.from_numpy(synth.normal_image((batch, side, side, 3), 0xC0FFEE + 20)).cuda()
+    batch_ms = {}
+    for lanes in (1, 4):
+        pla.set_op_concurrency(lanes)
+        for _ in range(2):
+            pla._lattice_filter_raw(b_img, b_img, True, 8.0, 0.125, 1.0, False)
+        torch.cuda.synchronize()
+        reps = max(3, args.steps // 5)
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            pla._lattice_filter_raw(b_img, b_img, True, 8.0, 0.125, 1.0, False)
+            pla._lattice_filter_raw(b_grad, b_img, True, 8.0, 0.125, 1.0, True)
+        torch.cuda.synchronize()
+        batch_ms["%d_at_a_time" % lanes] = 1e3 * (time.perf_counter() - t0) / reps
+    pla.set_op_concurrency(4)
+    del b_img, b_grad
+
+    return plain_ms, reuse_ms, op_ms, batch_ms
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -56,6 +132,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--size", type=int, default=1024, help="image side (default 1024)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and parity legs")
+    ap.add_argument("--headline-only", action="store_true",
+                    help="only the timed steps and the per-stage timing (what a rocprofv3 run of "
+                         "this file should see): no side legs, no CPU baseline")
     ap.add_argument("--calibrate-copy-mib", type=int, default=0,
                     help="only run device-to-device copies of this many MiB (a kernel of known "
                          "traffic, for scaling rocprofv3's FETCH_SIZE / WRITE_SIZE) and exit")
@@ -114,74 +193,12 @@ def main():
     pixels_per_step = 2 * n
     value = pixels_per_step / (ms_per_step * 1e-3) / 1e6
 
-    # the same without the grid hint (a caller of filter() that only has N points)
-    lat.set_point_grid(None)
-    for _ in range(2):
-        step()
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        step()
-    torch.cuda.synchronize()
-    plain_ms = 1e3 * (time.perf_counter() - t0) / args.steps
-    lat.set_point_grid((side, side))
-
-    # build once, apply forward and reverse (what a caller that keeps the lattice gets)
-    lat.build(d_pos)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        lat.apply(out_f, d_val, False)
-        lat.apply(out_r, d_grad, True)
-    torch.cuda.synchronize()
-    reuse_ms = 1e3 * (time.perf_counter() - t0) / args.steps
-
-    # the op's boundary: the reference image comes in, not a positions array.  First as the
-    # reference does it (feature kernel, then filter), then with the features built on the fly.
-    d_img = torch.from_numpy(np.ascontiguousarray(img.reshape(-1, 3))).cuda()
-    d_pos2 = torch.empty_like(d_pos)
-
-    def op_step_two_kernels():
-        for o, v, rev in ((out_f, d_val, False), (out_r, d_grad, True)):
-            pla.compute_positions(d_img, (side, side), 8.0, 0.125, out=d_pos2)
-            lat.filter(o, v, d_pos2, rev)
-
-    def op_step_fused():
-        for o, v, rev in ((out_f, d_val, False), (out_r, d_grad, True)):
-            lat.filter_image(o, v, d_img, (side, side), 8.0, 0.125, rev)
-
-    op_ms = {}
-    for name, fn in (("positions_then_filter", op_step_two_kernels), ("features_on_the_fly", op_step_fused)):
-        for _ in range(2):
-            fn()
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(args.steps):
-            fn()
-        torch.cuda.synchronize()
-        op_ms[name] = 1e3 * (time.perf_counter() - t0) / args.steps
-
-    # a batch through the op: four images, forward then reverse, one item at a time as the
-    # reference's loop runs them, and with the items spread over concurrent lattices
-    batch = 4
-    b_img = torch.from_numpy(np.stack([synth.blob_image(side, side, seed=0xC0FFEE + 10 + i)
-                                       for i in range(batch)])).cuda()
-    b_grad = torch.from_numpy(synth.normal_image((batch, side, side, 3), 0xC0FFEE + 20)).cuda()
-    batch_ms = {}
-    for lanes in (1, 4):
-        pla.set_op_concurrency(lanes)
-        for _ in range(2):
-            pla._lattice_filter_raw(b_img, b_img, True, 8.0, 0.125, 1.0, False)
-        torch.cuda.synchronize()
-        reps = max(3, args.steps // 5)
-        t0 = time.perf_counter()
-        for _ in range(reps):
-            pla._lattice_filter_raw(b_img, b_img, True, 8.0, 0.125, 1.0, False)
-            pla._lattice_filter_raw(b_grad, b_img, True, 8.0, 0.125, 1.0, True)
-        torch.cuda.synchronize()
-        batch_ms["%d_at_a_time" % lanes] = 1e3 * (time.perf_counter() - t0) / reps
-    pla.set_op_concurrency(4)
-    del b_img, b_grad
+    side_legs = not args.headline_only
+    plain_ms = reuse_ms = 0.0
+    op_ms, batch_ms, batch = {}, {}, 4
+    if side_legs:
+        plain_ms, reuse_ms, op_ms, batch_ms = run_side_legs(args, pla, synth, lat, step, img, d_pos,
+                                                            d_val, d_grad, out_f, out_r, side, batch)
 
     # per-kernel durations from HIP events on the lattice's stream
     lat.set_option(pla.PL_OPT_PROFILE, 1)
@@ -206,7 +223,7 @@ def main():
         dominant = "blur_axis"
     achieved = alg[dominant] / (per_launch_ms[dominant] * 1e-3) / 1e9
     kernel_name = {"build": "k_build<5, 4>" if fused else "k_build<5, 0>", "splat": "k_splat_dpp<4, 6>",
-                   "blur_axis": "k_blur2_element", "slice": "k_slice_point<4>"}[dominant]
+                   "blur_axis": "k_blur2_row<4>", "slice": "k_slice_point<4>"}[dominant]
     roofline = {"bound": "hbm", "kernel": kernel_name, "achieved": round(achieved, 2),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 5),
                 "traffic": measured_traffic(kernel_name, side),
@@ -231,25 +248,28 @@ def main():
                             "frac": round(filter_gbs / HBM_PEAK_GBS, 5)},
         "stage_ms": {k: round(v, 5) for k, v in stages.items()},
         "kernel_ms_per_filter": round(gpu_kernel_ms, 4),
-        "no_grid_hint": {"what": "same step, points treated as a plain list",
-                         "ms_per_step": round(plain_ms, 4),
-                         "value": round(pixels_per_step / (plain_ms * 1e-3) / 1e6, 3)},
-        "reuse": {"what": "build once, apply forward + reverse per step",
-                  "ms_per_step": round(reuse_ms, 4),
-                  "value": round(pixels_per_step / (reuse_ms * 1e-3) / 1e6, 3)},
-        "op_level": {"what": "reference image in, forward + reverse per step: feature kernel + "
-                             "filter(), and filter_image() (features built inside the first kernel)",
-                     "ms_per_step": {k: round(v, 4) for k, v in op_ms.items()},
-                     "value": {k: round(pixels_per_step / (v * 1e-3) / 1e6, 3)
-                               for k, v in op_ms.items()}},
-        "op_batch": {"what": "the op on a batch of %d such images, forward + reverse per step, "
-                             "items one at a time and four at a time" % batch,
-                     "ms_per_step": {k: round(v, 4) for k, v in batch_ms.items()},
-                     "value": {k: round(batch * pixels_per_step / (v * 1e-3) / 1e6, 3)
-                               for k, v in batch_ms.items()}},
     }
+    if side_legs:
+        result.update({
+            "no_grid_hint": {"what": "same step, points treated as a plain list",
+                             "ms_per_step": round(plain_ms, 4),
+                             "value": round(pixels_per_step / (plain_ms * 1e-3) / 1e6, 3)},
+            "reuse": {"what": "build once, apply forward + reverse per step",
+                      "ms_per_step": round(reuse_ms, 4),
+                      "value": round(pixels_per_step / (reuse_ms * 1e-3) / 1e6, 3)},
+            "op_level": {"what": "reference image in, forward + reverse per step: feature kernel + "
+                                 "filter(), and filter_image() (features built inside the first kernel)",
+                         "ms_per_step": {k: round(v, 4) for k, v in op_ms.items()},
+                         "value": {k: round(pixels_per_step / (v * 1e-3) / 1e6, 3)
+                                   for k, v in op_ms.items()}},
+            "op_batch": {"what": "the op on a batch of %d such images, forward + reverse per step, "
+                                 "items one at a time and four at a time" % batch,
+                         "ms_per_step": {k: round(v, 4) for k, v in batch_ms.items()},
+                         "value": {k: round(batch * pixels_per_step / (v * 1e-3) / 1e6, 3)
+                                   for k, v in batch_ms.items()}},
+        })
 
-    if not args.no_cpu:
+    if not args.no_cpu and not args.headline_only:
         import oracle
         ref = oracle.reference()
         cores = 1
