@@ -842,6 +842,111 @@ __global__ __launch_bounds__(kBlock) void k_splat_dpp_blocks(int vd, PointMap ma
     }
 }
 
+// Many channels (vd > 4, input rows of up to 64 channels): the lanes of a wavefront turn from
+// points into channels.  The wavefront first puts the input rows of its 64 points into LDS
+// (coalesced: consecutive lanes read consecutive floats); then, per simplex corner and per group
+// of points that share the vertex, lane c runs over the group's members, reads channel c of each
+// member's row from LDS and accumulates weight * value (channels past the input are the
+// homogeneous 1); one atomic instruction then adds the vd sums to the vertex row, consecutive
+// lanes on consecutive floats.  Against four channels at a time with a reduction tree per group
+// this is 1/6 of the instructions for vd = 22 and reads every input float from memory once.
+template <int W>
+__global__ __launch_bounds__(kBlock) void k_splat_channels(int d1, int vd, PointMap map,
+                                                            const float *__restrict__ input,
+                                                            int in_channels, ReplayEntry *replay,
+                                                            const int *__restrict__ cell_vertex,
+                                                            float *values, int xcd_aware) {
+    extern __shared__ float rows[];   // [kBlock][in_channels]
+    // workgroup (x, y): simplex corners 2y and 2y+1 of the points of block x.  With a few hundred
+    // thousand points there are too few wavefronts to hide the latencies of this serial code
+    // unless the corners are spread over several of them; each pays for putting the rows into LDS.
+    constexpr int kCorners = 2;
+    const unsigned vblock = xcd_contiguous_block(blockIdx.x, gridDim.x, xcd_aware);
+    const size_t t = (size_t)vblock * kBlock + threadIdx.x;
+    const size_t T = (size_t)gridDim.x * kBlock;
+    const int n = point_of_thread(map, vblock, threadIdx.x);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    float *wave_rows = rows + (size_t)wave * 64 * in_channels;
+
+    int vertex[kCorners];
+    float weight[kCorners];
+#pragma unroll
+    for (int i = 0; i < kCorners; ++i) {
+        const int r = blockIdx.y * kCorners + i;
+        vertex[i] = -1;
+        weight[i] = 0.0f;
+        if (r < d1) {
+            const ReplayEntry e = replay[(size_t)r * T + t];
+            vertex[i] = n >= 0 ? e.index : -1;
+            weight[i] = e.weight;
+            if (cell_vertex) {
+                if (vertex[i] >= 0) vertex[i] = cell_vertex[vertex[i]];
+                if (n >= 0) replay[(size_t)r * T + t].index = vertex[i];
+            }
+        }
+    }
+
+    // element i of the wavefront's 64 rows belongs to point i / in_channels, channel i % in_channels
+    {
+        int p = lane / in_channels, c = lane - p * in_channels;
+        const int step_p = 64 / in_channels, step_c = 64 - step_p * in_channels;
+        for (int i = lane; i < 64 * in_channels; i += 64) {
+            const int np = __shfl(n, p);
+            wave_rows[i] = np >= 0 ? input[(size_t)np * in_channels + c] : 0.0f;
+            p += step_p;
+            c += step_c;
+            if (c >= in_channels) {
+                c -= in_channels;
+                p += 1;
+            }
+        }
+    }
+    __syncthreads();
+
+    // W lanes per member (W = 16, 32 or 64, at least vd unless vd > 64): G = 64 / W members of a
+    // group are taken per step, member g by the lanes g*W .. g*W+W-1
+    constexpr int G = 64 / W;
+    const int sub = lane / W, c_in_w = lane % W;
+#pragma unroll
+    for (int i = 0; i < kCorners; ++i) {
+        const int v = vertex[i];
+        const float w = weight[i];
+        uint64_t remaining = wave_ballot(v >= 0);
+        while (remaining) {
+            const int first = __builtin_ctzll(remaining);
+            const int k = lane_value(v, first);
+            const uint64_t group = lanes_equal(v, k);
+            remaining &= ~group;
+            for (int c0 = 0; c0 < vd; c0 += W) {
+                const int c = c0 + c_in_w;
+                float acc = 0.0f;
+                uint64_t members = group;
+                while (members) {
+                    int m = first;
+                    float wm = 0.0f;
+#pragma unroll
+                    for (int g = 0; g < G; ++g) {
+                        const bool has = members != 0;
+                        const int mg = has ? __builtin_ctzll(members) : first;
+                        members &= members - 1;
+                        const float wg =
+                            __int_as_float(__builtin_amdgcn_readlane(__float_as_int(w), mg));
+                        if (sub == g) {
+                            m = mg;
+                            wm = has ? wg : 0.0f;
+                        }
+                    }
+                    const float x = c < in_channels ? wave_rows[m * in_channels + c] : 1.0f;
+                    acc += wm * x;
+                }
+                if (G >= 4) acc += __shfl_xor(acc, 16);
+                if (G >= 2) acc += __shfl_xor(acc, 32);
+                if (sub == 0 && c < vd) atomicAdd(values + ((unsigned)k * (unsigned)vd + (unsigned)c), acc);
+            }
+        }
+    }
+}
+
 // ------------------------------------------------------------------------------------------------
 // Stage 4: blur along one axis (reference: src/PermutohedralLatticeCPU.h:403-405, evaluated in
 // double and rounded once, as there).  The vertex count is read on the device.  The first blur
@@ -1025,26 +1130,41 @@ __global__ __launch_bounds__(kBlock) void k_slice_point(int d1, PointMap map,
     }
 }
 
-__global__ __launch_bounds__(kBlock) void k_slice_channel(int d1, int vd, PointMap map, size_t T,
+// Any vd: one thread per (point, channel).  The pd+1 replay rows, then the 2(pd+1) values, are
+// all requested before the first is used: with a run-time loop the passes waited for two memory
+// round trips per vertex, one after the other.
+template <int D1>
+__global__ __launch_bounds__(kBlock) void k_slice_channel(int vd, PointMap map, size_t T,
                                                            const ReplayEntry *__restrict__ replay,
                                                            const float *__restrict__ values,
                                                            float *__restrict__ output, int normalize) {
+    // workgroup (x, y): elements y*256 .. y*256+255 of the 256*out_ch (point, channel) pairs of
+    // point block x
     const int out_ch = normalize ? vd - 1 : vd;
-    const size_t g = (size_t)blockIdx.x * kBlock + threadIdx.x;
-    if (g >= T * out_ch) return;
-    const size_t t = g / (size_t)out_ch;
-    const int j = (int)(g - t * out_ch);
-    const int n = point_of_thread(map, (unsigned)(t / kBlock), (unsigned)(t % kBlock));
+    const unsigned element = blockIdx.y * kBlock + threadIdx.x;
+    const unsigned slot = element / (unsigned)out_ch;
+    if (slot >= kBlock) return;
+    const int j = (int)(element - slot * (unsigned)out_ch);
+    const size_t t = (size_t)blockIdx.x * kBlock + slot;
+    const int n = point_of_thread(map, blockIdx.x, slot);
     if (n < 0) return;
+    ReplayEntry e[D1];
+#pragma unroll
+    for (int r = 0; r < D1; ++r) e[r] = replay[(size_t)r * T + t];
+    float own[D1], last[D1];
+#pragma unroll
+    for (int r = 0; r < D1; ++r) {
+        const bool present = e[r].index >= 0;
+        const float *src = values + (size_t)(present ? e[r].index : 0) * vd;
+        own[r] = present ? src[j] : 0.0f;
+        last[r] = present ? src[vd - 1] : 0.0f;
+    }
     float acc = 0.0f, hom = 0.0f;
-    for (int r = 0; r < d1; ++r) {
-        const ReplayEntry e = replay[(size_t)r * T + t];
-        const int v = e.index;
-        if (v < 0) continue;
-        const float w = e.weight;
-        const float *src = values + (size_t)v * vd;
-        acc += w * src[j];
-        hom += w * src[vd - 1];
+#pragma unroll
+    for (int r = 0; r < D1; ++r) {
+        if (e[r].index < 0) continue;
+        acc += e[r].weight * own[r];
+        hom += e[r].weight * last[r];
     }
     const size_t o = (size_t)n * out_ch + j;
     if (normalize) {
@@ -1266,6 +1386,20 @@ hipError_t splat(int pd, int vd, const PointMap &map, const float *input, int in
     switch (vd) {
         PLK_SPLAT_DPP(2) PLK_SPLAT_DPP(3) PLK_SPLAT_DPP(4)
         default:
+            if (in_channels >= 1 && in_channels <= 64) {
+                const size_t lds = sizeof(float) * kBlock * (size_t)in_channels;
+                const dim3 grid2(map.n_blocks, (pd + 2) / 2);
+                if (vd <= 16)
+                    hipLaunchKernelGGL(k_splat_channels<16>, grid2, block, lds, s, pd + 1, vd, map, input,
+                                       in_channels, replay, cell_vertex, values, xcd_aware);
+                else if (vd <= 32)
+                    hipLaunchKernelGGL(k_splat_channels<32>, grid2, block, lds, s, pd + 1, vd, map, input,
+                                       in_channels, replay, cell_vertex, values, xcd_aware);
+                else
+                    hipLaunchKernelGGL(k_splat_channels<64>, grid2, block, lds, s, pd + 1, vd, map, input,
+                                       in_channels, replay, cell_vertex, values, xcd_aware);
+                break;
+            }
             PLK_DISPATCH_PD(pd, hipLaunchKernelGGL(k_splat_dpp_blocks<PD + 1>, grid, block, 0, s, vd,
                                                    map, input, in_channels, replay,
                                                    cell_vertex, values, xcd_aware));
@@ -1337,8 +1471,9 @@ hipError_t slice(int pd, int vd, const PointMap &map, const ReplayEntry *replay,
         PLK_SLICE(2) PLK_SLICE(3) PLK_SLICE(4) PLK_SLICE(5) PLK_SLICE(6) PLK_SLICE(7) PLK_SLICE(8)
         default: {
             const int out_ch = normalize ? vd - 1 : vd;
-            hipLaunchKernelGGL(k_slice_channel, dim3(blocks_for(T * out_ch)), block, 0, s, d1, vd, map,
-                               T, replay, values, output, normalize);
+            PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_slice_channel<PD + 1>),
+                                                   dim3(map.n_blocks, out_ch), block, 0, s, vd, map,
+                                                   T, replay, values, output, normalize));
         } break;
     }
 #undef PLK_SLICE
