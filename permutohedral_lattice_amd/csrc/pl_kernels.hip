@@ -1130,49 +1130,51 @@ __global__ __launch_bounds__(kBlock) void k_slice_point(int d1, PointMap map,
     }
 }
 
-// Any vd: one thread per (point, channel).  The pd+1 replay rows, then the 2(pd+1) values, are
-// all requested before the first is used: with a run-time loop the passes waited for two memory
-// round trips per vertex, one after the other.
+// Any vd: one thread per point and run of four channels.  The pd+1 replay rows, then the value
+// rows, are all requested before the first is used (with a run-time loop the passes waited for
+// two memory round trips per vertex, one after the other); four channels share the index
+// arithmetic and the replay loads.
 template <int D1>
-__global__ __launch_bounds__(kBlock) void k_slice_channel(int vd, PointMap map, size_t T,
-                                                           const ReplayEntry *__restrict__ replay,
-                                                           const float *__restrict__ values,
-                                                           float *__restrict__ output, int normalize) {
-    // workgroup (x, y): elements y*256 .. y*256+255 of the 256*out_ch (point, channel) pairs of
-    // point block x
+__global__ __launch_bounds__(kBlock) void k_slice_channels(int vd, PointMap map, size_t T,
+                                                            const ReplayEntry *__restrict__ replay,
+                                                            const float *__restrict__ values,
+                                                            float *__restrict__ output, int normalize) {
+    // workgroup (x, y): items y*256 .. y*256+255 of the 256*runs (point, run of channels) pairs
+    // of point block x
     const int out_ch = normalize ? vd - 1 : vd;
-    const unsigned element = blockIdx.y * kBlock + threadIdx.x;
-    const unsigned slot = element / (unsigned)out_ch;
+    const unsigned runs = (unsigned)(out_ch + 3) / 4u;
+    const unsigned item = blockIdx.y * kBlock + threadIdx.x;
+    const unsigned slot = item / runs;
     if (slot >= kBlock) return;
-    const int j = (int)(element - slot * (unsigned)out_ch);
+    const int j0 = 4 * (int)(item - slot * runs);
     const size_t t = (size_t)blockIdx.x * kBlock + slot;
     const int n = point_of_thread(map, blockIdx.x, slot);
     if (n < 0) return;
     ReplayEntry e[D1];
 #pragma unroll
     for (int r = 0; r < D1; ++r) e[r] = replay[(size_t)r * T + t];
-    float own[D1], last[D1];
+    float own[D1][4], last[D1];
 #pragma unroll
     for (int r = 0; r < D1; ++r) {
         const bool present = e[r].index >= 0;
         const float *src = values + (size_t)(present ? e[r].index : 0) * vd;
-        own[r] = present ? src[j] : 0.0f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) own[r][i] = (present && j0 + i < out_ch) ? src[j0 + i] : 0.0f;
         last[r] = present ? src[vd - 1] : 0.0f;
     }
-    float acc = 0.0f, hom = 0.0f;
+    float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f}, hom = 0.0f;
 #pragma unroll
     for (int r = 0; r < D1; ++r) {
         if (e[r].index < 0) continue;
-        acc += e[r].weight * own[r];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i] += e[r].weight * own[r][i];
         hom += e[r].weight * last[r];
     }
-    const size_t o = (size_t)n * out_ch + j;
-    if (normalize) {
-        const float scale = (float)(1.0 / (double)hom);
-        output[o] = acc * scale;
-    } else {
-        output[o] = acc;
-    }
+    const float scale = normalize ? (float)(1.0 / (double)hom) : 1.0f;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        if (j0 + i < out_ch)
+            output[(size_t)n * out_ch + j0 + i] = normalize ? acc[i] * scale : acc[i];
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -1471,9 +1473,9 @@ hipError_t slice(int pd, int vd, const PointMap &map, const ReplayEntry *replay,
         PLK_SLICE(2) PLK_SLICE(3) PLK_SLICE(4) PLK_SLICE(5) PLK_SLICE(6) PLK_SLICE(7) PLK_SLICE(8)
         default: {
             const int out_ch = normalize ? vd - 1 : vd;
-            PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_slice_channel<PD + 1>),
-                                                   dim3(map.n_blocks, out_ch), block, 0, s, vd, map,
-                                                   T, replay, values, output, normalize));
+            PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_slice_channels<PD + 1>),
+                                                   dim3(map.n_blocks, (out_ch + 3) / 4), block, 0, s,
+                                                   vd, map, T, replay, values, output, normalize));
         } break;
     }
 #undef PLK_SLICE
