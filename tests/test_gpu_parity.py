@@ -262,6 +262,44 @@ def test_two_axes_per_launch_is_bit_identical_to_one(pd, vd):
         assert_float_parity(results[(1, reverse)], oracle.Lattice(pd, vd, n).filter(val, pos, reverse))
 
 
+@pytest.mark.parametrize("pd,vd,shape", [(2, 6, (96, 70)), (3, 13, (40, 30, 20)), (2, 17, (70, 90)),
+                                         (5, 33, (64, 48)), (2, 40, (50, 60)), (3, 70, (3000,)),
+                                         (8, 5, (2500,))])
+def test_many_channels(pd, vd, shape):
+    """The kernels for more than four channels: 16, 32 and 64 lanes per member in the splat,
+    input rows beyond 64 channels, odd and even row lengths in the slice; filter and apply, with
+    and without a grid hint, normalised and as the bare linear operator."""
+    n = int(np.prod(shape))
+    rng = np.random.default_rng(pd * 1000 + vd)
+    # smooth positions over the grid plus noise, so that wavefronts see groups of several sizes
+    grid = np.stack(np.meshgrid(*[np.arange(s, dtype=np.float32) for s in shape], indexing="ij"), -1)
+    pos = np.concatenate([grid.reshape(n, -1) / (np.asarray(shape, np.float32) / 12.0),
+                          rng.uniform(0, 2.5, (n, pd)).astype(np.float32)], axis=1)[:, :pd]
+    pos = np.ascontiguousarray(pos, np.float32)
+    val = rng.uniform(0, 1, (n, vd - 1)).astype(np.float32)
+    want = {rev: oracle.Lattice(pd, vd, n).filter(val, pos, rev) for rev in (False, True)}
+    for hint in (None, shape if len(shape) > 1 else None):
+        lat = pla.PermutohedralLattice(pd, vd, n)
+        if hint:
+            lat.set_point_grid(hint)
+        got, _ = gpu_filter(pd, vd, pos, val, False, lattice=lat)
+        assert_float_parity(got, want[False])
+        out = torch.empty((n, vd - 1), dtype=torch.float32, device="cuda")
+        lat.apply(out, dev(val), True)
+        torch.cuda.synchronize()
+        assert_float_parity(host(out), want[True])
+    # bare operator: vd channels in and out, nothing divided; equals the oracle's raw filter
+    lat = pla.PermutohedralLattice(pd, vd, n)
+    lat.set_option(pla.PL_OPT_NORMALIZE, 0)
+    raw_in = rng.uniform(0, 1, (n, vd)).astype(np.float32)
+    out = torch.empty((n, vd), dtype=torch.float32, device="cuda")
+    lat.filter(out, dev(raw_in), dev(pos), False)
+    torch.cuda.synchronize()
+    want_raw = oracle.Lattice(pd, vd, n).filter_raw(raw_in, pos, False)
+    assert np.abs(host(out) - want_raw).max() <= MAX_ABS_TOL * max(1.0, float(np.abs(want_raw).max()))
+    assert rel_l2(host(out), want_raw) <= REL_L2_TOL
+
+
 def test_apply_before_build_is_an_error():
     lat = pla.PermutohedralLattice(2, 2, 16)
     x = torch.zeros((16, 1), device="cuda")
