@@ -93,6 +93,8 @@ int pl_filter(pl_handle h, float *output, const float *input, const float *posit
  * table) once; pl_apply then runs splat, blur, slice for any number of inputs, forward or reverse,
  * under those positions.  The reference rebuilds for every call
  * (src/LatticeFilterKernel.cpp:79, src/LatticeFilterKernel.cu:88); results are the same.
+ * pl_apply only launches kernels on the lattice's stream (no allocation, no wait, no memset):
+ * after the first pl_apply that follows a build, further ones may be captured in a HIP graph.
  */
 int pl_build(pl_handle h, const float *positions);
 int pl_apply(pl_handle h, float *output, const float *input, int reverse);
