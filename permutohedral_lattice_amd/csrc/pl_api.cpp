@@ -2,8 +2,8 @@
 // scratch memory, the build/apply orchestration and the LatticeFilter op loop.
 //
 // A filter call enqueues its kernels back to back: the vertex count of the lattice stays on the
-// device (every later kernel reads it there, launched for an upper bound of vertices), so the
-// host waits once, at the end, to learn whether the hash table was large enough.
+// device (every later kernel reads it there and is launched for an estimate of it), so the host
+// waits once, at the end, to learn whether the hash table was large enough.
 #include "permutohedral_lattice.h"
 
 #include <hip/hip_runtime.h>
@@ -117,7 +117,6 @@ struct pl_lattice {
         float *output = nullptr;
         const float *input = nullptr;
         int reverse = 0;
-        uint32_t cells = 0;
     } pending;
 
     void *dmalloc(size_t bytes) { return alloc.alloc(alloc.ctx, bytes); }
