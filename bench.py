@@ -274,7 +274,7 @@ def main():
         ref = oracle.reference()
         cores = 1
         times, outs = [], None
-        reps = 3 if n >= (1 << 20) else 5
+        reps = 9 if n >= (1 << 20) else 15
         for rep in range(reps + 1):  # first repetition is the warm-up
             t0 = time.perf_counter()
             if ref is not None:
