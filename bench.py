@@ -90,8 +90,19 @@ def run_side_legs(args, pla, synth, lat, step, img, d_pos, d_val, d_grad, out_f,
         for o, v, rev in ((out_f, d_val, False), (out_r, d_grad, True)):
             lat.filter_image(o, v, d_img, (side, side), 8.0, 0.125, rev)
 
+    # through the autograd function: backward applies the lattices forward built
+    x4 = d_val.view(1, side, side, 3).clone().requires_grad_(True)
+    ref4 = d_img.view(1, side, side, 3)
+    up4 = d_grad.view(1, side, side, 3)
+
+    def op_step_autograd():
+        y = pla.lattice_filter(x4, ref4, theta_alpha=8.0, theta_beta=0.125)
+        y.backward(up4)
+        x4.grad = None
+
     op_ms = {}
-    for name, fn in (("positions_then_filter", op_step_two_kernels), ("features_on_the_fly", op_step_fused)):
+    for name, fn in (("positions_then_filter", op_step_two_kernels), ("features_on_the_fly", op_step_fused),
+                     ("autograd_forward_backward", op_step_autograd)):
         for _ in range(2):
             fn()
         torch.cuda.synchronize()
@@ -258,7 +269,8 @@ def main():
                       "ms_per_step": round(reuse_ms, 4),
                       "value": round(pixels_per_step / (reuse_ms * 1e-3) / 1e6, 3)},
             "op_level": {"what": "reference image in, forward + reverse per step: feature kernel + "
-                                 "filter(), and filter_image() (features built inside the first kernel)",
+                                 "filter(), filter_image() (features built inside the first kernel), and "
+                                 "lattice_filter(...).backward(...) (backward applies forward's lattice)",
                          "ms_per_step": {k: round(v, 4) for k, v in op_ms.items()},
                          "value": {k: round(pixels_per_step / (v * 1e-3) / 1e6, 3)
                                    for k, v in op_ms.items()}},

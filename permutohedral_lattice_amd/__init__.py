@@ -284,14 +284,99 @@ def _lattice_filter_raw(input_image, reference_image, bilateral, theta_alpha, th
     return out
 
 
+class _LatticePool:
+    """Lattices kept between calls, so that the forward and the backward pass of one op call can
+    share what the forward pass built: the positions are the same, only the blur order differs
+    (the reference rebuilds the lattice in the backward pass, src/LatticeFilterKernel.cpp:79)."""
+
+    def __init__(self, max_idle_per_shape=4, max_lent=16):
+        self.idle, self.lent = {}, 0
+        self.max_idle_per_shape, self.max_lent = max_idle_per_shape, max_lent
+
+    @staticmethod
+    def _key(pd, vd, n, stream):
+        return (torch.cuda.current_device(), pd, vd, n, stream.cuda_stream)
+
+    def acquire(self, pd, vd, n, count):
+        """``count`` lattices for the current stream, or None when too many are lent out."""
+        if self.lent + count > self.max_lent:
+            return None
+        stream = torch.cuda.current_stream()
+        idle = self.idle.setdefault(self._key(pd, vd, n, stream), [])
+        lattices = [idle.pop() if idle else PermutohedralLattice(pd, vd, n, stream=stream)
+                    for _ in range(count)]
+        self.lent += count
+        return _LentLattices(self, lattices, self._key(pd, vd, n, stream))
+
+    def give_back(self, lattices, key):
+        self.lent -= len(lattices)
+        idle = self.idle.setdefault(key, [])
+        for lat in lattices:
+            if len(idle) < self.max_idle_per_shape:
+                idle.append(lat)
+            else:
+                lat.close()
+
+
+class _LentLattices:
+    """Returns its lattices to the pool when the autograd graph lets go of it."""
+
+    def __init__(self, pool, lattices, key):
+        self.pool, self.lattices, self.key = pool, lattices, key
+
+    def __del__(self):
+        if self.lattices is not None:
+            self.pool.give_back(self.lattices, self.key)
+            self.lattices = None
+
+
+_pool = _LatticePool()
+
+
 class _LatticeFilterFunction(torch.autograd.Function):
     @staticmethod
     def forward(ctx, input_image, reference_image, bilateral, theta_alpha, theta_beta, theta_gamma,
                 reverse):
         ctx.save_for_backward(reference_image)
         ctx.attrs = (bilateral, theta_alpha, theta_beta, theta_gamma)
+        ctx.lent = None
+        if ctx.needs_input_grad[0] and input_image.dim() >= 3 and input_image.shape[0] > 0:
+            out = _LatticeFilterFunction._forward_keeping_lattices(
+                ctx, input_image, reference_image, bilateral, theta_alpha, theta_beta, theta_gamma,
+                reverse)
+            if out is not None:
+                return out
         return _lattice_filter_raw(input_image, reference_image, bilateral, theta_alpha, theta_beta,
                                    theta_gamma, reverse)
+
+    @staticmethod
+    def _forward_keeping_lattices(ctx, input_image, reference_image, bilateral, theta_alpha,
+                                  theta_beta, theta_gamma, reverse):
+        """One lattice per batch item, built here and applied again (reversed) in backward."""
+        inp = input_image.contiguous()
+        sd = [int(s) for s in inp.shape[1:-1]]
+        n = 1
+        for s in sd:
+            n *= s
+        rc = int(reference_image.shape[-1]) if (bilateral and reference_image is not None) else 0
+        pd, vd = len(sd) + rc, int(inp.shape[-1]) + 1
+        if bilateral and (reference_image is None or rc < 1 or
+                          list(reference_image.shape[:-1]) != list(inp.shape[:-1])):
+            return None         # let the op report it
+        if not supported(pd, vd) or n == 0:
+            return None
+        lent = _pool.acquire(pd, vd, n, int(inp.shape[0]))
+        if lent is None:
+            return None
+        ref = reference_image.contiguous() if rc else None
+        out = torch.empty_like(inp)
+        spatial_std = theta_alpha if bilateral else theta_gamma
+        for b, lat in enumerate(lent.lattices):
+            lat.filter_image(out[b].view(n, vd - 1), inp[b].view(n, vd - 1),
+                             ref[b].view(n, rc) if rc else None, sd, spatial_std,
+                             theta_beta if bilateral else 1.0, reverse)
+        ctx.lent = lent
+        return out
 
     @staticmethod
     def backward(ctx, grad):
@@ -299,8 +384,16 @@ class _LatticeFilterFunction(torch.autograd.Function):
         # reverse=True, and zeros for the reference image (lattice_filter_op_loader.py:46-54)
         (reference_image,) = ctx.saved_tensors
         bilateral, theta_alpha, theta_beta, theta_gamma = ctx.attrs
-        grad_vals = _lattice_filter_raw(grad, reference_image, bilateral, theta_alpha, theta_beta,
-                                        theta_gamma, True)
+        lent = ctx.lent
+        if lent is not None and lent.lattices is not None and \
+                lent.key[-1] == torch.cuda.current_stream().cuda_stream:
+            g = grad.contiguous()
+            grad_vals = torch.empty_like(g)
+            for b, lat in enumerate(lent.lattices):
+                lat.apply(grad_vals[b].view(lat.N, lat.vd - 1), g[b].view(lat.N, lat.vd - 1), True)
+        else:
+            grad_vals = _lattice_filter_raw(grad, reference_image, bilateral, theta_alpha,
+                                            theta_beta, theta_gamma, True)
         grad_ref = torch.zeros_like(reference_image) if ctx.needs_input_grad[1] else None
         return grad_vals, grad_ref, None, None, None, None, None
 

@@ -157,3 +157,43 @@ def test_apply_can_be_captured_in_a_graph_and_replayed():
             lat.apply(eager, static_in, True)
         s.synchronize()
         close(eager.cpu().numpy(), oracle.Lattice(5, vd, n).filter(val, pos, True))
+
+
+def test_backward_reuses_the_lattices_of_forward():
+    """With an input that needs a gradient the op keeps the lattices it built: backward is then a
+    reversed apply under the same positions.  Same numbers as the op called twice; the lattices go
+    back to the pool when the graph is freed, and past the pool's limit the op rebuilds."""
+    import gc
+    b, h, w = 3, 80, 72
+    guide = np.stack([synth.blob_image(h, w, seed=70 + i) for i in range(b)])
+    inp = synth.uniform_image((b, h, w, 2), 73)
+    up = synth.normal_image(inp.shape, 74)
+    want = oracle.lattice_filter(inp, guide, True, 8.0, 0.125, 1.0, False)
+    want_grad = oracle.lattice_filter(up, guide, True, 8.0, 0.125, 1.0, True)
+    d_guide = dev(guide)
+    pool = pla._pool
+    gc.collect()
+    assert pool.lent == 0
+    x = dev(inp).requires_grad_(True)
+    y = pla.lattice_filter(x, d_guide, theta_alpha=8.0, theta_beta=0.125)
+    assert pool.lent == b
+    close(y.detach().cpu().numpy(), want)
+    y.backward(dev(up), retain_graph=True)
+    first = x.grad.clone()
+    close(first.cpu().numpy(), want_grad, scale=float(np.abs(want_grad).max()))
+    x.grad = None
+    y.backward(dev(up))                      # a second backward over the retained graph
+    close(x.grad.cpu().numpy(), want_grad, scale=float(np.abs(want_grad).max()))
+    del y
+    gc.collect()
+    assert pool.lent == 0
+    # more outputs alive than the pool lends lattices for: the rest are computed by the plain op
+    alive = [pla.lattice_filter(dev(inp).requires_grad_(True), d_guide, theta_alpha=8.0, theta_beta=0.125)
+             for _ in range(pool.max_lent // b + 2)]
+    assert pool.lent <= pool.max_lent
+    for y in alive:
+        close(y.detach().cpu().numpy(), want)
+    alive[-1].backward(dev(up))
+    del alive, y
+    gc.collect()
+    assert pool.lent == 0
