@@ -55,8 +55,12 @@ typedef enum pl_option {
     PL_OPT_TABLE_CELLS = 3, /* force the initial number of hash cells (power of two), 0 = automatic */
     PL_OPT_XCD_AWARE = 4,   /* 1 (default): kernels with atomic updates give each XCD a contiguous range
                                of points; 0: plain workgroup order (for measuring the difference) */
-    PL_OPT_PAIR_BLUR = 5    /* 1 (default): two blur axes per kernel launch; 0: one launch per axis
+    PL_OPT_PAIR_BLUR = 5,   /* 1 (default): two blur axes per kernel launch; 0: one launch per axis
                                (same results bit for bit; for measuring the difference) */
+    PL_OPT_GUESS_GRID = 6   /* 1 (default): a handle without pl_set_point_grid looks, the first time it
+                               sees positions, whether they describe a row-major image or volume (feature
+                               0 changing exactly every row length points ...) and if so orders its
+                               work as with the hint; 0: never (points are a plain list) */
 } pl_option;
 
 /* 1 when a lattice can be built for these dimensions, else 0.
@@ -107,6 +111,11 @@ int pl_apply(pl_handle h, float *output, const float *input, int reverse);
  * n_dims = 0 removes it.  pl_lattice_filter_op sets it by itself.
  */
 int pl_set_point_grid(pl_handle h, int n_dims, const int *dims);
+
+/* The grid the handle currently orders its work by: *n_dims = 0 (none), 2 or 3, extents in dims
+ * (leading extents of a longer hint folded into the first).  Given by pl_set_point_grid, by the
+ * *_image entry points, or found in the positions (PL_OPT_GUESS_GRID). */
+int pl_get_point_grid(pl_handle h, int *n_dims, int dims[3]);
 
 /* Number of lattice vertices of the last build (HashTableCPU::size(), src/PermutohedralLatticeCPU.h:151). */
 int pl_num_vertices(pl_handle h, int *num_vertices);

@@ -21,11 +21,12 @@ LIB_PATH = os.path.join(_HERE, "libpermutohedral_hip.so")
 
 PL_OK, PL_EINVAL, PL_EUNSUPPORTED, PL_ENOMEM, PL_EOVERFLOW, PL_EHIP, PL_ESTATE = 0, -1, -2, -3, -4, -5, -6
 PL_OPT_NORMALIZE, PL_OPT_PROFILE, PL_OPT_TABLE_CELLS, PL_OPT_XCD_AWARE, PL_OPT_PAIR_BLUR = 1, 2, 3, 4, 5
+PL_OPT_GUESS_GRID = 6
 
 # every symbol include/permutohedral_lattice.h declares
 EXPORTS = (
     "pl_supported", "pl_strerror", "pl_last_hip_error", "pl_create", "pl_destroy", "pl_filter",
-    "pl_build", "pl_apply", "pl_set_point_grid", "pl_num_vertices", "pl_set_option", "pl_stage_ms", "pl_debug_simplex",
+    "pl_build", "pl_apply", "pl_set_point_grid", "pl_get_point_grid", "pl_num_vertices", "pl_set_option", "pl_stage_ms", "pl_debug_simplex",
     "pl_debug_keys", "pl_debug_replay", "pl_compute_positions", "pl_filter_image", "pl_build_image",
     "pl_filter_begin", "pl_filter_image_begin", "pl_filter_end", "pl_lattice_filter_op",
     "pl_set_op_concurrency",
@@ -61,6 +62,7 @@ def _load():
     lib.pl_build.argtypes = [vp, vp]
     lib.pl_apply.argtypes = [vp, vp, vp, ci]
     lib.pl_set_point_grid.argtypes = [vp, ci, C.POINTER(ci)]
+    lib.pl_get_point_grid.argtypes = [vp, C.POINTER(ci), C.POINTER(ci)]
     lib.pl_num_vertices.argtypes = [vp, C.POINTER(ci)]
     lib.pl_set_option.argtypes = [vp, ci, C.c_long]
     lib.pl_stage_ms.argtypes = [vp, C.POINTER(cf)]
@@ -187,6 +189,13 @@ class PermutohedralLattice:
         dims = [int(d) for d in (dims or [])]
         arr = (C.c_int * max(1, len(dims)))(*dims)
         _check(_lib.pl_set_point_grid(self._h, len(dims), arr), "pl_set_point_grid")
+
+    @property
+    def point_grid(self):
+        """Extents of the grid the work is ordered by (given, or found in the positions); () if none."""
+        n, dims = C.c_int(), (C.c_int * 3)()
+        _check(_lib.pl_get_point_grid(self._h, C.byref(n), dims), "pl_get_point_grid")
+        return tuple(dims[i] for i in range(n.value))
 
     @property
     def num_vertices(self):

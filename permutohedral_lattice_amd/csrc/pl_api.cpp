@@ -107,6 +107,12 @@ struct pl_lattice {
     bool profile = false;
     bool xcd_aware = true;
     bool pair_blur = true;
+    // the grid the points form: given by the caller (pl_set_point_grid), or guessed once from the
+    // first positions the handle sees
+    bool grid_given = false;
+    bool guess_grid = true;
+    bool grid_guessed = false;             // a guess has been made (whatever came out)
+    plk::GridGuess *d_guess = nullptr;
     hipEvent_t ev[EV_COUNT] = {};
     bool ev_recorded[EV_COUNT] = {};
 
@@ -420,6 +426,7 @@ int pl_destroy(pl_handle h) {
     h->dfree(h->block_count);
     h->dfree(h->chunk_count);
     h->dfree(h->d_counters);
+    h->dfree(h->d_guess);
     if (h->h_status) (void)hipHostFree(h->h_status);
     for (int i = 0; i < EV_COUNT; ++i)
         if (h->ev[i]) (void)hipEventDestroy(h->ev[i]);
@@ -445,6 +452,9 @@ int pl_set_option(pl_handle h, int option, long value) {
         case PL_OPT_PAIR_BLUR:
             h->pair_blur = value != 0;
             return PL_OK;
+        case PL_OPT_GUESS_GRID:
+            h->guess_grid = value != 0;
+            return PL_OK;
         case PL_OPT_TABLE_CELLS:
             if (value < 0 || (value & (value - 1)) != 0) return PL_EINVAL;
             h->forced_cells = value;
@@ -468,8 +478,22 @@ int pl_set_point_grid(pl_handle h, int n_dims, const int *dims) {
         if (prod != (long long)h->N) return PL_EINVAL;
     }
     h->built = false;
+    h->grid_given = n_dims > 0;
     h->map = plk::make_point_map(h->N, n_dims, dims);
     return ensure_replay(h);
+}
+
+int pl_get_point_grid(pl_handle h, int *n_dims, int dims[3]) {
+    if (!h || !n_dims || !dims) return PL_EINVAL;
+    *n_dims = h->map.mode == 0 ? 0 : h->map.mode;
+    for (int i = 0; i < 3; ++i) dims[i] = 0;
+    if (h->map.mode == 2) {
+        dims[0] = h->map.dims[1];
+        dims[1] = h->map.dims[2];
+    } else if (h->map.mode == 3) {
+        for (int i = 0; i < 3; ++i) dims[i] = h->map.dims[i];
+    }
+    return PL_OK;
 }
 
 namespace {
@@ -478,6 +502,43 @@ plk::PointFeatures features_from_positions(const float *positions) {
     plk::PointFeatures f{};
     f.positions = positions;
     return f;
+}
+
+// A caller of filter(output, input, positions, reverse) has no way to say that its points are the
+// pixels of an image, but positions made by the reference's feature builder show it: the first
+// time a handle without a grid hint sees positions, two small kernels look for the row length
+// (and the slice size of a volume) and, if the points turn out to be a row-major grid, the
+// workgroups take tiles of it as with pl_set_point_grid.  One stream synchronisation, once per
+// handle; what is found only orders the work.
+int guess_point_grid(pl_lattice *h, const float *positions) {
+    if (h->grid_given || !h->guess_grid || h->grid_guessed || h->N < 4096) return PL_OK;
+    h->grid_guessed = true;
+    if (!h->d_guess) {
+        h->d_guess = (plk::GridGuess *)h->dmalloc(sizeof(plk::GridGuess));
+        if (!h->d_guess) return PL_ENOMEM;
+    }
+    plk::GridGuess guess{{h->N, h->N}, 0};
+    PL_HIP(hipMemcpyAsync(h->d_guess, &guess, sizeof(guess), hipMemcpyHostToDevice, h->stream));
+    PL_HIP(plk::guess_grid(positions, h->N, h->pd, h->d_guess, h->stream));
+    PL_HIP(hipMemcpyAsync(&guess, h->d_guess, sizeof(guess), hipMemcpyDeviceToHost, h->stream));
+    PL_HIP(hipStreamSynchronize(h->stream));
+    const int p0 = guess.period[0], p1 = h->pd >= 2 ? guess.period[1] : 1;
+    if (guess.mismatch || p0 < 8 || p0 >= h->N || h->N % p0 != 0) return PL_OK;
+    int dims[3], n_dims;
+    if (p1 == 1) {                      // feature 1 changes with every point: an image
+        n_dims = 2;
+        dims[0] = h->N / p0;
+        dims[1] = p0;
+    } else {                            // feature 1 changes every p1 points: a volume
+        if (p1 < 4 || p0 % p1 != 0 || p0 / p1 < 2) return PL_OK;
+        n_dims = 3;
+        dims[0] = h->N / p0;
+        dims[1] = p0 / p1;
+        dims[2] = p1;
+    }
+    if (dims[0] < 2) return PL_OK;
+    h->map = plk::make_point_map(h->N, n_dims, dims);
+    return ensure_replay(h);
 }
 
 // Checks the arguments of the *_image entry points, sets the grid hint and describes the features.
@@ -579,6 +640,8 @@ int filter_lattice(pl_lattice *h, float *output, const float *input,
 int pl_build(pl_handle h, const float *positions) {
     if (!h || (!positions && h->N > 0)) return PL_EINVAL;
     if (h->pending.active) return PL_ESTATE;
+    const int rc = guess_point_grid(h, positions);
+    if (rc != PL_OK) return rc;
     return build_lattice(h, features_from_positions(positions));
 }
 
@@ -604,6 +667,9 @@ int pl_apply(pl_handle h, float *output, const float *input, int reverse) {
 int pl_filter(pl_handle h, float *output, const float *input, const float *positions, int reverse) {
     if (!h) return PL_EINVAL;
     if (h->N > 0 && (!output || !input || !positions)) return PL_EINVAL;
+    if (h->pending.active) return PL_ESTATE;
+    const int rc = guess_point_grid(h, positions);
+    if (rc != PL_OK) return rc;
     return filter_lattice(h, output, input, features_from_positions(positions), reverse);
 }
 
@@ -623,6 +689,9 @@ int pl_filter_begin(pl_handle h, float *output, const float *input, const float 
                     int reverse) {
     if (!h) return PL_EINVAL;
     if (h->N > 0 && (!output || !input || !positions)) return PL_EINVAL;
+    if (h->pending.active) return PL_ESTATE;
+    const int rc = guess_point_grid(h, positions);
+    if (rc != PL_OK) return rc;
     return filter_begin(h, output, input, features_from_positions(positions), reverse);
 }
 

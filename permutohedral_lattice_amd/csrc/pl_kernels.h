@@ -173,6 +173,15 @@ hipError_t export_replay(int pd, const PointMap &map, const ReplayEntry *replay,
                          const int *cell_vertex, int *vertex,
                          float *weight, hipStream_t s);
 
+// First index at which feature 0 (period[0]) and feature 1 (period[1]) of consecutive points
+// differ, and whether all their changes lie exactly at the multiples of those indices.
+// *guess must be {N, N}, 0 before the call.
+struct GridGuess {
+    int period[2];
+    int mismatch;
+};
+hipError_t guess_grid(const float *positions, int N, int pd, GridGuess *guess, hipStream_t s);
+
 hipError_t compute_positions(const float *reference, float *positions, int N, int n_ref_channels,
                              int n_spatial_dims, const SpatialDims &dims, float spatial_std,
                              float feature_std, hipStream_t s);

@@ -1254,6 +1254,32 @@ __global__ __launch_bounds__(kBlock) void k_export_replay(int d1, PointMap map,
     }
 }
 
+// Is the list of points a row-major grid?  The feature builder of the reference puts the grid
+// coordinates first (src/PermutohedralLatticeCPU.h:464-469), so in positions that describe an
+// image feature 0 changes exactly every row length points, and feature 1 (the next slower
+// coordinate of a volume) every P1 points.  Pass 1 finds the first change of each, pass 2 checks
+// that the changes are exactly at the multiples of those periods.  The result only chooses the
+// order in which points are worked on, so a wrong guess costs time, never correctness.
+__global__ __launch_bounds__(kBlock) void k_first_changes(const float *__restrict__ positions, int N,
+                                                           int pd, GridGuess *guess) {
+    const int n = blockIdx.x * kBlock + threadIdx.x + 1;
+    if (n >= N) return;
+    const float *row = positions + (size_t)n * pd;
+    if (row[0] != row[0 - pd]) atomicMin(&guess->period[0], n);
+    if (pd >= 2 && row[1] != row[1 - pd]) atomicMin(&guess->period[1], n);
+}
+
+__global__ __launch_bounds__(kBlock) void k_check_periods(const float *__restrict__ positions, int N,
+                                                           int pd, GridGuess *guess) {
+    const int n = blockIdx.x * kBlock + threadIdx.x + 1;
+    if (n >= N) return;
+    const int p0 = guess->period[0], p1 = pd >= 2 ? guess->period[1] : 1;
+    const float *row = positions + (size_t)n * pd;
+    bool bad = (row[0] != row[0 - pd]) != (n % p0 == 0);
+    if (pd >= 2) bad = bad || ((row[1] != row[1 - pd]) != (n % p1 == 0));
+    if (bad) guess->mismatch = 1;
+}
+
 // reference: src/PermutohedralLatticeCPU.h:464-473 (IEEE float division, int -> float exact)
 __global__ __launch_bounds__(kBlock) void k_positions(const float *__restrict__ reference,
                                                        float *__restrict__ positions, int N, int rc,
@@ -1517,6 +1543,16 @@ hipError_t export_replay(int pd, const PointMap &map, const ReplayEntry *replay,
     if (map.n_blocks == 0) return hipSuccess;
     hipLaunchKernelGGL(k_export_replay, dim3(map.n_blocks), dim3(kBlock), 0, s, pd + 1, map,
                        replay, cell_vertex, vertex, weight);
+    return hipGetLastError();
+}
+
+hipError_t guess_grid(const float *positions, int N, int pd, GridGuess *guess, hipStream_t s) {
+    if (N < 2) return hipErrorInvalidValue;
+    // *guess must hold {N, N} and 0 (set by the caller)
+    hipLaunchKernelGGL(k_first_changes, dim3(blocks_for((size_t)N - 1)), dim3(kBlock), 0, s, positions,
+                       N, pd, guess);
+    hipLaunchKernelGGL(k_check_periods, dim3(blocks_for((size_t)N - 1)), dim3(kBlock), 0, s, positions,
+                       N, pd, guess);
     return hipGetLastError();
 }
 

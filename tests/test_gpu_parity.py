@@ -526,3 +526,60 @@ def test_reference_image_fixtures():
     diff = np.abs(q - im["filtered_grey"].astype(np.int64))
     assert diff.max() <= 1
     assert (diff != 0).mean() <= 1e-3
+
+
+# ---------------------------------------------------------------------------------------------
+# grid found in the positions
+# ---------------------------------------------------------------------------------------------
+
+@pytest.mark.parametrize("case", ["image", "image_ragged", "volume", "spatial_only", "scattered",
+                                  "image_with_repeated_row", "guessing_off"])
+def test_grid_is_found_in_positions_of_images_and_volumes(case):
+    """A handle that was given no grid recognises positions made by the feature builder (feature
+    0 changes exactly every row, feature 1 every point or every line of a volume) and orders its
+    work by tiles; anything else stays a plain list.  Results never depend on it."""
+    rng = np.random.default_rng(5)
+    if case in ("image", "guessing_off"):
+        img = synth.blob_image(96, 128, seed=81)
+        pd, vd, pos, val, want_grid = 5, 4, synth.bilateral_positions(img, 8.0, 0.125), img.reshape(-1, 3), (96, 128)
+    elif case == "image_ragged":
+        img = synth.blob_image(71, 103, seed=82)
+        pd, vd, pos, val, want_grid = 5, 4, synth.bilateral_positions(img, 5.0, 0.2), img.reshape(-1, 3), (71, 103)
+    elif case == "volume":
+        vol = synth.ellipsoid_volume(12, 24, 36, seed=83)
+        pd, vd, pos, val, want_grid = 4, 2, synth.bilateral_positions(vol, 5.0, 0.1), vol.reshape(-1, 1), (12, 24, 36)
+    elif case == "spatial_only":
+        pd, vd, pos, want_grid = 2, 3, synth.spatial_positions((80, 64), 3.0), (80, 64)
+        val = synth.uniform_image((80 * 64, 2), 84)
+    elif case == "scattered":
+        pd, vd, want_grid = 3, 3, ()
+        pos = rng.uniform(0, 9, (6000, 3)).astype(np.float32)
+        val = rng.uniform(0, 1, (6000, 2)).astype(np.float32)
+    else:   # two rows share their first feature: not the positions of an image
+        img = synth.blob_image(64, 96, seed=85)
+        pd, vd, val, want_grid = 5, 4, img.reshape(-1, 3), ()
+        pos = synth.bilateral_positions(img, 8.0, 0.125).copy()
+        pos.reshape(64, 96, 5)[17, :, 0] = pos.reshape(64, 96, 5)[16, 0, 0]
+    n = pos.shape[0]
+    lat = pla.PermutohedralLattice(pd, vd, n)
+    if case == "guessing_off":
+        lat.set_option(pla.PL_OPT_GUESS_GRID, 0)
+        want_grid = ()
+    assert lat.point_grid == ()
+    got, _ = gpu_filter(pd, vd, pos, val, False, lattice=lat)
+    assert lat.point_grid == want_grid
+    cpu = oracle.Lattice(pd, vd, n)
+    want = cpu.filter(val, pos, False)
+    assert_float_parity(got, want)
+    assert lat.num_vertices == cpu.num_vertices
+    got_r, _ = gpu_filter(pd, vd, pos, val, True, lattice=lat)
+    assert_float_parity(got_r, oracle.Lattice(pd, vd, n).filter(val, pos, True))
+    # an explicit hint replaces what was found, its removal leaves a plain list
+    if len(want_grid) == 2:
+        lat.set_point_grid(want_grid)
+        assert lat.point_grid == want_grid
+        lat.set_point_grid(None)
+        assert lat.point_grid == ()
+        got, _ = gpu_filter(pd, vd, pos, val, False, lattice=lat)
+        assert lat.point_grid == ()
+        assert_float_parity(got, want)
