@@ -77,7 +77,7 @@ struct pl_lattice {
     bool cell_values_clean = false;    // all zero
     uint32_t n_cells_alloc = 0;
     uint32_t n_cells = 0;              // in use by the last build
-    uint32_t max_cells = 0;            // enough for N*(pd+1) vertices at load 1/2
+    uint32_t max_cells = 0;            // enough for N*(pd+1) vertices
     long forced_cells = 0;
     bool table_clean = false;          // every cell of [0, n_cells) is empty
 

@@ -13,7 +13,7 @@ constexpr uint64_t kEmptyCell = ~0ull;
 
 // bits of Counters::flags
 enum : int {
-    kFlagTableFull = 1,   // a probe sequence wrapped, or more than cells/2 vertices were created
+    kFlagTableFull = 1,   // a probe sequence wrapped, or more vertices were created than the table may hold
     kFlagKeyRange = 2,    // a lattice coordinate does not fit its field of the packed key
 };
 
