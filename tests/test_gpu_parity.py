@@ -583,3 +583,27 @@ def test_grid_is_found_in_positions_of_images_and_volumes(case):
         got, _ = gpu_filter(pd, vd, pos, val, False, lattice=lat)
         assert lat.point_grid == ()
         assert_float_parity(got, want)
+
+
+def test_vertex_count_far_from_the_previous_one():
+    """The kernels over the vertices are launched for an estimate taken from the handle's previous
+    build; a lattice with twenty times as many vertices (or a twentieth) must come out the same."""
+    n = 40000
+    rng = np.random.default_rng(91)
+    val = rng.uniform(0, 1, (n, 3)).astype(np.float32)
+    few = rng.uniform(0, 1.5, (n, 5)).astype(np.float32)       # everything in a handful of simplices
+    many = rng.uniform(0, 14, (n, 5)).astype(np.float32)       # nearly every point alone
+    lat = pla.PermutohedralLattice(5, 4, n)
+    counts = []
+    for pos in (few, many, few, many):
+        cpu = oracle.Lattice(5, 4, n)
+        want = cpu.filter(val, pos, False)
+        got, _ = gpu_filter(5, 4, pos, val, False, lattice=lat)
+        assert lat.num_vertices == cpu.num_vertices
+        counts.append(lat.num_vertices)
+        assert_float_parity(got, want)
+        out = torch.empty((n, 3), dtype=torch.float32, device="cuda")
+        lat.apply(out, dev(val), True)
+        torch.cuda.synchronize()
+        assert_float_parity(host(out), oracle.Lattice(5, 4, n).filter(val, pos, True))
+    assert counts[1] > 20 * counts[0]
