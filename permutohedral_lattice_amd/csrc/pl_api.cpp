@@ -225,6 +225,10 @@ int enqueue_build(pl_lattice *h, const plk::PointFeatures &features, uint32_t ce
                   const float *splat_input) {
     int rc = ensure_table(h, cells);
     if (rc != PL_OK) return rc;
+    // the per-point arrays follow the point map; an allocation that failed when the map was set
+    // is made up for here
+    rc = ensure_replay(h);
+    if (rc != PL_OK) return rc;
     const bool fused = splat_input && plk::build_can_splat(h->vd);
     if (fused && !h->cell_values_clean) {
         PL_HIP(plk::fill_zero(h->cell_values, (size_t)h->n_cells_alloc * h->vd, h->stream));
