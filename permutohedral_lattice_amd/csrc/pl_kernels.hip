@@ -112,36 +112,33 @@ __device__ __forceinline__ void enclosing_simplex(const float (&pos)[PD], const 
         qsum += s.q[i];
     }
 
-    // rank[i] = number of coordinates with a larger residual; the pairwise i<j comparison with a
-    // strict < decides ties exactly as the sequential loop does
+    // rank[i] = number of coordinates with a larger residual.  One strict < per pair i < j decides
+    // ties exactly as the sequential loop does: true counts for i, false for j, so rank[i] starts
+    // at i (the pairs below it, all taken as false) and every true moves one count from j to i.
+    // The rounded point is qsum steps off the plane, which rotates the ranks by qsum.
     float d[D1];
-#pragma unroll
-    for (int i = 0; i < D1; ++i) d[i] = el[i] - rem[i];
+    int rk[D1];
 #pragma unroll
     for (int i = 0; i < D1; ++i) {
-        int rk = 0;
-#pragma unroll
-        for (int j = 0; j < D1; ++j) {
-            if (j > i) rk += (d[i] < d[j]) ? 1 : 0;
-            if (j < i) rk += (d[j] < d[i]) ? 0 : 1;
-        }
-        s.rank[i] = rk;
+        d[i] = el[i] - rem[i];
+        rk[i] = i + qsum;
     }
-
-    // the rounded point is qsum steps off the plane: rotate the ranks, wrap the coordinates
 #pragma unroll
     for (int i = 0; i < D1; ++i) {
-        int rk = s.rank[i] + qsum;
-        if (rk < 0) {
-            rk += D1;
-            s.q[i] += 1;
-            rem[i] += (float)D1;
-        } else if (rk > PD) {
-            rk -= D1;
-            s.q[i] -= 1;
-            rem[i] -= (float)D1;
+#pragma unroll
+        for (int j = i + 1; j < D1; ++j) {
+            const int lt = (d[i] < d[j]) ? 1 : 0;
+            rk[i] += lt;
+            rk[j] -= lt;
         }
-        s.rank[i] = rk;
+    }
+    // ranks that left 0..pd wrap round, and their coordinate moves one step
+#pragma unroll
+    for (int i = 0; i < D1; ++i) {
+        const int step = rk[i] < 0 ? 1 : (rk[i] > PD ? -1 : 0);
+        s.rank[i] = rk[i] + step * D1;
+        s.q[i] += step;
+        rem[i] += (float)(step * D1);
     }
 
     // barycentric weights.  by_rank[k] is the scaled residual of the coordinate of rank k; the
@@ -308,17 +305,18 @@ constexpr int kDppQuadSwap1 = 0xB1;   // quad_perm:[1,0,3,2]
 constexpr int kDppQuadSwap2 = 0x4E;   // quad_perm:[2,3,0,1]
 constexpr int kDppRowShr2 = 0x112, kDppRowShr4 = 0x114, kDppRowShr8 = 0x118;
 
-// Adds to the lanes of rows 1 and 3 (of 16 lanes) what the same lanes of rows 0 and 2 hold, then to
-// rows 2 and 3 what rows 0 and 1 hold: afterwards row 3 has the sum over the four rows, lane by
-// lane.  v_permlane16_swap / v_permlane32_swap are gfx950 instructions.
-__device__ __forceinline__ float add_rows_into_last(float x, int lane) {
+// Sum over the four rows (of 16 lanes) of the wavefront, lane by lane, delivered to every row.
+// v_permlane16_swap exchanges the odd rows of its first operand with the even rows of its second:
+// given x twice, the first result holds x's even rows in both rows of a pair and the second x's
+// odd rows, so their sum is the pair's sum in either row; v_permlane32_swap does the same with the
+// halves of the wavefront.  Both are gfx950 instructions.
+__device__ __forceinline__ float add_rows(float x) {
     const unsigned u = __float_as_uint(x);
-    const float from_even_row = __uint_as_float(__builtin_amdgcn_permlane16_swap(u, u, false, false)[0]);
-    if (lane & 16) x += from_even_row;
-    const unsigned w = __float_as_uint(x);
-    const float from_low_half = __uint_as_float(__builtin_amdgcn_permlane32_swap(w, w, false, false)[0]);
-    if (lane & 32) x += from_low_half;
-    return x;
+    const auto pair = __builtin_amdgcn_permlane16_swap(u, u, false, false);
+    const float y = __uint_as_float(pair[0]) + __uint_as_float(pair[1]);
+    const unsigned w = __float_as_uint(y);
+    const auto half = __builtin_amdgcn_permlane32_swap(w, w, false, false);
+    return __uint_as_float(half[0]) + __uint_as_float(half[1]);
 }
 
 // Sum over the lanes with `member` set of term[0..VD) (VD <= 4), delivered channel-wise to the
@@ -373,7 +371,7 @@ __device__ __forceinline__ float wave_sum_to_last_lanes(bool member, const QuadT
     }
     sum = add_from_lane<kDppRowShr4>(sum);
     sum = add_from_lane<kDppRowShr8>(sum);
-    return add_rows_into_last(sum, lane);
+    return add_rows(sum);
 }
 
 // ------------------------------------------------------------------------------------------------
