@@ -2,7 +2,8 @@
  * CPU oracle for the permutohedral-lattice filter.
  *
  * TEST INFRASTRUCTURE ONLY.  This is a plain-C restatement of the arithmetic of the
- * reference CPU path (src/PermutohedralLatticeCPU.h in the reference tree) for T = float.
+ * reference CPU path (src/PermutohedralLatticeCPU.h in the reference tree) for T = float and,
+ * with the suffix _f64, for T = double.
  * It exists to check the HIP library; nothing in the shipped library links, loads or
  * calls it, and it is never the thing whose speed is reported as the product's.
  *
@@ -95,6 +96,45 @@ int plo_lattice_filter_op(const float *input, const float *reference, float *out
                           int n_spatial_dims, const int *spatial_dims, int n_input_channels,
                           int n_reference_channels, int bilateral, float theta_alpha,
                           float theta_beta, float theta_gamma, int reverse);
+
+/* ------------------------------------------------------------------------------------------
+ * T = double (the op registers it, src/LatticeFilterKernel.cpp:196-208): the same functions,
+ * name by name, citing the same reference lines.  One difference is the reference's own: the
+ * scaled coordinate of the elevation is a float for every T (`float cf`, :226).
+ * ---------------------------------------------------------------------------------------- */
+typedef struct plo_lattice_f64 plo_lattice_f64;
+void plo_scale_factor_f64(int pd, double *scale);
+void plo_embed_f64(int pd, const double *scale, const double *position, double *elevated);
+void plo_simplex_f64(int pd, const double *elevated, double *rem0, short *rank);
+void plo_barycentric_f64(int pd, const double *elevated, const double *rem0, const short *rank,
+                         double *barycentric);
+void plo_vertex_key_f64(int pd, const double *rem0, const short *rank, int remainder, short *key);
+void plo_dump_simplex_f64(int pd, int N, const double *positions, short *rem0, short *rank,
+                          short *keys, double *barycentric, double *elevated);
+void plo_compute_positions_f64(const double *reference, double *positions, int num_super_pixels,
+                               int reference_channels, int n_sdims, const int *sdims,
+                               double spatial_std, double feature_std);
+plo_lattice_f64 *plo_create_f64(int pd, int vd, int N);
+void plo_destroy_f64(plo_lattice_f64 *l);
+void plo_splat_f64(plo_lattice_f64 *l, const double *positions, const double *values);
+void plo_blur_f64(plo_lattice_f64 *l, int reverse);
+void plo_slice_f64(plo_lattice_f64 *l, double *out, int normalize);
+void plo_filter_f64(plo_lattice_f64 *l, double *output, const double *input,
+                    const double *positions, int reverse);
+void plo_filter_raw_f64(plo_lattice_f64 *l, double *output, const double *input_vd,
+                        const double *positions, int reverse);
+void plo_set_reference_growth_quirk_f64(plo_lattice_f64 *l, int on);
+int plo_num_growths_f64(const plo_lattice_f64 *l);
+int plo_num_vertices_f64(const plo_lattice_f64 *l);
+const short *plo_keys_f64(const plo_lattice_f64 *l);
+const double *plo_values_f64(const plo_lattice_f64 *l);
+const int *plo_replay_vertex_f64(const plo_lattice_f64 *l);
+const double *plo_replay_weight_f64(const plo_lattice_f64 *l);
+void plo_stage_seconds_f64(const plo_lattice_f64 *l, double *splat, double *blur, double *slice);
+int plo_lattice_filter_op_f64(const double *input, const double *reference, double *output,
+                              int batch, int n_spatial_dims, const int *spatial_dims,
+                              int n_input_channels, int n_reference_channels, int bilateral,
+                              float theta_alpha, float theta_beta, float theta_gamma, int reverse);
 
 #ifdef __cplusplus
 }

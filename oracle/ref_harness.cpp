@@ -22,18 +22,17 @@ double now_seconds() {
     clock_gettime(CLOCK_MONOTONIC, &ts);
     return double(ts.tv_sec) + 1e-9 * double(ts.tv_nsec);
 }
-}  // namespace
 
-extern "C" {
-
-void plref_scale_factor(int pd, float *scale) {
-    PermutohedralLatticeCPU<float> lattice(pd, 2, 1);
+template <typename T>
+void scale_factor(int pd, T *scale) {
+    PermutohedralLatticeCPU<T> lattice(pd, 2, 1);
     for (int i = 0; i < pd; ++i) scale[i] = lattice.scaleFactor[i];
 }
 
-void plref_dump_simplex(int pd, int N, const float *positions, short *rem0, short *rank,
-                        short *keys, float *barycentric, float *elevated) {
-    PermutohedralLatticeCPU<float> lattice(pd, 2, 1);
+template <typename T>
+void dump_simplex(int pd, int N, const T *positions, short *rem0, short *rank, short *keys,
+                  T *barycentric, T *elevated) {
+    PermutohedralLatticeCPU<T> lattice(pd, 2, 1);
     const int d1 = pd + 1;
     for (int n = 0; n < N; ++n) {
         lattice.embed_position_vector(positions + size_t(n) * pd);
@@ -56,21 +55,23 @@ void plref_dump_simplex(int pd, int N, const float *positions, short *rem0, shor
     }
 }
 
-void plref_compute_positions(const float *reference, float *positions, int num_super_pixels,
+template <typename T>
+void compute_positions(const T *reference, T *positions, int num_super_pixels,
                              int reference_channels, int n_sdims, const int *sdims,
-                             float spatial_std, float feature_std) {
-    compute_kernel_cpu<float>(reference, positions, num_super_pixels, reference_channels, n_sdims,
+                             T spatial_std, T feature_std) {
+    compute_kernel_cpu<T>(reference, positions, num_super_pixels, reference_channels, n_sdims,
                               sdims, spatial_std, feature_std);
 }
 
 // One filter call on a fresh lattice.  Optional outputs: vertex count, keys (first-touch
 // order, caller provides N*(pd+1)*pd shorts at most), seconds for the whole call.
-void plref_filter(int pd, int vd, int N, float *output, const float *input,
-                  const float *positions, int reverse, int *num_vertices, short *keys_out,
+template <typename T>
+void filter(int pd, int vd, int N, T *output, const T *input,
+                  const T *positions, int reverse, int *num_vertices, short *keys_out,
                   double *seconds) {
     const double t0 = now_seconds();
     {
-        PermutohedralLatticeCPU<float> lattice(pd, vd, N);
+        PermutohedralLatticeCPU<T> lattice(pd, vd, N);
         lattice.filter(output, input, positions, reverse != 0);
         if (seconds) *seconds = now_seconds() - t0;
         if (num_vertices) *num_vertices = lattice.hashTable.size();
@@ -83,11 +84,12 @@ void plref_filter(int pd, int vd, int N, float *output, const float *input,
 
 // Stage-by-stage run exposing the vertex values after splat and after blur
 // (each M*vd floats, caller sizes them for N*(pd+1) vertices), and per-stage seconds.
-void plref_filter_stages(int pd, int vd, int N, float *output, const float *input,
-                         const float *positions, int reverse, int *num_vertices,
-                         float *values_after_splat, float *values_after_blur,
+template <typename T>
+void filter_stages(int pd, int vd, int N, T *output, const T *input,
+                         const T *positions, int reverse, int *num_vertices,
+                         T *values_after_splat, T *values_after_blur,
                          double *stage_seconds /* splat, blur, slice */) {
-    PermutohedralLatticeCPU<float> lattice(pd, vd, N);
+    PermutohedralLatticeCPU<T> lattice(pd, vd, N);
     double t0 = now_seconds();
     lattice.splat(positions, input);
     double t1 = now_seconds();
@@ -112,7 +114,8 @@ void plref_filter_stages(int pd, int vd, int N, float *output, const float *inpu
 
 // The op's per-batch-item loop (src/LatticeFilterKernel.cpp:111-179) driven through the
 // reference's own CPU functor bodies (compute_kernel_cpu + PermutohedralLatticeCPU::filter).
-int plref_lattice_filter_op(const float *input, const float *reference, float *output, int batch,
+template <typename T>
+int lattice_filter_op(const T *input, const T *reference, T *output, int batch,
                             int n_spatial_dims, const int *spatial_dims, int n_input_channels,
                             int n_reference_channels, int bilateral, float theta_alpha,
                             float theta_beta, float theta_gamma, int reverse) {
@@ -121,13 +124,13 @@ int plref_lattice_filter_op(const float *input, const float *reference, float *o
     const int vd = n_input_channels + 1;
     const int ref_ch = bilateral ? n_reference_channels : 0;
     const int pd = n_spatial_dims + ref_ch;
-    const float spatial_std = bilateral ? theta_alpha : theta_gamma;
-    const float feature_std = bilateral ? theta_beta : -1.0f;
-    float *positions = new float[size_t(N) * pd];
+    const T spatial_std = bilateral ? theta_alpha : theta_gamma;   // float attributes for every T
+    const T feature_std = bilateral ? theta_beta : -1.0f;
+    T *positions = new T[size_t(N) * pd];
     for (int b = 0; b < batch; ++b) {
-        compute_kernel_cpu<float>(reference + size_t(b) * N * ref_ch, positions, N, ref_ch,
+        compute_kernel_cpu<T>(reference + size_t(b) * N * ref_ch, positions, N, ref_ch,
                                   n_spatial_dims, spatial_dims, spatial_std, feature_std);
-        PermutohedralLatticeCPU<float> lattice(pd, vd, N);
+        PermutohedralLatticeCPU<T> lattice(pd, vd, N);
         lattice.filter(output + size_t(b) * N * n_input_channels,
                        input + size_t(b) * N * n_input_channels, positions, reverse != 0);
     }
@@ -135,4 +138,45 @@ int plref_lattice_filter_op(const float *input, const float *reference, float *o
     return 0;
 }
 
+
+}  // namespace
+
+// T = float: plref_<name>; T = double: plref_<name>_f64
+#define PLREF_EXPORTS(T, SUFFIX)                                                                   \
+    void plref_scale_factor##SUFFIX(int pd, T *scale) { scale_factor<T>(pd, scale); }              \
+    void plref_dump_simplex##SUFFIX(int pd, int N, const T *positions, short *rem0, short *rank,   \
+                                    short *keys, T *barycentric, T *elevated) {                    \
+        dump_simplex<T>(pd, N, positions, rem0, rank, keys, barycentric, elevated);                \
+    }                                                                                              \
+    void plref_compute_positions##SUFFIX(const T *reference, T *positions, int num_super_pixels,   \
+                                         int reference_channels, int n_sdims, const int *sdims,    \
+                                         T spatial_std, T feature_std) {                           \
+        compute_positions<T>(reference, positions, num_super_pixels, reference_channels, n_sdims,  \
+                             sdims, spatial_std, feature_std);                                     \
+    }                                                                                              \
+    void plref_filter##SUFFIX(int pd, int vd, int N, T *output, const T *input,                    \
+                              const T *positions, int reverse, int *num_vertices,                  \
+                              short *keys_out, double *seconds) {                                  \
+        filter<T>(pd, vd, N, output, input, positions, reverse, num_vertices, keys_out, seconds);  \
+    }                                                                                              \
+    void plref_filter_stages##SUFFIX(int pd, int vd, int N, T *output, const T *input,             \
+                                     const T *positions, int reverse, int *num_vertices,           \
+                                     T *values_after_splat, T *values_after_blur,                  \
+                                     double *stage_seconds) {                                      \
+        filter_stages<T>(pd, vd, N, output, input, positions, reverse, num_vertices,               \
+                         values_after_splat, values_after_blur, stage_seconds);                    \
+    }                                                                                              \
+    int plref_lattice_filter_op##SUFFIX(const T *input, const T *reference, T *output, int batch,  \
+                                        int n_spatial_dims, const int *spatial_dims,               \
+                                        int n_input_channels, int n_reference_channels,            \
+                                        int bilateral, float theta_alpha, float theta_beta,        \
+                                        float theta_gamma, int reverse) {                          \
+        return lattice_filter_op<T>(input, reference, output, batch, n_spatial_dims, spatial_dims, \
+                                    n_input_channels, n_reference_channels, bilateral,             \
+                                    theta_alpha, theta_beta, theta_gamma, reverse);                \
+    }
+
+extern "C" {
+PLREF_EXPORTS(float, )
+PLREF_EXPORTS(double, _f64)
 }  // extern "C"

@@ -20,9 +20,11 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs an MI355X (run with -m gpu on the GPU box)")
 
 
-def golden_lattice_cases():
-    return sorted(os.path.basename(p)[len("lattice_"):-len(".npz")]
-                  for p in glob.glob(os.path.join(GOLDEN, "lattice_*.npz")))
+def golden_lattice_cases(f64=False):
+    """Names of the lattice cases computed with T = float (default) or T = double (*_f64)."""
+    names = sorted(os.path.basename(p)[len("lattice_"):-len(".npz")]
+                   for p in glob.glob(os.path.join(GOLDEN, "lattice_*.npz")))
+    return [n for n in names if n.endswith("_f64") == f64]
 
 
 def load_golden(name):
@@ -30,6 +32,10 @@ def load_golden(name):
 
 
 def bits(a):
+    """Bit patterns: of doubles for a float64 array, of floats for anything else."""
+    a = np.asarray(a)
+    if a.dtype == np.float64:
+        return np.ascontiguousarray(a).view(np.uint64)
     return np.ascontiguousarray(a, np.float32).view(np.uint32)
 
 

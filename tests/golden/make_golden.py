@@ -22,16 +22,18 @@ from permutohedral_lattice_amd import synth  # noqa: E402
 REFERENCE_IMAGES = "/root/reference/Images"
 
 
-def lattice_case(ref, name, pd, vd, positions, values, per_point=True):
-    positions = np.ascontiguousarray(positions, np.float32)
-    values = np.ascontiguousarray(values, np.float32)
-    dump = ref.dump_simplex(positions)
+def lattice_case(ref, name, pd, vd, positions, values, per_point=True, dtype=np.float32):
+    """dtype: the reference's template parameter T.  float64 cases start from the same float32
+    inputs, widened, and are stored as lattice_<name>_f64.npz."""
+    positions = np.ascontiguousarray(positions, dtype)
+    values = np.ascontiguousarray(values, dtype)
+    dump = ref.dump_simplex(positions, dtype=dtype)
     if not per_point:  # large case: keep the per-point integers, drop the per-point floats
         dump["elevated"] = dump["elevated"][:0]
         dump["barycentric"] = dump["barycentric"][:0]
-    fwd = ref.filter_stages(pd, vd, values, positions, reverse=False)
-    rev = ref.filter_stages(pd, vd, values, positions, reverse=True)
-    _, m, keys, _ = ref.filter(pd, vd, values, positions, False)
+    fwd = ref.filter_stages(pd, vd, values, positions, reverse=False, dtype=dtype)
+    rev = ref.filter_stages(pd, vd, values, positions, reverse=True, dtype=dtype)
+    _, m, keys, _ = ref.filter(pd, vd, values, positions, False, dtype=dtype)
     assert m == fwd["M"] == rev["M"]
     out = dict(pd=np.int32(pd), vd=np.int32(vd), positions=positions, values=values,
                elevated=dump["elevated"], rem0=dump["rem0"], rank=dump["rank"], keys=dump["keys"],
@@ -39,6 +41,8 @@ def lattice_case(ref, name, pd, vd, positions, values, per_point=True):
                after_splat=fwd["after_splat"], after_blur_forward=fwd["after_blur"],
                after_blur_reverse=rev["after_blur"], output_forward=fwd["output"],
                output_reverse=rev["output"])
+    if np.dtype(dtype) == np.float64:
+        name += "_f64"
     path = os.path.join(HERE, "lattice_%s.npz" % name)
     np.savez_compressed(path, **out)
     print("%-28s N=%6d pd=%d vd=%2d M=%6d  %7.1f KB" % (name, positions.shape[0], pd, vd, m,
@@ -51,8 +55,9 @@ def main():
         raise SystemExit("oracle/_ref/libplref.so is missing: run `make -C oracle ref` first")
 
     # scale factors, bit patterns
-    np.savez(os.path.join(HERE, "scale_factor.npz"),
-             **{"pd%d" % pd: ref.scale_factor(pd) for pd in range(1, 9)})
+    factors = {"pd%d" % pd: ref.scale_factor(pd) for pd in range(1, 9)}
+    factors.update({"pd%d_f64" % pd: ref.scale_factor(pd, np.float64) for pd in range(1, 9)})
+    np.savez(os.path.join(HERE, "scale_factor.npz"), **factors)
 
     # feature builder: 2-D and 3-D, stds that are not powers of two
     rng = np.random.default_rng(11)
@@ -62,12 +67,16 @@ def main():
                                           ("2d_spatial", (12, 10), 0, 3.0, -1.0),
                                           ("2d_crf", (8, 8), 3, 80.0, 13.0)):
         n = int(np.prod(sdims))
+        # the op's attributes are floats for every T: the stds are float values also in double
+        s_std, f_std = float(np.float32(s_std)), float(np.float32(f_std))
         refimg = rng.uniform(0, 255 if f_std > 1 else 1, (n, max(rc, 1))).astype(np.float32)
         pos_cases[name + "_sdims"] = np.array(sdims, np.int32)
         pos_cases[name + "_rc"] = np.int32(rc)
         pos_cases[name + "_stds"] = np.array([s_std, f_std], np.float32)
         pos_cases[name + "_reference"] = refimg
         pos_cases[name + "_positions"] = ref.compute_positions(refimg, sdims, s_std, f_std, rc)
+        pos_cases[name + "_positions_f64"] = ref.compute_positions(refimg, sdims, s_std, f_std, rc,
+                                                                   dtype=np.float64)
     np.savez_compressed(os.path.join(HERE, "positions.npz"), **pos_cases)
 
     # lattice cases, one per (pd, vd) of the benchmark configurations, at small sizes
@@ -102,6 +111,17 @@ def main():
         lattice_case(ref, "random_pd%d_vd3" % pd, pd, 3,
                      rng.uniform(-6, 6, (700, pd)).astype(np.float32),
                      rng.uniform(0, 1, (700, 2)).astype(np.float32))
+
+    # T = double: the colour case, exact ties, the guided case and the highest dimension
+    lattice_case(ref, "bilateral_pd5_vd4", 5, 4, synth.bilateral_positions(img, 8.0, 0.125),
+                 img.reshape(-1, 3), dtype=np.float64)
+    lattice_case(ref, "ties_pd3_vd2", 3, 2, tie_pos, synth.uniform_image((tie_pos.shape[0], 1), 109),
+                 dtype=np.float64)
+    lattice_case(ref, "guided_pd5_vd2", 5, 2, synth.bilateral_positions(guide, 8.0, 0.125),
+                 synth.uniform_image((1600, 1), 104), dtype=np.float64)
+    rng = np.random.default_rng(118)
+    lattice_case(ref, "random_pd8_vd3", 8, 3, rng.uniform(-6, 6, (700, 8)).astype(np.float32),
+                 rng.uniform(0, 1, (700, 2)).astype(np.float32), dtype=np.float64)
 
     # the reference's image fixtures (Tests/bilateral_filter.py, Tests/greyscale_test.py)
     from PIL import Image

@@ -17,35 +17,45 @@ import oracle
 # golden vectors from the reference header
 # ---------------------------------------------------------------------------------------------
 
-def test_scale_factor_golden_and_closed_form():
+ALL_GOLDEN = golden_lattice_cases() + golden_lattice_cases(f64=True)
+
+
+@pytest.mark.parametrize("dtype,suffix,rtol", [(np.float32, "", 3e-7), (np.float64, "_f64", 1e-15)])
+def test_scale_factor_golden_and_closed_form(dtype, suffix, rtol):
     g = load_golden("scale_factor")
     for pd in range(1, 9):
-        sf = oracle.scale_factor(pd)
-        assert (bits(sf) == bits(g["pd%d" % pd])).all()
+        sf = oracle.scale_factor(pd, dtype)
+        assert sf.dtype == dtype
+        assert (bits(sf) == bits(g["pd%d%s" % (pd, suffix)])).all()
         closed = [(pd + 1) * math.sqrt(2.0 / 3.0) / math.sqrt((i + 1) * (i + 2)) for i in range(pd)]
-        assert np.allclose(sf, closed, rtol=3e-7, atol=0)
+        assert np.allclose(sf, closed, rtol=rtol, atol=0)
 
 
+@pytest.mark.parametrize("dtype,suffix", [(np.float32, ""), (np.float64, "_f64")])
 @pytest.mark.parametrize("name", ["2d_rgb", "3d_grey", "2d_spatial", "2d_crf"])
-def test_compute_positions_golden_and_closed_form(name):
+def test_compute_positions_golden_and_closed_form(name, dtype, suffix):
     g = load_golden("positions")
     sdims, rc = g[name + "_sdims"], int(g[name + "_rc"])
     s_std, f_std = [float(x) for x in g[name + "_stds"]]
     ref = g[name + "_reference"]
-    pos = oracle.compute_positions(ref, sdims, s_std, f_std, rc)
-    assert (bits(pos) == bits(g[name + "_positions"])).all()
+    pos = oracle.compute_positions(ref, sdims, s_std, f_std, rc, dtype=dtype)
+    assert pos.dtype == dtype
+    assert (bits(pos) == bits(g[name + "_positions" + suffix])).all()
     # closed form: coordinate / std in tensor order (last spatial dimension fastest)
-    grids = np.meshgrid(*[np.arange(s, dtype=np.float32) for s in sdims], indexing="ij")
+    grids = np.meshgrid(*[np.arange(s, dtype=dtype) for s in sdims], indexing="ij")
     for k, gk in enumerate(grids):
-        assert (bits(pos[:, k]) == bits(gk.reshape(-1) / np.float32(s_std))).all()
+        assert (bits(pos[:, k]) == bits(gk.reshape(-1) / dtype(s_std))).all()
     for c in range(rc):
-        assert (bits(pos[:, len(sdims) + c]) == bits(ref[:, c] / np.float32(f_std))).all()
+        assert (bits(pos[:, len(sdims) + c]) == bits(ref[:, c].astype(dtype) / dtype(f_std))).all()
 
 
-@pytest.mark.parametrize("name", golden_lattice_cases())
+@pytest.mark.parametrize("name", ALL_GOLDEN)
 def test_simplex_matches_reference_bit_exact(name):
     g = load_golden("lattice_" + name)
-    d = oracle.dump_simplex(g["positions"], want_elevated=True)
+    dtype = g["positions"].dtype
+    assert dtype == (np.float64 if name.endswith("_f64") else np.float32)
+    d = oracle.dump_simplex(g["positions"], want_elevated=True, dtype=dtype)
+    assert d["elevated"].dtype == dtype and d["barycentric"].dtype == dtype
     if g["elevated"].size:
         assert (bits(d["elevated"]) == bits(g["elevated"])).all()
         assert (bits(d["barycentric"]) == bits(g["barycentric"])).all()
@@ -54,15 +64,16 @@ def test_simplex_matches_reference_bit_exact(name):
     assert (d["keys"] == g["keys"]).all()
 
 
-@pytest.mark.parametrize("name", golden_lattice_cases())
+@pytest.mark.parametrize("name", ALL_GOLDEN)
 def test_filter_matches_reference_bit_exact(name):
     """With the reference's index-growth quirk reproduced, every stage is bit-identical."""
     g = load_golden("lattice_" + name)
     pd, vd = int(g["pd"]), int(g["vd"])
     n = g["positions"].shape[0]
+    dtype = g["positions"].dtype
     for reverse, blur_key, out_key in ((False, "after_blur_forward", "output_forward"),
                                        (True, "after_blur_reverse", "output_reverse")):
-        lat = oracle.Lattice(pd, vd, n, reference_growth_quirk=True)
+        lat = oracle.Lattice(pd, vd, n, reference_growth_quirk=True, dtype=dtype)
         lat.splat(g["values"], g["positions"])
         assert lat.num_vertices == int(g["num_vertices"])
         assert (lat.keys() == g["vertex_keys"]).all()
@@ -70,21 +81,22 @@ def test_filter_matches_reference_bit_exact(name):
         lat.blur(reverse)
         assert (bits(lat.values()) == bits(g[blur_key])).all()
         out = lat.slice()
+        assert out.dtype == dtype
         assert (bits(out) == bits(g[out_key])).all()
         # and through the one-call entry point
-        out2 = oracle.Lattice(pd, vd, n, reference_growth_quirk=True).filter(
+        out2 = oracle.Lattice(pd, vd, n, reference_growth_quirk=True, dtype=dtype).filter(
             g["values"], g["positions"], reverse)
         assert (bits(out2) == bits(g[out_key])).all()
 
 
-@pytest.mark.parametrize("name", golden_lattice_cases())
+@pytest.mark.parametrize("name", ALL_GOLDEN)
 def test_vertex_count_is_number_of_distinct_keys(name):
     """Without the quirk the lattice has exactly one vertex per distinct key; the reference has
     at most one more per doubling of its index, and the outputs barely move."""
     g = load_golden("lattice_" + name)
     pd, vd = int(g["pd"]), int(g["vd"])
     n = g["positions"].shape[0]
-    lat = oracle.Lattice(pd, vd, n)
+    lat = oracle.Lattice(pd, vd, n, dtype=g["positions"].dtype)
     out = lat.filter(g["values"], g["positions"])
     distinct = np.unique(g["keys"].reshape(-1, pd), axis=0)
     assert lat.num_vertices == len(distinct)
@@ -103,22 +115,24 @@ def test_growth_quirk_case_really_has_a_duplicate():
 
 
 @pytest.mark.skipif(not oracle.have_reference(), reason="reference build absent (oracle/_ref)")
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
 @pytest.mark.parametrize("pd,vd,n,seed", [(5, 4, 30000, 1), (2, 2, 50000, 2), (4, 2, 20000, 3),
                                           (3, 6, 9000, 4), (5, 22, 3000, 5)])
-def test_against_live_reference_build(pd, vd, n, seed):
+def test_against_live_reference_build(pd, vd, n, seed, dtype):
     ref = oracle.reference()
     rng = np.random.default_rng(seed)
-    pos = (rng.uniform(0, 30, (n, pd)) * rng.uniform(0.05, 1.0, pd)).astype(np.float32)
-    val = rng.uniform(0, 1, (n, vd - 1)).astype(np.float32)
-    d, r = oracle.dump_simplex(pos, want_elevated=True), ref.dump_simplex(pos)
+    pos = (rng.uniform(0, 30, (n, pd)) * rng.uniform(0.05, 1.0, pd)).astype(dtype)
+    val = rng.uniform(0, 1, (n, vd - 1)).astype(dtype)
+    d = oracle.dump_simplex(pos, want_elevated=True, dtype=dtype)
+    r = ref.dump_simplex(pos, dtype=dtype)
     for k in ("rem0", "rank", "keys"):
         assert (d[k] == r[k]).all()
     for k in ("elevated", "barycentric"):
         assert (bits(d[k]) == bits(r[k])).all()
     for reverse in (False, True):
-        lat = oracle.Lattice(pd, vd, n, reference_growth_quirk=True)
+        lat = oracle.Lattice(pd, vd, n, reference_growth_quirk=True, dtype=dtype)
         out = lat.filter(val, pos, reverse)
-        rout, m, keys, _ = ref.filter(pd, vd, val, pos, reverse)
+        rout, m, keys, _ = ref.filter(pd, vd, val, pos, reverse, dtype=dtype)
         assert lat.num_vertices == m
         assert (lat.keys() == keys).all()
         assert (bits(out) == bits(rout)).all()
@@ -148,13 +162,14 @@ def test_embedding_is_the_rotation_onto_the_hyperplane(pd):
     assert np.abs(el.sum(axis=1)).max() <= 1e-3
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
 @pytest.mark.parametrize("pd", [1, 2, 3, 4, 5, 6, 8])
-def test_simplex_invariants(pd):
+def test_simplex_invariants(pd, dtype):
     rng = np.random.default_rng(100 + pd)
-    pos = rng.uniform(-40, 40, (4000, pd)).astype(np.float32)
+    pos = rng.uniform(-40, 40, (4000, pd)).astype(dtype)
     # include exact ties: integer positions
     pos[:500] = np.round(pos[:500])
-    d = oracle.dump_simplex(pos, want_elevated=True)
+    d = oracle.dump_simplex(pos, want_elevated=True, dtype=dtype)
     d1 = pd + 1
     rem0, rank, el = d["rem0"].astype(np.int64), d["rank"].astype(np.int64), d["elevated"].astype(np.float64)
     assert (rem0 % d1 == 0).all()
@@ -205,7 +220,7 @@ class _DenseLattice:
 
     def __init__(self, positions):
         self.pd = positions.shape[1]
-        d = oracle.dump_simplex(positions)
+        d = oracle.dump_simplex(positions, dtype=positions.dtype)
         self.index = {}
         n, d1 = d["rank"].shape
         rows = []
@@ -241,22 +256,25 @@ class _DenseLattice:
         return self.W @ x
 
 
+@pytest.mark.parametrize("dtype,tol", [(np.float32, 2e-5), (np.float64, 1e-13)])
 @pytest.mark.parametrize("pd,vd,n", [(2, 3, 64), (3, 2, 80), (5, 4, 60)])
-def test_filter_equals_dense_brute_force(pd, vd, n):
+def test_filter_equals_dense_brute_force(pd, vd, n, dtype, tol):
+    """In double the oracle and the dense product agree to rounding: any difference in structure
+    (a wrong neighbour, a missing tap, the wrong axis order) would show at 1e-3."""
     rng = np.random.default_rng(pd * 10 + vd)
-    pos = rng.uniform(0, 4, (n, pd)).astype(np.float32)
-    val = rng.uniform(0, 1, (n, vd - 1)).astype(np.float32)
+    pos = rng.uniform(0, 4, (n, pd)).astype(dtype)
+    val = rng.uniform(0, 1, (n, vd - 1)).astype(dtype)
     dense = _DenseLattice(pos)
     hom = np.concatenate([val.astype(np.float64), np.ones((n, 1))], axis=1)
     for reverse in (False, True):
         raw = dense.apply(hom, reverse)
         expect = raw[:, :-1] / raw[:, -1:]
-        lat = oracle.Lattice(pd, vd, n)
+        lat = oracle.Lattice(pd, vd, n, dtype=dtype)
         out = lat.filter(val, pos, reverse)
         assert lat.num_vertices == len(dense.index)
-        assert np.abs(out - expect).max() <= 2e-5
-        raw_out = oracle.Lattice(pd, vd, n).filter_raw(hom.astype(np.float32), pos, reverse)
-        assert np.abs(raw_out - raw).max() <= 2e-5
+        assert np.abs(out - expect).max() <= tol
+        raw_out = oracle.Lattice(pd, vd, n, dtype=dtype).filter_raw(hom.astype(dtype), pos, reverse)
+        assert np.abs(raw_out - raw).max() <= tol
     # blur matrices are symmetric: the + neighbour of u is v iff the - neighbour of v is u
     for b in dense.B:
         assert np.abs(b - b.T).max() == 0.0
