@@ -216,6 +216,39 @@ int pl_lattice_filter_op(const float *input, const float *reference, float *outp
  */
 int pl_set_op_concurrency(int lanes);
 
+/* ------------------------------------------------------------------------------------------
+ * T = double.  The reference is a template over the value type and its op is registered for
+ * float and double (src/PermutohedralLatticeCPU.h:173, src/LatticeFilterKernel.cpp:196-208).
+ * A lattice made by pl_create_f64 takes positions, inputs and outputs as doubles through the
+ * calls below, which mean what their float namesakes mean; pl_destroy, pl_set_point_grid,
+ * pl_get_point_grid, pl_set_option, pl_num_vertices, pl_stage_ms and pl_debug_keys serve both
+ * kinds, every other float entry point returns PL_EINVAL for a lattice of doubles (and these for
+ * a lattice of floats).  The lattice (keys, vertex count) equals the CPU path's for T = double
+ * exactly; values agree to rounding of the sums (about 1e-15 relative), because the splat adds
+ * in another order than a sequential loop.  The float path is the one tuned for speed: this one
+ * uses the plain form of each value pass, and its points are not looked at for a grid (give one
+ * with pl_set_point_grid; the op does).
+ * ---------------------------------------------------------------------------------------- */
+int pl_create_f64(int pd, int vd, int N, pl_stream stream, const pl_alloc *alloc, pl_handle *out);
+int pl_filter_f64(pl_handle h, double *output, const double *input, const double *positions,
+                  int reverse);
+int pl_build_f64(pl_handle h, const double *positions);
+int pl_apply_f64(pl_handle h, double *output, const double *input, int reverse);
+int pl_debug_simplex_f64(pl_handle h, const double *positions, short *rem0, short *rank,
+                         short *keys, double *barycentric);
+/* compute_kernel<double> (src/PermutohedralLatticeCPU.h:452-474, src/LatticeFilterKernel.h:42-54) */
+int pl_compute_positions_f64(const double *reference, double *positions, int num_super_pixels,
+                             int n_reference_channels, int n_spatial_dims, const int *spatial_dims,
+                             double spatial_std, double feature_std, pl_stream stream);
+/* LatticeFilterOp<Device, double>::Compute (src/LatticeFilterKernel.cpp:98-181); the attributes
+ * are floats for every T (:36-38).  One lattice, the items one after the other; its scratch and
+ * the positions of an item come from alloc (NULL: hipMalloc) and go back before the call ends. */
+int pl_lattice_filter_op_f64(const double *input, const double *reference, double *output,
+                             int batch, int n_spatial_dims, const int *spatial_dims,
+                             int n_input_channels, int n_reference_channels, int bilateral,
+                             float theta_alpha, float theta_beta, float theta_gamma, int reverse,
+                             pl_stream stream, const pl_alloc *alloc);
+
 #ifdef __cplusplus
 }
 #endif

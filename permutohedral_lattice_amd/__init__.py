@@ -30,6 +30,8 @@ EXPORTS = (
     "pl_debug_keys", "pl_debug_replay", "pl_compute_positions", "pl_filter_image", "pl_build_image",
     "pl_filter_begin", "pl_filter_image_begin", "pl_filter_end", "pl_lattice_filter_op",
     "pl_set_op_concurrency",
+    "pl_create_f64", "pl_filter_f64", "pl_build_f64", "pl_apply_f64", "pl_debug_simplex_f64",
+    "pl_compute_positions_f64", "pl_lattice_filter_op_f64",
 )
 
 
@@ -78,6 +80,15 @@ def _load():
     lib.pl_set_op_concurrency.argtypes = [ci]
     lib.pl_lattice_filter_op.argtypes = [vp, vp, vp, ci, ci, C.POINTER(ci), ci, ci, ci, cf, cf, cf,
                                          ci, vp, vp]
+    # T = double
+    lib.pl_create_f64.argtypes = lib.pl_create.argtypes
+    lib.pl_filter_f64.argtypes = lib.pl_filter.argtypes
+    lib.pl_build_f64.argtypes = lib.pl_build.argtypes
+    lib.pl_apply_f64.argtypes = lib.pl_apply.argtypes
+    lib.pl_debug_simplex_f64.argtypes = lib.pl_debug_simplex.argtypes
+    lib.pl_compute_positions_f64.argtypes = [vp, vp, ci, ci, ci, C.POINTER(ci), C.c_double,
+                                             C.c_double, vp]
+    lib.pl_lattice_filter_op_f64.argtypes = lib.pl_lattice_filter_op.argtypes
     return lib
 
 
@@ -89,13 +100,25 @@ def _check(status, where):
         raise PermutohedralError(status, where)
 
 
-def _dev_f32(t, name, numel=None):
-    if not (isinstance(t, torch.Tensor) and t.is_cuda and t.dtype == torch.float32
-            and t.is_contiguous()):
-        raise TypeError("%s must be a contiguous float32 tensor on the GPU" % name)
+def _dev(t, name, numel=None, dtype=torch.float32):
+    if not (isinstance(t, torch.Tensor) and t.is_cuda and t.dtype == dtype and t.is_contiguous()):
+        raise TypeError("%s must be a contiguous %s tensor on the GPU" % (name, dtype))
     if numel is not None and t.numel() != numel:
         raise ValueError("%s has %d elements, expected %d" % (name, t.numel(), numel))
     return C.c_void_p(t.data_ptr())
+
+
+def _dev_f32(t, name, numel=None):
+    return _dev(t, name, numel, torch.float32)
+
+
+def _value_type(dtype):
+    """The reference's template parameter T: float (default) or double."""
+    if dtype in (None, torch.float32):
+        return torch.float32
+    if dtype == torch.float64:
+        return torch.float64
+    raise TypeError("the lattice is built for float32 and float64 values, not %s" % dtype)
 
 
 def _stream_ptr(stream=None):
@@ -109,15 +132,26 @@ def supported(pd, vd):
 
 class PermutohedralLattice:
     """Lattice for ``(pd, vd, N)``; ``vd`` counts the homogeneous channel.  All tensors are
-    contiguous float32 on the GPU; work is enqueued on the stream current at construction."""
+    contiguous tensors of ``dtype`` (float32, or float64 for the reference's ``T = double``) on
+    the GPU; work is enqueued on the stream current at construction."""
 
-    def __init__(self, pd, vd, N, stream=None):
+    def __init__(self, pd, vd, N, stream=None, dtype=torch.float32):
         self.pd, self.vd, self.N = int(pd), int(vd), int(N)
+        self.dtype = _value_type(dtype)
+        self._f64 = self.dtype == torch.float64
         self._h = C.c_void_p()
         self._stream = stream if stream is not None else torch.cuda.current_stream()
-        _check(_lib.pl_create(self.pd, self.vd, self.N, _stream_ptr(self._stream), None,
-                              C.byref(self._h)), "pl_create")
+        create = _lib.pl_create_f64 if self._f64 else _lib.pl_create
+        _check(create(self.pd, self.vd, self.N, _stream_ptr(self._stream), None, C.byref(self._h)),
+               "pl_create")
         self._normalize = True
+
+    def _t(self, t, name, numel):
+        return _dev(t, name, numel, self.dtype)
+
+    def _float_only(self, what):
+        if self._f64:
+            raise TypeError("%s is for lattices of float32 values" % what)
 
     def close(self):
         if getattr(self, "_h", None):
@@ -129,14 +163,16 @@ class PermutohedralLattice:
     # -- the reference's interface -------------------------------------------------------------
     def filter(self, output, input, positions, reverse=False):
         ch = self.vd - 1 if self._normalize else self.vd
-        _check(_lib.pl_filter(self._h, _dev_f32(output, "output", self.N * ch),
-                              _dev_f32(input, "input", self.N * ch),
-                              _dev_f32(positions, "positions", self.N * self.pd), int(bool(reverse))),
+        call = _lib.pl_filter_f64 if self._f64 else _lib.pl_filter
+        _check(call(self._h, self._t(output, "output", self.N * ch),
+                    self._t(input, "input", self.N * ch),
+                    self._t(positions, "positions", self.N * self.pd), int(bool(reverse))),
                "pl_filter")
         return output
 
     # -- the same in two halves: enqueue, and later wait and check ---------------------------------
     def filter_begin(self, output, input, positions, reverse=False):
+        self._float_only("filter_begin")
         ch = self.vd - 1 if self._normalize else self.vd
         self._in_flight = (output, input, positions)   # keep the tensors alive until filter_end
         _check(_lib.pl_filter_begin(self._h, _dev_f32(output, "output", self.N * ch),
@@ -150,16 +186,19 @@ class PermutohedralLattice:
 
     # -- build once, apply many ----------------------------------------------------------------
     def build(self, positions):
-        _check(_lib.pl_build(self._h, _dev_f32(positions, "positions", self.N * self.pd)), "pl_build")
+        call = _lib.pl_build_f64 if self._f64 else _lib.pl_build
+        _check(call(self._h, self._t(positions, "positions", self.N * self.pd)), "pl_build")
 
     def apply(self, output, input, reverse=False):
         ch = self.vd - 1 if self._normalize else self.vd
-        _check(_lib.pl_apply(self._h, _dev_f32(output, "output", self.N * ch),
-                             _dev_f32(input, "input", self.N * ch), int(bool(reverse))), "pl_apply")
+        call = _lib.pl_apply_f64 if self._f64 else _lib.pl_apply
+        _check(call(self._h, self._t(output, "output", self.N * ch),
+                    self._t(input, "input", self.N * ch), int(bool(reverse))), "pl_apply")
         return output
 
     # -- features built on the fly from the reference image and the grid coordinates ------------
     def _image_args(self, reference, spatial_dims):
+        self._float_only("the fused feature builder")
         dims = [int(d) for d in spatial_dims]
         rc = self.pd - len(dims)
         if rc < 0:
@@ -217,17 +256,17 @@ class PermutohedralLattice:
     # -- parity exports ------------------------------------------------------------------------
     def debug_simplex(self, positions):
         """-> dict of device tensors rem0 [N,pd+1] i16, rank [N,pd+1] i16, keys [N,pd+1,pd] i16,
-        barycentric [N,pd+1] f32."""
+        barycentric [N,pd+1] of the lattice's value type."""
         d1, dev = self.pd + 1, positions.device
         out = dict(rem0=torch.empty((self.N, d1), dtype=torch.int16, device=dev),
                    rank=torch.empty((self.N, d1), dtype=torch.int16, device=dev),
                    keys=torch.empty((self.N, d1, self.pd), dtype=torch.int16, device=dev),
-                   barycentric=torch.empty((self.N, d1), dtype=torch.float32, device=dev))
-        _check(_lib.pl_debug_simplex(self._h, _dev_f32(positions, "positions", self.N * self.pd),
-                                     C.c_void_p(out["rem0"].data_ptr()),
-                                     C.c_void_p(out["rank"].data_ptr()),
-                                     C.c_void_p(out["keys"].data_ptr()),
-                                     C.c_void_p(out["barycentric"].data_ptr())), "pl_debug_simplex")
+                   barycentric=torch.empty((self.N, d1), dtype=self.dtype, device=dev))
+        call = _lib.pl_debug_simplex_f64 if self._f64 else _lib.pl_debug_simplex
+        _check(call(self._h, self._t(positions, "positions", self.N * self.pd),
+                    C.c_void_p(out["rem0"].data_ptr()), C.c_void_p(out["rank"].data_ptr()),
+                    C.c_void_p(out["keys"].data_ptr()), C.c_void_p(out["barycentric"].data_ptr())),
+               "pl_debug_simplex")
         return out
 
     def debug_keys(self):
@@ -237,6 +276,7 @@ class PermutohedralLattice:
 
     def debug_replay(self):
         """-> (vertex [pd+1, N] i32, weight [pd+1, N] f32) of the last apply/filter."""
+        self._float_only("debug_replay")
         v = torch.empty((self.pd + 1, self.N), dtype=torch.int32, device="cuda")
         w = torch.empty((self.pd + 1, self.N), dtype=torch.float32, device="cuda")
         _check(_lib.pl_debug_replay(self._h, C.c_void_p(v.data_ptr()), C.c_void_p(w.data_ptr())),
@@ -249,9 +289,14 @@ def set_op_concurrency(lanes):
     _check(_lib.pl_set_op_concurrency(int(lanes)), "pl_set_op_concurrency")
 
 
-def compute_positions(reference, spatial_dims, spatial_std, feature_std=1.0, out=None):
+def compute_positions(reference, spatial_dims, spatial_std, feature_std=1.0, out=None, dtype=None):
     """Feature rows of one batch item.  ``reference``: ``[*spatial_dims, rc]`` device tensor, or
-    None for spatial-only features.  -> ``[N, k + rc]``."""
+    None for spatial-only features.  -> ``[N, k + rc]``, in ``dtype`` (default: the reference
+    tensor's, float32 without one)."""
+    if dtype is None:
+        dtype = out.dtype if out is not None else (reference.dtype if reference is not None
+                                                   else torch.float32)
+    dtype = _value_type(dtype)
     sd = [int(s) for s in spatial_dims]
     n = 1
     for s in sd:
@@ -259,12 +304,12 @@ def compute_positions(reference, spatial_dims, spatial_std, feature_std=1.0, out
     rc = 0 if reference is None else int(reference.shape[-1])
     pd = len(sd) + rc
     if out is None:
-        out = torch.empty((n, pd), dtype=torch.float32, device="cuda")
-    ref_ptr = None if reference is None else _dev_f32(reference, "reference", n * rc)
+        out = torch.empty((n, pd), dtype=dtype, device="cuda")
+    ref_ptr = None if reference is None else _dev(reference, "reference", n * rc, dtype)
     dims = (C.c_int * len(sd))(*sd)
-    _check(_lib.pl_compute_positions(ref_ptr, _dev_f32(out, "positions", n * pd), n, rc, len(sd), dims,
-                                     float(spatial_std), float(feature_std), _stream_ptr()),
-           "pl_compute_positions")
+    call = _lib.pl_compute_positions_f64 if dtype == torch.float64 else _lib.pl_compute_positions
+    _check(call(ref_ptr, _dev(out, "positions", n * pd, dtype), n, rc, len(sd), dims,
+                float(spatial_std), float(feature_std), _stream_ptr()), "pl_compute_positions")
     return out
 
 
@@ -273,6 +318,7 @@ def _lattice_filter_raw(input_image, reference_image, bilateral, theta_alpha, th
     if input_image.dim() < 3:
         raise ValueError("input_image must be [batch, spatial..., channels]")
     inp = input_image.contiguous()
+    dtype = _value_type(inp.dtype)
     sd = [int(s) for s in inp.shape[1:-1]]
     out = torch.empty_like(inp)
     ref_ptr, rc = None, 0
@@ -282,14 +328,13 @@ def _lattice_filter_raw(input_image, reference_image, bilateral, theta_alpha, th
         if bilateral:
             if list(ref.shape[:-1]) != list(inp.shape[:-1]):
                 raise ValueError("reference_image and input_image differ in batch or spatial shape")
-            ref_ptr = _dev_f32(ref, "reference_image")
+            ref_ptr = _dev(ref, "reference_image", None, dtype)
     dims = (C.c_int * len(sd))(*sd)
-    _check(_lib.pl_lattice_filter_op(_dev_f32(inp, "input_image"), ref_ptr,
-                                     C.c_void_p(out.data_ptr()), int(inp.shape[0]), len(sd), dims,
-                                     int(inp.shape[-1]), rc, int(bool(bilateral)),
-                                     float(theta_alpha), float(theta_beta), float(theta_gamma),
-                                     int(bool(reverse)), _stream_ptr(), None),
-           "pl_lattice_filter_op")
+    call = _lib.pl_lattice_filter_op_f64 if dtype == torch.float64 else _lib.pl_lattice_filter_op
+    _check(call(_dev(inp, "input_image", None, dtype), ref_ptr, C.c_void_p(out.data_ptr()),
+                int(inp.shape[0]), len(sd), dims, int(inp.shape[-1]), rc, int(bool(bilateral)),
+                float(theta_alpha), float(theta_beta), float(theta_gamma), int(bool(reverse)),
+                _stream_ptr(), None), "pl_lattice_filter_op")
     return out
 
 
@@ -349,7 +394,8 @@ class _LatticeFilterFunction(torch.autograd.Function):
         ctx.save_for_backward(reference_image)
         ctx.attrs = (bilateral, theta_alpha, theta_beta, theta_gamma)
         ctx.lent = None
-        if ctx.needs_input_grad[0] and input_image.dim() >= 3 and input_image.shape[0] > 0:
+        if (ctx.needs_input_grad[0] and input_image.dim() >= 3 and input_image.shape[0] > 0
+                and input_image.dtype == torch.float32):
             out = _LatticeFilterFunction._forward_keeping_lattices(
                 ctx, input_image, reference_image, bilateral, theta_alpha, theta_beta, theta_gamma,
                 reverse)

@@ -55,6 +55,13 @@ void compute_scale_factor(int pd, plk::ScaleFactor &sf) {
         sf.v[i] = (float)(1.0 / std::sqrt((double)((i + 1) * (i + 2))) * (double)inv_std_dev);
 }
 
+// T = double: all of it in double (src/PermutohedralLatticeCPU.h:209-214 with T = double)
+void compute_scale_factor(int pd, plk::ScaleFactor64 &sf) {
+    const double inv_std_dev = (double)(pd + 1) * std::sqrt(2.0 / 3.0);
+    for (int i = 0; i < plk::kMaxPd; ++i) sf.v[i] = 0.0;
+    for (int i = 0; i < pd; ++i) sf.v[i] = 1.0 / std::sqrt((double)((i + 1) * (i + 2))) * inv_std_dev;
+}
+
 enum { EV_T0, EV_CLEAR, EV_BUILD, EV_IDS, EV_NBR, EV_A0, EV_FILL, EV_SPLAT, EV_BLUR, EV_SLICE, EV_COUNT };
 
 }  // namespace
@@ -65,6 +72,11 @@ struct pl_lattice {
     hipStream_t stream = nullptr;
     pl_alloc alloc{};
     plk::ScaleFactor scale{};
+    // T = double (pl_create_f64): values, weights, inputs and outputs are doubles; the value
+    // arrays below are then arrays of double behind their float pointers
+    bool f64 = false;
+    plk::ScaleFactor64 scale64{};
+    double *weights64 = nullptr;       // barycentric weights, layout of the replay rows
 
     // hash table and the per-vertex arrays; a table of n_cells holds at most 3/4 n_cells vertices
     uint64_t *cell_keys = nullptr;     // [n_cells_alloc]
@@ -120,8 +132,9 @@ struct pl_lattice {
     struct Pending {
         bool active = false;
         plk::PointFeatures features{};
-        float *output = nullptr;
-        const float *input = nullptr;
+        const double *positions64 = nullptr;
+        void *output = nullptr;
+        const void *input = nullptr;
         int reverse = 0;
     } pending;
 
@@ -135,6 +148,7 @@ struct pl_lattice {
         if (profile && ev[which]) ev_recorded[which] = hipEventRecord(ev[which], stream) == hipSuccess;
     }
     plk::Counters *counters() { return d_counters + counter_set; }
+    size_t value_size() const { return f64 ? sizeof(double) : sizeof(float); }
     int max_vertices() const { return (int)plk::max_vertices_for(n_cells); }
     // what the grids of the kernels over the vertices are sized for: the count when the host
     // knows it, else the previous build's with a margin (the kernels cover any count)
@@ -169,13 +183,14 @@ int ensure_table(pl_lattice *h, uint32_t cells) {
     h->cell_vertex = (int *)h->dmalloc(sizeof(int) * (size_t)cells);
     h->vertex_keys = (uint64_t *)h->dmalloc(sizeof(uint64_t) * mv);
     h->vertex_cell = (int *)h->dmalloc(sizeof(int) * mv);
-    h->values[0] = (float *)h->dmalloc(sizeof(float) * mv * (size_t)h->vd);
-    h->values[1] = (float *)h->dmalloc(sizeof(float) * mv * (size_t)h->vd);
+    h->values[0] = (float *)h->dmalloc(h->value_size() * mv * (size_t)h->vd);
+    h->values[1] = (float *)h->dmalloc(h->value_size() * mv * (size_t)h->vd);
     h->neighbours = (int2 *)h->dmalloc(sizeof(int2) * mv * (size_t)(h->pd + 1));
-    if (plk::build_can_splat(h->vd))
+    const bool fused_splat = plk::build_can_splat(h->vd) && !h->f64;
+    if (fused_splat)
         h->cell_values = (float *)h->dmalloc(sizeof(float) * (size_t)cells * (size_t)h->vd);
     if (!h->cell_keys || !h->cell_vertex || !h->vertex_keys || !h->vertex_cell || !h->values[0] ||
-        !h->values[1] || !h->neighbours || (plk::build_can_splat(h->vd) && !h->cell_values))
+        !h->values[1] || !h->neighbours || (fused_splat && !h->cell_values))
         return PL_ENOMEM;
     h->n_cells_alloc = cells;
     return PL_OK;
@@ -186,6 +201,7 @@ int ensure_replay(pl_lattice *h) {
     if (want <= h->replay_capacity && h->replay) return PL_OK;
     PL_HIP(hipStreamSynchronize(h->stream));
     h->dfree(h->replay);
+    h->dfree(h->weights64);
     h->dfree(h->created_entries);
     h->dfree(h->block_count);
     h->dfree(h->chunk_count);
@@ -195,8 +211,9 @@ int ensure_replay(pl_lattice *h) {
     h->created_entries = (uint4 *)h->dmalloc(sizeof(uint4) * (want ? want : 1));
     h->block_count = (int *)h->dmalloc(sizeof(int) * (h->map.n_blocks ? h->map.n_blocks : 1));
     h->chunk_count = (int *)h->dmalloc(sizeof(int) * 2 * h->n_chunks);
-    if (!h->replay || !h->created_entries ||
-        !h->block_count || !h->chunk_count)
+    if (h->f64) h->weights64 = (double *)h->dmalloc(sizeof(double) * (want ? want : 1));
+    if (!h->replay || !h->created_entries || !h->block_count || !h->chunk_count ||
+        (h->f64 && !h->weights64))
         return PL_ENOMEM;
     PL_HIP(hipMemsetAsync(h->chunk_count, 0, sizeof(int) * 2 * h->n_chunks, h->stream));
     h->replay_capacity = want;
@@ -225,15 +242,16 @@ uint32_t initial_cells(const pl_lattice *h) {
 // Enqueue one build with a table of `cells` cells.  Nothing here waits for the device.
 // splat_input != nullptr: the build kernel also splats these values (when it can for this vd),
 // and the value table holds them when the build is done.
-int enqueue_build(pl_lattice *h, const plk::PointFeatures &features, uint32_t cells,
-                  const float *splat_input) {
+// A lattice for double values takes its positions from positions64 and never splats in the build.
+int enqueue_build(pl_lattice *h, const plk::PointFeatures &features, const double *positions64,
+                  uint32_t cells, const float *splat_input) {
     int rc = ensure_table(h, cells);
     if (rc != PL_OK) return rc;
     // the per-point arrays follow the point map; an allocation that failed when the map was set
     // is made up for here
     rc = ensure_replay(h);
     if (rc != PL_OK) return rc;
-    const bool fused = splat_input && plk::build_can_splat(h->vd);
+    const bool fused = splat_input && plk::build_can_splat(h->vd) && !h->f64;
     if (fused && !h->cell_values_clean) {
         PL_HIP(plk::fill_zero(h->cell_values, (size_t)h->n_cells_alloc * h->vd, h->stream));
         h->cell_values_clean = true;
@@ -252,15 +270,23 @@ int enqueue_build(pl_lattice *h, const plk::PointFeatures &features, uint32_t ce
                                      h->max_vertices()};
     const plk::CreatedLists lists{h->created_entries, h->block_count,
                                   h->chunk_count + (size_t)h->counter_set * h->n_chunks};
-    PL_HIP(plk::build(h->pd, features, h->map, h->scale, h->cell_keys, cells, h->counters(),
-                      h->replay, h->xcd_aware ? 1 : 0, fused ? h->vd : 0,
-                      splat_input, h->normalize ? h->vd - 1 : h->vd, h->cell_values, lists,
-                      h->stream));
+    if (h->f64) {
+        const plk::Points64 points{positions64, h->weights64, h->scale64};
+        PL_HIP(plk::build_f64(h->pd, points, h->map, h->cell_keys, cells, h->counters(), h->replay,
+                              h->xcd_aware ? 1 : 0, lists, h->stream));
+    } else {
+        PL_HIP(plk::build(h->pd, features, h->map, h->scale, h->cell_keys, cells, h->counters(),
+                          h->replay, h->xcd_aware ? 1 : 0, fused ? h->vd : 0,
+                          splat_input, h->normalize ? h->vd - 1 : h->vd, h->cell_values, lists,
+                          h->stream));
+    }
     h->mark(EV_BUILD);
+    // the numbering pass zeroes the vertices' value rows: a row of vd doubles is 2*vd zero floats
     PL_HIP(plk::number_vertices(h->pd, h->map, lists,
                                 h->chunk_count + (size_t)previous_set * h->n_chunks,
                                 (unsigned)h->n_chunks, vertices,
-                                h->values[0], h->vd, fused ? h->cell_values : nullptr, h->counters(),
+                                h->values[0], h->f64 ? 2 * h->vd : h->vd,
+                                fused ? h->cell_values : nullptr, h->counters(),
                                 h->d_counters + previous_set, h->h_status, h->stream));
     h->mark(EV_IDS);
     PL_HIP(plk::neighbours(h->pd, vertices, h->counters(), h->cell_keys, cells,
@@ -274,7 +300,47 @@ int enqueue_build(pl_lattice *h, const plk::PointFeatures &features, uint32_t ce
     return PL_OK;
 }
 
-int enqueue_apply(pl_lattice *h, float *output, const float *input, int reverse) {
+// The value passes for a lattice of doubles: plain splat, one blur launch per axis, slice.
+int enqueue_apply_f64(pl_lattice *h, double *output, const double *input, int reverse) {
+    const int pd = h->pd, vd = h->vd;
+    const int in_channels = h->normalize ? vd - 1 : vd;
+    const int mv = h->max_vertices();
+    double *values[2] = {reinterpret_cast<double *>(h->values[0]),
+                         reinterpret_cast<double *>(h->values[1])};
+    h->mark(EV_A0);
+    if (!h->values_zeroed)
+        PL_HIP(plk::fill_zero(h->values[0], (size_t)mv * vd * 2, h->stream));
+    h->mark(EV_FILL);
+    PL_HIP(plk::splat_f64(pd, vd, h->map, input, in_channels, h->replay, h->weights64,
+                          h->replay_holds_cells ? h->cell_vertex : nullptr, values[0],
+                          h->xcd_aware ? 1 : 0, h->stream));
+    h->replay_holds_cells = false;
+    h->values_zeroed = false;
+    h->mark(EV_SPLAT);
+    int cur = 0;
+    for (int step = 0; step <= pd; ++step) {
+        const int axis = reverse ? pd - step : step;
+        uint64_t *reset = (!h->table_clean && step == 0) ? h->cell_keys : nullptr;
+        PL_HIP(plk::blur_axis_f64(vd, h->counters(), mv, values[cur], values[1 - cur],
+                                  h->neighbours + (size_t)axis * mv, reset, h->vertex_cell,
+                                  h->launch_vertices(), h->stream));
+        if (reset) h->table_clean = true;
+        cur = 1 - cur;
+    }
+    h->mark(EV_BLUR);
+    PL_HIP(plk::slice_f64(pd, vd, h->map, h->replay, h->weights64, nullptr, values[cur], output,
+                          h->normalize ? 1 : 0, h->stream));
+    h->mark(EV_SLICE);
+    return PL_OK;
+}
+
+// output and input are arrays of the lattice's value type
+int enqueue_apply(pl_lattice *h, void *output_any, const void *input_any, int reverse) {
+    if (h->f64)
+        return enqueue_apply_f64(h, static_cast<double *>(output_any),
+                                 static_cast<const double *>(input_any), reverse);
+    float *output = static_cast<float *>(output_any);
+    const float *input = static_cast<const float *>(input_any);
     const int pd = h->pd, vd = h->vd;
     const int in_channels = h->normalize ? vd - 1 : vd;
     const int mv = h->max_vertices();
@@ -369,7 +435,8 @@ const char *pl_strerror(int status) {
 
 int pl_last_hip_error(void) { return g_last_hip_error; }
 
-int pl_create(int pd, int vd, int N, pl_stream stream, const pl_alloc *alloc, pl_handle *out) {
+static int create_lattice(int pd, int vd, int N, bool f64, pl_stream stream, const pl_alloc *alloc,
+                          pl_handle *out) {
     if (!out) return PL_EINVAL;
     *out = nullptr;
     if (N < 0 || pd < 1 || vd < 2) return PL_EINVAL;
@@ -384,6 +451,7 @@ int pl_create(int pd, int vd, int N, pl_stream stream, const pl_alloc *alloc, pl
     h->pd = pd;
     h->vd = vd;
     h->N = N;
+    h->f64 = f64;
     h->stream = (hipStream_t)stream;
     if (alloc) {
         h->alloc = *alloc;
@@ -393,6 +461,7 @@ int pl_create(int pd, int vd, int N, pl_stream stream, const pl_alloc *alloc, pl
         h->alloc.ctx = nullptr;
     }
     compute_scale_factor(pd, h->scale);
+    compute_scale_factor(pd, h->scale64);
     h->max_cells = pow2_at_least(rows * 2 < 4096 ? 4096 : rows * 2);  // holds N*(pd+1) vertices
     h->map = plk::make_point_map(N, 0, nullptr);
 
@@ -418,6 +487,14 @@ int pl_create(int pd, int vd, int N, pl_stream stream, const pl_alloc *alloc, pl
     return PL_OK;
 }
 
+int pl_create(int pd, int vd, int N, pl_stream stream, const pl_alloc *alloc, pl_handle *out) {
+    return create_lattice(pd, vd, N, false, stream, alloc, out);
+}
+
+int pl_create_f64(int pd, int vd, int N, pl_stream stream, const pl_alloc *alloc, pl_handle *out) {
+    return create_lattice(pd, vd, N, true, stream, alloc, out);
+}
+
 int pl_destroy(pl_handle h) {
     if (!h) return PL_OK;
     (void)hipStreamSynchronize(h->stream);
@@ -430,6 +507,7 @@ int pl_destroy(pl_handle h) {
     h->dfree(h->neighbours);
     h->dfree(h->cell_values);
     h->dfree(h->replay);
+    h->dfree(h->weights64);
     h->dfree(h->created_entries);
     h->dfree(h->block_count);
     h->dfree(h->chunk_count);
@@ -575,7 +653,8 @@ int features_from_image(pl_lattice *h, const float *reference, int n_reference_c
     return PL_OK;
 }
 
-int build_lattice(pl_lattice *h, const plk::PointFeatures &features) {
+int build_lattice(pl_lattice *h, const plk::PointFeatures &features,
+                  const double *positions64 = nullptr) {
     h->built = false;
     h->M = 0;
     for (int i = 0; i <= EV_NBR; ++i) h->ev_recorded[i] = false;
@@ -585,7 +664,7 @@ int build_lattice(pl_lattice *h, const plk::PointFeatures &features) {
     }
     uint32_t cells = initial_cells(h);
     for (;;) {
-        int rc = enqueue_build(h, features, cells, nullptr);
+        int rc = enqueue_build(h, features, positions64, cells, nullptr);
         if (rc != PL_OK) return rc;
         rc = verify_build(h, &cells);
         if (rc == PL_OK) return PL_OK;
@@ -596,8 +675,9 @@ int build_lattice(pl_lattice *h, const plk::PointFeatures &features) {
 // pl_filter in two halves.  begin: build and apply are enqueued together and the call returns.
 // end: waits for the lattice's stream; if the table turned out too small the whole call is
 // repeated with a larger one (the output is simply written again).
-int filter_begin(pl_lattice *h, float *output, const float *input,
-                 const plk::PointFeatures &features, int reverse) {
+int filter_begin(pl_lattice *h, void *output, const void *input,
+                 const plk::PointFeatures &features, int reverse,
+                 const double *positions64 = nullptr) {
     if (h->pending.active) return PL_ESTATE;
     h->built = false;
     h->M = 0;
@@ -607,12 +687,14 @@ int filter_begin(pl_lattice *h, float *output, const float *input,
         return PL_OK;
     }
     const uint32_t cells = initial_cells(h);
-    int rc = enqueue_build(h, features, cells, input);
+    // (only a lattice of floats splats in its build, and its input is then floats)
+    int rc = enqueue_build(h, features, positions64, cells, static_cast<const float *>(input));
     if (rc != PL_OK) return rc;
     rc = enqueue_apply(h, output, input, reverse);
     if (rc != PL_OK) return rc;
     h->pending.active = true;
     h->pending.features = features;
+    h->pending.positions64 = positions64;
     h->pending.output = output;
     h->pending.input = input;
     h->pending.reverse = reverse;
@@ -628,7 +710,8 @@ int filter_end(pl_lattice *h) {
             h->pending.active = false;
             return rc;
         }
-        rc = enqueue_build(h, h->pending.features, cells, h->pending.input);
+        rc = enqueue_build(h, h->pending.features, h->pending.positions64, cells,
+                           static_cast<const float *>(h->pending.input));
         if (rc == PL_OK) rc = enqueue_apply(h, h->pending.output, h->pending.input, h->pending.reverse);
         if (rc != PL_OK) {
             h->pending.active = false;
@@ -637,9 +720,10 @@ int filter_end(pl_lattice *h) {
     }
 }
 
-int filter_lattice(pl_lattice *h, float *output, const float *input,
-                   const plk::PointFeatures &features, int reverse) {
-    const int rc = filter_begin(h, output, input, features, reverse);
+int filter_lattice(pl_lattice *h, void *output, const void *input,
+                   const plk::PointFeatures &features, int reverse,
+                   const double *positions64 = nullptr) {
+    const int rc = filter_begin(h, output, input, features, reverse, positions64);
     return rc == PL_OK ? filter_end(h) : rc;
 }
 
@@ -647,6 +731,7 @@ int filter_lattice(pl_lattice *h, float *output, const float *input,
 
 int pl_build(pl_handle h, const float *positions) {
     if (!h || (!positions && h->N > 0)) return PL_EINVAL;
+    if (h->f64) return PL_EINVAL;   // a lattice of doubles: use the *_f64 entry points
     if (h->pending.active) return PL_ESTATE;
     const int rc = guess_point_grid(h, positions);
     if (rc != PL_OK) return rc;
@@ -657,6 +742,7 @@ int pl_build_image(pl_handle h, const float *reference, int n_reference_channels
                    int n_spatial_dims, const int *spatial_dims, float spatial_std,
                    float feature_std) {
     if (!h) return PL_EINVAL;
+    if (h->f64) return PL_EINVAL;   // a lattice of doubles: use the *_f64 entry points
     if (h->pending.active) return PL_ESTATE;
     plk::PointFeatures features;
     const int rc = features_from_image(h, reference, n_reference_channels, n_spatial_dims,
@@ -666,6 +752,7 @@ int pl_build_image(pl_handle h, const float *reference, int n_reference_channels
 
 int pl_apply(pl_handle h, float *output, const float *input, int reverse) {
     if (!h) return PL_EINVAL;
+    if (h->f64) return PL_EINVAL;   // a lattice of doubles: use the *_f64 entry points
     if (!h->built || !h->verified || h->pending.active) return PL_ESTATE;
     if (h->N == 0) return PL_OK;
     if (!output || !input) return PL_EINVAL;
@@ -674,6 +761,7 @@ int pl_apply(pl_handle h, float *output, const float *input, int reverse) {
 
 int pl_filter(pl_handle h, float *output, const float *input, const float *positions, int reverse) {
     if (!h) return PL_EINVAL;
+    if (h->f64) return PL_EINVAL;   // a lattice of doubles: use the *_f64 entry points
     if (h->N > 0 && (!output || !input || !positions)) return PL_EINVAL;
     if (h->pending.active) return PL_ESTATE;
     const int rc = guess_point_grid(h, positions);
@@ -685,6 +773,7 @@ int pl_filter_image(pl_handle h, float *output, const float *input, const float 
                     int n_reference_channels, int n_spatial_dims, const int *spatial_dims,
                     float spatial_std, float feature_std, int reverse) {
     if (!h) return PL_EINVAL;
+    if (h->f64) return PL_EINVAL;   // a lattice of doubles: use the *_f64 entry points
     if (h->pending.active) return PL_ESTATE;
     if (h->N > 0 && (!output || !input)) return PL_EINVAL;
     plk::PointFeatures features;
@@ -696,6 +785,7 @@ int pl_filter_image(pl_handle h, float *output, const float *input, const float 
 int pl_filter_begin(pl_handle h, float *output, const float *input, const float *positions,
                     int reverse) {
     if (!h) return PL_EINVAL;
+    if (h->f64) return PL_EINVAL;   // a lattice of doubles: use the *_f64 entry points
     if (h->N > 0 && (!output || !input || !positions)) return PL_EINVAL;
     if (h->pending.active) return PL_ESTATE;
     const int rc = guess_point_grid(h, positions);
@@ -707,12 +797,44 @@ int pl_filter_image_begin(pl_handle h, float *output, const float *input, const 
                           int n_reference_channels, int n_spatial_dims, const int *spatial_dims,
                           float spatial_std, float feature_std, int reverse) {
     if (!h) return PL_EINVAL;
+    if (h->f64) return PL_EINVAL;   // a lattice of doubles: use the *_f64 entry points
     if (h->pending.active) return PL_ESTATE;
     if (h->N > 0 && (!output || !input)) return PL_EINVAL;
     plk::PointFeatures features;
     const int rc = features_from_image(h, reference, n_reference_channels, n_spatial_dims,
                                        spatial_dims, spatial_std, feature_std, &features);
     return rc == PL_OK ? filter_begin(h, output, input, features, reverse) : rc;
+}
+
+// T = double: the same calls on a lattice made by pl_create_f64
+int pl_build_f64(pl_handle h, const double *positions) {
+    if (!h || !h->f64 || (!positions && h->N > 0)) return PL_EINVAL;
+    if (h->pending.active) return PL_ESTATE;
+    return build_lattice(h, plk::PointFeatures{}, positions);
+}
+
+int pl_apply_f64(pl_handle h, double *output, const double *input, int reverse) {
+    if (!h || !h->f64) return PL_EINVAL;
+    if (!h->built || !h->verified || h->pending.active) return PL_ESTATE;
+    if (h->N == 0) return PL_OK;
+    if (!output || !input) return PL_EINVAL;
+    return enqueue_apply(h, output, input, reverse);
+}
+
+int pl_filter_f64(pl_handle h, double *output, const double *input, const double *positions,
+                  int reverse) {
+    if (!h || !h->f64) return PL_EINVAL;
+    if (h->N > 0 && (!output || !input || !positions)) return PL_EINVAL;
+    if (h->pending.active) return PL_ESTATE;
+    return filter_lattice(h, output, input, plk::PointFeatures{}, reverse, positions);
+}
+
+int pl_debug_simplex_f64(pl_handle h, const double *positions, short *rem0, short *rank,
+                         short *keys, double *barycentric) {
+    if (!h || !h->f64 || (!positions && h->N > 0)) return PL_EINVAL;
+    PL_HIP(plk::debug_simplex_f64(h->pd, positions, h->N, h->scale64, rem0, rank, keys,
+                                  barycentric, h->stream));
+    return PL_OK;
 }
 
 int pl_filter_end(pl_handle h) {
@@ -745,6 +867,7 @@ int pl_stage_ms(pl_handle h, float ms[8]) {
 int pl_debug_simplex(pl_handle h, const float *positions, short *rem0, short *rank, short *keys,
                      float *barycentric) {
     if (!h || (!positions && h->N > 0)) return PL_EINVAL;
+    if (h->f64) return PL_EINVAL;   // a lattice of doubles: use the *_f64 entry points
     PL_HIP(plk::debug_simplex(h->pd, positions, h->N, h->scale, rem0, rank, keys, barycentric,
                               h->stream));
     return PL_OK;
@@ -759,6 +882,7 @@ int pl_debug_keys(pl_handle h, short *keys) {
 
 int pl_debug_replay(pl_handle h, int *vertex, float *weight) {
     if (!h) return PL_EINVAL;
+    if (h->f64) return PL_EINVAL;   // a lattice of doubles: use the *_f64 entry points
     if (!h->built || !h->verified) return PL_ESTATE;
     PL_HIP(plk::export_replay(h->pd, h->map, h->replay,
                               h->replay_holds_cells ? h->cell_vertex : nullptr, vertex, weight,
@@ -784,6 +908,27 @@ int pl_compute_positions(const float *reference, float *positions, int num_super
     PL_HIP(plk::compute_positions(reference, positions, num_super_pixels, n_reference_channels,
                                   n_spatial_dims, dims, spatial_std, feature_std,
                                   (hipStream_t)stream));
+    return PL_OK;
+}
+
+int pl_compute_positions_f64(const double *reference, double *positions, int num_super_pixels,
+                             int n_reference_channels, int n_spatial_dims, const int *spatial_dims,
+                             double spatial_std, double feature_std, pl_stream stream) {
+    if (num_super_pixels < 0 || n_reference_channels < 0 || n_spatial_dims < 0) return PL_EINVAL;
+    if (n_spatial_dims > plk::kMaxSpatialDims) return PL_EUNSUPPORTED;
+    if (n_spatial_dims + n_reference_channels < 1) return PL_EINVAL;
+    if (num_super_pixels == 0) return PL_OK;
+    if (!positions || (n_spatial_dims > 0 && !spatial_dims)) return PL_EINVAL;
+    if (n_reference_channels > 0 && !reference) return PL_EINVAL;
+    plk::SpatialDims dims{};
+    for (int i = 0; i < plk::kMaxSpatialDims; ++i) dims.v[i] = 1;
+    for (int i = 0; i < n_spatial_dims; ++i) {
+        if (spatial_dims[i] < 1) return PL_EINVAL;
+        dims.v[i] = spatial_dims[i];
+    }
+    PL_HIP(plk::compute_positions_f64(reference, positions, num_super_pixels, n_reference_channels,
+                                      n_spatial_dims, dims, spatial_std, feature_std,
+                                      (hipStream_t)stream));
     return PL_OK;
 }
 
@@ -958,4 +1103,65 @@ extern "C" int pl_set_op_concurrency(int lanes) {
     std::lock_guard<std::mutex> lock(g_op_cache_mutex);
     g_op_lanes = lanes;
     return PL_OK;
+}
+
+// The op for T = double (registered by the reference next to float,
+// src/LatticeFilterKernel.cpp:196-208): positions are built per item, as the reference does
+// (:153-160), and the items are filtered one after the other on one lattice, whose scratch and
+// the positions array come from `alloc` (NULL: hipMalloc) and are returned before the call ends.
+extern "C" int pl_lattice_filter_op_f64(const double *input, const double *reference, double *output,
+                                        int batch, int n_spatial_dims, const int *spatial_dims,
+                                        int n_input_channels, int n_reference_channels,
+                                        int bilateral, float theta_alpha, float theta_beta,
+                                        float theta_gamma, int reverse, pl_stream stream,
+                                        const pl_alloc *alloc) {
+    if (batch < 0 || n_spatial_dims < 1 || n_input_channels < 1 || !spatial_dims) return PL_EINVAL;
+    if (n_spatial_dims > plk::kMaxSpatialDims) return PL_EUNSUPPORTED;
+    if (alloc && (!alloc->alloc || !alloc->free)) return PL_EINVAL;
+    long long n = 1;
+    for (int i = 0; i < n_spatial_dims; ++i) {
+        if (spatial_dims[i] < 1) return PL_EINVAL;
+        n *= spatial_dims[i];
+        if (n > 2147483647LL) return PL_EOVERFLOW;
+    }
+    if (n * (long long)batch * n_input_channels > 2147483647LL) return PL_EOVERFLOW;
+    const int N = (int)n;
+    const int vd = n_input_channels + 1;
+    const int ref_ch = bilateral ? n_reference_channels : 0;
+    if (bilateral && (n_reference_channels < 1 || (!reference && batch > 0))) return PL_EINVAL;
+    const int pd = n_spatial_dims + ref_ch;
+    // the attributes are floats for every T (LatticeFilterKernel.cpp:36-38)
+    const double spatial_std = bilateral ? theta_alpha : theta_gamma;
+    const double feature_std = bilateral ? theta_beta : -1.0f;
+    if (!pl_supported(pd, vd)) return PL_EUNSUPPORTED;
+    if (batch == 0) return PL_OK;
+    if (!input || !output) return PL_EINVAL;
+
+    pl_alloc mem;
+    if (alloc) {
+        mem = *alloc;
+    } else {
+        mem.alloc = default_alloc;
+        mem.free = default_free;
+        mem.ctx = nullptr;
+    }
+    pl_handle lattice = nullptr;
+    int rc = pl_create_f64(pd, vd, N, stream, alloc, &lattice);
+    double *positions = nullptr;
+    if (rc == PL_OK) {
+        positions = (double *)mem.alloc(mem.ctx, sizeof(double) * (size_t)N * (size_t)pd);
+        if (!positions) rc = PL_ENOMEM;
+    }
+    if (rc == PL_OK) rc = pl_set_point_grid(lattice, n_spatial_dims, spatial_dims);
+    for (int b = 0; b < batch && rc == PL_OK; ++b) {
+        const double *ref_b = ref_ch ? reference + (size_t)b * N * ref_ch : nullptr;
+        rc = pl_compute_positions_f64(ref_b, positions, N, ref_ch, n_spatial_dims, spatial_dims,
+                                      spatial_std, feature_std, stream);
+        if (rc == PL_OK)
+            rc = pl_filter_f64(lattice, output + (size_t)b * N * n_input_channels,
+                               input + (size_t)b * N * n_input_channels, positions, reverse);
+    }
+    pl_destroy(lattice);   // synchronises the stream first
+    if (positions) mem.free(mem.ctx, positions);
+    return rc;
 }

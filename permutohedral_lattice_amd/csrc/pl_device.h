@@ -1,0 +1,373 @@
+// Device-side building blocks shared by the kernels for float values (pl_kernels.hip) and for
+// double values (pl_kernels_f64.hip): the packed vertex key and its hash, the simplex of a point,
+// the point <-> thread mapping, the wavefront election, the walk over vertex blocks, and the
+// host helpers that size grids.
+//
+// Translation units that include this must be compiled with -ffp-contract=off: the integer results
+// (nearest lattice point, rank permutation, vertex keys) are only equal to those of the reference
+// CPU path (src/PermutohedralLatticeCPU.h:220-304 of the reference tree) if every floating-point
+// operation of the embedding is a single IEEE operation.
+#ifndef PL_DEVICE_H
+#define PL_DEVICE_H
+
+#include <hip/hip_runtime.h>
+
+#include <cstdint>
+
+#include "pl_kernels.h"
+
+namespace plk {
+namespace device {
+
+constexpr int kBlock = 256;
+constexpr unsigned kXcds = 8;  // MI355X: 8 accelerator dies, each with its own L2
+
+// Workgroups are handed to the XCDs round-robin (workgroup b runs on XCD b % 8).  Points that are
+// close in memory share lattice vertices, so the kernels that update shared cells or values
+// atomically give each XCD one contiguous range of points: the contended lines then stay in
+// one L2 instead of migrating between dies.
+__device__ __forceinline__ unsigned xcd_contiguous_block(unsigned b, unsigned nb, int enabled) {
+    if (!enabled) return b;
+    const unsigned q = nb / kXcds, rem = nb % kXcds;
+    const unsigned xcd = b % kXcds, i = b / kXcds;
+    return xcd * q + (xcd < rem ? xcd : rem) + i;
+}
+
+template <int PD>
+struct KeyCodec {
+    static constexpr int kBits = (60 / PD) > 16 ? 16 : (60 / PD);
+    static constexpr int kBias = 1 << (kBits - 1);
+    // one step of margin on both sides so that a neighbour's coordinate never leaves its field
+    static constexpr int kMinQ = -kBias + 1;
+    static constexpr int kMaxQ = kBias - 2;
+    static constexpr uint64_t kFieldMask = (1ull << kBits) - 1ull;
+
+    __device__ static uint64_t pack(const int (&q)[PD], int r) {
+        uint64_t k = (uint64_t)(uint32_t)r << 60;
+#pragma unroll
+        for (int i = 0; i < PD; ++i) k |= (uint64_t)(uint32_t)(q[i] + kBias) << (i * kBits);
+        return k;
+    }
+    __device__ static void unpack(uint64_t k, int (&q)[PD], int &r) {
+        r = (int)(k >> 60);
+#pragma unroll
+        for (int i = 0; i < PD; ++i) q[i] = (int)((k >> (i * kBits)) & kFieldMask) - kBias;
+    }
+};
+
+__device__ __forceinline__ uint32_t hash_key(uint64_t k) {
+    uint32_t x = (uint32_t)k ^ ((uint32_t)(k >> 32) * 0x9E3779B1u);
+    x ^= x >> 16;
+    x *= 0x85EBCA6Bu;
+    x ^= x >> 13;
+    x *= 0xC2B2AE35u;
+    x ^= x >> 16;
+    return x;
+}
+
+// ------------------------------------------------------------------------------------------------
+// Per-point arithmetic: same operations, in the same precision and order, as
+// embed_position_vector / find_enclosing_simplex / compute_barycentric_coordinates of the
+// reference CPU path.  q[i] is rem0[i] / (pd+1).
+// ------------------------------------------------------------------------------------------------
+// T is the reference's value type
+template <int PD, typename T = float>
+struct Simplex {
+    int q[PD + 1];
+    int rank[PD + 1];
+    T weight[PD + 1];
+};
+
+template <int PD>
+__device__ __forceinline__ void enclosing_simplex(const float (&pos)[PD], const ScaleFactor &scale,
+                                                  Simplex<PD> &s) {
+    constexpr int D1 = PD + 1;
+    const double inv_d1 = 1.0 / (double)D1;
+
+    // elevate onto the hyperplane sum(x) = 0 (float, unfused)
+    float el[D1];
+    float running = 0.0f;
+#pragma unroll
+    for (int i = PD; i >= 1; --i) {
+        const float c = pos[i - 1] * scale.v[i - 1];
+        const float ic = (float)i * c;
+        el[i] = running - ic;
+        running = running + c;
+    }
+    el[0] = running;
+
+    // nearest remainder-0 point: round each coordinate to a multiple of pd+1, ties go down
+    float rem[D1];
+    int qsum = 0;
+#pragma unroll
+    for (int i = 0; i < D1; ++i) {
+        const float v = (float)((double)el[i] * inv_d1);
+        const float cu = ceilf(v), fl = floorf(v);
+        const float above = cu * (float)D1, below = fl * (float)D1;
+        const bool up = (above - el[i]) < (el[i] - below);
+        rem[i] = up ? above : below;
+        s.q[i] = (int)(up ? cu : fl);
+        qsum += s.q[i];
+    }
+
+    // rank[i] = number of coordinates with a larger residual.  One strict < per pair i < j decides
+    // ties exactly as the sequential loop does: true counts for i, false for j, so rank[i] starts
+    // at i (the pairs below it, all taken as false) and every true moves one count from j to i.
+    // The rounded point is qsum steps off the plane, which rotates the ranks by qsum.
+    float d[D1];
+    int rk[D1];
+#pragma unroll
+    for (int i = 0; i < D1; ++i) {
+        d[i] = el[i] - rem[i];
+        rk[i] = i + qsum;
+    }
+#pragma unroll
+    for (int i = 0; i < D1; ++i) {
+#pragma unroll
+        for (int j = i + 1; j < D1; ++j) {
+            const int lt = (d[i] < d[j]) ? 1 : 0;
+            rk[i] += lt;
+            rk[j] -= lt;
+        }
+    }
+    // ranks that left 0..pd wrap round, and their coordinate moves one step
+#pragma unroll
+    for (int i = 0; i < D1; ++i) {
+        const int step = rk[i] < 0 ? 1 : (rk[i] > PD ? -1 : 0);
+        s.rank[i] = rk[i] + step * D1;
+        s.q[i] += step;
+        rem[i] += (float)(step * D1);
+    }
+
+    // barycentric weights.  by_rank[k] is the scaled residual of the coordinate of rank k; the
+    // reference's scatter b[pd-rank] += delta, b[pd-rank+1] -= delta gives
+    // b[k] = by_rank[pd-k] - by_rank[pd-k+1] with one rounding, in either order of the two updates.
+    float by_rank[D1];
+#pragma unroll
+    for (int k = 0; k < D1; ++k) by_rank[k] = 0.0f;
+#pragma unroll
+    for (int i = 0; i < D1; ++i) {
+        const float delta = (float)((double)(el[i] - rem[i]) * inv_d1);
+#pragma unroll
+        for (int k = 0; k < D1; ++k) by_rank[k] = (s.rank[i] == k) ? delta : by_rank[k];
+    }
+#pragma unroll
+    for (int k = 1; k < D1; ++k) s.weight[k] = by_rank[PD - k] - by_rank[PD - k + 1];
+    s.weight[0] = (float)((double)by_rank[PD] + (1.0 + (double)(-by_rank[0])));
+}
+
+// The same for T = double.  All of it is double arithmetic except, as in the reference, the scaled
+// coordinate and its product with the index, which are floats for every T (`float cf`,
+// src/PermutohedralLatticeCPU.h:226).
+template <int PD>
+__device__ __forceinline__ void enclosing_simplex(const double (&pos)[PD], const ScaleFactor64 &scale,
+                                                  Simplex<PD, double> &s) {
+    constexpr int D1 = PD + 1;
+    const double inv_d1 = 1.0 / (double)D1;
+
+    double el[D1];
+    double running = 0.0;
+#pragma unroll
+    for (int i = PD; i >= 1; --i) {
+        const float c = (float)(pos[i - 1] * scale.v[i - 1]);
+        const float ic = (float)i * c;
+        el[i] = running - (double)ic;
+        running = running + (double)c;
+    }
+    el[0] = running;
+
+    double rem[D1];
+    int qsum = 0;
+#pragma unroll
+    for (int i = 0; i < D1; ++i) {
+        const double v = el[i] * inv_d1;
+        const double cu = ceil(v), fl = floor(v);
+        const double above = cu * (double)D1, below = fl * (double)D1;
+        const bool up = (above - el[i]) < (el[i] - below);
+        rem[i] = up ? above : below;
+        s.q[i] = (int)(up ? cu : fl);
+        qsum += s.q[i];
+    }
+
+    double d[D1];
+    int rk[D1];
+#pragma unroll
+    for (int i = 0; i < D1; ++i) {
+        d[i] = el[i] - rem[i];
+        rk[i] = i + qsum;
+    }
+#pragma unroll
+    for (int i = 0; i < D1; ++i) {
+#pragma unroll
+        for (int j = i + 1; j < D1; ++j) {
+            const int lt = (d[i] < d[j]) ? 1 : 0;
+            rk[i] += lt;
+            rk[j] -= lt;
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < D1; ++i) {
+        const int step = rk[i] < 0 ? 1 : (rk[i] > PD ? -1 : 0);
+        s.rank[i] = rk[i] + step * D1;
+        s.q[i] += step;
+        rem[i] += (double)(step * D1);
+    }
+
+    double by_rank[D1];
+#pragma unroll
+    for (int k = 0; k < D1; ++k) by_rank[k] = 0.0;
+#pragma unroll
+    for (int i = 0; i < D1; ++i) {
+        const double delta = (el[i] - rem[i]) * inv_d1;
+#pragma unroll
+        for (int k = 0; k < D1; ++k) by_rank[k] = (s.rank[i] == k) ? delta : by_rank[k];
+    }
+#pragma unroll
+    for (int k = 1; k < D1; ++k) s.weight[k] = by_rank[PD - k] - by_rank[PD - k + 1];
+    s.weight[0] = by_rank[PD] + (1.0 + (-by_rank[0]));
+}
+
+// q-coordinates of simplex vertex r: the coordinates ranked above pd-r drop by one step
+template <int PD, typename T>
+__device__ __forceinline__ void vertex_q(const Simplex<PD, T> &s, int r, int (&q)[PD]) {
+#pragma unroll
+    for (int i = 0; i < PD; ++i) q[i] = s.q[i] - ((s.rank[i] > PD - r) ? 1 : 0);
+}
+
+template <int PD, typename T>
+__device__ __forceinline__ bool simplex_in_key_range(const Simplex<PD, T> &s) {
+    bool ok = true;
+#pragma unroll
+    for (int i = 0; i < PD; ++i)
+        ok = ok && (s.q[i] - 1 >= KeyCodec<PD>::kMinQ) && (s.q[i] <= KeyCodec<PD>::kMaxQ);
+    return ok;
+}
+
+// ------------------------------------------------------------------------------------------------
+// Which point a thread works on.  Points that are neighbours in the image share lattice vertices,
+// and every duplicate that meets inside one wavefront is merged before it reaches memory, so a
+// wavefront should cover a compact tile of the image, not a run of 64 points of one row.  With a
+// grid hint (the op knows its spatial extents) a workgroup takes a 16x16 tile of a 2-D grid
+// (wavefronts 8x8) or a 4x8x8 tile of a 3-D grid (wavefronts 4x4x4); without one it takes 256
+// consecutive points.  The mapping only changes the order of work, never a result.
+// Per-point scratch (the replay arrays) is stored in thread order, so it stays coalesced.
+// ------------------------------------------------------------------------------------------------
+__device__ __forceinline__ int point_of_thread(const PointMap &m, unsigned vblock, unsigned tid) {
+    if (m.mode == 0) {
+        const size_t n = (size_t)vblock * kBlock + tid;
+        return n < (size_t)m.N ? (int)n : -1;
+    }
+    const unsigned wave = tid >> 6, lane = tid & 63;
+    const unsigned tiles_yx = (unsigned)m.tiles[1] * (unsigned)m.tiles[2];
+    const unsigned tz = vblock / tiles_yx;
+    const unsigned rest = vblock - tz * tiles_yx;
+    const unsigned ty = rest / (unsigned)m.tiles[2];
+    const unsigned tx = rest - ty * (unsigned)m.tiles[2];
+    unsigned z, y, x;
+    if (m.mode == 2) {
+        z = tz;
+        y = ty * 16 + (wave >> 1) * 8 + (lane >> 3);
+        x = tx * 16 + (wave & 1) * 8 + (lane & 7);
+    } else {
+        z = tz * 4 + (lane >> 4);
+        y = ty * 8 + (wave >> 1) * 4 + ((lane >> 2) & 3);
+        x = tx * 8 + (wave & 1) * 4 + (lane & 3);
+    }
+    if (z >= (unsigned)m.dims[0] || y >= (unsigned)m.dims[1] || x >= (unsigned)m.dims[2]) return -1;
+    return (int)(((size_t)z * m.dims[1] + y) * m.dims[2] + x);
+}
+
+// Mask of the lanes whose predicate holds (the compare result itself, no detour through 0/1)
+__device__ __forceinline__ uint64_t wave_ballot(bool predicate) {
+    return __builtin_amdgcn_ballot_w64(predicate);
+}
+
+// Mask of the (executing) lanes whose x equals the wavefront-uniform k, straight from the compare
+__device__ __forceinline__ uint64_t lanes_equal(uint64_t x, uint64_t k) {
+    return __builtin_amdgcn_uicmpl(x, k, 32 /* ICMP_EQ */);
+}
+__device__ __forceinline__ uint64_t lanes_equal(int x, int k) {
+    return __builtin_amdgcn_uicmp((unsigned)x, (unsigned)k, 32 /* ICMP_EQ */);
+}
+// A lane mask as a per-lane predicate
+__device__ __forceinline__ bool lane_in(uint64_t mask) {
+    return __builtin_amdgcn_inverse_ballot_w64(mask);
+}
+
+__device__ __forceinline__ int lane_value(int x, int lane) { return __builtin_amdgcn_readlane(x, lane); }
+__device__ __forceinline__ uint64_t lane_value(uint64_t x, int lane) {
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)x, lane);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(x >> 32), lane);
+    return ((uint64_t)hi << 32) | lo;
+}
+
+// Lanes that hold the same value of `x` elect the lowest of them as leader.  Returns the leader's
+// lane; inactive lanes get their own.  One iteration per distinct value in the wavefront, each a
+// v_readlane of the first unassigned lane's value, a compare and a ballot.
+template <typename T>
+__device__ __forceinline__ int wave_leader_of_equal(T x, bool active, int lane) {
+    int leader = lane;
+    const uint64_t among = wave_ballot(active);
+    uint64_t remaining = among;
+    while (remaining) {
+        const int first = __builtin_ctzll(remaining);
+        const uint64_t same = lanes_equal(x, lane_value(x, first)) & among;
+        if (lane_in(same)) leader = first;
+        remaining &= ~same;
+    }
+    return leader;
+}
+
+__device__ __forceinline__ int vertex_count(const Counters *counters, int max_vertices) {
+    const uint32_t m = counters->vertices;
+    return m < (uint32_t)max_vertices ? (int)m : max_vertices;
+}
+
+// The vertex count is only known on the device, so kernels over the vertices are launched for an
+// estimate (the count of the lattice's previous build, with a margin) and every workgroup walks
+// the blocks of 256 items in strides of the grid: a launch for the most vertices the table can
+// hold would spend more time dispatching empty workgroups than the passes spend working.
+// Workgroup b runs on XCD b % 8 and each XCD has its own L2, so the blocks are dealt out such
+// that every XCD gets one contiguous eighth of the items (the grid is a multiple of 8): with
+// vertex numbers that follow the image, the vertices a workgroup gathers from are then mostly
+// ones its own XCD works on.
+struct ItemBlocks {
+    unsigned n_active, chunk, k;
+    __device__ explicit ItemBlocks(size_t n_items)
+        : n_active((unsigned)((n_items + kBlock - 1) / kBlock)), chunk((n_active + 7u) / 8u),
+          k(blockIdx.x) {}
+    __device__ bool next(unsigned &block) {
+        while (k < 8u * chunk) {
+            block = (k & 7u) * chunk + (k >> 3);
+            k += gridDim.x;
+            if (block < n_active) return true;
+        }
+        return false;
+    }
+};
+
+inline unsigned blocks_for(size_t n, int block = kBlock) { return (unsigned)((n + block - 1) / block); }
+// grids of the kernels that walk their items with ItemBlocks: a multiple of 8
+inline unsigned vertex_blocks(size_t n_items) {
+    const unsigned b = (blocks_for(n_items) + 7u) & ~7u;
+    return b ? b : 8u;
+}
+
+#define PLK_DISPATCH_PD(pd, CALL)                 \
+    switch (pd) {                                 \
+        case 1: { constexpr int PD = 1; CALL; } break; \
+        case 2: { constexpr int PD = 2; CALL; } break; \
+        case 3: { constexpr int PD = 3; CALL; } break; \
+        case 4: { constexpr int PD = 4; CALL; } break; \
+        case 5: { constexpr int PD = 5; CALL; } break; \
+        case 6: { constexpr int PD = 6; CALL; } break; \
+        case 7: { constexpr int PD = 7; CALL; } break; \
+        case 8: { constexpr int PD = 8; CALL; } break; \
+        default: return hipErrorInvalidValue;     \
+    }
+
+
+}  // namespace device
+}  // namespace plk
+
+#endif

@@ -1,5 +1,5 @@
 // Internal launch interface between the host-side lattice object (pl_api.cpp) and the gfx950
-// kernels (pl_kernels.hip).  Not part of the public ABI.
+// kernels (pl_kernels.hip for float values, pl_kernels_f64.hip for double values).  Not part of the public ABI.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -54,6 +54,16 @@ struct ReplayEntry {
 
 struct ScaleFactor {
     float v[kMaxPd];
+};
+struct ScaleFactor64 {
+    double v[kMaxPd];
+};
+// What the build reads and writes for double values: positions N x pd, and the barycentric
+// weights in the layout of the replay rows.
+struct Points64 {
+    const double *positions;
+    double *weights;
+    ScaleFactor64 scale;
 };
 
 struct SpatialDims {
@@ -115,6 +125,12 @@ hipError_t build(int pd, const PointFeatures &features, const PointMap &map, con
                  int in_channels, float *cell_values, const CreatedLists &created_lists,
                  hipStream_t s);
 
+// The build for double values: the same kernel on points.positions with points.scale; replay[]
+// receives the cells (and the weights rounded to float), points.weights[r*T+t] the weights.
+hipError_t build_f64(int pd, const Points64 &points, const PointMap &map, uint64_t *cell_keys,
+                     uint32_t n_cells, Counters *counters, ReplayEntry *replay, int xcd_aware,
+                     const CreatedLists &created_lists, hipStream_t s);
+
 // Dense vertex numbers in the order of the build's workgroups (same map as the build):
 // cell_vertex[cell] := v, vertex_keys[v] := key, vertex_cell[v] := cell,
 // neighbours[a][v] := (-1, -1) for a <= pd, counters->vertices := M, and the vertex's row of
@@ -172,6 +188,25 @@ hipError_t export_keys(int pd, const uint64_t *vertex_keys, int M, short *keys, 
 hipError_t export_replay(int pd, const PointMap &map, const ReplayEntry *replay,
                          const int *cell_vertex, int *vertex,
                          float *weight, hipStream_t s);
+
+// The value passes for double values (pl_kernels_f64.hip): as splat, blur_axis, slice,
+// debug_simplex and compute_positions above, with `weights` (thread order, like the replay rows)
+// carrying the barycentric weights the double build wrote.
+hipError_t splat_f64(int pd, int vd, const PointMap &map, const double *input, int in_channels,
+                     ReplayEntry *replay, const double *weights, const int *cell_vertex,
+                     double *values, int xcd_aware, hipStream_t s);
+hipError_t blur_axis_f64(int vd, const Counters *counters, int max_vertices, const double *src,
+                         double *dst, const int2 *neighbours_of_axis, uint64_t *reset_cell_keys,
+                         const int *vertex_cell, int launch_vertices, hipStream_t s);
+hipError_t slice_f64(int pd, int vd, const PointMap &map, const ReplayEntry *replay,
+                     const double *weights, const int *cell_vertex, const double *values,
+                     double *output, int normalize, hipStream_t s);
+hipError_t debug_simplex_f64(int pd, const double *positions, int N, const ScaleFactor64 &scale,
+                             short *rem0, short *rank, short *keys, double *barycentric,
+                             hipStream_t s);
+hipError_t compute_positions_f64(const double *reference, double *positions, int N,
+                                 int n_ref_channels, int n_spatial_dims, const SpatialDims &dims,
+                                 double spatial_std, double feature_std, hipStream_t s);
 
 // First index at which feature 0 (period[0]) and feature 1 (period[1]) of consecutive points
 // differ, and whether all their changes lie exactly at the multiples of those indices.

@@ -1,0 +1,206 @@
+// gfx950 kernels of the permutohedral-lattice filter for T = double, the other value type the
+// reference registers (src/LatticeFilterKernel.cpp:196-208).
+//
+// The lattice itself (keys, hash table, vertex numbering, neighbour table) is what the float path
+// builds: the build kernel is instantiated for double positions in pl_kernels.hip, and the
+// numbering and neighbour passes do not look at values.  What is here are the passes that touch
+// values: splat, blur and slice on rows of doubles, the feature builder and the per-point dump.
+// They are the plain forms (one atomic per point, vertex and channel in the splat; one thread per
+// (vertex, channel) in the blur): the float path is the one tuned for speed.
+//
+// Arithmetic follows the reference CPU path with T = double: the three-tap blur and the reciprocal
+// of the slice are double expressions there for every T.  The splat adds in a different order
+// than the sequential CPU loop, so values agree to rounding (1e-16 relative per addition), not
+// bit for bit; the integers of the lattice agree exactly.
+#include "pl_device.h"
+#include "pl_kernels.h"
+
+namespace plk {
+
+namespace {
+
+using namespace device;
+
+// replay rows and weights are stored in thread order, [r][t], like the float path's
+template <int D1>
+__global__ __launch_bounds__(kBlock) void k_splat_f64(int vd, PointMap map,
+                                                       const double *__restrict__ input,
+                                                       int in_channels, ReplayEntry *replay,
+                                                       const double *__restrict__ weights,
+                                                       const int *__restrict__ cell_vertex,
+                                                       double *values, int xcd_aware) {
+    const unsigned vblock = xcd_contiguous_block(blockIdx.x, gridDim.x, xcd_aware);
+    const size_t t = (size_t)vblock * kBlock + threadIdx.x;
+    const size_t n_slots = (size_t)gridDim.x * kBlock;
+    const int n = point_of_thread(map, vblock, threadIdx.x);
+    if (n < 0) return;
+    const double *value = input + (size_t)n * in_channels;
+#pragma unroll
+    for (int r = 0; r < D1; ++r) {
+        int v = replay[(size_t)r * n_slots + t].index;
+        if (v < 0) continue;   // the build could not place this point's keys and has said so
+        if (cell_vertex) {
+            v = cell_vertex[v];
+            replay[(size_t)r * n_slots + t].index = v;
+        }
+        const double w = weights[(size_t)r * n_slots + t];
+        double *row = values + (size_t)v * vd;
+        for (int j = 0; j < in_channels; ++j) atomicAdd(row + j, w * value[j]);
+        if (in_channels == vd - 1) atomicAdd(row + vd - 1, w);   // homogeneous channel
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void k_blur_f64(const Counters *counters, int max_vertices,
+                                                      int vd, const double *__restrict__ src,
+                                                      double *__restrict__ dst,
+                                                      const int2 *__restrict__ nbr,
+                                                      uint64_t *reset_cell_keys,
+                                                      const int *__restrict__ vertex_cell) {
+    const int M = vertex_count(counters, max_vertices);
+    ItemBlocks blocks((size_t)M * vd);
+    unsigned eb;
+    while (blocks.next(eb)) {
+        const size_t e = (size_t)eb * kBlock + threadIdx.x;
+        if (e >= (size_t)M * vd) continue;
+        const int v = (int)(e / (size_t)vd);
+        const int j = (int)(e - (size_t)v * vd);
+        const int2 nb = nbr[v];
+        const double a = nb.x >= 0 ? src[(size_t)nb.x * vd + j] : 0.0;
+        const double b = nb.y >= 0 ? src[(size_t)nb.y * vd + j] : 0.0;
+        dst[e] = 0.25 * a + 0.5 * src[e] + 0.25 * b;
+        if (reset_cell_keys && j == 0) reset_cell_keys[vertex_cell[v]] = kEmptyCell;
+    }
+}
+
+// One thread per point and output channel: its channel's sum and the homogeneous channel's.
+template <int D1>
+__global__ __launch_bounds__(kBlock) void k_slice_f64(int vd, PointMap map,
+                                                       const ReplayEntry *__restrict__ replay,
+                                                       const double *__restrict__ weights,
+                                                       const int *__restrict__ cell_vertex,
+                                                       const double *__restrict__ values,
+                                                       double *__restrict__ output, int normalize) {
+    const int out_channels = normalize ? vd - 1 : vd;
+    const unsigned vblock = blockIdx.x;
+    const size_t t = (size_t)vblock * kBlock + threadIdx.x;
+    const size_t n_slots = (size_t)gridDim.x * kBlock;
+    const int n = point_of_thread(map, vblock, threadIdx.x);
+    if (n < 0) return;
+    const int j = blockIdx.y;
+    double sum = 0.0, homogeneous = 0.0;
+#pragma unroll
+    for (int r = 0; r < D1; ++r) {
+        int v = replay[(size_t)r * n_slots + t].index;
+        if (v < 0) continue;
+        if (cell_vertex) v = cell_vertex[v];
+        const double w = weights[(size_t)r * n_slots + t];
+        const double *row = values + (size_t)v * vd;
+        sum += w * row[j];
+        homogeneous += w * row[vd - 1];
+    }
+    output[(size_t)n * out_channels + j] = normalize ? sum * (1.0 / homogeneous) : sum;
+}
+
+template <int PD>
+__global__ __launch_bounds__(kBlock) void k_debug_simplex_f64(const double *__restrict__ positions,
+                                                               int N, ScaleFactor64 scale,
+                                                               short *rem0, short *rank, short *keys,
+                                                               double *barycentric) {
+    constexpr int D1 = PD + 1;
+    const int n = blockIdx.x * kBlock + threadIdx.x;
+    if (n >= N) return;
+    double pos[PD];
+#pragma unroll
+    for (int i = 0; i < PD; ++i) pos[i] = positions[(size_t)n * PD + i];
+    Simplex<PD, double> s;
+    enclosing_simplex<PD>(pos, scale, s);
+#pragma unroll
+    for (int i = 0; i < D1; ++i) {
+        if (rem0) rem0[(size_t)n * D1 + i] = (short)(s.q[i] * D1);
+        if (rank) rank[(size_t)n * D1 + i] = (short)s.rank[i];
+        if (barycentric) barycentric[(size_t)n * D1 + i] = s.weight[i];
+    }
+    if (keys) {
+#pragma unroll
+        for (int r = 0; r < D1; ++r) {
+            int q[PD];
+            vertex_q<PD>(s, r, q);
+#pragma unroll
+            for (int i = 0; i < PD; ++i)
+                keys[((size_t)n * D1 + r) * PD + i] = (short)(q[i] * D1 + r);
+        }
+    }
+}
+
+// reference: compute_kernel_cpu<double>, src/PermutohedralLatticeCPU.h:452-474
+__global__ __launch_bounds__(kBlock) void k_positions_f64(const double *__restrict__ reference,
+                                                           double *__restrict__ positions, int N,
+                                                           int rc, int nsd, SpatialDims dims,
+                                                           double spatial_std, double feature_std) {
+    const int n = blockIdx.x * kBlock + threadIdx.x;
+    if (n >= N) return;
+    const int pd = nsd + rc;
+    double *row = positions + (size_t)n * pd;
+    int stride = 1;
+    for (int s = nsd - 1; s >= 0; --s) {
+        const int coord = (n / stride) % dims.v[s];
+        row[s] = (double)coord / spatial_std;
+        stride *= dims.v[s];
+    }
+    for (int c = 0; c < rc; ++c) row[nsd + c] = reference[(size_t)n * rc + c] / feature_std;
+}
+
+}  // namespace
+
+hipError_t splat_f64(int pd, int vd, const PointMap &map, const double *input, int in_channels,
+                     ReplayEntry *replay, const double *weights, const int *cell_vertex,
+                     double *values, int xcd_aware, hipStream_t s) {
+    if (map.n_blocks == 0) return hipSuccess;
+    PLK_DISPATCH_PD(pd, hipLaunchKernelGGL(k_splat_f64<PD + 1>, dim3(map.n_blocks), dim3(kBlock), 0,
+                                           s, vd, map, input, in_channels, replay, weights,
+                                           cell_vertex, values, xcd_aware));
+    return hipGetLastError();
+}
+
+hipError_t blur_axis_f64(int vd, const Counters *counters, int max_vertices, const double *src,
+                         double *dst, const int2 *neighbours_of_axis, uint64_t *reset_cell_keys,
+                         const int *vertex_cell, int launch_vertices, hipStream_t s) {
+    if (max_vertices <= 0) return hipSuccess;
+    hipLaunchKernelGGL(k_blur_f64, dim3(vertex_blocks((size_t)launch_vertices * vd)), dim3(kBlock),
+                       0, s, counters, max_vertices, vd, src, dst, neighbours_of_axis,
+                       reset_cell_keys, vertex_cell);
+    return hipGetLastError();
+}
+
+hipError_t slice_f64(int pd, int vd, const PointMap &map, const ReplayEntry *replay,
+                     const double *weights, const int *cell_vertex, const double *values,
+                     double *output, int normalize, hipStream_t s) {
+    if (map.n_blocks == 0) return hipSuccess;
+    const unsigned out_channels = (unsigned)(normalize ? vd - 1 : vd);
+    PLK_DISPATCH_PD(pd, hipLaunchKernelGGL(k_slice_f64<PD + 1>, dim3(map.n_blocks, out_channels),
+                                           dim3(kBlock), 0, s, vd, map, replay, weights,
+                                           cell_vertex, values, output, normalize));
+    return hipGetLastError();
+}
+
+hipError_t debug_simplex_f64(int pd, const double *positions, int N, const ScaleFactor64 &scale,
+                             short *rem0, short *rank, short *keys, double *barycentric,
+                             hipStream_t s) {
+    if (N <= 0) return hipSuccess;
+    PLK_DISPATCH_PD(pd, hipLaunchKernelGGL(k_debug_simplex_f64<PD>, dim3(blocks_for((size_t)N)),
+                                           dim3(kBlock), 0, s, positions, N, scale, rem0, rank,
+                                           keys, barycentric));
+    return hipGetLastError();
+}
+
+hipError_t compute_positions_f64(const double *reference, double *positions, int N,
+                                 int n_ref_channels, int n_spatial_dims, const SpatialDims &dims,
+                                 double spatial_std, double feature_std, hipStream_t s) {
+    if (N <= 0) return hipSuccess;
+    hipLaunchKernelGGL(k_positions_f64, dim3(blocks_for((size_t)N)), dim3(kBlock), 0, s, reference,
+                       positions, N, n_ref_channels, n_spatial_dims, dims, spatial_std,
+                       feature_std);
+    return hipGetLastError();
+}
+
+}  // namespace plk
