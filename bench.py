@@ -143,7 +143,28 @@ def run_side_legs(args, pla, synth, lat, step, img, d_pos, d_val, d_grad, out_f,
     pla.set_op_concurrency(4)
     del b_img, b_grad
 
-    return plain_ms, reuse_ms, op_ms, batch_ms
+    # the same step on a lattice of doubles (the reference's T = double), grid hint set
+    lat64 = pla.PermutohedralLattice(lat.pd, lat.vd, lat.N, dtype=torch.float64)
+    lat64.set_point_grid((side, side))
+    pos64, val64, grad64 = d_pos.double(), d_val.double(), d_grad.double()
+    out64 = torch.empty_like(val64)
+
+    def step64():
+        lat64.filter(out64, val64, pos64, False)
+        lat64.filter(out64, grad64, pos64, True)
+
+    for _ in range(2):
+        step64()
+    torch.cuda.synchronize()
+    reps = max(3, args.steps // 5)
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        step64()
+    torch.cuda.synchronize()
+    double_ms = 1e3 * (time.perf_counter() - t0) / reps
+    lat64.close()
+
+    return plain_ms, reuse_ms, op_ms, batch_ms, double_ms
 
 
 def main():
@@ -215,10 +236,10 @@ def main():
     value = pixels_per_step / (ms_per_step * 1e-3) / 1e6
 
     side_legs = not args.headline_only
-    plain_ms, reuse_ms = {}, 0.0
+    plain_ms, reuse_ms, double_ms = {}, 0.0, 0.0
     op_ms, batch_ms, batch = {}, {}, 4
     if side_legs:
-        plain_ms, reuse_ms, op_ms, batch_ms = run_side_legs(args, pla, synth, lat, step, img, d_pos,
+        plain_ms, reuse_ms, op_ms, batch_ms, double_ms = run_side_legs(args, pla, synth, lat, step, img, d_pos,
                                                             d_val, d_grad, out_f, out_r, side, batch)
 
     # per-kernel durations from HIP events on the lattice's stream
@@ -290,6 +311,9 @@ def main():
                          "ms_per_step": {k: round(v, 4) for k, v in batch_ms.items()},
                          "value": {k: round(batch * pixels_per_step / (v * 1e-3) / 1e6, 3)
                                    for k, v in batch_ms.items()}},
+            "double": {"what": "same step on a lattice of doubles (plain value passes, not the tuned ones)",
+                       "ms_per_step": round(double_ms, 4),
+                       "value": round(pixels_per_step / (double_ms * 1e-3) / 1e6, 3)},
         })
 
     if not args.no_cpu and not args.headline_only:

@@ -10,7 +10,9 @@
 //        OpKernelContext* becomes an optional allocator);
 //   * lattice_filter(...) -- LatticeFilterOp::Compute (src/LatticeFilterKernel.cpp:98-181).
 //
-// Errors are thrown as PermutohedralError (the reference GPU path calls exit()).  Only T = float.
+// Errors are thrown as PermutohedralError (the reference GPU path calls exit()).  T = float and
+// T = double, the two types the reference registers (src/LatticeFilterKernel.cpp:196-208); the
+// fused feature builder (filter_image, build_image) exists for float only.
 #ifndef PERMUTOHEDRAL_LATTICE_HPP
 #define PERMUTOHEDRAL_LATTICE_HPP
 
@@ -99,6 +101,38 @@ private:
     pl_handle handle_ = nullptr;
 };
 
+template <>
+class PermutohedralLatticeHIP<double> {
+public:
+    PermutohedralLatticeHIP(int pd, int vd, int N, pl_stream stream = nullptr,
+                            const pl_alloc *allocator = nullptr) {
+        check(pl_create_f64(pd, vd, N, stream, allocator, &handle_), "pl_create_f64");
+    }
+    ~PermutohedralLatticeHIP() { pl_destroy(handle_); }
+    PermutohedralLatticeHIP(const PermutohedralLatticeHIP &) = delete;
+    PermutohedralLatticeHIP &operator=(const PermutohedralLatticeHIP &) = delete;
+
+    void filter(double *output, const double *input, const double *positions, bool reverse) {
+        check(pl_filter_f64(handle_, output, input, positions, reverse ? 1 : 0), "pl_filter_f64");
+    }
+    void build(const double *positions) { check(pl_build_f64(handle_, positions), "pl_build_f64"); }
+    void apply(double *output, const double *input, bool reverse) {
+        check(pl_apply_f64(handle_, output, input, reverse ? 1 : 0), "pl_apply_f64");
+    }
+    void set_point_grid(int n_dims, const int *dims) {
+        check(pl_set_point_grid(handle_, n_dims, dims), "pl_set_point_grid");
+    }
+    int size() const {
+        int m = 0;
+        check(pl_num_vertices(handle_, &m), "pl_num_vertices");
+        return m;
+    }
+    pl_handle handle() const { return handle_; }
+
+private:
+    pl_handle handle_ = nullptr;
+};
+
 template <typename Device, typename T>
 struct LatticeFilter;
 template <typename Device, typename T>
@@ -125,6 +159,29 @@ struct ComputeKernel<HipDevice, float> {
     }
 };
 
+template <>
+struct LatticeFilter<HipDevice, double> {
+    void operator()(const HipDevice &d, const pl_alloc *allocator, double *output,
+                    const double *input, const double *positions, int num_super_pixels, int pd,
+                    int vd, bool reverse) {
+        PermutohedralLatticeHIP<double> lattice(pd, vd, num_super_pixels, d.stream(), allocator);
+        lattice.filter(output, input, positions, reverse);
+    }
+};
+
+template <>
+struct ComputeKernel<HipDevice, double> {
+    void operator()(const HipDevice &d, const pl_alloc * /*allocator*/,
+                    const double *reference_image, double *positions, int num_super_pixels,
+                    int n_spatial_dims, int *spatial_dims, int n_reference_channels,
+                    double spatial_std, double features_std) {
+        check(pl_compute_positions_f64(reference_image, positions, num_super_pixels,
+                                       n_reference_channels, n_spatial_dims, spatial_dims,
+                                       spatial_std, features_std, d.stream()),
+              "pl_compute_positions_f64");
+    }
+};
+
 // The op on channels-last device tensors [batch, s_1..s_k, C]; attrs as in REGISTER_OP("LatticeFilter").
 inline void lattice_filter(const HipDevice &d, const float *input_image, const float *reference_image,
                            float *output, int batch, int n_spatial_dims, const int *spatial_dims,
@@ -136,6 +193,19 @@ inline void lattice_filter(const HipDevice &d, const float *input_image, const f
                                theta_alpha, theta_beta, theta_gamma, reverse ? 1 : 0, d.stream(),
                                allocator),
           "pl_lattice_filter_op");
+}
+
+inline void lattice_filter(const HipDevice &d, const double *input_image,
+                           const double *reference_image, double *output, int batch,
+                           int n_spatial_dims, const int *spatial_dims, int n_input_channels,
+                           int n_reference_channels, bool bilateral = true, float theta_alpha = 1.0f,
+                           float theta_beta = 1.0f, float theta_gamma = 1.0f, bool reverse = false,
+                           const pl_alloc *allocator = nullptr) {
+    check(pl_lattice_filter_op_f64(input_image, reference_image, output, batch, n_spatial_dims,
+                                   spatial_dims, n_input_channels, n_reference_channels,
+                                   bilateral ? 1 : 0, theta_alpha, theta_beta, theta_gamma,
+                                   reverse ? 1 : 0, d.stream(), allocator),
+          "pl_lattice_filter_op_f64");
 }
 
 }  // namespace permutohedral

@@ -212,7 +212,8 @@ int pl_lattice_filter_op(const float *input, const float *reference, float *outp
 /*
  * How many batch items pl_lattice_filter_op (with alloc = NULL) keeps in flight at once, each on a
  * lattice and a stream of its own (1..8, default 4; 1 = one after the other as the reference's
- * loop, src/LatticeFilterKernel.cpp:152-179).  Process-wide.
+ * loop, src/LatticeFilterKernel.cpp:152-179).  Items of more than 2^19 points run at most two at
+ * a time whatever is set: their kernels fill the GPU.  Process-wide.
  */
 int pl_set_op_concurrency(int lanes);
 

@@ -125,3 +125,30 @@ def test_op_with_caller_scratch_returns_everything_before_it_returns():
     got = out.cpu().numpy()
     assert np.abs(got - want).max() <= MAX_ABS_TOL and rel_l2(got, want) <= REL_L2_TOL
     assert scratch.n_alloc > 0 and not scratch.live and scratch.n_free == scratch.n_alloc
+
+
+def test_double_op_with_caller_scratch_returns_everything_before_it_returns():
+    b, h, w = 2, 40, 44
+    guide = np.stack([synth.blob_image(h, w, seed=99 + i) for i in range(b)]).astype(np.float64)
+    inp = synth.uniform_image((b, h, w, 2), 101).astype(np.float64)
+    want = oracle.lattice_filter(inp, guide, True, 8.0, 0.125, 1.0, False)
+    scratch = TorchScratch()
+    d_in, d_ref = dev(inp), dev(guide)
+    out = torch.empty_like(d_in)
+    dims = (C.c_int * 2)(h, w)
+    rc = pla._lib.pl_lattice_filter_op_f64(d_in.data_ptr(), d_ref.data_ptr(), out.data_ptr(), b, 2,
+                                           dims, 2, 3, 1, 8.0, 0.125, 1.0, 0, None,
+                                           C.byref(scratch.struct))
+    assert rc == pla.PL_OK
+    torch.cuda.synchronize()
+    assert np.abs(out.cpu().numpy() - want).max() <= 1e-12
+    assert scratch.n_alloc > 0 and not scratch.live and scratch.n_free == scratch.n_alloc
+    # and a failing allocator is reported, with nothing kept
+    for fail_after in (0, 2, 7, 11):
+        short = TorchScratch(fail_after=fail_after)
+        rc = pla._lib.pl_lattice_filter_op_f64(d_in.data_ptr(), d_ref.data_ptr(), out.data_ptr(), b,
+                                               2, dims, 2, 3, 1, 8.0, 0.125, 1.0, 0, None,
+                                               C.byref(short.struct))
+        assert rc in (pla.PL_ENOMEM, pla.PL_OK)
+        assert not short.live and short.n_free == short.n_alloc
+    assert rc == pla.PL_ENOMEM      # eleven allocations are not enough for a lattice
