@@ -7,6 +7,8 @@
 // is its own guide, pixels are scaled by 1/255 (Tests/utils.h:9-23), filtered with pd = 5, vd = 4,
 // and written back as int(value * 255) clamped to 0..255 (Tests/utils.h:26-40).  With a fifth
 // argument that image is filtered under the first one as guide (Tests/greyscale_test.py).
+// Like the reference's program (Tests/test_bilateral_gpu.cpp:43-49) it then repeats the filter in
+// double precision and reports the time; the file written holds the float result.
 // Reads uncompressed 24-bit and 8-bit (palette) BMP files, writes 24-bit ones.
 #include <chrono>
 #include <cstdint>
@@ -113,9 +115,10 @@ void hip_check(hipError_t e, const char *what) {
     if (e != hipSuccess) throw std::runtime_error(std::string(what) + ": " + hipGetErrorString(e));
 }
 
+template <typename T = float>
 struct DeviceBuffer {
-    float *p = nullptr;
-    explicit DeviceBuffer(size_t n) { hip_check(hipMalloc((void **)&p, n * sizeof(float)), "hipMalloc"); }
+    T *p = nullptr;
+    explicit DeviceBuffer(size_t n) { hip_check(hipMalloc((void **)&p, n * sizeof(T)), "hipMalloc"); }
     ~DeviceBuffer() { (void)hipFree(p); }
 };
 
@@ -144,7 +147,7 @@ int main(int argc, char **argv) {
         const std::vector<float> guide_flat = to_unit_floats(guide), flat = to_unit_floats(source);
         std::vector<float> filtered(flat.size());
 
-        DeviceBuffer d_guide(flat.size()), d_in(flat.size()), d_out(flat.size());
+        DeviceBuffer<> d_guide(flat.size()), d_in(flat.size()), d_out(flat.size());
         hip_check(hipMemcpy(d_guide.p, guide_flat.data(), flat.size() * sizeof(float), hipMemcpyHostToDevice), "copy in");
         hip_check(hipMemcpy(d_in.p, flat.data(), flat.size() * sizeof(float), hipMemcpyHostToDevice), "copy in");
 
@@ -156,6 +159,36 @@ int main(int argc, char **argv) {
         std::printf("Measured from function call: %f seconds (%d x %d, %d lattice vertices)\n", seconds,
                     guide.width, guide.height, lattice.size());
         hip_check(hipMemcpy(filtered.data(), d_out.p, flat.size() * sizeof(float), hipMemcpyDeviceToHost), "copy out");
+
+        {
+            std::printf("Testing for double precision\n");
+            const std::vector<double> guide64(guide_flat.begin(), guide_flat.end());
+            const std::vector<double> flat64(flat.begin(), flat.end());
+            std::vector<double> filtered64(flat.size());
+            DeviceBuffer<double> d_guide64(flat.size()), d_in64(flat.size()), d_out64(flat.size());
+            DeviceBuffer<double> d_positions64((size_t)n * 5);
+            hip_check(hipMemcpy(d_guide64.p, guide64.data(), flat.size() * sizeof(double), hipMemcpyHostToDevice), "copy in");
+            hip_check(hipMemcpy(d_in64.p, flat64.data(), flat.size() * sizeof(double), hipMemcpyHostToDevice), "copy in");
+            permutohedral::PermutohedralLatticeHIP<double> lattice64(5, 4, n);
+            lattice64.set_point_grid(2, sdims);
+            int dims[2] = {sdims[0], sdims[1]};
+            const auto begin64 = std::chrono::steady_clock::now();
+            permutohedral::ComputeKernel<permutohedral::HipDevice, double>()(
+                permutohedral::HipDevice{}, nullptr, d_guide64.p, d_positions64.p, n, 2, dims, 3,
+                (double)theta_alpha, (double)theta_beta);
+            lattice64.filter(d_out64.p, d_in64.p, d_positions64.p, false);
+            hip_check(hipDeviceSynchronize(), "filter");
+            const double seconds64 =
+                std::chrono::duration<double>(std::chrono::steady_clock::now() - begin64).count();
+            hip_check(hipMemcpy(filtered64.data(), d_out64.p, flat.size() * sizeof(double), hipMemcpyDeviceToHost), "copy out");
+            double max_diff = 0.0;
+            for (size_t i = 0; i < filtered.size(); ++i) {
+                const double diff = filtered64[i] - (double)filtered[i];
+                max_diff = diff > max_diff ? diff : (-diff > max_diff ? -diff : max_diff);
+            }
+            std::printf("Measured from function call: %f seconds (%d lattice vertices, "
+                        "max |double - float| %.3g)\n", seconds64, lattice64.size(), max_diff);
+        }
 
         Image out = source;
         for (size_t i = 0; i < filtered.size(); ++i) {
