@@ -311,7 +311,7 @@ def main():
                          "ms_per_step": {k: round(v, 4) for k, v in batch_ms.items()},
                          "value": {k: round(batch * pixels_per_step / (v * 1e-3) / 1e6, 3)
                                    for k, v in batch_ms.items()}},
-            "double": {"what": "same step on a lattice of doubles (plain value passes, not the tuned ones)",
+            "double": {"what": "same step on a lattice of doubles (the reference's T = double)",
                        "ms_per_step": round(double_ms, 4),
                        "value": round(pixels_per_step / (double_ms * 1e-3) / 1e6, 3)},
         })

@@ -226,9 +226,9 @@ int pl_set_op_concurrency(int lanes);
  * kinds, every other float entry point returns PL_EINVAL for a lattice of doubles (and these for
  * a lattice of floats).  The lattice (keys, vertex count) equals the CPU path's for T = double
  * exactly; values agree to rounding of the sums (about 1e-15 relative), because the splat adds
- * in another order than a sequential loop.  The float path is the one tuned for speed: this one
- * uses the plain form of each value pass, and its points are not looked at for a grid (give one
- * with pl_set_point_grid; the op does).
+ * in another order than a sequential loop.  The float path is the one tuned for speed (this one
+ * runs at roughly half of it), and the points of a lattice of doubles are not looked at for a
+ * grid (give one with pl_set_point_grid; the op does).
  * ---------------------------------------------------------------------------------------- */
 int pl_create_f64(int pd, int vd, int N, pl_stream stream, const pl_alloc *alloc, pl_handle *out);
 int pl_filter_f64(pl_handle h, double *output, const double *input, const double *positions,

@@ -5,8 +5,9 @@
 // builds: the build kernel is instantiated for double positions in pl_kernels.hip, and the
 // numbering and neighbour passes do not look at values.  What is here are the passes that touch
 // values: splat, blur and slice on rows of doubles, the feature builder and the per-point dump.
-// They are the plain forms (one atomic per point, vertex and channel in the splat; one thread per
-// (vertex, channel) in the blur): the float path is the one tuned for speed.
+// They are simple forms (the splat sums per wavefront and vertex before it adds, channel by
+// channel; one thread per (vertex, channel) in the blur, per (point, channel) in the slice): the
+// float path is the one tuned for speed.
 //
 // Arithmetic follows the reference CPU path with T = double: the three-tap blur and the reciprocal
 // of the slice are double expressions there for every T.  The splat adds in a different order
@@ -21,7 +22,55 @@ namespace {
 
 using namespace device;
 
-// replay rows and weights are stored in thread order, [r][t], like the float path's
+// The double of another lane (by DPP control; both words moved alike)
+template <int CTRL>
+__device__ __forceinline__ double from_lane_f64(double x) {
+    const int lo = __builtin_amdgcn_update_dpp(0, __double2loint(x), CTRL, 0xf, 0xf, false);
+    const int hi = __builtin_amdgcn_update_dpp(0, __double2hiint(x), CTRL, 0xf, 0xf, false);
+    return __hiloint2double(hi, lo);
+}
+// Sums over the wavefront of four terms per lane (zero where `member` is false), delivered to
+// every quad of lanes: lane q of a quad returns the sum of channel channel_of_quad_lane(q).  The
+// terms are reduce-scattered inside each quad (two exchanges, after which a lane holds one
+// channel), then summed across the quads of a row by rotations and across the rows with
+// v_permlane16_swap and v_permlane32_swap (given x twice, the first result holds the even rows /
+// lower half in both places and the second the odd rows / upper half: their sum is the pair's).
+__device__ __forceinline__ int channel_of_quad_lane(int lane) {
+    return ((lane & 1) << 1) | ((lane >> 1) & 1);
+}
+__device__ __forceinline__ double wave_sums_to_quads_f64(bool member, const double (&term)[4],
+                                                         int lane) {
+    const bool bit0 = lane & 1, bit1 = lane & 2;
+    const double keep_a = member ? (bit0 ? term[2] : term[0]) : 0.0;
+    const double keep_b = member ? (bit0 ? term[3] : term[1]) : 0.0;
+    const double send_a = member ? (bit0 ? term[0] : term[2]) : 0.0;
+    const double send_b = member ? (bit0 ? term[1] : term[3]) : 0.0;
+    const double ya = keep_a + from_lane_f64<0xB1>(send_a);   // quad_perm:[1,0,3,2]
+    const double yb = keep_b + from_lane_f64<0xB1>(send_b);
+    double x = (bit1 ? yb : ya) + from_lane_f64<0x4E>(bit1 ? ya : yb);   // quad_perm:[2,3,0,1]
+    x += from_lane_f64<0x124>(x);   // row_ror:4
+    x += from_lane_f64<0x128>(x);   // row_ror:8
+    {
+        const unsigned lo = (unsigned)__double2loint(x), hi = (unsigned)__double2hiint(x);
+        const auto l = __builtin_amdgcn_permlane16_swap(lo, lo, false, false);
+        const auto h = __builtin_amdgcn_permlane16_swap(hi, hi, false, false);
+        x = __hiloint2double((int)h[0], (int)l[0]) + __hiloint2double((int)h[1], (int)l[1]);
+    }
+    {
+        const unsigned lo = (unsigned)__double2loint(x), hi = (unsigned)__double2hiint(x);
+        const auto l = __builtin_amdgcn_permlane32_swap(lo, lo, false, false);
+        const auto h = __builtin_amdgcn_permlane32_swap(hi, hi, false, false);
+        x = __hiloint2double((int)h[0], (int)l[0]) + __hiloint2double((int)h[1], (int)l[1]);
+    }
+    return x;
+}
+
+// Splat.  As in the float path the contributions of a wavefront to one vertex are summed before
+// they leave it (points that are neighbours in the image share vertices, and what bounds a splat
+// is the number of atomic requests): for each distinct vertex of the wavefront and each channel
+// four channels at a time are summed over the members, and the first four lanes add the four
+// sums to the vertex row with one atomic instruction.  replay rows and weights are stored in thread order, [r][t],
+// like the float path's.
 template <int D1>
 __global__ __launch_bounds__(kBlock) void k_splat_f64(int vd, PointMap map,
                                                        const double *__restrict__ input,
@@ -33,20 +82,54 @@ __global__ __launch_bounds__(kBlock) void k_splat_f64(int vd, PointMap map,
     const size_t t = (size_t)vblock * kBlock + threadIdx.x;
     const size_t n_slots = (size_t)gridDim.x * kBlock;
     const int n = point_of_thread(map, vblock, threadIdx.x);
-    if (n < 0) return;
-    const double *value = input + (size_t)n * in_channels;
+    const int lane = threadIdx.x & 63;
+    // every lane stays for the sums; lanes without a point, or whose keys the build could not
+    // place (it has said so), carry vertex -1 and belong to no group
+    int vertex[D1];
+    double weight[D1];
 #pragma unroll
     for (int r = 0; r < D1; ++r) {
-        int v = replay[(size_t)r * n_slots + t].index;
-        if (v < 0) continue;   // the build could not place this point's keys and has said so
-        if (cell_vertex) {
-            v = cell_vertex[v];
-            replay[(size_t)r * n_slots + t].index = v;
+        vertex[r] = n >= 0 ? replay[(size_t)r * n_slots + t].index : -1;
+        weight[r] = weights[(size_t)r * n_slots + t];
+    }
+    if (cell_vertex) {
+#pragma unroll
+        for (int r = 0; r < D1; ++r) {
+            if (vertex[r] >= 0) {
+                vertex[r] = cell_vertex[vertex[r]];
+                replay[(size_t)r * n_slots + t].index = vertex[r];
+            }
         }
-        const double w = weights[(size_t)r * n_slots + t];
-        double *row = values + (size_t)v * vd;
-        for (int j = 0; j < in_channels; ++j) atomicAdd(row + j, w * value[j]);
-        if (in_channels == vd - 1) atomicAdd(row + vd - 1, w);   // homogeneous channel
+    }
+    const double *value = input + (size_t)(n >= 0 ? n : 0) * in_channels;
+    // four channels at a time: their values are loaded once, then every corner's groups are
+    // walked with the four sums of a group going to lanes 0..3 and out in one instruction
+    for (int first_channel = 0; first_channel < vd; first_channel += 4) {
+        const int channels = vd - first_channel < 4 ? vd - first_channel : 4;
+        double val[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c) {
+            const int j = first_channel + c;
+            // the homogeneous channel is the bare weight when vd-1 channels are given
+            val[c] = (n >= 0 && j < in_channels) ? value[j] : 1.0;
+        }
+#pragma unroll
+        for (int r = 0; r < D1; ++r) {
+            const int v = vertex[r];
+            const double w = weight[r];
+            const double term[4] = {w * val[0], w * val[1], w * val[2], w * val[3]};
+            const int my_channel = channel_of_quad_lane(lane);
+            uint64_t remaining = wave_ballot(v >= 0);
+            while (remaining) {
+                const int first = __builtin_ctzll(remaining);
+                const int k = lane_value(v, first);
+                const uint64_t group = lanes_equal(v, k);
+                remaining &= ~group;
+                const double sum = wave_sums_to_quads_f64(lane_in(group), term, lane);
+                if (lane < 4 && my_channel < channels)
+                    atomicAdd(values + (size_t)k * vd + first_channel + my_channel, sum);
+            }
+        }
     }
 }
 
@@ -72,7 +155,62 @@ __global__ __launch_bounds__(kBlock) void k_blur_f64(const Counters *counters, i
     }
 }
 
-// One thread per point and output channel: its channel's sum and the homogeneous channel's.
+// Slice, up to eight channels: one thread per point, the row sums in registers.
+template <int D1>
+__global__ __launch_bounds__(kBlock) void k_slice_point_f64(int vd, PointMap map,
+                                                             const ReplayEntry *__restrict__ replay,
+                                                             const double *__restrict__ weights,
+                                                             const int *__restrict__ cell_vertex,
+                                                             const double *__restrict__ values,
+                                                             double *__restrict__ output,
+                                                             int normalize) {
+    constexpr int kMaxChannels = 8;
+    const unsigned vblock = blockIdx.x;
+    const size_t t = (size_t)vblock * kBlock + threadIdx.x;
+    const size_t n_slots = (size_t)gridDim.x * kBlock;
+    const int n = point_of_thread(map, vblock, threadIdx.x);
+    if (n < 0) return;
+    int vertex[D1];
+    double weight[D1];
+#pragma unroll
+    for (int r = 0; r < D1; ++r) {
+        vertex[r] = replay[(size_t)r * n_slots + t].index;
+        weight[r] = weights[(size_t)r * n_slots + t];
+    }
+    if (cell_vertex) {
+#pragma unroll
+        for (int r = 0; r < D1; ++r)
+            if (vertex[r] >= 0) vertex[r] = cell_vertex[vertex[r]];
+    }
+    double sum[kMaxChannels];
+#pragma unroll
+    for (int j = 0; j < kMaxChannels; ++j) sum[j] = 0.0;
+#pragma unroll
+    for (int r = 0; r < D1; ++r) {
+        if (vertex[r] < 0) continue;
+        const double *row = values + (size_t)vertex[r] * vd;
+#pragma unroll
+        for (int j = 0; j < kMaxChannels; ++j)
+            if (j < vd) sum[j] += weight[r] * row[j];
+    }
+    if (normalize) {
+        double homogeneous = 0.0;
+#pragma unroll
+        for (int j = 0; j < kMaxChannels; ++j)
+            if (j == vd - 1) homogeneous = sum[j];
+        const double scale = 1.0 / homogeneous;
+#pragma unroll
+        for (int j = 0; j < kMaxChannels; ++j)
+            if (j < vd - 1) output[(size_t)n * (vd - 1) + j] = sum[j] * scale;
+    } else {
+#pragma unroll
+        for (int j = 0; j < kMaxChannels; ++j)
+            if (j < vd) output[(size_t)n * vd + j] = sum[j];
+    }
+}
+
+// More channels: one thread per point and output channel, its channel's sum and the homogeneous
+// channel's.
 template <int D1>
 __global__ __launch_bounds__(kBlock) void k_slice_f64(int vd, PointMap map,
                                                        const ReplayEntry *__restrict__ replay,
@@ -176,6 +314,12 @@ hipError_t slice_f64(int pd, int vd, const PointMap &map, const ReplayEntry *rep
                      const double *weights, const int *cell_vertex, const double *values,
                      double *output, int normalize, hipStream_t s) {
     if (map.n_blocks == 0) return hipSuccess;
+    if (vd <= 8) {
+        PLK_DISPATCH_PD(pd, hipLaunchKernelGGL(k_slice_point_f64<PD + 1>, dim3(map.n_blocks),
+                                               dim3(kBlock), 0, s, vd, map, replay, weights,
+                                               cell_vertex, values, output, normalize));
+        return hipGetLastError();
+    }
     const unsigned out_channels = (unsigned)(normalize ? vd - 1 : vd);
     PLK_DISPATCH_PD(pd, hipLaunchKernelGGL(k_slice_f64<PD + 1>, dim3(map.n_blocks, out_channels),
                                            dim3(kBlock), 0, s, vd, map, replay, weights,
