@@ -242,8 +242,9 @@ int pl_compute_positions_f64(const double *reference, double *positions, int num
                              int n_reference_channels, int n_spatial_dims, const int *spatial_dims,
                              double spatial_std, double feature_std, pl_stream stream);
 /* LatticeFilterOp<Device, double>::Compute (src/LatticeFilterKernel.cpp:98-181); the attributes
- * are floats for every T (:36-38).  One lattice, the items one after the other; its scratch and
- * the positions of an item come from alloc (NULL: hipMalloc) and go back before the call ends. */
+ * are floats for every T (:36-38).  One lattice, the items one after the other.  With alloc its
+ * scratch and the positions of an item come from there and go back before the call ends; with
+ * NULL the library keeps them between calls, as pl_lattice_filter_op does. */
 int pl_lattice_filter_op_f64(const double *input, const double *reference, double *output,
                              int batch, int n_spatial_dims, const int *spatial_dims,
                              int n_input_channels, int n_reference_channels, int bilateral,

@@ -957,8 +957,10 @@ struct OpLane {
 struct OpCacheEntry {
     int device, pd, vd, N;
     hipStream_t stream;
+    bool f64;                       // lattices of doubles
     std::vector<OpLane> lanes;
     hipEvent_t fork = nullptr;
+    double *positions64 = nullptr;  // [N*pd], the positions of the item being filtered (doubles only)
 };
 std::mutex g_op_cache_mutex;
 std::vector<OpCacheEntry> g_op_cache;
@@ -973,7 +975,23 @@ void destroy_entry(OpCacheEntry &e) {
         if (lane.owns_stream && lane.stream) (void)hipStreamDestroy(lane.stream);
     }
     if (e.fork) (void)hipEventDestroy(e.fork);
+    if (e.positions64) (void)hipFree(e.positions64);
+    e.positions64 = nullptr;
     e.lanes.clear();
+}
+
+// The cached lattices for this device, shape, stream and value type (g_op_cache_mutex held).
+OpCacheEntry *op_cache_entry(int device, int pd, int vd, int N, hipStream_t stream, bool f64) {
+    for (auto &e : g_op_cache)
+        if (e.device == device && e.pd == pd && e.vd == vd && e.N == N && e.stream == stream &&
+            e.f64 == f64)
+            return &e;
+    if (g_op_cache.size() >= kOpCacheMax) {
+        destroy_entry(g_op_cache.front());
+        g_op_cache.erase(g_op_cache.begin());
+    }
+    g_op_cache.push_back(OpCacheEntry{device, pd, vd, N, stream, f64, {}, nullptr, nullptr});
+    return &g_op_cache.back();
 }
 
 // Lattices and streams for `want` concurrent items.
@@ -986,7 +1004,8 @@ int ensure_lanes(OpCacheEntry &e, int want) {
             PL_HIP(hipStreamCreateWithFlags(&lane.stream, hipStreamNonBlocking));
             lane.owns_stream = true;
         }
-        int rc = pl_create(e.pd, e.vd, e.N, (pl_stream)lane.stream, nullptr, &lane.lattice);
+        int rc = e.f64 ? pl_create_f64(e.pd, e.vd, e.N, (pl_stream)lane.stream, nullptr, &lane.lattice)
+                       : pl_create(e.pd, e.vd, e.N, (pl_stream)lane.stream, nullptr, &lane.lattice);
         if (rc == PL_OK && hipEventCreateWithFlags(&lane.done, hipEventDisableTiming) != hipSuccess)
             rc = PL_EHIP;
         if (rc != PL_OK) {
@@ -1048,21 +1067,7 @@ extern "C" int pl_lattice_filter_op(const float *input, const float *reference, 
 
     // held for the whole call: cached lattices are not re-entrant
     std::lock_guard<std::mutex> lock(g_op_cache_mutex);
-    OpCacheEntry *entry = nullptr;
-    for (auto &e : g_op_cache)
-        if (e.device == device && e.pd == pd && e.vd == vd && e.N == N &&
-            e.stream == (hipStream_t)stream) {
-            entry = &e;
-            break;
-        }
-    if (!entry) {
-        if (g_op_cache.size() >= kOpCacheMax) {
-            destroy_entry(g_op_cache.front());
-            g_op_cache.erase(g_op_cache.begin());
-        }
-        g_op_cache.push_back(OpCacheEntry{device, pd, vd, N, (hipStream_t)stream, {}, nullptr});
-        entry = &g_op_cache.back();
-    }
+    OpCacheEntry *entry = op_cache_entry(device, pd, vd, N, (hipStream_t)stream, false);
     // Items in flight: small items leave most of the GPU idle and gain from four at a time
     // (512x512: 1.44 -> 0.87 ms for eight items forward + reverse); the kernels of an item of a
     // million points fill it, and more than two such items only crowd each other (1.37 / 1.21 /
@@ -1112,8 +1117,10 @@ extern "C" int pl_set_op_concurrency(int lanes) {
 
 // The op for T = double (registered by the reference next to float,
 // src/LatticeFilterKernel.cpp:196-208): positions are built per item, as the reference does
-// (:153-160), and the items are filtered one after the other on one lattice, whose scratch and
-// the positions array come from `alloc` (NULL: hipMalloc) and are returned before the call ends.
+// (:153-160), and the items are filtered one after the other on one lattice.  With a caller's
+// allocator its scratch and the positions array come from there and are returned before the call
+// ends; without one the lattice and the positions array are kept between calls like the float
+// op's.
 extern "C" int pl_lattice_filter_op_f64(const double *input, const double *reference, double *output,
                                         int batch, int n_spatial_dims, const int *spatial_dims,
                                         int n_input_channels, int n_reference_channels,
@@ -1142,31 +1149,42 @@ extern "C" int pl_lattice_filter_op_f64(const double *input, const double *refer
     if (batch == 0) return PL_OK;
     if (!input || !output) return PL_EINVAL;
 
-    pl_alloc mem;
+    // pl_filter_f64 returns after the build, the only reader of the positions, has been waited
+    // for, so the next item may overwrite them
+    auto filter_items = [&](pl_handle lattice, double *positions) {
+        int rc = pl_set_point_grid(lattice, n_spatial_dims, spatial_dims);
+        for (int b = 0; b < batch && rc == PL_OK; ++b) {
+            const double *ref_b = ref_ch ? reference + (size_t)b * N * ref_ch : nullptr;
+            rc = pl_compute_positions_f64(ref_b, positions, N, ref_ch, n_spatial_dims,
+                                          spatial_dims, spatial_std, feature_std, stream);
+            if (rc == PL_OK)
+                rc = pl_filter_f64(lattice, output + (size_t)b * N * n_input_channels,
+                                   input + (size_t)b * N * n_input_channels, positions, reverse);
+        }
+        return rc;
+    };
+    const size_t position_bytes = sizeof(double) * (size_t)N * (size_t)pd;
+
     if (alloc) {
-        mem = *alloc;
-    } else {
-        mem.alloc = default_alloc;
-        mem.free = default_free;
-        mem.ctx = nullptr;
+        pl_handle lattice = nullptr;
+        int rc = pl_create_f64(pd, vd, N, stream, alloc, &lattice);
+        double *positions = nullptr;
+        if (rc == PL_OK) {
+            positions = (double *)alloc->alloc(alloc->ctx, position_bytes);
+            if (!positions) rc = PL_ENOMEM;
+        }
+        if (rc == PL_OK) rc = filter_items(lattice, positions);
+        pl_destroy(lattice);   // synchronises the stream first
+        if (positions) alloc->free(alloc->ctx, positions);
+        return rc;
     }
-    pl_handle lattice = nullptr;
-    int rc = pl_create_f64(pd, vd, N, stream, alloc, &lattice);
-    double *positions = nullptr;
-    if (rc == PL_OK) {
-        positions = (double *)mem.alloc(mem.ctx, sizeof(double) * (size_t)N * (size_t)pd);
-        if (!positions) rc = PL_ENOMEM;
-    }
-    if (rc == PL_OK) rc = pl_set_point_grid(lattice, n_spatial_dims, spatial_dims);
-    for (int b = 0; b < batch && rc == PL_OK; ++b) {
-        const double *ref_b = ref_ch ? reference + (size_t)b * N * ref_ch : nullptr;
-        rc = pl_compute_positions_f64(ref_b, positions, N, ref_ch, n_spatial_dims, spatial_dims,
-                                      spatial_std, feature_std, stream);
-        if (rc == PL_OK)
-            rc = pl_filter_f64(lattice, output + (size_t)b * N * n_input_channels,
-                               input + (size_t)b * N * n_input_channels, positions, reverse);
-    }
-    pl_destroy(lattice);   // synchronises the stream first
-    if (positions) mem.free(mem.ctx, positions);
-    return rc;
+
+    int device = 0;
+    PL_HIP(hipGetDevice(&device));
+    std::lock_guard<std::mutex> lock(g_op_cache_mutex);
+    OpCacheEntry *entry = op_cache_entry(device, pd, vd, N, (hipStream_t)stream, true);
+    int rc = ensure_lanes(*entry, 1);
+    if (rc != PL_OK) return rc;
+    if (!entry->positions64) PL_HIP(hipMalloc((void **)&entry->positions64, position_bytes));
+    return filter_items(entry->lanes[0].lattice, entry->positions64);
 }
