@@ -1185,6 +1185,10 @@ extern "C" int pl_lattice_filter_op_f64(const double *input, const double *refer
     OpCacheEntry *entry = op_cache_entry(device, pd, vd, N, (hipStream_t)stream, true);
     int rc = ensure_lanes(*entry, 1);
     if (rc != PL_OK) return rc;
-    if (!entry->positions64) PL_HIP(hipMalloc((void **)&entry->positions64, position_bytes));
+    if (!entry->positions64 &&
+        hip_failed(hipMalloc((void **)&entry->positions64, position_bytes))) {
+        entry->positions64 = nullptr;
+        return PL_ENOMEM;
+    }
     return filter_items(entry->lanes[0].lattice, entry->positions64);
 }
