@@ -157,6 +157,12 @@ __device__ __forceinline__ float wave_sum_to_last_lanes(bool member, const QuadT
 // atomic instruction per group, to the row of the key's CELL in cell_values (the vertices are not
 // numbered yet); the numbering pass moves the rows into the dense value table.  One kernel then
 // does the work of two, shares the deduplication between them and never reads the replay arrays.
+// Address of a hash cell as the table's base plus a 32-bit byte offset (tables stay below 2^29
+// cells): one address register per cell instead of two.
+__device__ __forceinline__ uint64_t *cell_at(uint64_t *cell_keys, uint32_t cell) {
+    return reinterpret_cast<uint64_t *>(reinterpret_cast<char *>(cell_keys) + (cell << 3));
+}
+
 // T = double (SPLAT_VD == 0 only): positions, scale factors and the weights written are those of
 // `points64`; the replay rows then carry the cells only.
 template <int PD, int SPLAT_VD, typename T = float>
@@ -198,6 +204,12 @@ __global__ __launch_bounds__(kBlock) void k_build(PointFeatures features, PointM
         enclosing_simplex<PD>(pos, scale, s);
     }
 
+    // The weights are wanted after the insertion only, and the compiler would carry the residuals
+    // and ranks they come from (twice as many registers) across it instead: have them now.
+    if constexpr (!kDouble) {
+#pragma unroll
+        for (int r = 0; r < D1; ++r) asm volatile("" : "+v"(s.weight[r]));
+    }
     const bool in_range = simplex_in_key_range<PD>(s);
     if (valid && !in_range) atomicOr(&counters->flags, kFlagKeyRange);
     const bool active = valid && in_range;
@@ -206,13 +218,16 @@ __global__ __launch_bounds__(kBlock) void k_build(PointFeatures features, PointM
     // (the lowest that holds it) and its cell is broadcast to the others.  Only leaders touch the
     // table.
     uint64_t key[D1];
-    int leader[D1];
+    // (leader lanes are kept five to a register, six bits each: registers decide how many
+    // wavefronts a CU holds)
+    unsigned leaders[(D1 + 4) / 5] = {};
+    auto leader_of = [&](int r) { return (int)((leaders[r / 5] >> (6 * (r % 5))) & 63u); };
 #pragma unroll
     for (int r = 0; r < D1; ++r) {
         int q[PD];
         vertex_q<PD>(s, r, q);
         key[r] = KeyCodec<PD>::pack(q, r);
-        leader[r] = wave_leader_of_equal(key[r], active, lane);
+        leaders[r / 5] |= (unsigned)wave_leader_of_equal(key[r], active, lane) << (6 * (r % 5));
     }
 
     // Insertion of a lane's pd+1 keys proceeds in rounds over all of them at once, so that the
@@ -222,36 +237,35 @@ __global__ __launch_bounds__(kBlock) void k_build(PointFeatures features, PointM
     // so a stale load can at worst report "empty" and the compare-and-swap returns the truth.
     uint32_t cell[D1];
     uint64_t seen[D1];
-    bool open[D1];
+    unsigned open = 0;      // bit r: this lane still has to place key r
     unsigned created = 0;   // bit r: this lane's swap made the vertex of rank r
-    bool any_open = false;
 #pragma unroll
     for (int r = 0; r < D1; ++r) {
-        open[r] = active && leader[r] == lane;
+        if (active && leader_of(r) == lane) open |= 1u << r;
         cell[r] = hash_key(key[r]) & mask;
-        any_open = any_open || open[r];
     }
+    bool any_open = open != 0;
     for (uint32_t probe = 0; any_open && probe <= mask; ++probe) {
 #pragma unroll
-        for (int r = 0; r < D1; ++r) seen[r] = open[r] ? cell_keys[cell[r]] : key[r];
+        for (int r = 0; r < D1; ++r)
+            seen[r] = (open >> r) & 1u ? *cell_at(cell_keys, cell[r]) : key[r];
 #pragma unroll
         for (int r = 0; r < D1; ++r)
-            if (open[r] && seen[r] == kEmptyCell)
-                seen[r] = atomicCAS((unsigned long long *)(cell_keys + cell[r]),
+            if (((open >> r) & 1u) && seen[r] == kEmptyCell)
+                seen[r] = atomicCAS((unsigned long long *)cell_at(cell_keys, cell[r]),
                                     (unsigned long long)kEmptyCell, (unsigned long long)key[r]);
-        any_open = false;
 #pragma unroll
         for (int r = 0; r < D1; ++r) {
-            if (open[r]) {
+            if ((open >> r) & 1u) {
                 if (seen[r] == kEmptyCell || seen[r] == key[r]) {
                     if (seen[r] == kEmptyCell) created |= 1u << r;
-                    open[r] = false;              // swapped in, or already there
+                    open &= ~(1u << r);           // swapped in, or already there
                 } else {
                     cell[r] = (cell[r] + 1u) & mask;
-                    any_open = true;
                 }
             }
         }
+        any_open = open != 0;
     }
     if (any_open) atomicOr(&counters->flags, kFlagTableFull);
 
@@ -301,8 +315,9 @@ __global__ __launch_bounds__(kBlock) void k_build(PointFeatures features, PointM
 
 #pragma unroll
     for (int r = 0; r < D1; ++r) {
-        const int own = open[r] ? -1 : (int)cell[r];
-        const int c = __shfl(own, leader[r]);
+        const int own = (open >> r) & 1u ? -1 : (int)cell[r];
+        const int leader = leader_of(r);
+        const int c = __shfl(own, leader);
         replay[(size_t)r * n_slots + t] = ReplayEntry{active ? c : -1, valid ? (float)s.weight[r] : 0.0f};
         if constexpr (kDouble) points64.weights[(size_t)r * n_slots + t] = valid ? s.weight[r] : 0.0;
         if (SPLAT_VD) {
@@ -315,7 +330,7 @@ __global__ __launch_bounds__(kBlock) void k_build(PointFeatures features, PointM
             uint64_t remaining = among;
             while (remaining) {
                 const int first = __builtin_ctzll(remaining);
-                const uint64_t group = lanes_equal(leader[r], first) & among;
+                const uint64_t group = lanes_equal(leader, first) & among;
                 remaining &= ~group;
                 const bool same = lane_in(group);
                 const int group_cell = lane_value(own, first);
