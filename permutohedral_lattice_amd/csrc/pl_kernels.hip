@@ -206,10 +206,8 @@ __global__ __launch_bounds__(kBlock) void k_build(PointFeatures features, PointM
 
     // The weights are wanted after the insertion only, and the compiler would carry the residuals
     // and ranks they come from (twice as many registers) across it instead: have them now.
-    if constexpr (!kDouble) {
 #pragma unroll
-        for (int r = 0; r < D1; ++r) asm volatile("" : "+v"(s.weight[r]));
-    }
+    for (int r = 0; r < D1; ++r) asm volatile("" : "+v"(s.weight[r]));
     const bool in_range = simplex_in_key_range<PD>(s);
     if (valid && !in_range) atomicOr(&counters->flags, kFlagKeyRange);
     const bool active = valid && in_range;
