@@ -307,7 +307,8 @@ def main():
                          "value": {k: round(pixels_per_step / (v * 1e-3) / 1e6, 3)
                                    for k, v in op_ms.items()}},
             "op_batch": {"what": "the op on a batch of %d such images, forward + reverse per step, "
-                                 "items one at a time and four at a time" % batch,
+                                 "items one at a time, and with the op's concurrency set to four (of items this "
+                                 "large it then runs two at a time)" % batch,
                          "ms_per_step": {k: round(v, 4) for k, v in batch_ms.items()},
                          "value": {k: round(batch * pixels_per_step / (v * 1e-3) / 1e6, 3)
                                    for k, v in batch_ms.items()}},
