@@ -87,8 +87,11 @@ int pl_destroy(pl_handle h);
  * row-major, one row per point.  reverse != 0 visits the blur axes pd..0 (the gradient pass).
  * Stands in for filter(output, input, positions, reverse)
  * (src/PermutohedralLatticeCPU.h:442-446, src/PermutohedralLatticeGPU.cuh:453-479).
- * Equivalent to pl_build followed by pl_apply.  Returns after the result of the build has been
- * checked on the host (one stream synchronisation); the remaining work may still be in flight.
+ * Equivalent to pl_build followed by pl_apply.  Everything is enqueued at once; the call returns
+ * when the build has reported whether its hash table was large enough (one wait for an event
+ * behind the build's kernels; if it was not, the call is repeated with a larger table), while
+ * the blur and the slice may still be running.  The output is complete in the order of the
+ * lattice's stream, as with the reference's GPU path.
  */
 int pl_filter(pl_handle h, float *output, const float *input, const float *positions, int reverse);
 
@@ -179,8 +182,8 @@ int pl_build_image(pl_handle h, const float *reference, int n_reference_channels
 /*
  * pl_filter / pl_filter_image in two halves, for callers that keep several lattices (each on a
  * stream of its own) in flight: *_begin enqueues the whole call on the lattice's stream and
- * returns at once; pl_filter_end waits for that stream and, should the hash table have turned
- * out too small, repeats the call with a larger one before it returns.  The arguments of *_begin
+ * returns at once; pl_filter_end waits for the build's report and, should the hash table have
+ * turned out too small, repeats the call with a larger one before it returns.  The arguments of *_begin
  * must stay valid until pl_filter_end; between the two only pl_filter_end and pl_destroy may be
  * called on the handle (anything else returns PL_ESTATE).  pl_filter_end with nothing in flight
  * returns PL_OK.  The reference's filter (src/PermutohedralLatticeGPU.cuh:454-479) enqueues on
@@ -201,7 +204,8 @@ int pl_filter_end(pl_handle h);
  * (src/LatticeFilterKernel.cpp:98-181); its gradient is the same call on the upstream gradient
  * with reverse = 1 (lattice_filter_op_loader.py:32-54).  Scratch comes from alloc; with NULL the
  * library keeps lattices of its own between calls and runs several batch items at a time (see
- * pl_set_op_concurrency).  Returns when the results are complete.
+ * pl_set_op_concurrency).  Returns when every item's build has been checked; the output is
+ * complete in the order of `stream`.
  */
 int pl_lattice_filter_op(const float *input, const float *reference, float *output, int batch,
                          int n_spatial_dims, const int *spatial_dims, int n_input_channels,

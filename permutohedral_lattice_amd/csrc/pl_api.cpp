@@ -107,6 +107,7 @@ struct pl_lattice {
     plk::Counters *d_counters = nullptr;   // two sets, used by alternate builds
     int counter_set = 0;                   // the set of the last build
     plk::HostStatus *h_status = nullptr;   // pinned, written by the device
+    hipEvent_t status_written = nullptr;   // recorded behind the kernel that writes h_status
 
     int M = 0;
     int last_M = -1;
@@ -288,6 +289,7 @@ int enqueue_build(pl_lattice *h, const plk::PointFeatures &features, const doubl
                                 h->values[0], h->f64 ? 2 * h->vd : h->vd,
                                 fused ? h->cell_values : nullptr, h->counters(),
                                 h->d_counters + previous_set, h->h_status, h->stream));
+    PL_HIP(hipEventRecord(h->status_written, h->stream));
     h->mark(EV_IDS);
     PL_HIP(plk::neighbours(h->pd, vertices, h->counters(), h->cell_keys, cells,
                            h->launch_vertices(), h->stream));
@@ -388,11 +390,13 @@ int enqueue_apply(pl_lattice *h, void *output_any, const void *input_any, int re
     return PL_OK;
 }
 
-// Wait for the stream and read what the last build reported.  PL_OK: it fitted, h->M is valid.
+// Wait until the last build has reported (not for what was enqueued behind it: the host learns
+// whether the table was large enough while the blur and the slice still run, and the caller's next
+// call is enqueued behind them without a gap).  PL_OK: it fitted, h->M is valid.
 // Otherwise *retry_cells is the table size to try next (0: give up with the returned status).
 int verify_build(pl_lattice *h, uint32_t *retry_cells) {
     *retry_cells = 0;
-    PL_HIP(hipStreamSynchronize(h->stream));
+    PL_HIP(hipEventSynchronize(h->status_written));
     const int flags = h->h_status->flags;
     const int m = h->h_status->num_vertices;
     if (flags & plk::kFlagKeyRange) {
@@ -477,6 +481,8 @@ static int create_lattice(int pd, int vd, int N, bool f64, pl_stream stream, con
     if (rc == PL_OK &&
         hip_failed(hipHostMalloc((void **)&h->h_status, sizeof(plk::HostStatus), hipHostMallocDefault)))
         rc = PL_EHIP;
+    if (rc == PL_OK && hip_failed(hipEventCreateWithFlags(&h->status_written, hipEventDisableTiming)))
+        rc = PL_EHIP;
     if (rc != PL_OK) {
         pl_destroy(h);
         return rc;
@@ -514,6 +520,7 @@ int pl_destroy(pl_handle h) {
     h->dfree(h->d_counters);
     h->dfree(h->d_guess);
     if (h->h_status) (void)hipHostFree(h->h_status);
+    if (h->status_written) (void)hipEventDestroy(h->status_written);
     for (int i = 0; i < EV_COUNT; ++i)
         if (h->ev[i]) (void)hipEventDestroy(h->ev[i]);
     delete h;
