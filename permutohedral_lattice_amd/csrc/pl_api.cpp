@@ -3,7 +3,8 @@
 //
 // A filter call enqueues its kernels back to back: the vertex count of the lattice stays on the
 // device (every later kernel reads it there and is launched for an estimate of it), so the host
-// waits once, at the end, to learn whether the hash table was large enough.
+// waits once, for an event behind the build's kernels, to learn whether the hash table was large
+// enough, and is back at the caller while the blur and the slice still run.
 #include "permutohedral_lattice.h"
 
 #include <hip/hip_runtime.h>
