@@ -111,3 +111,43 @@ def test_full_size_properties(name):
         # the control: forward order on both sides is a different number
         wrong = _dot(xa, yb)
         assert abs(lhs - wrong) > 1e-4 * abs(lhs)
+
+
+def test_full_size_properties_in_double():
+    """The headline configuration on a lattice of doubles: the same size-independent properties,
+    at double precision."""
+    pd, vd, shape, pos = _positions("north_star_1024_rgb")
+    n = pos.shape[0]
+    gen = torch.Generator(device="cuda").manual_seed(4321)
+    d_pos = torch.from_numpy(pos).cuda().double()
+    lat = pla.PermutohedralLattice(pd, vd, n, dtype=torch.float64)
+    lat.set_point_grid(shape)
+    d = lat.debug_simplex(d_pos)
+    rem0, rank, keys, bary = d["rem0"].int(), d["rank"].int(), d["keys"], d["barycentric"]
+    assert int((rem0 % (pd + 1)).abs().max()) == 0
+    assert int(rem0.sum(dim=1).abs().max()) == 0
+    assert int((rank.sum(dim=1) - pd * (pd + 1) // 2).abs().max()) == 0
+    assert float(bary.min()) >= -1e-14
+    assert float((bary.sum(dim=1) - 1.0).abs().max()) <= 1e-14
+    distinct = torch.unique(keys.reshape(-1, pd), dim=0).shape[0]
+    del d, rem0, rank, keys, bary
+
+    const = torch.full((n, vd - 1), 0.625, dtype=torch.float64, device="cuda")
+    out = torch.empty_like(const)
+    lat.filter(out, const, d_pos, False)
+    torch.cuda.synchronize()
+    assert lat.num_vertices == distinct
+    assert float((out - 0.625).abs().max()) <= 1e-13
+
+    lat.set_option(pla.PL_OPT_NORMALIZE, 0)
+    lat.build(d_pos)
+    xa = torch.randn((n, vd), generator=gen, device="cuda", dtype=torch.float64)
+    xb = torch.randn((n, vd), generator=gen, device="cuda", dtype=torch.float64)
+    ya, rev_b, yb = (torch.empty_like(xa) for _ in range(3))
+    lat.apply(ya, xa, False)
+    lat.apply(rev_b, xb, True)
+    lat.apply(yb, xb, False)
+    torch.cuda.synchronize()
+    lhs, rhs, wrong = _dot(ya, xb), _dot(xa, rev_b), _dot(xa, yb)
+    assert abs(lhs - rhs) <= 1e-11 * max(abs(lhs), abs(rhs))      # reverse is the adjoint of forward
+    assert abs(lhs - wrong) > 1e-4 * abs(lhs)                     # and forward is not
