@@ -874,9 +874,12 @@ __global__ __launch_bounds__(kBlock) void k_slice_point(int d1, PointMap map,
                                                          const int *__restrict__ cell_vertex,
                                                          const float *__restrict__ values,
                                                          float *__restrict__ output, int normalize) {
-    const size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    // each XCD takes one contiguous range of the tiles: the value rows it gathers (vertex numbers
+    // follow the tiles) are then in its own L2 and not in all eight
+    const unsigned vblock = xcd_contiguous_block(blockIdx.x, gridDim.x, 1);
+    const size_t t = (size_t)vblock * kBlock + threadIdx.x;
     const size_t T = (size_t)gridDim.x * kBlock;
-    const int n = point_of_thread(map, blockIdx.x, threadIdx.x);
+    const int n = point_of_thread(map, vblock, threadIdx.x);
     if (n < 0) return;
     float acc[VD];
 #pragma unroll
@@ -919,8 +922,9 @@ __global__ __launch_bounds__(kBlock) void k_slice_channels(int vd, PointMap map,
     const unsigned slot = item / runs;
     if (slot >= kBlock) return;
     const int j0 = kSliceRun * (int)(item - slot * runs);
-    const size_t t = (size_t)blockIdx.x * kBlock + slot;
-    const int n = point_of_thread(map, blockIdx.x, slot);
+    const unsigned vblock = xcd_contiguous_block(blockIdx.x, gridDim.x, 1);   // as in k_slice_point
+    const size_t t = (size_t)vblock * kBlock + slot;
+    const int n = point_of_thread(map, vblock, slot);
     if (n < 0) return;
     ReplayEntry e[D1];
 #pragma unroll

@@ -165,7 +165,8 @@ __global__ __launch_bounds__(kBlock) void k_slice_point_f64(int vd, PointMap map
                                                              double *__restrict__ output,
                                                              int normalize) {
     constexpr int kMaxChannels = 8;
-    const unsigned vblock = blockIdx.x;
+    // each XCD takes one contiguous range of the tiles, whose vertices' rows are then in its L2
+    const unsigned vblock = xcd_contiguous_block(blockIdx.x, gridDim.x, 1);
     const size_t t = (size_t)vblock * kBlock + threadIdx.x;
     const size_t n_slots = (size_t)gridDim.x * kBlock;
     const int n = point_of_thread(map, vblock, threadIdx.x);
@@ -219,7 +220,8 @@ __global__ __launch_bounds__(kBlock) void k_slice_f64(int vd, PointMap map,
                                                        const double *__restrict__ values,
                                                        double *__restrict__ output, int normalize) {
     const int out_channels = normalize ? vd - 1 : vd;
-    const unsigned vblock = blockIdx.x;
+    // each XCD takes one contiguous range of the tiles, whose vertices' rows are then in its L2
+    const unsigned vblock = xcd_contiguous_block(blockIdx.x, gridDim.x, 1);
     const size_t t = (size_t)vblock * kBlock + threadIdx.x;
     const size_t n_slots = (size_t)gridDim.x * kBlock;
     const int n = point_of_thread(map, vblock, threadIdx.x);
