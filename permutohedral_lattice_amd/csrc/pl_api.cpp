@@ -272,15 +272,32 @@ int enqueue_build(pl_lattice *h, const plk::PointFeatures &features, const doubl
                                      h->max_vertices()};
     const plk::CreatedLists lists{h->created_entries, h->block_count,
                                   h->chunk_count + (size_t)h->counter_set * h->n_chunks};
+    // keys go to the part of the table that belongs to their band of rows when the points are
+    // known to be a grid (and feature 0 then runs with its slowest extent)
+    plk::RegionSource regions{};
+    regions.enabled = h->xcd_aware && h->map.mode != 0;
+    regions.N = h->N;
+    regions.pd = h->pd;
+    regions.scale0 = h->f64 ? (float)h->scale64.v[0] : h->scale.v[0];
+    regions.positions = h->f64 ? nullptr : features.positions;
+    regions.positions64 = h->f64 ? positions64 : nullptr;
+    if (!h->f64 && !features.positions) {
+        if (features.n_spatial_dims > 0) {
+            regions.first = 0.0f;
+            regions.last = (float)(features.dims.v[0] - 1) / features.spatial_std;
+        } else {
+            regions.enabled = 0;
+        }
+    }
     if (h->f64) {
         const plk::Points64 points{positions64, h->weights64, h->scale64};
         PL_HIP(plk::build_f64(h->pd, points, h->map, h->cell_keys, cells, h->counters(), h->replay,
-                              h->xcd_aware ? 1 : 0, lists, h->stream));
+                              h->xcd_aware ? 1 : 0, lists, regions, h->stream));
     } else {
         PL_HIP(plk::build(h->pd, features, h->map, h->scale, h->cell_keys, cells, h->counters(),
                           h->replay, h->xcd_aware ? 1 : 0, fused ? h->vd : 0,
                           splat_input, h->normalize ? h->vd - 1 : h->vd, h->cell_values, lists,
-                          h->stream));
+                          regions, h->stream));
     }
     h->mark(EV_BUILD);
     // the numbering pass zeroes the vertices' value rows: a row of vd doubles is 2*vd zero floats
@@ -293,7 +310,7 @@ int enqueue_build(pl_lattice *h, const plk::PointFeatures &features, const doubl
     PL_HIP(hipEventRecord(h->status_written, h->stream));
     h->mark(EV_IDS);
     PL_HIP(plk::neighbours(h->pd, vertices, h->counters(), h->cell_keys, cells,
-                           h->launch_vertices(), h->stream));
+                           h->launch_vertices(), regions, h->stream));
     h->mark(EV_NBR);
     h->replay_holds_cells = true;
     h->values_zeroed = !fused;

@@ -65,6 +65,53 @@ __device__ __forceinline__ uint32_t hash_key(uint64_t k) {
     return x;
 }
 
+// Keys spread over the table by where they lie along feature 0.  Every XCD has an L2 of its own,
+// and the kernels deal their work out so that an XCD handles one band of image rows (one
+// contiguous eighth of the tiles, of the vertices): if a vertex's cell is taken from the eighth of
+// the table that belongs to its band, what an XCD looks up -- its own vertices and their
+// neighbours -- lies in an eighth of the table instead of all over it.  Feature 0 can be read off a
+// key: the first two coordinates of an elevated point differ by twice its scaled feature 0, and a
+// vertex is within pd+1 of the points that touch it.  The band only picks the leading bits of the
+// cell; probing runs on over the whole table, so any spread of the keys is handled, evenly or not.
+struct KeyRegions {
+    float lo, per_unit;   // band = (scaled feature 0 - lo) * per_unit, clamped to 0..7; per_unit 0: one band
+};
+__device__ __forceinline__ KeyRegions key_regions(const RegionSource &src) {
+    KeyRegions regions{0.0f, 0.0f};
+    if (!src.enabled || src.N < 2) return regions;
+    float a = src.first, b = src.last;
+    if (src.positions) {
+        a = src.positions[0];
+        b = src.positions[(size_t)(src.N - 1) * src.pd];
+    } else if (src.positions64) {
+        a = (float)src.positions64[0];
+        b = (float)src.positions64[(size_t)(src.N - 1) * src.pd];
+    }
+    a *= src.scale0;
+    b *= src.scale0;
+    const float lo = fminf(a, b), span = fmaxf(a, b) - lo;
+    // bands narrower than a few lattice steps would scatter a point's vertices over several
+    if (!(span >= 32.0f * (float)(src.pd + 1))) return regions;
+    regions.lo = lo;
+    regions.per_unit = 8.0f / span;
+    return regions;
+}
+template <int PD>
+__device__ __forceinline__ uint32_t cell_of_key(uint64_t key, uint32_t mask, const KeyRegions &regions) {
+    const uint32_t h = hash_key(key);
+    if (regions.per_unit == 0.0f) return h & mask;
+    int q[PD], r;
+    KeyCodec<PD>::unpack(key, q, r);
+    // scaled feature 0 of the points around this vertex: half the difference of its first two
+    // coordinates (for pd = 1 the second coordinate is minus the first)
+    const float c = PD >= 2 ? 0.5f * (float)((q[0] - q[PD >= 2 ? 1 : 0]) * (PD + 1))
+                            : (float)(q[0] * (PD + 1) + r);
+    int band = (int)((c - regions.lo) * regions.per_unit);
+    band = band < 0 ? 0 : (band > 7 ? 7 : band);
+    const uint32_t low = mask >> 3;   // the table has at least 4096 cells
+    return ((uint32_t)band * (low + 1u)) | (h & low);
+}
+
 // ------------------------------------------------------------------------------------------------
 // Per-point arithmetic: same operations, in the same precision and order, as
 // embed_position_vector / find_enclosing_simplex / compute_barycentric_coordinates of the

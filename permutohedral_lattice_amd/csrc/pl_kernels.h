@@ -101,6 +101,18 @@ struct PointMap {
     unsigned n_blocks;
 };
 
+// Where feature 0 of the first and of the last point can be read (one of the two pointers, or
+// the two values themselves when the features are built on the fly), for spreading the keys over
+// the hash table by it: see KeyRegions in pl_device.h.  enabled == 0: plain hashing.
+struct RegionSource {
+    const float *positions;
+    const double *positions64;
+    float first, last;
+    float scale0;          // scale factor of feature 0
+    int N, pd;
+    int enabled;
+};
+
 // Bits per lattice coordinate in the packed 64-bit key, and the coordinate range that fits.
 int key_field_bits(int pd);
 
@@ -123,13 +135,14 @@ hipError_t build(int pd, const PointFeatures &features, const PointMap &map, con
                  uint64_t *cell_keys, uint32_t n_cells, Counters *counters, ReplayEntry *replay,
                  int xcd_aware, int splat_vd, const float *input,
                  int in_channels, float *cell_values, const CreatedLists &created_lists,
-                 hipStream_t s);
+                 const RegionSource &regions, hipStream_t s);
 
 // The build for double values: the same kernel on points.positions with points.scale; replay[]
 // receives the cells (and the weights rounded to float), points.weights[r*T+t] the weights.
 hipError_t build_f64(int pd, const Points64 &points, const PointMap &map, uint64_t *cell_keys,
                      uint32_t n_cells, Counters *counters, ReplayEntry *replay, int xcd_aware,
-                     const CreatedLists &created_lists, hipStream_t s);
+                     const CreatedLists &created_lists, const RegionSource &regions,
+                     hipStream_t s);
 
 // Dense vertex numbers in the order of the build's workgroups (same map as the build):
 // cell_vertex[cell] := v, vertex_keys[v] := key, vertex_cell[v] := cell,
@@ -146,9 +159,10 @@ hipError_t number_vertices(int pd, const PointMap &map, const CreatedLists &list
 // below the vertex count; entries of absent neighbours keep their -1.
 // launch_vertices (here and below): the vertex count the grid is sized for; any count is
 // covered, a wrong estimate only costs time.
+// regions: the same as the build's, so that keys are looked for where it put them.
 hipError_t neighbours(int pd, const VertexTables &vertices, const Counters *counters,
                       const uint64_t *cell_keys, uint32_t n_cells, int launch_vertices,
-                      hipStream_t s);
+                      const RegionSource &regions, hipStream_t s);
 
 hipError_t fill_zero(float *p, size_t n, hipStream_t s);
 

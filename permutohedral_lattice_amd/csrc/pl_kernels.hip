@@ -173,7 +173,7 @@ __global__ __launch_bounds__(kBlock) void k_build(PointFeatures features, PointM
                                                    int xcd_aware, const float *__restrict__ input,
                                                    int in_channels, float *cell_values,
                                                    CreatedLists created_lists,
-                                                   Points64 points64) {
+                                                   Points64 points64, RegionSource region_source) {
     constexpr bool kDouble = sizeof(T) == sizeof(double);
     static_assert(!kDouble || SPLAT_VD == 0, "the fused splat is for float values");
     constexpr int D1 = PD + 1;
@@ -233,6 +233,7 @@ __global__ __launch_bounds__(kBlock) void k_build(PointFeatures features, PointM
     // cell of every unresolved key, swaps the key into the cells seen empty, and steps the
     // keys that met another key to their next cell.  Cells only ever change from empty to a key,
     // so a stale load can at worst report "empty" and the compare-and-swap returns the truth.
+    const KeyRegions regions = key_regions(region_source);
     uint32_t cell[D1];
     uint64_t seen[D1];
     unsigned open = 0;      // bit r: this lane still has to place key r
@@ -240,7 +241,7 @@ __global__ __launch_bounds__(kBlock) void k_build(PointFeatures features, PointM
 #pragma unroll
     for (int r = 0; r < D1; ++r) {
         if (active && leader_of(r) == lane) open |= 1u << r;
-        cell[r] = hash_key(key[r]) & mask;
+        cell[r] = cell_of_key<PD>(key[r], mask, regions);
     }
     bool any_open = open != 0;
     for (uint32_t probe = 0; any_open && probe <= mask; ++probe) {
@@ -356,7 +357,9 @@ __global__ __launch_bounds__(64) void k_number_vertices(CreatedLists lists, int 
                                                         float *cell_values, Counters *counters,
                                                         Counters *next_counters,
                                                         HostStatus *host_status) {
-    const unsigned b = blockIdx.x;
+    // (an XCD takes the lists of one contiguous range of tiles: their cells are in its part of the
+    // table and their vertex numbers in one range)
+    const unsigned b = xcd_contiguous_block(blockIdx.x, gridDim.x, 1);
     const int lane = threadIdx.x;
     const unsigned chunk = b / kBlocksPerChunk;
     // vertices of the workgroups before this one: whole chunks, then the rest one by one
@@ -428,8 +431,9 @@ template <int PD>
 __global__ __launch_bounds__(kBlock) void k_neighbours(VertexTables vertices,
                                                         const Counters *counters,
                                                         const uint64_t *__restrict__ cell_keys,
-                                                        uint32_t mask) {
+                                                        uint32_t mask, RegionSource region_source) {
     constexpr int D1 = PD + 1;
+    const KeyRegions regions = key_regions(region_source);
     const int max_vertices = vertices.max_vertices;
     const int M = vertex_count(counters, max_vertices);
     const unsigned runs = (unsigned)((M + kBlock - 1) / kBlock);
@@ -450,7 +454,7 @@ __global__ __launch_bounds__(kBlock) void k_neighbours(VertexTables vertices,
         qp[i] = q[i] + (wrap_up ? (on_axis ? 0 : 1) : (on_axis ? -1 : 0));
     }
     const uint64_t want = KeyCodec<PD>::pack(qp, wrap_up ? 0 : r + 1);
-    uint32_t h = hash_key(want) & mask;
+    uint32_t h = cell_of_key<PD>(want, mask, regions);
     int u = -1;
     for (uint32_t probe = 0; probe <= mask; ++probe) {
         const uint64_t cur = cell_keys[h];
@@ -1120,14 +1124,14 @@ hipError_t build(int pd, const PointFeatures &features, const PointMap &map, con
                  uint64_t *cell_keys, uint32_t n_cells, Counters *counters, ReplayEntry *replay,
                  int xcd_aware, int splat_vd, const float *input,
                  int in_channels, float *cell_values, const CreatedLists &created_lists,
-                 hipStream_t s) {
+                 const RegionSource &regions, hipStream_t s) {
     if (map.n_blocks == 0) return hipSuccess;
 #define PLK_BUILD(SPLAT_VD)                                                                        \
     PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_build<PD, SPLAT_VD>), dim3(map.n_blocks),            \
                                            dim3(kBlock), 0, s, features, map, scale, cell_keys,    \
                                            n_cells - 1u, counters, replay,                         \
                                            xcd_aware, input, in_channels, cell_values,             \
-                                           created_lists, Points64{}))
+                                           created_lists, Points64{}, regions))
     switch (splat_vd) {
         case 0: PLK_BUILD(0); break;
         case 2: PLK_BUILD(2); break;
@@ -1141,13 +1145,14 @@ hipError_t build(int pd, const PointFeatures &features, const PointMap &map, con
 
 hipError_t build_f64(int pd, const Points64 &points, const PointMap &map, uint64_t *cell_keys,
                      uint32_t n_cells, Counters *counters, ReplayEntry *replay, int xcd_aware,
-                     const CreatedLists &created_lists, hipStream_t s) {
+                     const CreatedLists &created_lists, const RegionSource &regions,
+                     hipStream_t s) {
     if (map.n_blocks == 0) return hipSuccess;
     PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_build<PD, 0, double>), dim3(map.n_blocks),
                                            dim3(kBlock), 0, s, PointFeatures{}, map, ScaleFactor{},
                                            cell_keys, n_cells - 1u, counters, replay, xcd_aware,
                                            (const float *)nullptr, 0, (float *)nullptr,
-                                           created_lists, points));
+                                           created_lists, points, regions));
     return hipGetLastError();
 }
 
@@ -1165,12 +1170,12 @@ hipError_t number_vertices(int pd, const PointMap &map, const CreatedLists &list
 
 hipError_t neighbours(int pd, const VertexTables &vertices, const Counters *counters,
                       const uint64_t *cell_keys, uint32_t n_cells, int launch_vertices,
-                      hipStream_t s) {
+                      const RegionSource &regions, hipStream_t s) {
     if (vertices.max_vertices <= 0) return hipErrorInvalidValue;
     const size_t items = (size_t)(pd + 1) * ((size_t)launch_vertices + kBlock);
     PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_neighbours<PD>), dim3(vertex_blocks(items)),
                                            dim3(kBlock), 0, s, vertices, counters, cell_keys,
-                                           n_cells - 1u));
+                                           n_cells - 1u, regions));
     return hipGetLastError();
 }
 
