@@ -71,8 +71,12 @@ __device__ __forceinline__ uint32_t hash_key(uint64_t k) {
 // the table that belongs to its band, what an XCD looks up -- its own vertices and their
 // neighbours -- lies in an eighth of the table instead of all over it.  Feature 0 can be read off a
 // key: the first two coordinates of an elevated point differ by twice its scaled feature 0, and a
-// vertex is within pd+1 of the points that touch it.  The band only picks the leading bits of the
-// cell; probing runs on over the whole table, so any spread of the keys is handled, evenly or not.
+// vertex is within pd+1 of the points that touch it.
+// Only the first two cells of a key's probe sequence are in its band's part (an aligned pair, so
+// one 16-byte piece of a line); after them the sequence is the plain one, from the key's hash over
+// the whole table.  With the table a fifth full that places 19 keys of 20 in their band, and an
+// input whose vertices crowd into one band (an image that is flat but for a few rows) costs every
+// key two more probe steps and nothing else.
 struct KeyRegions {
     float lo, per_unit;   // band = (scaled feature 0 - lo) * per_unit, clamped to 0..7; per_unit 0: one band
 };
@@ -109,7 +113,13 @@ __device__ __forceinline__ uint32_t cell_of_key(uint64_t key, uint32_t mask, con
     int band = (int)((c - regions.lo) * regions.per_unit);
     band = band < 0 ? 0 : (band > 7 ? 7 : band);
     const uint32_t low = mask >> 3;   // the table has at least 4096 cells
-    return ((uint32_t)band * (low + 1u)) | (h & low);
+    return (((uint32_t)band * (low + 1u)) | (h & low)) & ~1u;
+}
+// The cell after `cell`, the step-th of key's probe sequence (step counts from 0).
+__device__ __forceinline__ uint32_t next_cell(uint32_t cell, uint32_t step, uint64_t key, uint32_t mask,
+                                             const KeyRegions &regions) {
+    if (regions.per_unit != 0.0f && step == 1u) return hash_key(key) & mask;
+    return (cell + 1u) & mask;
 }
 
 // ------------------------------------------------------------------------------------------------

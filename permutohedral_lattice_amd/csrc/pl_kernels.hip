@@ -244,7 +244,7 @@ __global__ __launch_bounds__(kBlock) void k_build(PointFeatures features, PointM
         cell[r] = cell_of_key<PD>(key[r], mask, regions);
     }
     bool any_open = open != 0;
-    for (uint32_t probe = 0; any_open && probe <= mask; ++probe) {
+    for (uint32_t probe = 0; any_open && probe <= mask + 2u; ++probe) {
 #pragma unroll
         for (int r = 0; r < D1; ++r)
             seen[r] = (open >> r) & 1u ? *cell_at(cell_keys, cell[r]) : key[r];
@@ -260,7 +260,7 @@ __global__ __launch_bounds__(kBlock) void k_build(PointFeatures features, PointM
                     if (seen[r] == kEmptyCell) created |= 1u << r;
                     open &= ~(1u << r);           // swapped in, or already there
                 } else {
-                    cell[r] = (cell[r] + 1u) & mask;
+                    cell[r] = next_cell(cell[r], probe, key[r], mask, regions);
                 }
             }
         }
@@ -456,14 +456,14 @@ __global__ __launch_bounds__(kBlock) void k_neighbours(VertexTables vertices,
     const uint64_t want = KeyCodec<PD>::pack(qp, wrap_up ? 0 : r + 1);
     uint32_t h = cell_of_key<PD>(want, mask, regions);
     int u = -1;
-    for (uint32_t probe = 0; probe <= mask; ++probe) {
+    for (uint32_t probe = 0; probe <= mask + 2u; ++probe) {
         const uint64_t cur = cell_keys[h];
         if (cur == want) {
             u = vertices.cell_vertex[h];
             break;
         }
         if (cur == kEmptyCell) break;
-        h = (h + 1u) & mask;
+        h = next_cell(h, probe, want, mask, regions);
     }
     if (u >= 0) {
         int *entries = reinterpret_cast<int *>(vertices.neighbours);

@@ -216,6 +216,44 @@ def test_point_grid_hint_changes_nothing_but_the_order_of_work(dims, pd, vd):
     assert_float_parity(again, want)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_points_crowded_into_one_band_of_the_first_feature(dtype):
+    """With a grid hint the hash table is divided by bands of feature 0 between the first and the
+    last point.  Here those two points are far apart and every other point sits in a narrow range
+    between them, so that all vertices fall into one band, more of them than that band's part of
+    the table holds: the keys must spill over the whole table, the result must not change, and the
+    call must not take longer than a few probe steps per key (a chain through a full part of the
+    table would take minutes)."""
+    import time
+    dims, pd, vd = (256, 256), 3, 2
+    n = dims[0] * dims[1]
+    rng = np.random.default_rng(77)
+    pos = rng.uniform(0, 1, (n, pd)) * np.array([10.0, 60.0, 60.0]) + np.array([245.0, 0.0, 0.0])
+    pos[0, 0], pos[-1, 0] = 0.0, 500.0
+    pos = pos.astype(dtype)
+    val = rng.uniform(0, 1, (n, vd - 1)).astype(dtype)
+    torch_dtype = torch.float32 if dtype == np.float32 else torch.float64
+    cpu = oracle.Lattice(pd, vd, n, dtype=dtype)
+    want = cpu.filter(val, pos)
+    lat = pla.PermutohedralLattice(pd, vd, n, dtype=torch_dtype)
+    lat.set_point_grid(dims)
+    out = torch.empty((n, vd - 1), dtype=torch_dtype, device="cuda")
+    d_val, d_pos = dev(val), dev(pos)
+    for _ in range(3):          # the table has its final size from the second call on
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        lat.filter(out, d_val, d_pos, False)
+        torch.cuda.synchronize()
+        elapsed = time.perf_counter() - t0
+        assert elapsed < 2.0
+        assert lat.num_vertices == cpu.num_vertices
+        if dtype == np.float32:
+            assert_float_parity(host(out), want)
+        else:
+            assert np.abs(host(out) - want).max() <= 1e-12
+    assert (sorted_keys(host(lat.debug_keys()))[0] == sorted_keys(cpu.keys())[0]).all()
+
+
 def test_point_grid_must_match_the_number_of_points():
     lat = pla.PermutohedralLattice(2, 2, 100)
     with pytest.raises(pla.PermutohedralError) as e:
