@@ -57,10 +57,14 @@ typedef enum pl_option {
                                of points; 0: plain workgroup order (for measuring the difference) */
     PL_OPT_PAIR_BLUR = 5,   /* 1 (default): two blur axes per kernel launch; 0: one launch per axis
                                (same results bit for bit; for measuring the difference) */
-    PL_OPT_GUESS_GRID = 6   /* 1 (default): a handle without pl_set_point_grid looks, the first time it
+    PL_OPT_GUESS_GRID = 6,  /* 1 (default): a handle without pl_set_point_grid looks, the first time it
                                sees positions, whether they describe a row-major image or volume (feature
                                0 changing exactly every row length points ...) and if so orders its
                                work as with the hint; 0: never (points are a plain list) */
+    PL_OPT_MERGE_TILES = 7  /* 1 (default): when the points are a grid, a workgroup of the build merges
+                               the keys and sums of its tile in LDS before they go to the hash table;
+                               0: every wavefront goes to the table itself (same results; for
+                               measuring the difference) */
 } pl_option;
 
 /* 1 when a lattice can be built for these dimensions, else 0.

@@ -22,6 +22,7 @@ LIB_PATH = os.path.join(_HERE, "libpermutohedral_hip.so")
 PL_OK, PL_EINVAL, PL_EUNSUPPORTED, PL_ENOMEM, PL_EOVERFLOW, PL_EHIP, PL_ESTATE = 0, -1, -2, -3, -4, -5, -6
 PL_OPT_NORMALIZE, PL_OPT_PROFILE, PL_OPT_TABLE_CELLS, PL_OPT_XCD_AWARE, PL_OPT_PAIR_BLUR = 1, 2, 3, 4, 5
 PL_OPT_GUESS_GRID = 6
+PL_OPT_MERGE_TILES = 7
 
 # every symbol include/permutohedral_lattice.h declares
 EXPORTS = (

@@ -120,6 +120,8 @@ struct pl_lattice {
     bool normalize = true;
     bool profile = false;
     bool xcd_aware = true;
+    bool merge_tiles = true;      // option: workgroups merge their keys in LDS when the points are a grid
+    bool tiles_fit = true;        // cleared when a build found a tile with too many distinct keys
     bool pair_blur = true;
     // the grid the points form: given by the caller (pl_set_point_grid), or guessed once from the
     // first positions the handle sees
@@ -289,15 +291,17 @@ int enqueue_build(pl_lattice *h, const plk::PointFeatures &features, const doubl
             regions.enabled = 0;
         }
     }
+    // tiles of an image share most of their vertices among their four wavefronts
+    const bool merge = h->merge_tiles && h->tiles_fit && h->map.mode != 0;
     if (h->f64) {
         const plk::Points64 points{positions64, h->weights64, h->scale64};
         PL_HIP(plk::build_f64(h->pd, points, h->map, h->cell_keys, cells, h->counters(), h->replay,
-                              h->xcd_aware ? 1 : 0, lists, regions, h->stream));
+                              h->xcd_aware ? 1 : 0, lists, regions, merge, h->stream));
     } else {
         PL_HIP(plk::build(h->pd, features, h->map, h->scale, h->cell_keys, cells, h->counters(),
                           h->replay, h->xcd_aware ? 1 : 0, fused ? h->vd : 0,
                           splat_input, h->normalize ? h->vd - 1 : h->vd, h->cell_values, lists,
-                          regions, h->stream));
+                          regions, merge, h->stream));
     }
     h->mark(EV_BUILD);
     // the numbering pass zeroes the vertices' value rows: a row of vd doubles is 2*vd zero floats
@@ -420,6 +424,16 @@ int verify_build(pl_lattice *h, uint32_t *retry_cells) {
     if (flags & plk::kFlagKeyRange) {
         h->built = false;
         h->table_clean = false;
+        return PL_EOVERFLOW;
+    }
+    if (flags & plk::kFlagTileFull) {
+        // a tile with more distinct keys than the merging build's LDS table holds: this lattice
+        // builds without merging from now on (until its point grid is set anew)
+        h->built = false;
+        h->table_clean = false;
+        h->cell_values_clean = false;
+        h->tiles_fit = false;
+        *retry_cells = h->n_cells;
         return PL_EOVERFLOW;
     }
     if ((flags & plk::kFlagTableFull) || (uint32_t)m > plk::max_vertices_for(h->n_cells)) {
@@ -565,6 +579,9 @@ int pl_set_option(pl_handle h, int option, long value) {
             return PL_OK;
         case PL_OPT_GUESS_GRID:
             h->guess_grid = value != 0;
+            return PL_OK;
+        case PL_OPT_MERGE_TILES:
+            h->merge_tiles = value != 0;
             return PL_OK;
         case PL_OPT_TABLE_CELLS:
             if (value < 0 || (value & (value - 1)) != 0) return PL_EINVAL;

@@ -15,6 +15,7 @@ constexpr uint64_t kEmptyCell = ~0ull;
 enum : int {
     kFlagTableFull = 1,   // a probe sequence wrapped, or more vertices were created than the table may hold
     kFlagKeyRange = 2,    // a lattice coordinate does not fit its field of the packed key
+    kFlagTileFull = 4,    // a workgroup of the merging build has more distinct keys than its LDS table holds
 };
 
 // Device-side state of one build.  Kernels after the numbering pass read the vertex count from
@@ -135,14 +136,14 @@ hipError_t build(int pd, const PointFeatures &features, const PointMap &map, con
                  uint64_t *cell_keys, uint32_t n_cells, Counters *counters, ReplayEntry *replay,
                  int xcd_aware, int splat_vd, const float *input,
                  int in_channels, float *cell_values, const CreatedLists &created_lists,
-                 const RegionSource &regions, hipStream_t s);
+                 const RegionSource &regions, bool merge_in_workgroup, hipStream_t s);
 
 // The build for double values: the same kernel on points.positions with points.scale; replay[]
 // receives the cells (and the weights rounded to float), points.weights[r*T+t] the weights.
 hipError_t build_f64(int pd, const Points64 &points, const PointMap &map, uint64_t *cell_keys,
                      uint32_t n_cells, Counters *counters, ReplayEntry *replay, int xcd_aware,
                      const CreatedLists &created_lists, const RegionSource &regions,
-                     hipStream_t s);
+                     bool merge_in_workgroup, hipStream_t s);
 
 // Dense vertex numbers in the order of the build's workgroups (same map as the build):
 // cell_vertex[cell] := v, vertex_keys[v] := key, vertex_cell[v] := cell,

@@ -341,6 +341,231 @@ __global__ __launch_bounds__(kBlock) void k_build(PointFeatures features, PointM
     }
 }
 
+// The same stage with the keys and sums of a whole workgroup merged in LDS before they go to the
+// table: for an image tile of 16x16 pixels the four wavefronts hold about 165 (wavefront, vertex)
+// pairs but only about 100 distinct vertices, and what limits the build is the number of requests
+// to the L2 atomic unit (one per compare-and-swap, one per row of sums).  Each wavefront elects
+// its leaders and sums its groups as above, but the leaders place their keys in a small hash table
+// in LDS and the sums are added to the rows of the LDS slots; then every occupied slot is placed
+// in the table in HBM by one thread, and its row goes out with one request.  A workgroup whose
+// distinct keys do not fit the LDS table raises kFlagTileFull and the host repeats the build with
+// k_build.  Three barriers; every thread reaches each of them.
+constexpr int kTileSlots = 2 * kBlock;    // LDS slots per workgroup (at most 6 * kBlock keys exist)
+constexpr int kTileProbeLimit = 48;
+
+template <int PD, int SPLAT_VD, typename T = float>
+__global__ __launch_bounds__(kBlock) void k_build_tile(PointFeatures features, PointMap map,
+                                                        ScaleFactor scale, uint64_t *cell_keys,
+                                                        uint32_t mask, Counters *counters,
+                                                        ReplayEntry *__restrict__ replay,
+                                                        int xcd_aware, const float *__restrict__ input,
+                                                        int in_channels, float *cell_values,
+                                                        CreatedLists created_lists,
+                                                        Points64 points64, RegionSource region_source) {
+    constexpr bool kDouble = sizeof(T) == sizeof(double);
+    static_assert(!kDouble || SPLAT_VD == 0, "the fused splat is for float values");
+    constexpr int D1 = PD + 1;
+    constexpr int VD = SPLAT_VD ? SPLAT_VD : 2;
+    constexpr int P = VD == 2 ? 2 : 4;      // floats per LDS row of sums
+    __shared__ uint64_t slot_key[kTileSlots];
+    __shared__ int slot_cell[kTileSlots];
+    __shared__ float slot_sum[SPLAT_VD ? kTileSlots * P : 1];
+    __shared__ int group_created;
+    const int tid = threadIdx.x;
+    for (int i = tid; i < kTileSlots; i += kBlock) slot_key[i] = kEmptyCell;
+    if (SPLAT_VD)
+        for (int i = tid; i < kTileSlots * P; i += kBlock) slot_sum[i] = 0.0f;
+    if (tid == 0) group_created = 0;
+
+    const unsigned vblock = xcd_contiguous_block(blockIdx.x, gridDim.x, xcd_aware);
+    const size_t t = (size_t)vblock * kBlock + tid;   // slot in the replay arrays
+    const size_t n_slots = (size_t)gridDim.x * kBlock;
+    const int n = point_of_thread(map, vblock, tid);
+    const int lane = tid & 63;
+    const bool valid = n >= 0;
+
+    Simplex<PD, T> s;
+    if constexpr (kDouble) {
+        double pos[PD];
+#pragma unroll
+        for (int i = 0; i < PD; ++i) pos[i] = valid ? points64.positions[(size_t)n * PD + i] : 0.0;
+        enclosing_simplex<PD>(pos, points64.scale, s);
+    } else {
+        float pos[PD];
+#pragma unroll
+        for (int i = 0; i < PD; ++i) pos[i] = 0.0f;
+        if (valid) load_features<PD>(features, n, pos);
+        enclosing_simplex<PD>(pos, scale, s);
+    }
+#pragma unroll
+    for (int r = 0; r < D1; ++r) asm volatile("" : "+v"(s.weight[r]));
+    const bool in_range = simplex_in_key_range<PD>(s);
+    if (valid && !in_range) atomicOr(&counters->flags, kFlagKeyRange);
+    const bool active = valid && in_range;
+
+    unsigned leaders[(D1 + 4) / 5] = {};
+    auto leader_of = [&](int r) { return (int)((leaders[r / 5] >> (6 * (r % 5))) & 63u); };
+    int slot[D1];           // the LDS slot of key r, at first in the lanes of the leaders only
+    __syncthreads();        // the LDS table is empty
+    {
+        uint64_t key[D1];
+        unsigned open = 0;
+#pragma unroll
+        for (int r = 0; r < D1; ++r) {
+            int q[PD];
+            vertex_q<PD>(s, r, q);
+            key[r] = KeyCodec<PD>::pack(q, r);
+            const int leader = wave_leader_of_equal(key[r], active, lane);
+            leaders[r / 5] |= (unsigned)leader << (6 * (r % 5));
+            if (active && leader == lane) open |= 1u << r;
+            slot[r] = (int)((hash_key(key[r]) >> 20) & (kTileSlots - 1));
+        }
+        bool any_open = open != 0;
+        for (int probe = 0; any_open && probe < kTileProbeLimit; ++probe) {
+#pragma unroll
+            for (int r = 0; r < D1; ++r) {
+                if ((open >> r) & 1u) {
+                    const uint64_t seen =
+                        atomicCAS((unsigned long long *)&slot_key[slot[r]],
+                                  (unsigned long long)kEmptyCell, (unsigned long long)key[r]);
+                    if (seen == kEmptyCell || seen == key[r])
+                        open &= ~(1u << r);
+                    else
+                        slot[r] = (slot[r] + 1) & (kTileSlots - 1);
+                }
+            }
+            any_open = open != 0;
+        }
+        if (any_open) atomicOr(&counters->flags, kFlagTileFull);
+#pragma unroll
+        for (int r = 0; r < D1; ++r)
+            if ((open >> r) & 1u) slot[r] = -1;
+    }
+
+    float val[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (SPLAT_VD) {
+#pragma unroll
+        for (int j = 0; j < SPLAT_VD; ++j) val[j] = 1.0f;  // homogeneous channel when vd-1 are given
+        if (valid) {
+#pragma unroll
+            for (int j = 0; j < SPLAT_VD; ++j)
+                if (j < in_channels) val[j] = input[(size_t)n * in_channels + j];
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < D1; ++r) {
+        const int leader = leader_of(r);
+        const int own = slot[r];
+        slot[r] = active ? __shfl(own, leader) : -1;
+        if (SPLAT_VD) {
+            const float w = (float)s.weight[r];
+            const float term[4] = {w * val[0], w * val[1], w * val[2], w * val[3]};
+            const QuadTerms quad = quad_terms<VD>(term, lane);
+            const uint64_t among = wave_ballot(active);
+            uint64_t remaining = among;
+            while (remaining) {
+                const int first = __builtin_ctzll(remaining);
+                const uint64_t group = lanes_equal(leader, first) & among;
+                remaining &= ~group;
+                const bool same = lane_in(group);
+                const int group_slot = lane_value(own, first);
+                const float sum = wave_sum_to_last_lanes<VD>(same, quad, lane);
+                if (group_slot >= 0 && lane >= 64 - P && channel_of_lane<VD>(lane) < VD)
+                    atomicAdd(&slot_sum[group_slot * P + channel_of_lane<VD>(lane)], sum);
+            }
+        }
+    }
+    __syncthreads();        // the keys and sums of all four wavefronts are in the LDS table
+
+    // Every occupied slot goes to the table in HBM: thread i takes slots i and i + kBlock, in
+    // rounds over both as in k_build.
+    constexpr int H = kTileSlots / kBlock;
+    const KeyRegions regions = key_regions(region_source);
+    {
+        uint64_t key[H], seen[H];
+        uint32_t cell[H];
+        unsigned open = 0, created = 0;
+#pragma unroll
+        for (int h = 0; h < H; ++h) {
+            key[h] = slot_key[tid + h * kBlock];
+            if (key[h] != kEmptyCell) open |= 1u << h;
+            cell[h] = cell_of_key<PD>(key[h], mask, regions);
+        }
+        bool any_open = open != 0;
+        for (uint32_t probe = 0; any_open && probe <= mask + 2u; ++probe) {
+#pragma unroll
+            for (int h = 0; h < H; ++h)
+                seen[h] = (open >> h) & 1u ? *cell_at(cell_keys, cell[h]) : key[h];
+#pragma unroll
+            for (int h = 0; h < H; ++h)
+                if (((open >> h) & 1u) && seen[h] == kEmptyCell)
+                    seen[h] = atomicCAS((unsigned long long *)cell_at(cell_keys, cell[h]),
+                                        (unsigned long long)kEmptyCell, (unsigned long long)key[h]);
+#pragma unroll
+            for (int h = 0; h < H; ++h) {
+                if ((open >> h) & 1u) {
+                    if (seen[h] == kEmptyCell || seen[h] == key[h]) {
+                        if (seen[h] == kEmptyCell) created |= 1u << h;
+                        open &= ~(1u << h);
+                    } else {
+                        cell[h] = next_cell(cell[h], probe, key[h], mask, regions);
+                    }
+                }
+            }
+            any_open = open != 0;
+        }
+        if (any_open) atomicOr(&counters->flags, kFlagTableFull);
+#pragma unroll
+        for (int h = 0; h < H; ++h)
+            slot_cell[tid + h * kBlock] = (open >> h) & 1u ? -1 : (int)cell[h];
+
+        // the vertices this workgroup created, as in k_build
+        int offset[H];
+        int total = 0;
+#pragma unroll
+        for (int h = 0; h < H; ++h) {
+            const uint64_t b = wave_ballot((created >> h) & 1u);
+            offset[h] = total + (int)__builtin_amdgcn_mbcnt_hi(
+                                    (uint32_t)(b >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)b, 0u));
+            total += __builtin_popcountll(b);
+        }
+        int base = 0;
+        if (lane == 0 && total) base = atomicAdd(&group_created, total);
+        base = __builtin_amdgcn_readfirstlane(base);
+        const size_t list = (size_t)vblock * (kBlock * D1);
+#pragma unroll
+        for (int h = 0; h < H; ++h) {
+            if ((created >> h) & 1u) {
+                created_lists.entries[list + base + offset[h]] =
+                    make_uint4((uint32_t)key[h], (uint32_t)(key[h] >> 32), cell[h], 0u);
+            }
+        }
+    }
+    __syncthreads();        // every slot's cell is known, and so is the number of vertices created
+    if (tid == 0) {
+        const int sum = group_created;
+        created_lists.block_count[vblock] = sum;
+        if (sum) atomicAdd(&created_lists.chunk_count[vblock / kBlocksPerChunk], sum);
+    }
+    if (SPLAT_VD) {
+        // rows of sums: P consecutive lanes per slot, one request per row
+#pragma unroll
+        for (int i = 0; i < kTileSlots * P / kBlock; ++i) {
+            const int sl = i * (kBlock / P) + tid / P;
+            const int channel = tid % P;
+            const int cell = slot_cell[sl];
+            if (slot_key[sl] != kEmptyCell && cell >= 0 && channel < VD)
+                atomicAdd(cell_values + (size_t)cell * VD + channel, slot_sum[sl * P + channel]);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < D1; ++r) {
+        const int c = slot[r] >= 0 ? slot_cell[slot[r]] : -1;
+        replay[(size_t)r * n_slots + t] = ReplayEntry{c, valid ? (float)s.weight[r] : 0.0f};
+        if constexpr (kDouble) points64.weights[(size_t)r * n_slots + t] = valid ? s.weight[r] : 0.0;
+    }
+}
+
 // Dense vertex numbering in the order of the build's workgroups, i.e. of the image tiles: the
 // vertices a workgroup created follow those of the workgroups before it.  Vertices that are close
 // in the lattice were created by the same or a neighbouring tile, so their numbers are close, and
@@ -1124,14 +1349,17 @@ hipError_t build(int pd, const PointFeatures &features, const PointMap &map, con
                  uint64_t *cell_keys, uint32_t n_cells, Counters *counters, ReplayEntry *replay,
                  int xcd_aware, int splat_vd, const float *input,
                  int in_channels, float *cell_values, const CreatedLists &created_lists,
-                 const RegionSource &regions, hipStream_t s) {
+                 const RegionSource &regions, bool merge_in_workgroup, hipStream_t s) {
     if (map.n_blocks == 0) return hipSuccess;
+#define PLK_BUILD_ARGS                                                                             \
+    dim3(map.n_blocks), dim3(kBlock), 0, s, features, map, scale, cell_keys, n_cells - 1u,         \
+        counters, replay, xcd_aware, input, in_channels, cell_values, created_lists, Points64{},   \
+        regions
 #define PLK_BUILD(SPLAT_VD)                                                                        \
-    PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_build<PD, SPLAT_VD>), dim3(map.n_blocks),            \
-                                           dim3(kBlock), 0, s, features, map, scale, cell_keys,    \
-                                           n_cells - 1u, counters, replay,                         \
-                                           xcd_aware, input, in_channels, cell_values,             \
-                                           created_lists, Points64{}, regions))
+    if (merge_in_workgroup)                                                                        \
+        PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_build_tile<PD, SPLAT_VD>), PLK_BUILD_ARGS))      \
+    else                                                                                           \
+        PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_build<PD, SPLAT_VD>), PLK_BUILD_ARGS))
     switch (splat_vd) {
         case 0: PLK_BUILD(0); break;
         case 2: PLK_BUILD(2); break;
@@ -1140,19 +1368,24 @@ hipError_t build(int pd, const PointFeatures &features, const PointMap &map, con
         default: return hipErrorInvalidValue;
     }
 #undef PLK_BUILD
+#undef PLK_BUILD_ARGS
     return hipGetLastError();
 }
 
 hipError_t build_f64(int pd, const Points64 &points, const PointMap &map, uint64_t *cell_keys,
                      uint32_t n_cells, Counters *counters, ReplayEntry *replay, int xcd_aware,
                      const CreatedLists &created_lists, const RegionSource &regions,
-                     hipStream_t s) {
+                     bool merge_in_workgroup, hipStream_t s) {
     if (map.n_blocks == 0) return hipSuccess;
-    PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_build<PD, 0, double>), dim3(map.n_blocks),
-                                           dim3(kBlock), 0, s, PointFeatures{}, map, ScaleFactor{},
-                                           cell_keys, n_cells - 1u, counters, replay, xcd_aware,
-                                           (const float *)nullptr, 0, (float *)nullptr,
-                                           created_lists, points, regions));
+#define PLK_BUILD_ARGS                                                                             \
+    dim3(map.n_blocks), dim3(kBlock), 0, s, PointFeatures{}, map, ScaleFactor{}, cell_keys,        \
+        n_cells - 1u, counters, replay, xcd_aware, (const float *)nullptr, 0, (float *)nullptr,    \
+        created_lists, points, regions
+    if (merge_in_workgroup)
+        PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_build_tile<PD, 0, double>), PLK_BUILD_ARGS))
+    else
+        PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_build<PD, 0, double>), PLK_BUILD_ARGS))
+#undef PLK_BUILD_ARGS
     return hipGetLastError();
 }
 
