@@ -103,7 +103,7 @@ __device__ __forceinline__ KeyRegions key_regions(const RegionSource &src) {
 template <int PD>
 __device__ __forceinline__ uint32_t cell_of_key(uint64_t key, uint32_t mask, const KeyRegions &regions) {
     const uint32_t h = hash_key(key);
-    if (regions.per_unit == 0.0f) return h & mask;
+    if (regions.per_unit == 0.0f) return h & mask & ~1u;
     int q[PD], r;
     KeyCodec<PD>::unpack(key, q, r);
     // scaled feature 0 of the points around this vertex: half the difference of its first two
@@ -115,11 +115,18 @@ __device__ __forceinline__ uint32_t cell_of_key(uint64_t key, uint32_t mask, con
     const uint32_t low = mask >> 3;   // the table has at least 4096 cells
     return (((uint32_t)band * (low + 1u)) | (h & low)) & ~1u;
 }
-// The cell after `cell`, the step-th of key's probe sequence (step counts from 0).
+// A probe sequence is a sequence of aligned pairs of cells (16 bytes, one load), walked first cell
+// first.  The cell after `cell`, the step-th of key's sequence (step counts from 0):
 __device__ __forceinline__ uint32_t next_cell(uint32_t cell, uint32_t step, uint64_t key, uint32_t mask,
                                              const KeyRegions &regions) {
-    if (regions.per_unit != 0.0f && step == 1u) return hash_key(key) & mask;
+    if (regions.per_unit != 0.0f && step == 1u) return hash_key(key) & mask & ~1u;
     return (cell + 1u) & mask;
+}
+// and the pair after the pair that starts at `cell`, the index-th pair of the sequence
+__device__ __forceinline__ uint32_t next_pair(uint32_t cell, uint32_t index, uint64_t key, uint32_t mask,
+                                             const KeyRegions &regions) {
+    if (regions.per_unit != 0.0f && index == 0u) return hash_key(key) & mask & ~1u;
+    return (cell + 2u) & mask;
 }
 
 // ------------------------------------------------------------------------------------------------

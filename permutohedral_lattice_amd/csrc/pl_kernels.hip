@@ -482,34 +482,60 @@ __global__ __launch_bounds__(kBlock) void k_build_tile(PointFeatures features, P
     constexpr int H = kTileSlots / kBlock;
     const KeyRegions regions = key_regions(region_source);
     {
-        uint64_t key[H], seen[H];
-        uint32_t cell[H];
+        // A round looks at the pair of cells a key has come to (one 16-byte load), takes the key's
+        // cell if it is there, else swaps the key into the pair's first empty cell, else moves on
+        // to the next pair.  A swap lost to another key looks at the same pair again: each turn
+        // either moves on or sees a cell of the pair filled for good.
+        uint64_t key[H];
+        uint32_t cell[H], pair_index[H];
+        ulonglong2 seen[H];
         unsigned open = 0, created = 0;
 #pragma unroll
         for (int h = 0; h < H; ++h) {
             key[h] = slot_key[tid + h * kBlock];
             if (key[h] != kEmptyCell) open |= 1u << h;
             cell[h] = cell_of_key<PD>(key[h], mask, regions);
+            pair_index[h] = 0;
         }
         bool any_open = open != 0;
-        for (uint32_t probe = 0; any_open && probe <= mask + 2u; ++probe) {
+        for (uint32_t turn = 0; any_open && turn <= 2u * mask + 8u; ++turn) {
 #pragma unroll
             for (int h = 0; h < H; ++h)
-                seen[h] = (open >> h) & 1u ? *cell_at(cell_keys, cell[h]) : key[h];
-#pragma unroll
-            for (int h = 0; h < H; ++h)
-                if (((open >> h) & 1u) && seen[h] == kEmptyCell)
-                    seen[h] = atomicCAS((unsigned long long *)cell_at(cell_keys, cell[h]),
-                                        (unsigned long long)kEmptyCell, (unsigned long long)key[h]);
+                if ((open >> h) & 1u)
+                    seen[h] = *reinterpret_cast<const ulonglong2 *>(cell_at(cell_keys, cell[h]));
+            int target[H];
 #pragma unroll
             for (int h = 0; h < H; ++h) {
+                target[h] = -1;
                 if ((open >> h) & 1u) {
-                    if (seen[h] == kEmptyCell || seen[h] == key[h]) {
-                        if (seen[h] == kEmptyCell) created |= 1u << h;
+                    if (seen[h].x == key[h]) {
                         open &= ~(1u << h);
+                    } else if (seen[h].x == kEmptyCell) {
+                        target[h] = 0;
+                    } else if (seen[h].y == key[h]) {
+                        cell[h] += 1u;
+                        open &= ~(1u << h);
+                    } else if (seen[h].y == kEmptyCell) {
+                        target[h] = 1;
                     } else {
-                        cell[h] = next_cell(cell[h], probe, key[h], mask, regions);
+                        cell[h] = next_pair(cell[h], pair_index[h], key[h], mask, regions);
+                        pair_index[h] += 1u;
                     }
+                }
+            }
+            uint64_t found[H];
+#pragma unroll
+            for (int h = 0; h < H; ++h)
+                if (target[h] >= 0)
+                    found[h] = atomicCAS(
+                        (unsigned long long *)cell_at(cell_keys, cell[h] + (uint32_t)target[h]),
+                        (unsigned long long)kEmptyCell, (unsigned long long)key[h]);
+#pragma unroll
+            for (int h = 0; h < H; ++h) {
+                if (target[h] >= 0 && (found[h] == kEmptyCell || found[h] == key[h])) {
+                    if (found[h] == kEmptyCell) created |= 1u << h;
+                    cell[h] += (uint32_t)target[h];
+                    open &= ~(1u << h);
                 }
             }
             any_open = open != 0;
@@ -681,14 +707,14 @@ __global__ __launch_bounds__(kBlock) void k_neighbours(VertexTables vertices,
     const uint64_t want = KeyCodec<PD>::pack(qp, wrap_up ? 0 : r + 1);
     uint32_t h = cell_of_key<PD>(want, mask, regions);
     int u = -1;
-    for (uint32_t probe = 0; probe <= mask + 2u; ++probe) {
-        const uint64_t cur = cell_keys[h];
-        if (cur == want) {
-            u = vertices.cell_vertex[h];
+    for (uint32_t index = 0; index <= (mask >> 1) + 1u; ++index) {
+        const ulonglong2 cur = *reinterpret_cast<const ulonglong2 *>(cell_keys + h);
+        if (cur.x == want || (cur.x != kEmptyCell && cur.y == want)) {
+            u = vertices.cell_vertex[cur.x == want ? h : h + 1u];
             break;
         }
-        if (cur == kEmptyCell) break;
-        h = next_cell(h, probe, want, mask, regions);
+        if (cur.x == kEmptyCell || cur.y == kEmptyCell) break;
+        h = next_pair(h, index, want, mask, regions);
     }
     if (u >= 0) {
         int *entries = reinterpret_cast<int *>(vertices.neighbours);
