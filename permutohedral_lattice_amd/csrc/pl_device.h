@@ -381,6 +381,22 @@ __device__ __forceinline__ int wave_leader_of_equal(T x, bool active, int lane) 
     }
     return leader;
 }
+// The same, and the mask of the lanes whose group has at most small_size members.
+template <typename T>
+__device__ __forceinline__ int wave_leader_of_equal(T x, bool active, int lane, int small_size, uint64_t &small) {
+    int leader = lane;
+    small = 0;
+    const uint64_t among = wave_ballot(active);
+    uint64_t remaining = among;
+    while (remaining) {
+        const int first = __builtin_ctzll(remaining);
+        const uint64_t same = lanes_equal(x, lane_value(x, first)) & among;
+        if (lane_in(same)) leader = first;
+        remaining &= ~same;
+        if (__builtin_popcountll(same) <= small_size) small |= same;
+    }
+    return leader;
+}
 
 __device__ __forceinline__ int vertex_count(const Counters *counters, int max_vertices) {
     const uint32_t m = counters->vertices;

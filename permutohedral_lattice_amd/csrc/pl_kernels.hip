@@ -406,6 +406,10 @@ __global__ __launch_bounds__(kBlock) void k_build_tile(PointFeatures features, P
     unsigned leaders[(D1 + 4) / 5] = {};
     auto leader_of = [&](int r) { return (int)((leaders[r / 5] >> (6 * (r % 5))) & 63u); };
     int slot[D1];           // the LDS slot of key r, at first in the lanes of the leaders only
+    // Groups of a few lanes add their terms to the slot's row one by one; the tree that sums a
+    // group costs the same for two lanes as for sixty-four, and half the groups have four or fewer.
+    constexpr int kSmallGroup = SPLAT_VD ? 4 : 0;
+    uint64_t small[D1];
     __syncthreads();        // the LDS table is empty
     {
         uint64_t key[D1];
@@ -415,7 +419,7 @@ __global__ __launch_bounds__(kBlock) void k_build_tile(PointFeatures features, P
             int q[PD];
             vertex_q<PD>(s, r, q);
             key[r] = KeyCodec<PD>::pack(q, r);
-            const int leader = wave_leader_of_equal(key[r], active, lane);
+            const int leader = wave_leader_of_equal(key[r], active, lane, kSmallGroup, small[r]);
             leaders[r / 5] |= (unsigned)leader << (6 * (r % 5));
             if (active && leader == lane) open |= 1u << r;
             slot[r] = (int)((hash_key(key[r]) >> 20) & (kTileSlots - 1));
@@ -461,7 +465,7 @@ __global__ __launch_bounds__(kBlock) void k_build_tile(PointFeatures features, P
             const float w = (float)s.weight[r];
             const float term[4] = {w * val[0], w * val[1], w * val[2], w * val[3]};
             const QuadTerms quad = quad_terms<VD>(term, lane);
-            const uint64_t among = wave_ballot(active);
+            const uint64_t among = wave_ballot(active) & ~small[r];
             uint64_t remaining = among;
             while (remaining) {
                 const int first = __builtin_ctzll(remaining);
@@ -472,6 +476,10 @@ __global__ __launch_bounds__(kBlock) void k_build_tile(PointFeatures features, P
                 const float sum = wave_sum_to_last_lanes<VD>(same, quad, lane);
                 if (group_slot >= 0 && lane >= 64 - P && channel_of_lane<VD>(lane) < VD)
                     atomicAdd(&slot_sum[group_slot * P + channel_of_lane<VD>(lane)], sum);
+            }
+            if (lane_in(small[r]) && slot[r] >= 0) {
+#pragma unroll
+                for (int j = 0; j < VD; ++j) atomicAdd(&slot_sum[slot[r] * P + j], term[j]);
             }
         }
     }
