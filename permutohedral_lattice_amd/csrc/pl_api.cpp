@@ -86,7 +86,7 @@ struct pl_lattice {
     int *vertex_cell = nullptr;        // [3/4 n_cells_alloc]
     float *values[2] = {nullptr, nullptr};  // [3/4 n_cells_alloc * vd]
     int2 *neighbours = nullptr;        // [(pd+1) * 3/4 n_cells_alloc]
-    float *cell_values = nullptr;      // [n_cells_alloc * vd], rows by hash cell (fused build+splat)
+    float *cell_values = nullptr;      // [n_cells_alloc * vd] values, rows by hash cell (fused build+splat)
     bool cell_values_clean = false;    // all zero
     uint32_t n_cells_alloc = 0;
     uint32_t n_cells = 0;              // in use by the last build
@@ -190,9 +190,9 @@ int ensure_table(pl_lattice *h, uint32_t cells) {
     h->values[0] = (float *)h->dmalloc(h->value_size() * mv * (size_t)h->vd);
     h->values[1] = (float *)h->dmalloc(h->value_size() * mv * (size_t)h->vd);
     h->neighbours = (int2 *)h->dmalloc(sizeof(int2) * mv * (size_t)(h->pd + 1));
-    const bool fused_splat = plk::build_can_splat(h->vd) && !h->f64;
+    const bool fused_splat = plk::build_can_splat(h->vd);
     if (fused_splat)
-        h->cell_values = (float *)h->dmalloc(sizeof(float) * (size_t)cells * (size_t)h->vd);
+        h->cell_values = (float *)h->dmalloc(h->value_size() * (size_t)cells * (size_t)h->vd);
     if (!h->cell_keys || !h->cell_vertex || !h->vertex_keys || !h->vertex_cell || !h->values[0] ||
         !h->values[1] || !h->neighbours || (fused_splat && !h->cell_values))
         return PL_ENOMEM;
@@ -248,16 +248,21 @@ uint32_t initial_cells(const pl_lattice *h) {
 // and the value table holds them when the build is done.
 // A lattice for double values takes its positions from positions64 and never splats in the build.
 int enqueue_build(pl_lattice *h, const plk::PointFeatures &features, const double *positions64,
-                  uint32_t cells, const float *splat_input) {
+                  uint32_t cells, const void *splat_input) {
     int rc = ensure_table(h, cells);
     if (rc != PL_OK) return rc;
     // the per-point arrays follow the point map; an allocation that failed when the map was set
     // is made up for here
     rc = ensure_replay(h);
     if (rc != PL_OK) return rc;
-    const bool fused = splat_input && plk::build_can_splat(h->vd) && !h->f64;
+    // tiles of an image share most of their vertices among their four wavefronts
+    const bool merge = h->merge_tiles && h->tiles_fit && h->map.mode != 0;
+    // (a lattice of doubles splats in its build only in the merging kernel)
+    const bool fused = splat_input && plk::build_can_splat(h->vd) && (!h->f64 || merge);
+    const size_t floats_per_value = h->f64 ? 2 : 1;
     if (fused && !h->cell_values_clean) {
-        PL_HIP(plk::fill_zero(h->cell_values, (size_t)h->n_cells_alloc * h->vd, h->stream));
+        PL_HIP(plk::fill_zero(h->cell_values, (size_t)h->n_cells_alloc * h->vd * floats_per_value,
+                              h->stream));
         h->cell_values_clean = true;
     }
     h->mark(EV_T0);
@@ -291,16 +296,18 @@ int enqueue_build(pl_lattice *h, const plk::PointFeatures &features, const doubl
             regions.enabled = 0;
         }
     }
-    // tiles of an image share most of their vertices among their four wavefronts
-    const bool merge = h->merge_tiles && h->tiles_fit && h->map.mode != 0;
     if (h->f64) {
         const plk::Points64 points{positions64, h->weights64, h->scale64};
         PL_HIP(plk::build_f64(h->pd, points, h->map, h->cell_keys, cells, h->counters(), h->replay,
-                              h->xcd_aware ? 1 : 0, lists, regions, merge, h->stream));
+                              h->xcd_aware ? 1 : 0, lists, regions, merge, fused ? h->vd : 0,
+                              static_cast<const double *>(splat_input),
+                              h->normalize ? h->vd - 1 : h->vd,
+                              reinterpret_cast<double *>(h->cell_values), h->stream));
     } else {
         PL_HIP(plk::build(h->pd, features, h->map, h->scale, h->cell_keys, cells, h->counters(),
                           h->replay, h->xcd_aware ? 1 : 0, fused ? h->vd : 0,
-                          splat_input, h->normalize ? h->vd - 1 : h->vd, h->cell_values, lists,
+                          static_cast<const float *>(splat_input),
+                          h->normalize ? h->vd - 1 : h->vd, h->cell_values, lists,
                           regions, merge, h->stream));
     }
     h->mark(EV_BUILD);
@@ -332,14 +339,19 @@ int enqueue_apply_f64(pl_lattice *h, double *output, const double *input, int re
     double *values[2] = {reinterpret_cast<double *>(h->values[0]),
                          reinterpret_cast<double *>(h->values[1])};
     h->mark(EV_A0);
-    if (!h->values_zeroed)
-        PL_HIP(plk::fill_zero(h->values[0], (size_t)mv * vd * 2, h->stream));
-    h->mark(EV_FILL);
-    PL_HIP(plk::splat_f64(pd, vd, h->map, input, in_channels, h->replay, h->weights64,
-                          h->replay_holds_cells ? h->cell_vertex : nullptr, values[0],
-                          h->xcd_aware ? 1 : 0, h->stream));
-    h->replay_holds_cells = false;
+    if (!h->values_splatted) {
+        if (!h->values_zeroed)
+            PL_HIP(plk::fill_zero(h->values[0], (size_t)mv * vd * 2, h->stream));
+        h->mark(EV_FILL);
+        PL_HIP(plk::splat_f64(pd, vd, h->map, input, in_channels, h->replay, h->weights64,
+                              h->replay_holds_cells ? h->cell_vertex : nullptr, values[0],
+                              h->xcd_aware ? 1 : 0, h->stream));
+        h->replay_holds_cells = false;
+    } else {
+        h->mark(EV_FILL);
+    }
     h->values_zeroed = false;
+    h->values_splatted = false;
     h->mark(EV_SPLAT);
     int cur = 0;
     for (int step = 0; step <= pd; ++step) {
@@ -352,7 +364,8 @@ int enqueue_apply_f64(pl_lattice *h, double *output, const double *input, int re
         cur = 1 - cur;
     }
     h->mark(EV_BLUR);
-    PL_HIP(plk::slice_f64(pd, vd, h->map, h->replay, h->weights64, nullptr, values[cur], output,
+    PL_HIP(plk::slice_f64(pd, vd, h->map, h->replay, h->weights64,
+                          h->replay_holds_cells ? h->cell_vertex : nullptr, values[cur], output,
                           h->normalize ? 1 : 0, h->stream));
     h->mark(EV_SLICE);
     return PL_OK;
@@ -730,7 +743,7 @@ int filter_begin(pl_lattice *h, void *output, const void *input,
     }
     const uint32_t cells = initial_cells(h);
     // (only a lattice of floats splats in its build, and its input is then floats)
-    int rc = enqueue_build(h, features, positions64, cells, static_cast<const float *>(input));
+    int rc = enqueue_build(h, features, positions64, cells, input);
     if (rc != PL_OK) return rc;
     rc = enqueue_apply(h, output, input, reverse);
     if (rc != PL_OK) return rc;
@@ -753,7 +766,7 @@ int filter_end(pl_lattice *h) {
             return rc;
         }
         rc = enqueue_build(h, h->pending.features, h->pending.positions64, cells,
-                           static_cast<const float *>(h->pending.input));
+                           h->pending.input);
         if (rc == PL_OK) rc = enqueue_apply(h, h->pending.output, h->pending.input, h->pending.reverse);
         if (rc != PL_OK) {
             h->pending.active = false;

@@ -143,7 +143,8 @@ hipError_t build(int pd, const PointFeatures &features, const PointMap &map, con
 hipError_t build_f64(int pd, const Points64 &points, const PointMap &map, uint64_t *cell_keys,
                      uint32_t n_cells, Counters *counters, ReplayEntry *replay, int xcd_aware,
                      const CreatedLists &created_lists, const RegionSource &regions,
-                     bool merge_in_workgroup, hipStream_t s);
+                     bool merge_in_workgroup, int splat_vd, const double *input, int in_channels,
+                     double *cell_values, hipStream_t s);
 
 // Dense vertex numbers in the order of the build's workgroups (same map as the build):
 // cell_vertex[cell] := v, vertex_keys[v] := key, vertex_cell[v] := cell,

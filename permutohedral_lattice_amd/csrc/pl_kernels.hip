@@ -170,13 +170,15 @@ __global__ __launch_bounds__(kBlock) void k_build(PointFeatures features, PointM
                                                    ScaleFactor scale, uint64_t *cell_keys,
                                                    uint32_t mask, Counters *counters,
                                                    ReplayEntry *__restrict__ replay,
-                                                   int xcd_aware, const float *__restrict__ input,
-                                                   int in_channels, float *cell_values,
+                                                   int xcd_aware, const void *__restrict__ input_any,
+                                                   int in_channels, void *cell_values_any,
                                                    CreatedLists created_lists,
                                                    Points64 points64, RegionSource region_source) {
     constexpr bool kDouble = sizeof(T) == sizeof(double);
     static_assert(!kDouble || SPLAT_VD == 0, "the fused splat is for float values");
     constexpr int D1 = PD + 1;
+    const float *__restrict__ input = static_cast<const float *>(input_any);
+    float *cell_values = static_cast<float *>(cell_values_any);
     __shared__ int group_created, waves_done;
     if (threadIdx.x == 0) {
         group_created = 0;
@@ -358,23 +360,24 @@ __global__ __launch_bounds__(kBlock) void k_build_tile(PointFeatures features, P
                                                         ScaleFactor scale, uint64_t *cell_keys,
                                                         uint32_t mask, Counters *counters,
                                                         ReplayEntry *__restrict__ replay,
-                                                        int xcd_aware, const float *__restrict__ input,
-                                                        int in_channels, float *cell_values,
+                                                        int xcd_aware, const void *__restrict__ input_any,
+                                                        int in_channels, void *cell_values_any,
                                                         CreatedLists created_lists,
                                                         Points64 points64, RegionSource region_source) {
     constexpr bool kDouble = sizeof(T) == sizeof(double);
-    static_assert(!kDouble || SPLAT_VD == 0, "the fused splat is for float values");
     constexpr int D1 = PD + 1;
     constexpr int VD = SPLAT_VD ? SPLAT_VD : 2;
-    constexpr int P = VD == 2 ? 2 : 4;      // floats per LDS row of sums
+    constexpr int P = (VD == 2 && !kDouble) ? 2 : 4;      // values per LDS row of sums
+    const T *__restrict__ input = static_cast<const T *>(input_any);
+    T *cell_values = static_cast<T *>(cell_values_any);
     __shared__ uint64_t slot_key[kTileSlots];
     __shared__ int slot_cell[kTileSlots];
-    __shared__ float slot_sum[SPLAT_VD ? kTileSlots * P : 1];
+    __shared__ T slot_sum[SPLAT_VD ? kTileSlots * P : 1];
     __shared__ int group_created;
     const int tid = threadIdx.x;
     for (int i = tid; i < kTileSlots; i += kBlock) slot_key[i] = kEmptyCell;
     if (SPLAT_VD)
-        for (int i = tid; i < kTileSlots * P; i += kBlock) slot_sum[i] = 0.0f;
+        for (int i = tid; i < kTileSlots * P; i += kBlock) slot_sum[i] = (T)0;
     if (tid == 0) group_created = 0;
 
     const unsigned vblock = xcd_contiguous_block(blockIdx.x, gridDim.x, xcd_aware);
@@ -446,10 +449,10 @@ __global__ __launch_bounds__(kBlock) void k_build_tile(PointFeatures features, P
             if ((open >> r) & 1u) slot[r] = -1;
     }
 
-    float val[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    T val[4] = {(T)0, (T)0, (T)0, (T)0};
     if (SPLAT_VD) {
 #pragma unroll
-        for (int j = 0; j < SPLAT_VD; ++j) val[j] = 1.0f;  // homogeneous channel when vd-1 are given
+        for (int j = 0; j < SPLAT_VD; ++j) val[j] = (T)1;  // homogeneous channel when vd-1 are given
         if (valid) {
 #pragma unroll
             for (int j = 0; j < SPLAT_VD; ++j)
@@ -462,20 +465,32 @@ __global__ __launch_bounds__(kBlock) void k_build_tile(PointFeatures features, P
         const int own = slot[r];
         slot[r] = active ? __shfl(own, leader) : -1;
         if (SPLAT_VD) {
-            const float w = (float)s.weight[r];
-            const float term[4] = {w * val[0], w * val[1], w * val[2], w * val[3]};
-            const QuadTerms quad = quad_terms<VD>(term, lane);
+            const T w = s.weight[r];
+            const T term[4] = {w * val[0], w * val[1], w * val[2], w * val[3]};
             const uint64_t among = wave_ballot(active) & ~small[r];
             uint64_t remaining = among;
-            while (remaining) {
-                const int first = __builtin_ctzll(remaining);
-                const uint64_t group = lanes_equal(leader, first) & among;
-                remaining &= ~group;
-                const bool same = lane_in(group);
-                const int group_slot = lane_value(own, first);
-                const float sum = wave_sum_to_last_lanes<VD>(same, quad, lane);
-                if (group_slot >= 0 && lane >= 64 - P && channel_of_lane<VD>(lane) < VD)
-                    atomicAdd(&slot_sum[group_slot * P + channel_of_lane<VD>(lane)], sum);
+            if constexpr (kDouble) {
+                while (remaining) {
+                    const int first = __builtin_ctzll(remaining);
+                    const uint64_t group = lanes_equal(leader, first) & among;
+                    remaining &= ~group;
+                    const int group_slot = lane_value(own, first);
+                    const double sum = wave_sums_to_quads_f64(lane_in(group), term, lane);
+                    if (group_slot >= 0 && lane < 4 && channel_of_quad_lane(lane) < VD)
+                        atomicAdd(&slot_sum[group_slot * P + channel_of_quad_lane(lane)], sum);
+                }
+            } else {
+                const QuadTerms quad = quad_terms<VD>(term, lane);
+                while (remaining) {
+                    const int first = __builtin_ctzll(remaining);
+                    const uint64_t group = lanes_equal(leader, first) & among;
+                    remaining &= ~group;
+                    const bool same = lane_in(group);
+                    const int group_slot = lane_value(own, first);
+                    const float sum = wave_sum_to_last_lanes<VD>(same, quad, lane);
+                    if (group_slot >= 0 && lane >= 64 - P && channel_of_lane<VD>(lane) < VD)
+                        atomicAdd(&slot_sum[group_slot * P + channel_of_lane<VD>(lane)], sum);
+                }
             }
             if (lane_in(small[r]) && slot[r] >= 0) {
 #pragma unroll
@@ -656,6 +671,12 @@ __global__ __launch_bounds__(64) void k_number_vertices(CreatedLists lists, int 
                 float4 *from = reinterpret_cast<float4 *>(cell_values) + cell;
                 reinterpret_cast<float4 *>(values)[v] = *from;
                 *from = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            } else if (cell_values && vd == 8) {
+                float4 *from = reinterpret_cast<float4 *>(cell_values) + 2 * (size_t)cell;
+                float4 *to = reinterpret_cast<float4 *>(values) + 2 * (size_t)v;
+                to[0] = from[0];
+                to[1] = from[1];
+                from[0] = from[1] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
             } else if (cell_values && vd == 2) {
                 float2 *from = reinterpret_cast<float2 *>(cell_values) + cell;
                 reinterpret_cast<float2 *>(values)[v] = *from;
@@ -1387,8 +1408,8 @@ hipError_t build(int pd, const PointFeatures &features, const PointMap &map, con
     if (map.n_blocks == 0) return hipSuccess;
 #define PLK_BUILD_ARGS                                                                             \
     dim3(map.n_blocks), dim3(kBlock), 0, s, features, map, scale, cell_keys, n_cells - 1u,         \
-        counters, replay, xcd_aware, input, in_channels, cell_values, created_lists, Points64{},   \
-        regions
+        counters, replay, xcd_aware, (const void *)input, in_channels, (void *)cell_values,        \
+        created_lists, Points64{}, regions
 #define PLK_BUILD(SPLAT_VD)                                                                        \
     if (merge_in_workgroup)                                                                        \
         PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_build_tile<PD, SPLAT_VD>), PLK_BUILD_ARGS))      \
@@ -1409,16 +1430,28 @@ hipError_t build(int pd, const PointFeatures &features, const PointMap &map, con
 hipError_t build_f64(int pd, const Points64 &points, const PointMap &map, uint64_t *cell_keys,
                      uint32_t n_cells, Counters *counters, ReplayEntry *replay, int xcd_aware,
                      const CreatedLists &created_lists, const RegionSource &regions,
-                     bool merge_in_workgroup, hipStream_t s) {
+                     bool merge_in_workgroup, int splat_vd, const double *input, int in_channels,
+                     double *cell_values, hipStream_t s) {
     if (map.n_blocks == 0) return hipSuccess;
+    if (splat_vd && !merge_in_workgroup) return hipErrorInvalidValue;
 #define PLK_BUILD_ARGS                                                                             \
     dim3(map.n_blocks), dim3(kBlock), 0, s, PointFeatures{}, map, ScaleFactor{}, cell_keys,        \
-        n_cells - 1u, counters, replay, xcd_aware, (const float *)nullptr, 0, (float *)nullptr,    \
-        created_lists, points, regions
-    if (merge_in_workgroup)
-        PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_build_tile<PD, 0, double>), PLK_BUILD_ARGS))
-    else
+        n_cells - 1u, counters, replay, xcd_aware, (const void *)input, in_channels,               \
+        (void *)cell_values, created_lists, points, regions
+#define PLK_BUILD(SPLAT_VD)                                                                        \
+    PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_build_tile<PD, SPLAT_VD, double>), PLK_BUILD_ARGS))
+    if (merge_in_workgroup) {
+        switch (splat_vd) {
+            case 0: PLK_BUILD(0); break;
+            case 2: PLK_BUILD(2); break;
+            case 3: PLK_BUILD(3); break;
+            case 4: PLK_BUILD(4); break;
+            default: return hipErrorInvalidValue;
+        }
+    } else {
         PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_build<PD, 0, double>), PLK_BUILD_ARGS))
+    }
+#undef PLK_BUILD
 #undef PLK_BUILD_ARGS
     return hipGetLastError();
 }

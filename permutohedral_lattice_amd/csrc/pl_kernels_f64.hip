@@ -22,49 +22,6 @@ namespace {
 
 using namespace device;
 
-// The double of another lane (by DPP control; both words moved alike)
-template <int CTRL>
-__device__ __forceinline__ double from_lane_f64(double x) {
-    const int lo = __builtin_amdgcn_update_dpp(0, __double2loint(x), CTRL, 0xf, 0xf, false);
-    const int hi = __builtin_amdgcn_update_dpp(0, __double2hiint(x), CTRL, 0xf, 0xf, false);
-    return __hiloint2double(hi, lo);
-}
-// Sums over the wavefront of four terms per lane (zero where `member` is false), delivered to
-// every quad of lanes: lane q of a quad returns the sum of channel channel_of_quad_lane(q).  The
-// terms are reduce-scattered inside each quad (two exchanges, after which a lane holds one
-// channel), then summed across the quads of a row by rotations and across the rows with
-// v_permlane16_swap and v_permlane32_swap (given x twice, the first result holds the even rows /
-// lower half in both places and the second the odd rows / upper half: their sum is the pair's).
-__device__ __forceinline__ int channel_of_quad_lane(int lane) {
-    return ((lane & 1) << 1) | ((lane >> 1) & 1);
-}
-__device__ __forceinline__ double wave_sums_to_quads_f64(bool member, const double (&term)[4],
-                                                         int lane) {
-    const bool bit0 = lane & 1, bit1 = lane & 2;
-    const double keep_a = member ? (bit0 ? term[2] : term[0]) : 0.0;
-    const double keep_b = member ? (bit0 ? term[3] : term[1]) : 0.0;
-    const double send_a = member ? (bit0 ? term[0] : term[2]) : 0.0;
-    const double send_b = member ? (bit0 ? term[1] : term[3]) : 0.0;
-    const double ya = keep_a + from_lane_f64<0xB1>(send_a);   // quad_perm:[1,0,3,2]
-    const double yb = keep_b + from_lane_f64<0xB1>(send_b);
-    double x = (bit1 ? yb : ya) + from_lane_f64<0x4E>(bit1 ? ya : yb);   // quad_perm:[2,3,0,1]
-    x += from_lane_f64<0x124>(x);   // row_ror:4
-    x += from_lane_f64<0x128>(x);   // row_ror:8
-    {
-        const unsigned lo = (unsigned)__double2loint(x), hi = (unsigned)__double2hiint(x);
-        const auto l = __builtin_amdgcn_permlane16_swap(lo, lo, false, false);
-        const auto h = __builtin_amdgcn_permlane16_swap(hi, hi, false, false);
-        x = __hiloint2double((int)h[0], (int)l[0]) + __hiloint2double((int)h[1], (int)l[1]);
-    }
-    {
-        const unsigned lo = (unsigned)__double2loint(x), hi = (unsigned)__double2hiint(x);
-        const auto l = __builtin_amdgcn_permlane32_swap(lo, lo, false, false);
-        const auto h = __builtin_amdgcn_permlane32_swap(hi, hi, false, false);
-        x = __hiloint2double((int)h[0], (int)l[0]) + __hiloint2double((int)h[1], (int)l[1]);
-    }
-    return x;
-}
-
 // Splat.  As in the float path the contributions of a wavefront to one vertex are summed before
 // they leave it (points that are neighbours in the image share vertices, and what bounds a splat
 // is the number of atomic requests): for each distinct vertex of the wavefront and each channel
