@@ -354,12 +354,22 @@ int enqueue_apply_f64(pl_lattice *h, double *output, const double *input, int re
     h->values_splatted = false;
     h->mark(EV_SPLAT);
     int cur = 0;
-    for (int step = 0; step <= pd; ++step) {
+    for (int step = 0; step <= pd;) {
         const int axis = reverse ? pd - step : step;
         uint64_t *reset = (!h->table_clean && step == 0) ? h->cell_keys : nullptr;
-        PL_HIP(plk::blur_axis_f64(vd, h->counters(), mv, values[cur], values[1 - cur],
-                                  h->neighbours + (size_t)axis * mv, reset, h->vertex_cell,
-                                  h->launch_vertices(), h->stream));
+        if (h->pair_blur && step + 1 <= pd) {
+            const int next_axis = reverse ? axis - 1 : axis + 1;
+            PL_HIP(plk::blur_two_axes_f64(vd, h->counters(), mv, values[cur], values[1 - cur],
+                                          h->neighbours + (size_t)axis * mv,
+                                          h->neighbours + (size_t)next_axis * mv, reset,
+                                          h->vertex_cell, h->launch_vertices(), h->stream));
+            step += 2;
+        } else {
+            PL_HIP(plk::blur_axis_f64(vd, h->counters(), mv, values[cur], values[1 - cur],
+                                      h->neighbours + (size_t)axis * mv, reset, h->vertex_cell,
+                                      h->launch_vertices(), h->stream));
+            step += 1;
+        }
         if (reset) h->table_clean = true;
         cur = 1 - cur;
     }

@@ -1078,41 +1078,45 @@ __global__ __launch_bounds__(kBlock) void k_blur2_element(const Counters *counte
 // vertex numbers that follow the image the rows a thread gathers are near each other, and a
 // quarter of the memory instructions moves the same bytes (34 -> 25 us for the three launches
 // of pd = 5, vd = 4).  Same arithmetic per channel, same results.
-template <int VD>
-struct alignas(VD == 3 ? 4 : 4 * VD) ValueRow {
-    float c[VD];
+// (S = double: the rows of a lattice of doubles)
+__device__ __forceinline__ double blur_tap(double a, double self, double b) {
+    return 0.25 * a + 0.5 * self + 0.25 * b;
+}
+template <int VD, typename S = float>
+struct alignas(VD == 3 ? sizeof(S) : sizeof(S) * VD) ValueRow {
+    S c[VD];
 };
 
-template <int VD>
-__device__ __forceinline__ ValueRow<VD> blur_rows(const ValueRow<VD> &a, const ValueRow<VD> &self,
-                                                  const ValueRow<VD> &b) {
-    ValueRow<VD> out;
+template <int VD, typename S = float>
+__device__ __forceinline__ ValueRow<VD, S> blur_rows(const ValueRow<VD, S> &a, const ValueRow<VD, S> &self,
+                                                  const ValueRow<VD, S> &b) {
+    ValueRow<VD, S> out;
 #pragma unroll
     for (int j = 0; j < VD; ++j) out.c[j] = blur_tap(a.c[j], self.c[j], b.c[j]);
     return out;
 }
 
-template <int VD>
-__device__ __forceinline__ ValueRow<VD> row_or_zero(const ValueRow<VD> *__restrict__ src, int u) {
+template <int VD, typename S = float>
+__device__ __forceinline__ ValueRow<VD, S> row_or_zero(const ValueRow<VD, S> *__restrict__ src, int u) {
     if (u >= 0) return src[u];
-    ValueRow<VD> zero;
+    ValueRow<VD, S> zero;
 #pragma unroll
-    for (int j = 0; j < VD; ++j) zero.c[j] = 0.0f;
+    for (int j = 0; j < VD; ++j) zero.c[j] = (S)0;
     return zero;
 }
 
-template <int VD>
-__device__ __forceinline__ ValueRow<VD> blur_row_of(const ValueRow<VD> *__restrict__ src,
+template <int VD, typename S = float>
+__device__ __forceinline__ ValueRow<VD, S> blur_row_of(const ValueRow<VD, S> *__restrict__ src,
                                                     const int2 *__restrict__ nbr_a, int u) {
-    if (u < 0) return row_or_zero<VD>(src, -1);
+    if (u < 0) return row_or_zero<VD, S>(src, -1);
     const int2 nb = nbr_a[u];
-    return blur_rows<VD>(row_or_zero<VD>(src, nb.x), src[u], row_or_zero<VD>(src, nb.y));
+    return blur_rows<VD, S>(row_or_zero<VD, S>(src, nb.x), src[u], row_or_zero<VD, S>(src, nb.y));
 }
 
-template <int VD>
+template <int VD, typename S = float>
 __global__ __launch_bounds__(kBlock) void k_blur_row(const Counters *counters, int max_vertices,
-                                                      const ValueRow<VD> *__restrict__ src,
-                                                      ValueRow<VD> *__restrict__ dst,
+                                                      const ValueRow<VD, S> *__restrict__ src,
+                                                      ValueRow<VD, S> *__restrict__ dst,
                                                       const int2 *__restrict__ nbr,
                                                       uint64_t *reset_cell_keys,
                                                       const int *__restrict__ vertex_cell) {
@@ -1122,15 +1126,15 @@ __global__ __launch_bounds__(kBlock) void k_blur_row(const Counters *counters, i
     while (blocks.next(vb)) {
         const int v = (int)(vb * kBlock + threadIdx.x);
         if (v >= M) continue;
-        dst[v] = blur_row_of<VD>(src, nbr, v);
+        dst[v] = blur_row_of<VD, S>(src, nbr, v);
         if (reset_cell_keys) reset_cell_keys[vertex_cell[v]] = kEmptyCell;
     }
 }
 
-template <int VD>
+template <int VD, typename S = float>
 __global__ __launch_bounds__(kBlock) void k_blur2_row(const Counters *counters, int max_vertices,
-                                                       const ValueRow<VD> *__restrict__ src,
-                                                       ValueRow<VD> *__restrict__ dst,
+                                                       const ValueRow<VD, S> *__restrict__ src,
+                                                       ValueRow<VD, S> *__restrict__ dst,
                                                        const int2 *__restrict__ nbr_a,
                                                        const int2 *__restrict__ nbr_b,
                                                        uint64_t *reset_cell_keys,
@@ -1142,8 +1146,8 @@ __global__ __launch_bounds__(kBlock) void k_blur2_row(const Counters *counters, 
         const int v = (int)(vb * kBlock + threadIdx.x);
         if (v >= M) continue;
         const int2 nb = nbr_b[v];
-        dst[v] = blur_rows<VD>(blur_row_of<VD>(src, nbr_a, nb.x), blur_row_of<VD>(src, nbr_a, v),
-                               blur_row_of<VD>(src, nbr_a, nb.y));
+        dst[v] = blur_rows<VD, S>(blur_row_of<VD, S>(src, nbr_a, nb.x), blur_row_of<VD, S>(src, nbr_a, v),
+                               blur_row_of<VD, S>(src, nbr_a, nb.y));
         if (reset_cell_keys) reset_cell_keys[vertex_cell[v]] = kEmptyCell;
     }
 }
@@ -1566,6 +1570,46 @@ hipError_t blur_two_axes(int vd, const Counters *counters, int max_vertices, con
                        counters, max_vertices, vd, src, dst, nbr_first, nbr_second, reset_cell_keys,
                        vertex_cell);
     return hipGetLastError();
+}
+
+// Rows of two to four doubles, one thread per vertex row as for floats.
+hipError_t blur_axis_rows_f64(int vd, const Counters *counters, int max_vertices, const double *src,
+                              double *dst, const int2 *nbr, uint64_t *reset_cell_keys,
+                              const int *vertex_cell, int launch_vertices, hipStream_t s) {
+    if (max_vertices <= 0) return hipSuccess;
+#define PLK_BLUR_ROW(VD)                                                                          \
+    case VD:                                                                                      \
+        hipLaunchKernelGGL((k_blur_row<VD, double>), dim3(vertex_blocks((size_t)launch_vertices)), \
+                           dim3(kBlock), 0, s, counters, max_vertices,                            \
+                           reinterpret_cast<const ValueRow<VD, double> *>(src),                   \
+                           reinterpret_cast<ValueRow<VD, double> *>(dst), nbr, reset_cell_keys,   \
+                           vertex_cell);                                                          \
+        return hipGetLastError();
+    switch (vd) {
+        PLK_BLUR_ROW(2) PLK_BLUR_ROW(3) PLK_BLUR_ROW(4)
+        default: return hipErrorInvalidValue;
+    }
+#undef PLK_BLUR_ROW
+}
+
+hipError_t blur_two_axes_rows_f64(int vd, const Counters *counters, int max_vertices,
+                                  const double *src, double *dst, const int2 *nbr_first,
+                                  const int2 *nbr_second, uint64_t *reset_cell_keys,
+                                  const int *vertex_cell, int launch_vertices, hipStream_t s) {
+    if (max_vertices <= 0) return hipSuccess;
+#define PLK_BLUR2_ROW(VD)                                                                         \
+    case VD:                                                                                      \
+        hipLaunchKernelGGL((k_blur2_row<VD, double>), dim3(vertex_blocks((size_t)launch_vertices)), \
+                           dim3(kBlock), 0, s, counters, max_vertices,                            \
+                           reinterpret_cast<const ValueRow<VD, double> *>(src),                   \
+                           reinterpret_cast<ValueRow<VD, double> *>(dst), nbr_first, nbr_second,  \
+                           reset_cell_keys, vertex_cell);                                         \
+        return hipGetLastError();
+    switch (vd) {
+        PLK_BLUR2_ROW(2) PLK_BLUR2_ROW(3) PLK_BLUR2_ROW(4)
+        default: return hipErrorInvalidValue;
+    }
+#undef PLK_BLUR2_ROW
 }
 
 hipError_t slice(int pd, int vd, const PointMap &map, const ReplayEntry *replay,
