@@ -131,6 +131,32 @@ __device__ __forceinline__ uint32_t next_pair(uint32_t cell, uint32_t index, uin
 
 // ------------------------------------------------------------------------------------------------
 // Per-point arithmetic: same operations, in the same precision and order, as
+// x[0] >= x[1] >= ... in place.  Six values take the 12-comparator network; other counts an
+// odd-even transposition sort.
+template <typename S>
+__device__ __forceinline__ void order_pair(S &hi, S &lo) {
+    const bool swap = hi < lo;
+    const S a = swap ? lo : hi, b = swap ? hi : lo;
+    hi = a;
+    lo = b;
+}
+template <int N, typename S>
+__device__ __forceinline__ void sort_descending(S (&x)[N]) {
+    if constexpr (N == 6) {
+        order_pair(x[0], x[5]); order_pair(x[1], x[3]); order_pair(x[2], x[4]);
+        order_pair(x[1], x[2]); order_pair(x[3], x[4]);
+        order_pair(x[0], x[3]); order_pair(x[2], x[5]);
+        order_pair(x[0], x[1]); order_pair(x[2], x[3]); order_pair(x[4], x[5]);
+        order_pair(x[1], x[2]); order_pair(x[3], x[4]);
+    } else {
+#pragma unroll
+        for (int round = 0; round < N; ++round) {
+#pragma unroll
+            for (int i = round & 1; i + 1 < N; i += 2) order_pair(x[i], x[i + 1]);
+        }
+    }
+}
+
 // embed_position_vector / find_enclosing_simplex / compute_barycentric_coordinates of the
 // reference CPU path.  q[i] is rem0[i] / (pd+1).
 // ------------------------------------------------------------------------------------------------
@@ -206,15 +232,13 @@ __device__ __forceinline__ void enclosing_simplex(const float (&pos)[PD], const 
     // barycentric weights.  by_rank[k] is the scaled residual of the coordinate of rank k; the
     // reference's scatter b[pd-rank] += delta, b[pd-rank+1] -= delta gives
     // b[k] = by_rank[pd-k] - by_rank[pd-k+1] with one rounding, in either order of the two updates.
+    // The ranks order the coordinates by falling residual (a coordinate that wrapped moved a whole
+    // step, past all that did not), so by_rank is the residuals sorted, largest first; equal
+    // residuals are equal in either place.  Sorted by a network of compare-and-swaps.
     float by_rank[D1];
 #pragma unroll
-    for (int k = 0; k < D1; ++k) by_rank[k] = 0.0f;
-#pragma unroll
-    for (int i = 0; i < D1; ++i) {
-        const float delta = (float)((double)(el[i] - rem[i]) * inv_d1);
-#pragma unroll
-        for (int k = 0; k < D1; ++k) by_rank[k] = (s.rank[i] == k) ? delta : by_rank[k];
-    }
+    for (int i = 0; i < D1; ++i) by_rank[i] = (float)((double)(el[i] - rem[i]) * inv_d1);
+    sort_descending<D1>(by_rank);
 #pragma unroll
     for (int k = 1; k < D1; ++k) s.weight[k] = by_rank[PD - k] - by_rank[PD - k + 1];
     s.weight[0] = (float)((double)by_rank[PD] + (1.0 + (double)(-by_rank[0])));
@@ -277,15 +301,11 @@ __device__ __forceinline__ void enclosing_simplex(const double (&pos)[PD], const
         rem[i] += (double)(step * D1);
     }
 
+    // (the residuals sorted, largest first, as in the float version)
     double by_rank[D1];
 #pragma unroll
-    for (int k = 0; k < D1; ++k) by_rank[k] = 0.0;
-#pragma unroll
-    for (int i = 0; i < D1; ++i) {
-        const double delta = (el[i] - rem[i]) * inv_d1;
-#pragma unroll
-        for (int k = 0; k < D1; ++k) by_rank[k] = (s.rank[i] == k) ? delta : by_rank[k];
-    }
+    for (int i = 0; i < D1; ++i) by_rank[i] = (el[i] - rem[i]) * inv_d1;
+    sort_descending<D1>(by_rank);
 #pragma unroll
     for (int k = 1; k < D1; ++k) s.weight[k] = by_rank[PD - k] - by_rank[PD - k + 1];
     s.weight[0] = by_rank[PD] + (1.0 + (-by_rank[0]));
