@@ -5,9 +5,9 @@
 // builds: the build kernel is instantiated for double positions in pl_kernels.hip, and the
 // numbering and neighbour passes do not look at values.  What is here are the passes that touch
 // values: splat, blur and slice on rows of doubles, the feature builder and the per-point dump.
-// They are simple forms (the splat sums per wavefront and vertex before it adds, channel by
-// channel; one thread per (vertex, channel) in the blur, per (point, channel) in the slice): the
-// float path is the one tuned for speed.
+// The splat here serves pl_apply_f64 and more than four channels (with up to four, pl_filter_f64
+// splats in the merging build kernel, as the float path does); the blur kernels here serve more
+// than four channels (up to four use the float path's row kernels over the value type).
 //
 // Arithmetic follows the reference CPU path with T = double: the three-tap blur and the reciprocal
 // of the slice are double expressions there for every T.  The splat adds in a different order
