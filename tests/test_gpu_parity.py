@@ -254,6 +254,43 @@ def test_points_crowded_into_one_band_of_the_first_feature(dtype):
     assert (sorted_keys(host(lat.debug_keys()))[0] == sorted_keys(cpu.keys())[0]).all()
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_merging_build_equals_the_plain_build(dtype):
+    """With a grid hint the build merges each tile's keys and sums in LDS before they go to the
+    hash table (PL_OPT_MERGE_TILES); without the option every wavefront goes to the table itself.
+    Same vertices, same replay rows, same outputs to rounding, for a smooth image (tiles share
+    most vertices) and for one with noise in every feature (a tile then has more distinct keys
+    than its LDS table holds, and the lattice must fall back by itself, for this and later calls)."""
+    h, w, pd, vd = 96, 112, 5, 4
+    n = h * w
+    torch_dtype = torch.float32 if dtype == np.float32 else torch.float64
+    img = synth.blob_image(h, w, seed=91)
+    smooth = synth.bilateral_positions(img, 8.0, 0.125)
+    rng = np.random.default_rng(92)
+    noisy = np.concatenate([smooth[:, :2], rng.uniform(0, 40, (n, 3)).astype(np.float32)], axis=1)
+    val = img.reshape(-1, 3).astype(dtype)
+    for pos in (smooth.astype(dtype), noisy.astype(dtype)):
+        cpu = oracle.Lattice(pd, vd, n, dtype=dtype)
+        want = cpu.filter(val, pos)
+        outs = {}
+        for merge in (1, 0):
+            lat = pla.PermutohedralLattice(pd, vd, n, dtype=torch_dtype)
+            lat.set_point_grid((h, w))
+            lat.set_option(pla.PL_OPT_MERGE_TILES, merge)
+            out = torch.empty((n, vd - 1), dtype=torch_dtype, device="cuda")
+            for _ in range(2):      # the second call runs on what the first one learnt
+                lat.filter(out, dev(val), dev(pos), False)
+                torch.cuda.synchronize()
+                assert lat.num_vertices == cpu.num_vertices
+            assert (sorted_keys(host(lat.debug_keys()))[0] == sorted_keys(cpu.keys())[0]).all()
+            outs[merge] = host(out).copy()
+            if dtype == np.float32:
+                assert_float_parity(outs[merge], want)
+            else:
+                assert np.abs(outs[merge] - want).max() <= 1e-12
+        assert np.abs(outs[1] - outs[0]).max() <= (2e-6 if dtype == np.float32 else 1e-13)
+
+
 def test_point_grid_must_match_the_number_of_points():
     lat = pla.PermutohedralLattice(2, 2, 100)
     with pytest.raises(pla.PermutohedralError) as e:
