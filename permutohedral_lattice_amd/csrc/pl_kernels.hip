@@ -1156,7 +1156,7 @@ __global__ __launch_bounds__(kBlock) void k_blur2_row(const Counters *counters, 
 // Stage 5: slice (reference: src/PermutohedralLatticeCPU.h:333-352)
 // ------------------------------------------------------------------------------------------------
 // cell_vertex != nullptr: the replay rows still hold hash cells (nothing has translated them yet)
-template <int VD>
+template <int VD, int D1 = 0>
 __global__ __launch_bounds__(kBlock) void k_slice_point(int d1, PointMap map,
                                                          const ReplayEntry *__restrict__ replay,
                                                          const int *__restrict__ cell_vertex,
@@ -1172,15 +1172,40 @@ __global__ __launch_bounds__(kBlock) void k_slice_point(int d1, PointMap map,
     float acc[VD];
 #pragma unroll
     for (int j = 0; j < VD; ++j) acc[j] = 0.0f;
-    for (int r = 0; r < d1; ++r) {
-        const ReplayEntry e = replay[(size_t)r * T + t];
-        int v = e.index;
-        if (v < 0) continue;
-        if (cell_vertex) v = cell_vertex[v];
-        const float w = e.weight;
-        const float *src = values + (size_t)v * VD;
+    if constexpr (D1 > 0) {
+        // all replay rows, then all translations, then all value rows: three round trips to
+        // memory instead of three per corner (what a point waits for when many workgroups queue
+        // behind each other, as for a volume of millions of voxels)
+        ReplayEntry e[D1];
+        int v[D1];
 #pragma unroll
-        for (int j = 0; j < VD; ++j) acc[j] += w * src[j];
+        for (int r = 0; r < D1; ++r) e[r] = replay[(size_t)r * T + t];
+#pragma unroll
+        for (int r = 0; r < D1; ++r) {
+            v[r] = e[r].index;
+            if (cell_vertex && v[r] >= 0) v[r] = cell_vertex[v[r]];
+        }
+        ValueRow<VD> row[D1];
+#pragma unroll
+        for (int r = 0; r < D1; ++r)
+            row[r] = reinterpret_cast<const ValueRow<VD> *>(values)[v[r] >= 0 ? v[r] : 0];
+#pragma unroll
+        for (int r = 0; r < D1; ++r) {
+            if (v[r] < 0) continue;
+#pragma unroll
+            for (int j = 0; j < VD; ++j) acc[j] += e[r].weight * row[r].c[j];
+        }
+    } else {
+        for (int r = 0; r < d1; ++r) {
+            const ReplayEntry e = replay[(size_t)r * T + t];
+            int v = e.index;
+            if (v < 0) continue;
+            if (cell_vertex) v = cell_vertex[v];
+            const float w = e.weight;
+            const float *src = values + (size_t)v * VD;
+#pragma unroll
+            for (int j = 0; j < VD; ++j) acc[j] += w * src[j];
+        }
     }
     if (normalize) {
         const float scale = (float)(1.0 / (double)acc[VD - 1]);
@@ -1624,8 +1649,15 @@ hipError_t slice(int pd, int vd, const PointMap &map, const ReplayEntry *replay,
         hipLaunchKernelGGL(k_slice_point<VD>, grid, block, 0, s, d1, map, replay,              \
                            cell_vertex, values, output, normalize);                            \
         break;
+#define PLK_SLICE_ROWS(VD)                                                                     \
+    case VD:                                                                                   \
+        PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_slice_point<VD, PD + 1>), grid, block, 0, s, \
+                                               d1, map, replay, cell_vertex, values, output,   \
+                                               normalize));                                    \
+        break;
     switch (vd) {
-        PLK_SLICE(2) PLK_SLICE(3) PLK_SLICE(4) PLK_SLICE(5) PLK_SLICE(6) PLK_SLICE(7) PLK_SLICE(8)
+        PLK_SLICE_ROWS(2) PLK_SLICE_ROWS(3) PLK_SLICE_ROWS(4)
+        PLK_SLICE(5) PLK_SLICE(6) PLK_SLICE(7) PLK_SLICE(8)
         default: {
             const int out_ch = normalize ? vd - 1 : vd;
             PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_slice_channels<PD + 1>),
@@ -1634,6 +1666,7 @@ hipError_t slice(int pd, int vd, const PointMap &map, const ReplayEntry *replay,
         } break;
     }
 #undef PLK_SLICE
+#undef PLK_SLICE_ROWS
     return hipGetLastError();
 }
 
