@@ -226,6 +226,10 @@ hipError_t blur_two_axes_f64(int vd, const Counters *counters, int max_vertices,
                              double *dst, const int2 *nbr_first, const int2 *nbr_second,
                              uint64_t *reset_cell_keys, const int *vertex_cell,
                              int launch_vertices, hipStream_t s);
+// (vd 2..4: in pl_kernels.hip, rows of doubles gathered whole)
+hipError_t slice_rows_f64(int pd, int vd, const PointMap &map, const ReplayEntry *replay,
+                          const double *weights, const int *cell_vertex, const double *values,
+                          double *output, int normalize, hipStream_t s);
 hipError_t slice_f64(int pd, int vd, const PointMap &map, const ReplayEntry *replay,
                      const double *weights, const int *cell_vertex, const double *values,
                      double *output, int normalize, hipStream_t s);

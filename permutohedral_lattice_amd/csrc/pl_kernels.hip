@@ -1217,6 +1217,56 @@ __global__ __launch_bounds__(kBlock) void k_slice_point(int d1, PointMap map,
     }
 }
 
+// The same for rows of doubles (weights64[r*T+t]: the barycentric weights as doubles; the replay
+// rows give the vertices).  Arithmetic as in k_slice_point_f64.
+template <int VD, int D1>
+__global__ __launch_bounds__(kBlock) void k_slice_rows_f64(PointMap map,
+                                                            const ReplayEntry *__restrict__ replay,
+                                                            const double *__restrict__ weights64,
+                                                            const int *__restrict__ cell_vertex,
+                                                            const double *__restrict__ values,
+                                                            double *__restrict__ output,
+                                                            int normalize) {
+    const unsigned vblock = xcd_contiguous_block(blockIdx.x, gridDim.x, 1);
+    const size_t t = (size_t)vblock * kBlock + threadIdx.x;
+    const size_t T = (size_t)gridDim.x * kBlock;
+    const int n = point_of_thread(map, vblock, threadIdx.x);
+    if (n < 0) return;
+    int v[D1];
+    double w[D1];
+#pragma unroll
+    for (int r = 0; r < D1; ++r) {
+        v[r] = replay[(size_t)r * T + t].index;
+        w[r] = weights64[(size_t)r * T + t];
+    }
+    if (cell_vertex) {
+#pragma unroll
+        for (int r = 0; r < D1; ++r)
+            if (v[r] >= 0) v[r] = cell_vertex[v[r]];
+    }
+    ValueRow<VD, double> row[D1];
+#pragma unroll
+    for (int r = 0; r < D1; ++r)
+        row[r] = reinterpret_cast<const ValueRow<VD, double> *>(values)[v[r] >= 0 ? v[r] : 0];
+    double sum[VD];
+#pragma unroll
+    for (int j = 0; j < VD; ++j) sum[j] = 0.0;
+#pragma unroll
+    for (int r = 0; r < D1; ++r) {
+        if (v[r] < 0) continue;
+#pragma unroll
+        for (int j = 0; j < VD; ++j) sum[j] += w[r] * row[r].c[j];
+    }
+    if (normalize) {
+        const double scale = 1.0 / sum[VD - 1];
+#pragma unroll
+        for (int j = 0; j < VD - 1; ++j) output[(size_t)n * (VD - 1) + j] = sum[j] * scale;
+    } else {
+#pragma unroll
+        for (int j = 0; j < VD; ++j) output[(size_t)n * VD + j] = sum[j];
+    }
+}
+
 // Any vd: one thread per point and run of four channels.  The pd+1 replay rows, then the value
 // rows, are all requested before the first is used (with a run-time loop the passes waited for
 // two memory round trips per vertex, one after the other); the channels of a run share the index
@@ -1666,6 +1716,25 @@ hipError_t slice(int pd, int vd, const PointMap &map, const ReplayEntry *replay,
         } break;
     }
 #undef PLK_SLICE
+#undef PLK_SLICE_ROWS
+    return hipGetLastError();
+}
+
+hipError_t slice_rows_f64(int pd, int vd, const PointMap &map, const ReplayEntry *replay,
+                          const double *weights, const int *cell_vertex, const double *values,
+                          double *output, int normalize, hipStream_t s) {
+    if (map.n_blocks == 0) return hipSuccess;
+    const dim3 grid(map.n_blocks), block(kBlock);
+#define PLK_SLICE_ROWS(VD)                                                                     \
+    case VD:                                                                                   \
+        PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_slice_rows_f64<VD, PD + 1>), grid, block, 0, \
+                                               s, map, replay, weights, cell_vertex, values,   \
+                                               output, normalize));                            \
+        break;
+    switch (vd) {
+        PLK_SLICE_ROWS(2) PLK_SLICE_ROWS(3) PLK_SLICE_ROWS(4)
+        default: return hipErrorInvalidValue;
+    }
 #undef PLK_SLICE_ROWS
     return hipGetLastError();
 }

@@ -326,6 +326,8 @@ hipError_t slice_f64(int pd, int vd, const PointMap &map, const ReplayEntry *rep
                      const double *weights, const int *cell_vertex, const double *values,
                      double *output, int normalize, hipStream_t s) {
     if (map.n_blocks == 0) return hipSuccess;
+    if (vd >= 2 && vd <= 4)
+        return slice_rows_f64(pd, vd, map, replay, weights, cell_vertex, values, output, normalize, s);
     if (vd <= 8) {
         PLK_DISPATCH_PD(pd, hipLaunchKernelGGL(k_slice_point_f64<PD + 1>, dim3(map.n_blocks),
                                                dim3(kBlock), 0, s, vd, map, replay, weights,
