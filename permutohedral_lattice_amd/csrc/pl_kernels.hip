@@ -1096,21 +1096,26 @@ __device__ __forceinline__ ValueRow<VD, S> blur_rows(const ValueRow<VD, S> &a, c
     return out;
 }
 
-template <int VD, typename S = float>
-__device__ __forceinline__ ValueRow<VD, S> row_or_zero(const ValueRow<VD, S> *__restrict__ src, int u) {
-    if (u >= 0) return src[u];
-    ValueRow<VD, S> zero;
+// Loads never depend on a branch: an absent neighbour (-1) reads row 0 and its values are then
+// replaced by zeros, so that all the loads of one level of the gather are in flight together
+// (with a branch per neighbour each load is waited for before the next is asked for: thirteen
+// round trips in a row for two axes instead of three).  The empty asm statements keep the
+// compiler from moving the loads back under the conditions.
+template <int VD, typename S, int N>
+__device__ __forceinline__ void gather_rows(const ValueRow<VD, S> *__restrict__ src,
+                                            const int (&u)[N], ValueRow<VD, S> (&row)[N]) {
 #pragma unroll
-    for (int j = 0; j < VD; ++j) zero.c[j] = (S)0;
-    return zero;
-}
-
-template <int VD, typename S = float>
-__device__ __forceinline__ ValueRow<VD, S> blur_row_of(const ValueRow<VD, S> *__restrict__ src,
-                                                    const int2 *__restrict__ nbr_a, int u) {
-    if (u < 0) return row_or_zero<VD, S>(src, -1);
-    const int2 nb = nbr_a[u];
-    return blur_rows<VD, S>(row_or_zero<VD, S>(src, nb.x), src[u], row_or_zero<VD, S>(src, nb.y));
+    for (int k = 0; k < N; ++k) row[k] = src[u[k] >= 0 ? u[k] : 0];
+#pragma unroll
+    for (int k = 0; k < N; ++k) {
+#pragma unroll
+        for (int j = 0; j < VD; ++j) asm volatile("" : "+v"(row[k].c[j]));
+    }
+#pragma unroll
+    for (int k = 0; k < N; ++k) {
+#pragma unroll
+        for (int j = 0; j < VD; ++j) row[k].c[j] = u[k] >= 0 ? row[k].c[j] : (S)0;
+    }
 }
 
 template <int VD, typename S = float>
@@ -1126,7 +1131,11 @@ __global__ __launch_bounds__(kBlock) void k_blur_row(const Counters *counters, i
     while (blocks.next(vb)) {
         const int v = (int)(vb * kBlock + threadIdx.x);
         if (v >= M) continue;
-        dst[v] = blur_row_of<VD, S>(src, nbr, v);
+        const int2 nb = nbr[v];
+        const int u[3] = {nb.x, v, nb.y};
+        ValueRow<VD, S> row[3];
+        gather_rows<VD, S, 3>(src, u, row);
+        dst[v] = blur_rows<VD, S>(row[0], row[1], row[2]);
         if (reset_cell_keys) reset_cell_keys[vertex_cell[v]] = kEmptyCell;
     }
 }
@@ -1145,9 +1154,22 @@ __global__ __launch_bounds__(kBlock) void k_blur2_row(const Counters *counters, 
     while (blocks.next(vb)) {
         const int v = (int)(vb * kBlock + threadIdx.x);
         if (v >= M) continue;
+        // level 1: the vertex's neighbours along both axes; level 2: the a-neighbours of its
+        // b-neighbours; level 3: nine rows
         const int2 nb = nbr_b[v];
-        dst[v] = blur_rows<VD, S>(blur_row_of<VD, S>(src, nbr_a, nb.x), blur_row_of<VD, S>(src, nbr_a, v),
-                               blur_row_of<VD, S>(src, nbr_a, nb.y));
+        const int2 na_self = nbr_a[v];
+        int2 na_x = nbr_a[nb.x >= 0 ? nb.x : 0];
+        int2 na_y = nbr_a[nb.y >= 0 ? nb.y : 0];
+        asm volatile("" : "+v"(na_x.x), "+v"(na_x.y), "+v"(na_y.x), "+v"(na_y.y));
+        // (an absent b-neighbour stands for three zero rows, whose tap is zero)
+        const int u[9] = {nb.x >= 0 ? na_x.x : -1, nb.x, nb.x >= 0 ? na_x.y : -1,
+                          na_self.x,               v,    na_self.y,
+                          nb.y >= 0 ? na_y.x : -1, nb.y, nb.y >= 0 ? na_y.y : -1};
+        ValueRow<VD, S> row[9];
+        gather_rows<VD, S, 9>(src, u, row);
+        dst[v] = blur_rows<VD, S>(blur_rows<VD, S>(row[0], row[1], row[2]),
+                                  blur_rows<VD, S>(row[3], row[4], row[5]),
+                                  blur_rows<VD, S>(row[6], row[7], row[8]));
         if (reset_cell_keys) reset_cell_keys[vertex_cell[v]] = kEmptyCell;
     }
 }
