@@ -214,14 +214,7 @@ hipError_t splat_f64(int pd, int vd, const PointMap &map, const double *input, i
 hipError_t blur_axis_f64(int vd, const Counters *counters, int max_vertices, const double *src,
                          double *dst, const int2 *neighbours_of_axis, uint64_t *reset_cell_keys,
                          const int *vertex_cell, int launch_vertices, hipStream_t s);
-// (vd 2..4: one thread per vertex row, in pl_kernels.hip beside the float kernels they share)
-hipError_t blur_axis_rows_f64(int vd, const Counters *counters, int max_vertices, const double *src,
-                              double *dst, const int2 *nbr, uint64_t *reset_cell_keys,
-                              const int *vertex_cell, int launch_vertices, hipStream_t s);
-hipError_t blur_two_axes_rows_f64(int vd, const Counters *counters, int max_vertices,
-                                  const double *src, double *dst, const int2 *nbr_first,
-                                  const int2 *nbr_second, uint64_t *reset_cell_keys,
-                                  const int *vertex_cell, int launch_vertices, hipStream_t s);
+// (in pl_kernels.hip: the float kernels over the value type)
 hipError_t blur_two_axes_f64(int vd, const Counters *counters, int max_vertices, const double *src,
                              double *dst, const int2 *nbr_first, const int2 *nbr_second,
                              uint64_t *reset_cell_keys, const int *vertex_cell,

@@ -1012,10 +1012,53 @@ __device__ __forceinline__ float blur_tap(float a, float self, float b) {
     return (float)(0.25 * (double)a + 0.5 * (double)self + 0.25 * (double)b);
 }
 
+// (S = double: the values of a lattice of doubles)
+__device__ __forceinline__ double blur_tap(double a, double self, double b) {
+    return 0.25 * a + 0.5 * self + 0.25 * b;
+}
+
+// Loads never depend on a branch: an absent neighbour (-1) reads vertex 0 and the value is then
+// replaced by zero, so that all the loads of one level of the gather are in flight together
+// (with a branch per neighbour each load is waited for before the next is asked for: thirteen
+// round trips in a row for two axes instead of three).  The empty asm statements keep the
+// compiler from moving the loads back under the conditions.
+template <typename S, int N>
+__device__ __forceinline__ void gather_elements(const S *__restrict__ src, int vd, int j,
+                                                const int (&u)[N], S (&x)[N]) {
+#pragma unroll
+    for (int k = 0; k < N; ++k) x[k] = src[(size_t)(u[k] >= 0 ? u[k] : 0) * vd + j];
+#pragma unroll
+    for (int k = 0; k < N; ++k) asm volatile("" : "+v"(x[k]));
+#pragma unroll
+    for (int k = 0; k < N; ++k) x[k] = u[k] >= 0 ? x[k] : (S)0;
+}
+
+// The vertices whose values the taps along axis a, then axis b at vertex v combine (nine; -1
+// where there is none: an absent b-neighbour stands for three zeros, whose tap is zero).
+__device__ __forceinline__ void two_axis_sources(const int2 *__restrict__ nbr_a,
+                                                 const int2 *__restrict__ nbr_b, int v,
+                                                 int (&u)[9]) {
+    const int2 nb = nbr_b[v];
+    const int2 na_self = nbr_a[v];
+    int2 na_x = nbr_a[nb.x >= 0 ? nb.x : 0];
+    int2 na_y = nbr_a[nb.y >= 0 ? nb.y : 0];
+    asm volatile("" : "+v"(na_x.x), "+v"(na_x.y), "+v"(na_y.x), "+v"(na_y.y));
+    u[0] = nb.x >= 0 ? na_x.x : -1;
+    u[1] = nb.x;
+    u[2] = nb.x >= 0 ? na_x.y : -1;
+    u[3] = na_self.x;
+    u[4] = v;
+    u[5] = na_self.y;
+    u[6] = nb.y >= 0 ? na_y.x : -1;
+    u[7] = nb.y;
+    u[8] = nb.y >= 0 ? na_y.y : -1;
+}
+
 // one thread per (vertex, channel), any vd
+template <typename S>
 __global__ __launch_bounds__(kBlock) void k_blur_element(const Counters *counters, int max_vertices,
-                                                          int vd, const float *__restrict__ src,
-                                                          float *__restrict__ dst,
+                                                          int vd, const S *__restrict__ src,
+                                                          S *__restrict__ dst,
                                                           const int2 *__restrict__ nbr,
                                                           uint64_t *reset_cell_keys,
                                                           const int *__restrict__ vertex_cell) {
@@ -1028,32 +1071,23 @@ __global__ __launch_bounds__(kBlock) void k_blur_element(const Counters *counter
         const int v = (int)(e / (size_t)vd);
         const int j = (int)(e - (size_t)v * vd);
         const int2 nb = nbr[v];
-        const float a = nb.x >= 0 ? src[(size_t)nb.x * vd + j] : 0.0f;
-        const float b = nb.y >= 0 ? src[(size_t)nb.y * vd + j] : 0.0f;
-        dst[e] = blur_tap(a, src[e], b);
+        const int u[3] = {nb.x, v, nb.y};
+        S x[3];
+        gather_elements<S, 3>(src, vd, j, u, x);
+        dst[e] = blur_tap(x[0], x[1], x[2]);
         if (reset_cell_keys && j == 0) reset_cell_keys[vertex_cell[v]] = kEmptyCell;
     }
 }
 
 // Two axes in one launch.  Every kernel boundary costs a cold L2 and a round of dependent loads,
 // and a blur pass has almost no work, so axis a and then axis b are applied together: the value
-// after axis a is evaluated (and rounded to float, as the separate pass would store it) at the
-// vertex and at its two b-neighbours, then the b tap combines the three.  An absent b-neighbour
-// contributes zero, whatever its own a-neighbours hold.  Same arithmetic, same results.
-// One thread per (vertex, channel): with a few hundred thousand vertices the passes are bound by
-// latency, and more threads hide more of it (41 us against 48 us for one thread per vertex row).
-__device__ __forceinline__ float blur_element_of(const float *__restrict__ src,
-                                                 const int2 *__restrict__ nbr_a, int u, int vd, int j) {
-    if (u < 0) return 0.0f;
-    const int2 nb = nbr_a[u];
-    const float a = nb.x >= 0 ? src[(size_t)nb.x * vd + j] : 0.0f;
-    const float b = nb.y >= 0 ? src[(size_t)nb.y * vd + j] : 0.0f;
-    return blur_tap(a, src[(size_t)u * vd + j], b);
-}
-
+// after axis a is evaluated (and rounded to the value type, as the separate pass would store it)
+// at the vertex and at its two b-neighbours, then the b tap combines the three.  An absent
+// b-neighbour contributes zero, whatever its own a-neighbours hold.  Same arithmetic, same results.
+template <typename S>
 __global__ __launch_bounds__(kBlock) void k_blur2_element(const Counters *counters, int max_vertices,
-                                                           int vd, const float *__restrict__ src,
-                                                           float *__restrict__ dst,
+                                                           int vd, const S *__restrict__ src,
+                                                           S *__restrict__ dst,
                                                            const int2 *__restrict__ nbr_a,
                                                            const int2 *__restrict__ nbr_b,
                                                            uint64_t *reset_cell_keys,
@@ -1066,10 +1100,12 @@ __global__ __launch_bounds__(kBlock) void k_blur2_element(const Counters *counte
         if (e >= (size_t)M * vd) continue;
         const int v = (int)(e / (size_t)vd);
         const int j = (int)(e - (size_t)v * vd);
-        const int2 nb = nbr_b[v];
-        dst[e] = blur_tap(blur_element_of(src, nbr_a, nb.x, vd, j),
-                          blur_element_of(src, nbr_a, v, vd, j),
-                          blur_element_of(src, nbr_a, nb.y, vd, j));
+        int u[9];
+        two_axis_sources(nbr_a, nbr_b, v, u);
+        S x[9];
+        gather_elements<S, 9>(src, vd, j, u, x);
+        dst[e] = blur_tap(blur_tap(x[0], x[1], x[2]), blur_tap(x[3], x[4], x[5]),
+                          blur_tap(x[6], x[7], x[8]));
         if (reset_cell_keys && j == 0) reset_cell_keys[vertex_cell[v]] = kEmptyCell;
     }
 }
@@ -1078,10 +1114,6 @@ __global__ __launch_bounds__(kBlock) void k_blur2_element(const Counters *counte
 // vertex numbers that follow the image the rows a thread gathers are near each other, and a
 // quarter of the memory instructions moves the same bytes (34 -> 25 us for the three launches
 // of pd = 5, vd = 4).  Same arithmetic per channel, same results.
-// (S = double: the rows of a lattice of doubles)
-__device__ __forceinline__ double blur_tap(double a, double self, double b) {
-    return 0.25 * a + 0.5 * self + 0.25 * b;
-}
 template <int VD, typename S = float>
 struct alignas(VD == 3 ? sizeof(S) : sizeof(S) * VD) ValueRow {
     S c[VD];
@@ -1156,15 +1188,8 @@ __global__ __launch_bounds__(kBlock) void k_blur2_row(const Counters *counters, 
         if (v >= M) continue;
         // level 1: the vertex's neighbours along both axes; level 2: the a-neighbours of its
         // b-neighbours; level 3: nine rows
-        const int2 nb = nbr_b[v];
-        const int2 na_self = nbr_a[v];
-        int2 na_x = nbr_a[nb.x >= 0 ? nb.x : 0];
-        int2 na_y = nbr_a[nb.y >= 0 ? nb.y : 0];
-        asm volatile("" : "+v"(na_x.x), "+v"(na_x.y), "+v"(na_y.x), "+v"(na_y.y));
-        // (an absent b-neighbour stands for three zero rows, whose tap is zero)
-        const int u[9] = {nb.x >= 0 ? na_x.x : -1, nb.x, nb.x >= 0 ? na_x.y : -1,
-                          na_self.x,               v,    na_self.y,
-                          nb.y >= 0 ? na_y.x : -1, nb.y, nb.y >= 0 ? na_y.y : -1};
+        int u[9];
+        two_axis_sources(nbr_a, nbr_b, v, u);
         ValueRow<VD, S> row[9];
         gather_rows<VD, S, 9>(src, u, row);
         dst[v] = blur_rows<VD, S>(blur_rows<VD, S>(row[0], row[1], row[2]),
@@ -1640,7 +1665,7 @@ hipError_t blur_axis(int vd, const Counters *counters, int max_vertices, const f
         default: break;
     }
 #undef PLK_BLUR_ROW
-    hipLaunchKernelGGL(k_blur_element, dim3(vertex_blocks((size_t)launch_vertices * vd)), dim3(kBlock), 0, s,
+    hipLaunchKernelGGL(k_blur_element<float>, dim3(vertex_blocks((size_t)launch_vertices * vd)), dim3(kBlock), 0, s,
                        counters, max_vertices, vd, src, dst, nbr, reset_cell_keys, vertex_cell);
     return hipGetLastError();
 }
@@ -1663,14 +1688,14 @@ hipError_t blur_two_axes(int vd, const Counters *counters, int max_vertices, con
         default: break;
     }
 #undef PLK_BLUR2_ROW
-    hipLaunchKernelGGL(k_blur2_element, dim3(vertex_blocks((size_t)launch_vertices * vd)), dim3(kBlock), 0, s,
+    hipLaunchKernelGGL(k_blur2_element<float>, dim3(vertex_blocks((size_t)launch_vertices * vd)), dim3(kBlock), 0, s,
                        counters, max_vertices, vd, src, dst, nbr_first, nbr_second, reset_cell_keys,
                        vertex_cell);
     return hipGetLastError();
 }
 
-// Rows of two to four doubles, one thread per vertex row as for floats.
-hipError_t blur_axis_rows_f64(int vd, const Counters *counters, int max_vertices, const double *src,
+// The blur of a lattice of doubles: the same kernels over the value type.
+hipError_t blur_axis_f64(int vd, const Counters *counters, int max_vertices, const double *src,
                               double *dst, const int2 *nbr, uint64_t *reset_cell_keys,
                               const int *vertex_cell, int launch_vertices, hipStream_t s) {
     if (max_vertices <= 0) return hipSuccess;
@@ -1684,12 +1709,16 @@ hipError_t blur_axis_rows_f64(int vd, const Counters *counters, int max_vertices
         return hipGetLastError();
     switch (vd) {
         PLK_BLUR_ROW(2) PLK_BLUR_ROW(3) PLK_BLUR_ROW(4)
-        default: return hipErrorInvalidValue;
+        default: break;
     }
 #undef PLK_BLUR_ROW
+    hipLaunchKernelGGL(k_blur_element<double>, dim3(vertex_blocks((size_t)launch_vertices * vd)),
+                       dim3(kBlock), 0, s, counters, max_vertices, vd, src, dst, nbr,
+                       reset_cell_keys, vertex_cell);
+    return hipGetLastError();
 }
 
-hipError_t blur_two_axes_rows_f64(int vd, const Counters *counters, int max_vertices,
+hipError_t blur_two_axes_f64(int vd, const Counters *counters, int max_vertices,
                                   const double *src, double *dst, const int2 *nbr_first,
                                   const int2 *nbr_second, uint64_t *reset_cell_keys,
                                   const int *vertex_cell, int launch_vertices, hipStream_t s) {
@@ -1704,9 +1733,13 @@ hipError_t blur_two_axes_rows_f64(int vd, const Counters *counters, int max_vert
         return hipGetLastError();
     switch (vd) {
         PLK_BLUR2_ROW(2) PLK_BLUR2_ROW(3) PLK_BLUR2_ROW(4)
-        default: return hipErrorInvalidValue;
+        default: break;
     }
 #undef PLK_BLUR2_ROW
+    hipLaunchKernelGGL(k_blur2_element<double>, dim3(vertex_blocks((size_t)launch_vertices * vd)),
+                       dim3(kBlock), 0, s, counters, max_vertices, vd, src, dst, nbr_first,
+                       nbr_second, reset_cell_keys, vertex_cell);
+    return hipGetLastError();
 }
 
 hipError_t slice(int pd, int vd, const PointMap &map, const ReplayEntry *replay,

@@ -90,64 +90,6 @@ __global__ __launch_bounds__(kBlock) void k_splat_f64(int vd, PointMap map,
     }
 }
 
-__global__ __launch_bounds__(kBlock) void k_blur_f64(const Counters *counters, int max_vertices,
-                                                      int vd, const double *__restrict__ src,
-                                                      double *__restrict__ dst,
-                                                      const int2 *__restrict__ nbr,
-                                                      uint64_t *reset_cell_keys,
-                                                      const int *__restrict__ vertex_cell) {
-    const int M = vertex_count(counters, max_vertices);
-    ItemBlocks blocks((size_t)M * vd);
-    unsigned eb;
-    while (blocks.next(eb)) {
-        const size_t e = (size_t)eb * kBlock + threadIdx.x;
-        if (e >= (size_t)M * vd) continue;
-        const int v = (int)(e / (size_t)vd);
-        const int j = (int)(e - (size_t)v * vd);
-        const int2 nb = nbr[v];
-        const double a = nb.x >= 0 ? src[(size_t)nb.x * vd + j] : 0.0;
-        const double b = nb.y >= 0 ? src[(size_t)nb.y * vd + j] : 0.0;
-        dst[e] = 0.25 * a + 0.5 * src[e] + 0.25 * b;
-        if (reset_cell_keys && j == 0) reset_cell_keys[vertex_cell[v]] = kEmptyCell;
-    }
-}
-
-// Two axes in one launch, as in the float path: the value after axis a at the vertex and at its two
-// b-neighbours (doubles, exactly what the separate pass would have stored), then the b tap.
-__device__ __forceinline__ double blur_element_of_f64(const double *__restrict__ src,
-                                                      const int2 *__restrict__ nbr_a, int u, int vd,
-                                                      int j) {
-    if (u < 0) return 0.0;
-    const int2 nb = nbr_a[u];
-    const double a = nb.x >= 0 ? src[(size_t)nb.x * vd + j] : 0.0;
-    const double b = nb.y >= 0 ? src[(size_t)nb.y * vd + j] : 0.0;
-    return 0.25 * a + 0.5 * src[(size_t)u * vd + j] + 0.25 * b;
-}
-
-__global__ __launch_bounds__(kBlock) void k_blur2_f64(const Counters *counters, int max_vertices,
-                                                       int vd, const double *__restrict__ src,
-                                                       double *__restrict__ dst,
-                                                       const int2 *__restrict__ nbr_a,
-                                                       const int2 *__restrict__ nbr_b,
-                                                       uint64_t *reset_cell_keys,
-                                                       const int *__restrict__ vertex_cell) {
-    const int M = vertex_count(counters, max_vertices);
-    ItemBlocks blocks((size_t)M * vd);
-    unsigned eb;
-    while (blocks.next(eb)) {
-        const size_t e = (size_t)eb * kBlock + threadIdx.x;
-        if (e >= (size_t)M * vd) continue;
-        const int v = (int)(e / (size_t)vd);
-        const int j = (int)(e - (size_t)v * vd);
-        const int2 nb = nbr_b[v];
-        const double a = blur_element_of_f64(src, nbr_a, nb.x, vd, j);
-        const double self = blur_element_of_f64(src, nbr_a, v, vd, j);
-        const double b = blur_element_of_f64(src, nbr_a, nb.y, vd, j);
-        dst[e] = 0.25 * a + 0.5 * self + 0.25 * b;
-        if (reset_cell_keys && j == 0) reset_cell_keys[vertex_cell[v]] = kEmptyCell;
-    }
-}
-
 // Slice, up to eight channels: one thread per point, the row sums in registers.
 template <int D1>
 __global__ __launch_bounds__(kBlock) void k_slice_point_f64(int vd, PointMap map,
@@ -292,33 +234,6 @@ hipError_t splat_f64(int pd, int vd, const PointMap &map, const double *input, i
     PLK_DISPATCH_PD(pd, hipLaunchKernelGGL(k_splat_f64<PD + 1>, dim3(map.n_blocks), dim3(kBlock), 0,
                                            s, vd, map, input, in_channels, replay, weights,
                                            cell_vertex, values, xcd_aware));
-    return hipGetLastError();
-}
-
-hipError_t blur_axis_f64(int vd, const Counters *counters, int max_vertices, const double *src,
-                         double *dst, const int2 *neighbours_of_axis, uint64_t *reset_cell_keys,
-                         const int *vertex_cell, int launch_vertices, hipStream_t s) {
-    if (max_vertices <= 0) return hipSuccess;
-    if (vd >= 2 && vd <= 4)
-        return blur_axis_rows_f64(vd, counters, max_vertices, src, dst, neighbours_of_axis,
-                                  reset_cell_keys, vertex_cell, launch_vertices, s);
-    hipLaunchKernelGGL(k_blur_f64, dim3(vertex_blocks((size_t)launch_vertices * vd)), dim3(kBlock),
-                       0, s, counters, max_vertices, vd, src, dst, neighbours_of_axis,
-                       reset_cell_keys, vertex_cell);
-    return hipGetLastError();
-}
-
-hipError_t blur_two_axes_f64(int vd, const Counters *counters, int max_vertices, const double *src,
-                             double *dst, const int2 *nbr_first, const int2 *nbr_second,
-                             uint64_t *reset_cell_keys, const int *vertex_cell,
-                             int launch_vertices, hipStream_t s) {
-    if (max_vertices <= 0) return hipSuccess;
-    if (vd >= 2 && vd <= 4)
-        return blur_two_axes_rows_f64(vd, counters, max_vertices, src, dst, nbr_first, nbr_second,
-                                      reset_cell_keys, vertex_cell, launch_vertices, s);
-    hipLaunchKernelGGL(k_blur2_f64, dim3(vertex_blocks((size_t)launch_vertices * vd)), dim3(kBlock),
-                       0, s, counters, max_vertices, vd, src, dst, nbr_first, nbr_second,
-                       reset_cell_keys, vertex_cell);
     return hipGetLastError();
 }
 
