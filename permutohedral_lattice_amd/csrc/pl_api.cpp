@@ -357,7 +357,18 @@ int enqueue_apply_f64(pl_lattice *h, double *output, const double *input, int re
     for (int step = 0; step <= pd;) {
         const int axis = reverse ? pd - step : step;
         uint64_t *reset = (!h->table_clean && step == 0) ? h->cell_keys : nullptr;
-        if (h->pair_blur && step + 1 <= pd) {
+        const int left = pd + 1 - step;
+        // (three axes in one launch pay only when they are all there is: pd = 2; otherwise 27 row
+        // gathers per vertex cost more than the launch they save)
+        if (h->pair_blur && plk::blur_can_take_three_axes(vd) && left == 3 && step == 0) {
+            const int d = reverse ? -1 : 1;
+            PL_HIP(plk::blur_three_axes_f64(vd, h->counters(), mv, values[cur], values[1 - cur],
+                                            h->neighbours + (size_t)axis * mv,
+                                            h->neighbours + (size_t)(axis + d) * mv,
+                                            h->neighbours + (size_t)(axis + 2 * d) * mv, reset,
+                                            h->vertex_cell, h->launch_vertices(), h->stream));
+            step += 3;
+        } else if (h->pair_blur && step + 1 <= pd) {
             const int next_axis = reverse ? axis - 1 : axis + 1;
             PL_HIP(plk::blur_two_axes_f64(vd, h->counters(), mv, values[cur], values[1 - cur],
                                           h->neighbours + (size_t)axis * mv,
@@ -411,7 +422,18 @@ int enqueue_apply(pl_lattice *h, void *output_any, const void *input_any, int re
         const int axis = reverse ? pd - step : step;
         // the first blur after a build also empties the vertices' hash cells
         uint64_t *reset = (!h->table_clean && step == 0) ? h->cell_keys : nullptr;
-        if (h->pair_blur && step + 1 <= pd) {
+        const int left = pd + 1 - step;
+        // (three axes in one launch pay only when they are all there is: pd = 2; otherwise 27 row
+        // gathers per vertex cost more than the launch they save)
+        if (h->pair_blur && plk::blur_can_take_three_axes(vd) && left == 3 && step == 0) {
+            const int d = reverse ? -1 : 1;
+            PL_HIP(plk::blur_three_axes(vd, h->counters(), mv, h->values[cur], h->values[1 - cur],
+                                        h->neighbours + (size_t)axis * mv,
+                                        h->neighbours + (size_t)(axis + d) * mv,
+                                        h->neighbours + (size_t)(axis + 2 * d) * mv, reset,
+                                        h->vertex_cell, h->launch_vertices(), h->stream));
+            step += 3;
+        } else if (h->pair_blur && step + 1 <= pd) {
             const int next_axis = reverse ? axis - 1 : axis + 1;
             PL_HIP(plk::blur_two_axes(vd, h->counters(), mv, h->values[cur], h->values[1 - cur],
                                       h->neighbours + (size_t)axis * mv,

@@ -188,6 +188,17 @@ hipError_t blur_two_axes(int vd, const Counters *counters, int max_vertices, con
                          uint64_t *reset_cell_keys, const int *vertex_cell, int launch_vertices,
                          hipStream_t s);
 
+// Three axes in one launch (vd 2..4 only: blur_can_take_three_axes), bit for bit three blur_axis.
+bool blur_can_take_three_axes(int vd);
+hipError_t blur_three_axes(int vd, const Counters *counters, int max_vertices, const float *src,
+                           float *dst, const int2 *nbr_first, const int2 *nbr_second,
+                           const int2 *nbr_third, uint64_t *reset_cell_keys, const int *vertex_cell,
+                           int launch_vertices, hipStream_t s);
+hipError_t blur_three_axes_f64(int vd, const Counters *counters, int max_vertices, const double *src,
+                               double *dst, const int2 *nbr_first, const int2 *nbr_second,
+                               const int2 *nbr_third, uint64_t *reset_cell_keys,
+                               const int *vertex_cell, int launch_vertices, hipStream_t s);
+
 // Stage 5.  normalize: divide by the homogeneous channel and write vd-1 channels; else write vd.
 // cell_vertex != nullptr: the replay rows still hold hash cells (vd <= 8 only).
 hipError_t slice(int pd, int vd, const PointMap &map, const ReplayEntry *replay,

@@ -1199,6 +1199,70 @@ __global__ __launch_bounds__(kBlock) void k_blur2_row(const Counters *counters, 
     }
 }
 
+// Three axes in one launch: four levels of loads (1, 3, 9 neighbour pairs, 27 rows) instead of
+// three launches' worth.  u[3i..3i+2] are the sources of the a-tap at the i-th of the nine
+// vertices the b- and c-taps combine.
+__device__ __forceinline__ void three_axis_sources(const int2 *__restrict__ nbr_a,
+                                                   const int2 *__restrict__ nbr_b,
+                                                   const int2 *__restrict__ nbr_c, int v,
+                                                   int (&u)[27]) {
+    const int2 nc = nbr_c[v];
+    const int w[3] = {nc.x, v, nc.y};
+    int2 nbw[3];
+#pragma unroll
+    for (int k = 0; k < 3; ++k) nbw[k] = nbr_b[w[k] >= 0 ? w[k] : 0];
+#pragma unroll
+    for (int k = 0; k < 3; ++k) asm volatile("" : "+v"(nbw[k].x), "+v"(nbw[k].y));
+    int m[9];
+#pragma unroll
+    for (int k = 0; k < 3; ++k) {
+        m[3 * k] = w[k] >= 0 ? nbw[k].x : -1;
+        m[3 * k + 1] = w[k];
+        m[3 * k + 2] = w[k] >= 0 ? nbw[k].y : -1;
+    }
+    int2 nam[9];
+#pragma unroll
+    for (int i = 0; i < 9; ++i) nam[i] = nbr_a[m[i] >= 0 ? m[i] : 0];
+#pragma unroll
+    for (int i = 0; i < 9; ++i) asm volatile("" : "+v"(nam[i].x), "+v"(nam[i].y));
+#pragma unroll
+    for (int i = 0; i < 9; ++i) {
+        u[3 * i] = m[i] >= 0 ? nam[i].x : -1;
+        u[3 * i + 1] = m[i];
+        u[3 * i + 2] = m[i] >= 0 ? nam[i].y : -1;
+    }
+}
+
+template <int VD, typename S = float>
+__global__ __launch_bounds__(kBlock) void k_blur3_row(const Counters *counters, int max_vertices,
+                                                       const ValueRow<VD, S> *__restrict__ src,
+                                                       ValueRow<VD, S> *__restrict__ dst,
+                                                       const int2 *__restrict__ nbr_a,
+                                                       const int2 *__restrict__ nbr_b,
+                                                       const int2 *__restrict__ nbr_c,
+                                                       uint64_t *reset_cell_keys,
+                                                       const int *__restrict__ vertex_cell) {
+    const int M = vertex_count(counters, max_vertices);
+    ItemBlocks blocks((size_t)M);
+    unsigned vb;
+    while (blocks.next(vb)) {
+        const int v = (int)(vb * kBlock + threadIdx.x);
+        if (v >= M) continue;
+        int u[27];
+        three_axis_sources(nbr_a, nbr_b, nbr_c, v, u);
+        ValueRow<VD, S> row[27];
+        gather_rows<VD, S, 27>(src, u, row);
+        ValueRow<VD, S> after_a[9];
+#pragma unroll
+        for (int i = 0; i < 9; ++i)
+            after_a[i] = blur_rows<VD, S>(row[3 * i], row[3 * i + 1], row[3 * i + 2]);
+        dst[v] = blur_rows<VD, S>(blur_rows<VD, S>(after_a[0], after_a[1], after_a[2]),
+                                  blur_rows<VD, S>(after_a[3], after_a[4], after_a[5]),
+                                  blur_rows<VD, S>(after_a[6], after_a[7], after_a[8]));
+        if (reset_cell_keys) reset_cell_keys[vertex_cell[v]] = kEmptyCell;
+    }
+}
+
 // ------------------------------------------------------------------------------------------------
 // Stage 5: slice (reference: src/PermutohedralLatticeCPU.h:333-352)
 // ------------------------------------------------------------------------------------------------
@@ -1740,6 +1804,43 @@ hipError_t blur_two_axes_f64(int vd, const Counters *counters, int max_vertices,
                        dim3(kBlock), 0, s, counters, max_vertices, vd, src, dst, nbr_first,
                        nbr_second, reset_cell_keys, vertex_cell);
     return hipGetLastError();
+}
+
+bool blur_can_take_three_axes(int vd) { return vd >= 2 && vd <= 4; }
+
+template <typename S>
+static hipError_t blur_three_axes_of(int vd, const Counters *counters, int max_vertices, const S *src,
+                                     S *dst, const int2 *nbr_first, const int2 *nbr_second,
+                                     const int2 *nbr_third, uint64_t *reset_cell_keys,
+                                     const int *vertex_cell, int launch_vertices, hipStream_t s) {
+    if (max_vertices <= 0) return hipSuccess;
+#define PLK_BLUR3_ROW(VD)                                                                         \
+    case VD:                                                                                      \
+        hipLaunchKernelGGL((k_blur3_row<VD, S>), dim3(vertex_blocks((size_t)launch_vertices)),    \
+                           dim3(kBlock), 0, s, counters, max_vertices,                            \
+                           reinterpret_cast<const ValueRow<VD, S> *>(src),                        \
+                           reinterpret_cast<ValueRow<VD, S> *>(dst), nbr_first, nbr_second,       \
+                           nbr_third, reset_cell_keys, vertex_cell);                              \
+        return hipGetLastError();
+    switch (vd) {
+        PLK_BLUR3_ROW(2) PLK_BLUR3_ROW(3) PLK_BLUR3_ROW(4)
+        default: return hipErrorInvalidValue;
+    }
+#undef PLK_BLUR3_ROW
+}
+hipError_t blur_three_axes(int vd, const Counters *counters, int max_vertices, const float *src,
+                           float *dst, const int2 *nbr_first, const int2 *nbr_second,
+                           const int2 *nbr_third, uint64_t *reset_cell_keys, const int *vertex_cell,
+                           int launch_vertices, hipStream_t s) {
+    return blur_three_axes_of<float>(vd, counters, max_vertices, src, dst, nbr_first, nbr_second,
+                                     nbr_third, reset_cell_keys, vertex_cell, launch_vertices, s);
+}
+hipError_t blur_three_axes_f64(int vd, const Counters *counters, int max_vertices, const double *src,
+                               double *dst, const int2 *nbr_first, const int2 *nbr_second,
+                               const int2 *nbr_third, uint64_t *reset_cell_keys,
+                               const int *vertex_cell, int launch_vertices, hipStream_t s) {
+    return blur_three_axes_of<double>(vd, counters, max_vertices, src, dst, nbr_first, nbr_second,
+                                      nbr_third, reset_cell_keys, vertex_cell, launch_vertices, s);
 }
 
 hipError_t slice(int pd, int vd, const PointMap &map, const ReplayEntry *replay,
