@@ -265,7 +265,7 @@ def main():
         dominant = "blur_axis"
     achieved = alg[dominant] / (per_launch_ms[dominant] * 1e-3) / 1e9
     kernel_name = {"build": "k_build_tile<5, 4, float>" if fused else "k_build_tile<5, 0, float>", "splat": "k_splat_dpp<4, 6>",
-                   "blur_axis": "k_blur2_row<4, float>", "slice": "k_slice_point<4>"}[dominant]
+                   "blur_axis": "k_blur2_row<4, float>", "slice": "k_slice_point<4, 6>"}[dominant]
     roofline = {"bound": "hbm", "kernel": kernel_name, "achieved": round(achieved, 2),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 5),
                 "traffic": measured_traffic(kernel_name, side),
