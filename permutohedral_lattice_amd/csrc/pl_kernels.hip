@@ -942,18 +942,33 @@ __global__ __launch_bounds__(kBlock) void k_splat_channels(int d1, int vd, Point
     }
 
     // element i of the wavefront's 64 rows belongs to point i / in_channels, channel i % in_channels
+    // (eight loads asked for before the first is stored: a point without data reads point 0 and
+    // stores zero, so that no load waits behind a branch)
     {
         int p = lane / in_channels, c = lane - p * in_channels;
         const int step_p = 64 / in_channels, step_c = 64 - step_p * in_channels;
-        for (int i = lane; i < 64 * in_channels; i += 64) {
-            const int np = __shfl(n, p);
-            wave_rows[i] = np >= 0 ? input[(size_t)np * in_channels + c] : 0.0f;
-            p += step_p;
-            c += step_c;
-            if (c >= in_channels) {
-                c -= in_channels;
-                p += 1;
+        constexpr int kBatch = 8;
+        for (int i0 = lane; i0 < 64 * in_channels; i0 += 64 * kBatch) {
+            float x[kBatch];
+            bool has[kBatch];
+#pragma unroll
+            for (int k = 0; k < kBatch; ++k) {
+                const bool inside = i0 + 64 * k < 64 * in_channels;
+                const int np = __shfl(n, inside ? p : 0);
+                has[k] = inside && np >= 0;
+                x[k] = input[(size_t)(has[k] ? np : 0) * in_channels + (has[k] ? c : 0)];
+                p += step_p;
+                c += step_c;
+                if (c >= in_channels) {
+                    c -= in_channels;
+                    p += 1;
+                }
             }
+#pragma unroll
+            for (int k = 0; k < kBatch; ++k) asm volatile("" : "+v"(x[k]));
+#pragma unroll
+            for (int k = 0; k < kBatch; ++k)
+                if (i0 + 64 * k < 64 * in_channels) wave_rows[i0 + 64 * k] = has[k] ? x[k] : 0.0f;
         }
     }
     __syncthreads();
