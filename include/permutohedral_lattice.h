@@ -55,8 +55,9 @@ typedef enum pl_option {
     PL_OPT_TABLE_CELLS = 3, /* force the initial number of hash cells (power of two), 0 = automatic */
     PL_OPT_XCD_AWARE = 4,   /* 1 (default): kernels with atomic updates give each XCD a contiguous range
                                of points; 0: plain workgroup order (for measuring the difference) */
-    PL_OPT_PAIR_BLUR = 5,   /* 1 (default): two blur axes per kernel launch; 0: one launch per axis
-                               (same results bit for bit; for measuring the difference) */
+    PL_OPT_PAIR_BLUR = 5,   /* 1 (default): two blur axes per kernel launch (all three when pd = 2 and
+                               vd <= 4); 0: one launch per axis (same results bit for bit; for measuring
+                               the difference) */
     PL_OPT_GUESS_GRID = 6,  /* 1 (default): a handle without pl_set_point_grid looks, the first time it
                                sees positions, whether they describe a row-major image or volume (feature
                                0 changing exactly every row length points ...) and if so orders its
