@@ -121,7 +121,12 @@ struct pl_lattice {
     bool profile = false;
     bool xcd_aware = true;
     bool merge_tiles = true;      // option: workgroups merge their keys in LDS when the points are a grid
-    bool tiles_fit = true;        // cleared when a build found a tile with too many distinct keys
+    // A build that found a tile with too many distinct keys for its LDS table switches merging off
+    // for the next tiles_backoff builds of this lattice (doubled every time it happens again, up
+    // to 1024): inputs change, and one noisy image must not slow a long-lived lattice for good.
+    int tiles_off_for = 0;
+    int tiles_backoff = 32;
+    bool last_build_merged = false;
     bool pair_blur = true;
     // the grid the points form: given by the caller (pl_set_point_grid), or guessed once from the
     // first positions the handle sees
@@ -256,7 +261,9 @@ int enqueue_build(pl_lattice *h, const plk::PointFeatures &features, const doubl
     rc = ensure_replay(h);
     if (rc != PL_OK) return rc;
     // tiles of an image share most of their vertices among their four wavefronts
-    const bool merge = h->merge_tiles && h->tiles_fit && h->map.mode != 0;
+    const bool merge = h->merge_tiles && h->tiles_off_for == 0 && h->map.mode != 0;
+    if (h->tiles_off_for > 0) h->tiles_off_for -= 1;
+    h->last_build_merged = merge;
     // (a lattice of doubles splats in its build only in the merging kernel)
     const bool fused = splat_input && plk::build_can_splat(h->vd) && (!h->f64 || merge);
     const size_t floats_per_value = h->f64 ? 2 : 1;
@@ -472,12 +479,13 @@ int verify_build(pl_lattice *h, uint32_t *retry_cells) {
         return PL_EOVERFLOW;
     }
     if (flags & plk::kFlagTileFull) {
-        // a tile with more distinct keys than the merging build's LDS table holds: this lattice
-        // builds without merging from now on (until its point grid is set anew)
+        // a tile with more distinct keys than the merging build's LDS table holds: this call is
+        // repeated, and the next builds of this lattice run, without merging
         h->built = false;
         h->table_clean = false;
         h->cell_values_clean = false;
-        h->tiles_fit = false;
+        h->tiles_off_for = h->tiles_backoff;
+        h->tiles_backoff = h->tiles_backoff >= 512 ? 1024 : h->tiles_backoff * 2;
         *retry_cells = h->n_cells;
         return PL_EOVERFLOW;
     }
@@ -492,6 +500,7 @@ int verify_build(pl_lattice *h, uint32_t *retry_cells) {
     h->M = m;
     h->last_M = m;
     h->verified = true;
+    if (h->last_build_merged) h->tiles_backoff = 32;
     return PL_OK;
 }
 

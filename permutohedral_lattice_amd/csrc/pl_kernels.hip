@@ -351,7 +351,7 @@ __global__ __launch_bounds__(kBlock) void k_build(PointFeatures features, PointM
 // in LDS and the sums are added to the rows of the LDS slots; then every occupied slot is placed
 // in the table in HBM by one thread, and its row goes out with one request.  A workgroup whose
 // distinct keys do not fit the LDS table raises kFlagTileFull and the host repeats the build with
-// k_build.  Three barriers; every thread reaches each of them.
+// k_build (and uses it for a while).  Three barriers; every thread reaches each of them.
 constexpr int kTileSlots = 2 * kBlock;    // LDS slots per workgroup (at most 6 * kBlock keys exist)
 constexpr int kTileProbeLimit = 48;
 

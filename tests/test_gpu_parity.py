@@ -260,7 +260,8 @@ def test_merging_build_equals_the_plain_build(dtype):
     hash table (PL_OPT_MERGE_TILES); without the option every wavefront goes to the table itself.
     Same vertices, same replay rows, same outputs to rounding, for a smooth image (tiles share
     most vertices) and for one with noise in every feature (a tile then has more distinct keys
-    than its LDS table holds, and the lattice must fall back by itself, for this and later calls)."""
+    than its LDS table holds, and the lattice must fall back by itself, for this and later calls;
+    after 32 builds it tries merging again, which must again give the right answer)."""
     h, w, pd, vd = 96, 112, 5, 4
     n = h * w
     torch_dtype = torch.float32 if dtype == np.float32 else torch.float64
@@ -269,7 +270,8 @@ def test_merging_build_equals_the_plain_build(dtype):
     rng = np.random.default_rng(92)
     noisy = np.concatenate([smooth[:, :2], rng.uniform(0, 40, (n, 3)).astype(np.float32)], axis=1)
     val = img.reshape(-1, 3).astype(dtype)
-    for pos in (smooth.astype(dtype), noisy.astype(dtype)):
+    noisy_pos = noisy.astype(dtype)
+    for pos in (smooth.astype(dtype), noisy_pos):
         cpu = oracle.Lattice(pd, vd, n, dtype=dtype)
         want = cpu.filter(val, pos)
         outs = {}
@@ -278,7 +280,7 @@ def test_merging_build_equals_the_plain_build(dtype):
             lat.set_point_grid((h, w))
             lat.set_option(pla.PL_OPT_MERGE_TILES, merge)
             out = torch.empty((n, vd - 1), dtype=torch_dtype, device="cuda")
-            for _ in range(2):      # the second call runs on what the first one learnt
+            for _ in range(36 if pos is noisy_pos and merge else 2):   # later calls run on what the first learnt
                 lat.filter(out, dev(val), dev(pos), False)
                 torch.cuda.synchronize()
                 assert lat.num_vertices == cpu.num_vertices
