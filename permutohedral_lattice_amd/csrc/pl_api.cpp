@@ -224,7 +224,7 @@ int ensure_replay(pl_lattice *h) {
     if (!h->replay || !h->created_entries || !h->block_count || !h->chunk_count ||
         (h->f64 && !h->weights64))
         return PL_ENOMEM;
-    PL_HIP(hipMemsetAsync(h->chunk_count, 0, sizeof(int) * 2 * h->n_chunks, h->stream));
+    PL_HIP(plk::fill_zero(reinterpret_cast<float *>(h->chunk_count), 2 * h->n_chunks, h->stream));
     h->replay_capacity = want;
     return PL_OK;
 }
@@ -328,7 +328,7 @@ int enqueue_build(pl_lattice *h, const plk::PointFeatures &features, const doubl
     PL_HIP(hipEventRecord(h->status_written, h->stream));
     h->mark(EV_IDS);
     PL_HIP(plk::neighbours(h->pd, vertices, h->counters(), h->cell_keys, cells,
-                           h->launch_vertices(), regions, h->stream));
+                           h->launch_vertices(), h->stream));
     h->mark(EV_NBR);
     h->replay_holds_cells = true;
     h->values_zeroed = !fused;
@@ -474,8 +474,11 @@ int verify_build(pl_lattice *h, uint32_t *retry_cells) {
     const int flags = h->h_status->flags;
     const int m = h->h_status->num_vertices;
     if (flags & plk::kFlagKeyRange) {
+        // (the build may also have overflowed the table, and then rows of sums of the vertices
+        // beyond its capacity are still where the fused splat put them)
         h->built = false;
         h->table_clean = false;
+        h->cell_values_clean = false;
         return PL_EOVERFLOW;
     }
     if (flags & plk::kFlagTileFull) {
@@ -552,7 +555,11 @@ static int create_lattice(int pd, int vd, int N, bool f64, pl_stream stream, con
     }
     compute_scale_factor(pd, h->scale);
     compute_scale_factor(pd, h->scale64);
-    h->max_cells = pow2_at_least(rows * 2 < 4096 ? 4096 : rows * 2);  // holds N*(pd+1) vertices
+    // holds N*(pd+1) vertices, up to the size the kernels address cells in (32-bit byte offsets
+    // of 8-byte cells, cell_at in pl_kernels.hip); a lattice with more vertices than 3/4 of that
+    // is refused with PL_EOVERFLOW when a build finds them
+    h->max_cells = pow2_at_least(rows * 2 < 4096 ? 4096 : rows * 2);
+    if (h->max_cells > plk::kMaxCells) h->max_cells = plk::kMaxCells;
     h->map = plk::make_point_map(N, 0, nullptr);
 
     int rc = PL_OK;
@@ -562,7 +569,8 @@ static int create_lattice(int pd, int vd, int N, bool f64, pl_stream stream, con
         h->d_counters = (plk::Counters *)h->dmalloc(2 * sizeof(plk::Counters));
         if (!h->d_counters) rc = PL_ENOMEM;
     }
-    if (rc == PL_OK && hip_failed(hipMemsetAsync(h->d_counters, 0, 2 * sizeof(plk::Counters), h->stream)))
+    if (rc == PL_OK && hip_failed(plk::fill_zero(reinterpret_cast<float *>(h->d_counters),
+                                                 2 * sizeof(plk::Counters) / sizeof(float), h->stream)))
         rc = PL_EHIP;
     if (rc == PL_OK &&
         hip_failed(hipHostMalloc((void **)&h->h_status, sizeof(plk::HostStatus), hipHostMallocDefault)))
@@ -1245,8 +1253,8 @@ extern "C" int pl_lattice_filter_op_f64(const double *input, const double *refer
     if (batch == 0) return PL_OK;
     if (!input || !output) return PL_EINVAL;
 
-    // pl_filter_f64 returns after the build, the only reader of the positions, has been waited
-    // for, so the next item may overwrite them
+    // pl_filter_f64 returns after the build has been waited for, and the build's kernel is the
+    // only reader of the positions, so the next item may overwrite them
     auto filter_items = [&](pl_handle lattice, double *positions) {
         int rc = pl_set_point_grid(lattice, n_spatial_dims, spatial_dims);
         for (int b = 0; b < batch && rc == PL_OK; ++b) {

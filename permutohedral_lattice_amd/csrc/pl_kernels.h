@@ -10,6 +10,7 @@ namespace plk {
 constexpr int kMaxPd = 8;          // feature dimensions the build/neighbour kernels are instantiated for
 constexpr int kMaxSpatialDims = 8;
 constexpr uint64_t kEmptyCell = ~0ull;
+constexpr uint32_t kMaxCells = 1u << 28;   // cells are addressed by 32-bit byte offsets (8 bytes each)
 
 // bits of Counters::flags
 enum : int {
@@ -23,6 +24,10 @@ enum : int {
 struct Counters {
     unsigned int vertices;   // set by the numbering pass (may exceed what the table can hold)
     int flags;
+    // how the build spread its keys over the table (KeyRegions in pl_device.h), written by the
+    // build for the passes that look keys up after it: they must not read the caller's positions
+    // again, which only have to stay valid until the build has run
+    float region_lo, region_per_unit;
 };
 
 // What the numbering pass writes to pinned host memory about the build.
@@ -161,10 +166,10 @@ hipError_t number_vertices(int pd, const PointMap &map, const CreatedLists &list
 // below the vertex count; entries of absent neighbours keep their -1.
 // launch_vertices (here and below): the vertex count the grid is sized for; any count is
 // covered, a wrong estimate only costs time.
-// regions: the same as the build's, so that keys are looked for where it put them.
+// Keys are looked for where the build put them: counters->region_* as the build left them.
 hipError_t neighbours(int pd, const VertexTables &vertices, const Counters *counters,
                       const uint64_t *cell_keys, uint32_t n_cells, int launch_vertices,
-                      const RegionSource &regions, hipStream_t s);
+                      hipStream_t s);
 
 hipError_t fill_zero(float *p, size_t n, hipStream_t s);
 

@@ -236,6 +236,10 @@ __global__ __launch_bounds__(kBlock) void k_build(PointFeatures features, PointM
     // keys that met another key to their next cell.  Cells only ever change from empty to a key,
     // so a stale load can at worst report "empty" and the compare-and-swap returns the truth.
     const KeyRegions regions = key_regions(region_source);
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        counters->region_lo = regions.lo;
+        counters->region_per_unit = regions.per_unit;
+    }
     uint32_t cell[D1];
     uint64_t seen[D1];
     unsigned open = 0;      // bit r: this lane still has to place key r
@@ -504,6 +508,10 @@ __global__ __launch_bounds__(kBlock) void k_build_tile(PointFeatures features, P
     // rounds over both as in k_build.
     constexpr int H = kTileSlots / kBlock;
     const KeyRegions regions = key_regions(region_source);
+    if (blockIdx.x == 0 && tid == 0) {
+        counters->region_lo = regions.lo;
+        counters->region_per_unit = regions.per_unit;
+    }
     {
         // A round looks at the pair of cells a key has come to (one 16-byte load), takes the key's
         // cell if it is there, else swaps the key into the pair's first empty cell, else moves on
@@ -711,9 +719,9 @@ template <int PD>
 __global__ __launch_bounds__(kBlock) void k_neighbours(VertexTables vertices,
                                                         const Counters *counters,
                                                         const uint64_t *__restrict__ cell_keys,
-                                                        uint32_t mask, RegionSource region_source) {
+                                                        uint32_t mask) {
     constexpr int D1 = PD + 1;
-    const KeyRegions regions = key_regions(region_source);
+    const KeyRegions regions{counters->region_lo, counters->region_per_unit};
     const int max_vertices = vertices.max_vertices;
     const int M = vertex_count(counters, max_vertices);
     const unsigned runs = (unsigned)((M + kBlock - 1) / kBlock);
@@ -1592,7 +1600,18 @@ PointMap make_point_map(int N, int n_dims, const int *dims) {
             m.dims[0] = (int)lead; m.dims[1] = H; m.dims[2] = W;
             m.tiles[0] = (int)((lead + 3) / 4); m.tiles[1] = (H + 7) / 8; m.tiles[2] = (W + 7) / 8;
         }
-        m.n_blocks = (unsigned)((size_t)m.tiles[0] * m.tiles[1] * m.tiles[2]);
+        const size_t tiles = (size_t)m.tiles[0] * m.tiles[1] * m.tiles[2];
+        // An extent much shorter than its tile edge (a grid of N x 2 points) would leave most
+        // lanes of every tile without a point and multiply the per-point scratch: such points are
+        // taken as a plain list.
+        if (tiles > 2 * (((size_t)N + kBlock - 1) / kBlock)) {
+            m.mode = 0;
+            m.dims[0] = m.dims[1] = 1;
+            m.dims[2] = N;
+            m.tiles[0] = m.tiles[1] = m.tiles[2] = 1;
+        } else {
+            m.n_blocks = (unsigned)tiles;
+        }
     }
     if (N == 0) m.n_blocks = 0;
     return m;
@@ -1675,12 +1694,12 @@ hipError_t number_vertices(int pd, const PointMap &map, const CreatedLists &list
 
 hipError_t neighbours(int pd, const VertexTables &vertices, const Counters *counters,
                       const uint64_t *cell_keys, uint32_t n_cells, int launch_vertices,
-                      const RegionSource &regions, hipStream_t s) {
+                      hipStream_t s) {
     if (vertices.max_vertices <= 0) return hipErrorInvalidValue;
     const size_t items = (size_t)(pd + 1) * ((size_t)launch_vertices + kBlock);
     PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_neighbours<PD>), dim3(vertex_blocks(items)),
                                            dim3(kBlock), 0, s, vertices, counters, cell_keys,
-                                           n_cells - 1u, regions));
+                                           n_cells - 1u));
     return hipGetLastError();
 }
 

@@ -454,6 +454,31 @@ def test_coordinates_beyond_the_packed_key_range_are_reported():
     assert_float_parity(got, oracle.Lattice(4, 2, n).filter(val, pos4))
 
 
+def test_handle_filters_correctly_after_a_refused_call_that_also_overflowed_its_table():
+    """A call refused for a coordinate out of range, whose build had overflowed a small table as
+    well, must not leave sums behind that the next call on the handle adds its own to."""
+    rng = np.random.default_rng(41)
+    n = 64 * 64
+    img = rng.uniform(0, 1, (64, 64, 3)).astype(np.float32)      # noise: many vertices
+    pos = synth.bilateral_positions(img, 2.0, 0.05)
+    bad = pos.copy()
+    bad[n // 2, 0] = 3.0e6                                        # beyond the reference's short keys
+    val = rng.uniform(0, 1, (n, 3)).astype(np.float32)
+    lat = pla.PermutohedralLattice(5, 4, n)
+    lat.set_point_grid((64, 64))
+    lat.set_option(pla.PL_OPT_TABLE_CELLS, 4096)
+    out = torch.empty((n, 3), dtype=torch.float32, device="cuda")
+    with pytest.raises(pla.PermutohedralError) as e:
+        lat.filter(out, dev(val), dev(bad))
+    assert e.value.status == pla.PL_EOVERFLOW
+    cpu = oracle.Lattice(5, 4, n)
+    want = cpu.filter(val, pos)
+    for _ in range(2):
+        got, _ = gpu_filter(5, 4, pos, val, lattice=lat)
+        assert lat.num_vertices == cpu.num_vertices
+        assert_float_parity(got, want)
+
+
 def test_large_lattice_coordinates_pd5_within_range():
     rng = np.random.default_rng(18)
     n = 20000
