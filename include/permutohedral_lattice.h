@@ -26,7 +26,8 @@ typedef enum pl_status {
     PL_ENOMEM = -3,       /* allocator returned NULL */
     PL_EOVERFLOW = -4,    /* sizes do not fit int32, or lattice coordinates do not fit the packed key */
     PL_EHIP = -5,         /* a HIP runtime call failed; pl_last_hip_error() has the code */
-    PL_ESTATE = -6        /* pl_apply before pl_build, and the like */
+    PL_ESTATE = -6,       /* pl_apply before pl_build, and the like */
+    PL_ETOOLARGE = -7     /* pl_filter_static: the lattice does not fit the library's static scratch */
 } pl_status;
 
 /* Opaque lattice object. */
@@ -99,6 +100,23 @@ int pl_destroy(pl_handle h);
  * lattice's stream, as with the reference's GPU path.
  */
 int pl_filter(pl_handle h, float *output, const float *input, const float *positions, int reverse);
+
+/*
+ * pl_filter for callers that cannot allocate (code under HIP graph capture elsewhere in the
+ * process, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the
+ * reference, whose lattice objects allocate in their constructors
+ * (src/PermutohedralLatticeGPU.cuh:434-451).  No handle: the lattice lives for the length of the call
+ * in a static device array of 64 MiB inside the library (one copy per GPU the library runs on,
+ * held until the process ends), and the call makes no hipMalloc, hipFree, hipHostMalloc or event.
+ * Limits: N*(pd+1) <= 131072 (e.g. 21845 points at pd = 5) and vd <= 8, float values; beyond them
+ * PL_ETOOLARGE.  The hash table is sized for N*(pd+1) vertices, so no input makes it overflow.
+ * The points are taken as a plain list (no grid is looked for).  Same results as pl_filter; the
+ * call returns when its work on `stream` is complete.  All calls on a GPU share that GPU's array
+ * and what the last call left in it (each call clears what it needs to be zero), so calls that
+ * overlapped on one GPU would race: the library takes a lock for the length of each call.
+ */
+int pl_filter_static(int pd, int vd, int N, float *output, const float *input,
+                     const float *positions, int reverse, pl_stream stream);
 
 /*
  * Build the lattice for positions[N*pd] (embed, enclosing simplex, hash insertion, neighbour

@@ -20,6 +20,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "libpermutohedral_hip.so")
 
 PL_OK, PL_EINVAL, PL_EUNSUPPORTED, PL_ENOMEM, PL_EOVERFLOW, PL_EHIP, PL_ESTATE = 0, -1, -2, -3, -4, -5, -6
+PL_ETOOLARGE = -7
 PL_OPT_NORMALIZE, PL_OPT_PROFILE, PL_OPT_TABLE_CELLS, PL_OPT_XCD_AWARE, PL_OPT_PAIR_BLUR = 1, 2, 3, 4, 5
 PL_OPT_GUESS_GRID = 6
 PL_OPT_MERGE_TILES = 7
@@ -27,7 +28,7 @@ PL_OPT_MERGE_TILES = 7
 # every symbol include/permutohedral_lattice.h declares
 EXPORTS = (
     "pl_supported", "pl_strerror", "pl_last_hip_error", "pl_create", "pl_destroy", "pl_filter",
-    "pl_build", "pl_apply", "pl_set_point_grid", "pl_get_point_grid", "pl_num_vertices", "pl_set_option", "pl_stage_ms", "pl_debug_simplex",
+    "pl_filter_static", "pl_build", "pl_apply", "pl_set_point_grid", "pl_get_point_grid", "pl_num_vertices", "pl_set_option", "pl_stage_ms", "pl_debug_simplex",
     "pl_debug_keys", "pl_debug_replay", "pl_compute_positions", "pl_filter_image", "pl_build_image",
     "pl_filter_begin", "pl_filter_image_begin", "pl_filter_end", "pl_lattice_filter_op",
     "pl_set_op_concurrency",
@@ -62,6 +63,7 @@ def _load():
     lib.pl_create.argtypes = [ci, ci, ci, vp, vp, C.POINTER(vp)]
     lib.pl_destroy.argtypes = [vp]
     lib.pl_filter.argtypes = [vp, vp, vp, vp, ci]
+    lib.pl_filter_static.argtypes = [ci, ci, ci, vp, vp, vp, ci, vp]
     lib.pl_build.argtypes = [vp, vp]
     lib.pl_apply.argtypes = [vp, vp, vp, ci]
     lib.pl_set_point_grid.argtypes = [vp, ci, C.POINTER(ci)]
@@ -283,6 +285,18 @@ class PermutohedralLattice:
         _check(_lib.pl_debug_replay(self._h, C.c_void_p(v.data_ptr()), C.c_void_p(w.data_ptr())),
                "pl_debug_replay")
         return v, w
+
+
+def filter_static(output, input, positions, pd, vd, reverse=False, stream=None):
+    """``filter`` without a lattice object and without any allocation: the lattice lives in a
+    static device array inside the library for the length of the call (N*(pd+1) <= 131072,
+    vd <= 8, float32; ``PL_ETOOLARGE`` beyond)."""
+    n = int(positions.shape[0]) if positions.dim() == 2 else positions.numel() // int(pd)
+    _check(_lib.pl_filter_static(int(pd), int(vd), n, _dev_f32(output, "output", n * (vd - 1)),
+                                 _dev_f32(input, "input", n * (vd - 1)),
+                                 _dev_f32(positions, "positions", n * pd), int(bool(reverse)),
+                                 _stream_ptr(stream)), "pl_filter_static")
+    return output
 
 
 def set_op_concurrency(lanes):

@@ -109,6 +109,9 @@ struct pl_lattice {
     int counter_set = 0;                   // the set of the last build
     plk::HostStatus *h_status = nullptr;   // pinned, written by the device
     hipEvent_t status_written = nullptr;   // recorded behind the kernel that writes h_status
+    // a lattice in the library's static scratch (pl_filter_static) owns no pinned memory and no
+    // event: h_status is device memory there, copied to the host when the build is verified
+    bool status_on_device = false;
 
     int M = 0;
     int last_M = -1;
@@ -325,7 +328,7 @@ int enqueue_build(pl_lattice *h, const plk::PointFeatures &features, const doubl
                                 h->values[0], h->f64 ? 2 * h->vd : h->vd,
                                 fused ? h->cell_values : nullptr, h->counters(),
                                 h->d_counters + previous_set, h->h_status, h->stream));
-    PL_HIP(hipEventRecord(h->status_written, h->stream));
+    if (!h->status_on_device) PL_HIP(hipEventRecord(h->status_written, h->stream));
     h->mark(EV_IDS);
     PL_HIP(plk::neighbours(h->pd, vertices, h->counters(), h->cell_keys, cells,
                            h->launch_vertices(), h->stream));
@@ -470,9 +473,16 @@ int enqueue_apply(pl_lattice *h, void *output_any, const void *input_any, int re
 // Otherwise *retry_cells is the table size to try next (0: give up with the returned status).
 int verify_build(pl_lattice *h, uint32_t *retry_cells) {
     *retry_cells = 0;
-    PL_HIP(hipEventSynchronize(h->status_written));
-    const int flags = h->h_status->flags;
-    const int m = h->h_status->num_vertices;
+    plk::HostStatus status;
+    if (h->status_on_device) {
+        PL_HIP(hipMemcpyAsync(&status, h->h_status, sizeof(status), hipMemcpyDeviceToHost, h->stream));
+        PL_HIP(hipStreamSynchronize(h->stream));
+    } else {
+        PL_HIP(hipEventSynchronize(h->status_written));
+        status = *h->h_status;
+    }
+    const int flags = status.flags;
+    const int m = status.num_vertices;
     if (flags & plk::kFlagKeyRange) {
         // (the build may also have overflowed the table, and then rows of sums of the vertices
         // beyond its capacity are still where the fused splat put them)
@@ -522,6 +532,8 @@ const char *pl_strerror(int status) {
         case PL_EOVERFLOW: return "size or lattice coordinate out of range";
         case PL_EHIP: return "HIP runtime error";
         case PL_ESTATE: return "call out of order";
+        case PL_ETOOLARGE:
+            return "too large for the static scratch of pl_filter_static (N*(pd+1) <= 131072, vd <= 8)";
         default: return "unknown status";
     }
 }
@@ -1295,4 +1307,107 @@ extern "C" int pl_lattice_filter_op_f64(const double *input, const double *refer
         return PL_ENOMEM;
     }
     return filter_items(entry->lanes[0].lattice, entry->positions64);
+}
+
+// ------------------------------------------------------------------------------------------------
+// pl_filter_static: pl_filter on a lattice whose every array lies in a static device array, for
+// callers that cannot allocate.  No hipMalloc, hipFree, hipHostMalloc or event creation anywhere
+// on this path; the lattice object itself is static host memory.
+// ------------------------------------------------------------------------------------------------
+namespace {
+
+constexpr size_t kStaticScratchBytes = (size_t)64 << 20;
+constexpr long long kStaticMaxRows = 1 << 17;   // N * (pd + 1)
+constexpr int kStaticMaxVd = 8;
+constexpr int kStaticMaxDevices = 32;
+
+// Every GPU the library runs on holds its own copy of this array, at its own address, until the
+// process ends.  In host code the name is a stand-in for the symbol, never an address to pass on:
+// the address on the current device comes from hipGetSymbolAddress (static_scratch_of).
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+
+struct StaticLattice {
+    unsigned char *base = nullptr;   // address of `scratch` on this device
+    size_t used = 0;
+    pl_lattice lattice;
+};
+StaticLattice g_static[kStaticMaxDevices];
+std::mutex g_static_mutex;
+
+void *static_alloc(void *ctx, size_t bytes) {
+    StaticLattice *st = static_cast<StaticLattice *>(ctx);
+    const size_t start = (st->used + 255) & ~(size_t)255;
+    if (start + bytes > kStaticScratchBytes) return nullptr;
+    st->used = start + bytes;
+    return st->base + start;
+}
+void static_free(void *, void *) {}
+
+// The address of `scratch` on the current device, asked for once per device.
+int static_scratch_of(int device, StaticLattice **out) {
+    if (device < 0 || device >= kStaticMaxDevices) return PL_EUNSUPPORTED;
+    StaticLattice *st = &g_static[device];
+    if (!st->base) {
+        void *ptr = nullptr;
+        PL_HIP(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
+        if (!ptr) return PL_EHIP;
+        st->base = static_cast<unsigned char *>(ptr);
+    }
+    *out = st;
+    return PL_OK;
+}
+
+}  // namespace
+
+extern "C" int pl_filter_static(int pd, int vd, int N, float *output, const float *input,
+                                const float *positions, int reverse, pl_stream stream) {
+    if (N < 0 || pd < 1 || vd < 2) return PL_EINVAL;
+    if (!pl_supported(pd, vd)) return PL_EUNSUPPORTED;
+    if ((long long)N * (pd + 1) > kStaticMaxRows || vd > kStaticMaxVd) return PL_ETOOLARGE;
+    if (N == 0) return PL_OK;
+    if (!output || !input || !positions) return PL_EINVAL;
+
+    // one call at a time per process: the calls share the lattice object below, and on a GPU the
+    // array itself (the call returns when its work on the stream is done, see verify_build)
+    std::lock_guard<std::mutex> lock(g_static_mutex);
+    int device = 0;
+    PL_HIP(hipGetDevice(&device));
+    StaticLattice *st = nullptr;
+    int rc = static_scratch_of(device, &st);
+    if (rc != PL_OK) return rc;
+
+    // A fresh lattice over the array: whatever the last call left there is cleared by the build
+    // as for memory that has just been allocated (hash cells, rows of sums, counters, chunk sums).
+    st->used = 0;
+    st->lattice = pl_lattice();
+    pl_lattice *h = &st->lattice;
+    h->pd = pd;
+    h->vd = vd;
+    h->N = N;
+    h->device = device;
+    h->stream = (hipStream_t)stream;
+    h->alloc.alloc = static_alloc;
+    h->alloc.free = static_free;
+    h->alloc.ctx = st;
+    compute_scale_factor(pd, h->scale);
+    compute_scale_factor(pd, h->scale64);
+    // a table that holds N*(pd+1) vertices, the most there can be: no build is ever repeated
+    const uint64_t rows = (uint64_t)N * (uint64_t)(pd + 1);
+    h->max_cells = pow2_at_least(rows * 2 < 4096 ? 4096 : rows * 2);
+    h->forced_cells = (long)h->max_cells;
+    h->guess_grid = false;   // (looking for a grid in the positions would allocate and wait)
+    h->map = plk::make_point_map(N, 0, nullptr);
+    h->status_on_device = true;
+    rc = ensure_replay(h);
+    if (rc != PL_OK) return rc;
+    h->d_counters = (plk::Counters *)h->dmalloc(2 * sizeof(plk::Counters));
+    h->h_status = (plk::HostStatus *)h->dmalloc(sizeof(plk::HostStatus));
+    if (!h->d_counters || !h->h_status) return PL_ENOMEM;
+    PL_HIP(plk::fill_zero(reinterpret_cast<float *>(h->d_counters),
+                          2 * sizeof(plk::Counters) / sizeof(float), h->stream));
+    rc = filter_lattice(h, output, input, features_from_positions(positions), reverse);
+    // verify_build has waited for the stream; after an error make sure nothing is left running
+    // on an array the next call will overwrite
+    if (rc != PL_OK) (void)hipStreamSynchronize(h->stream);
+    return rc;
 }

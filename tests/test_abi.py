@@ -37,11 +37,11 @@ def test_supported_dimensions():
 
 def test_strerror_covers_every_status():
     seen = set()
-    for code in range(0, -7, -1):
+    for code in range(0, -8, -1):
         msg = pla._lib.pl_strerror(code).decode()
         assert msg and msg != "unknown status"
         seen.add(msg)
-    assert len(seen) == 7
+    assert len(seen) == 8
     assert pla._lib.pl_strerror(-99).decode() == "unknown status"
 
 
