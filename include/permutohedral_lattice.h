@@ -63,10 +63,14 @@ typedef enum pl_option {
                                sees positions, whether they describe a row-major image or volume (feature
                                0 changing exactly every row length points ...) and if so orders its
                                work as with the hint; 0: never (points are a plain list) */
-    PL_OPT_MERGE_TILES = 7  /* 1 (default): when the points are a grid, a workgroup of the build merges
+    PL_OPT_MERGE_TILES = 7, /* 1 (default): when the points are a grid, a workgroup of the build merges
                                the keys and sums of its tile in LDS before they go to the hash table;
                                0: every wavefront goes to the table itself (same results; for
                                measuring the difference) */
+    PL_OPT_STOP_AFTER = 8   /* 0 (default): a filter or apply runs to the end.  1: it ends behind the
+                               splat, 2: behind the blur; the output is then not written and
+                               pl_debug_values gives the vertex values of that stage (for checking the
+                               stages one by one against src/PermutohedralLatticeCPU.h:306-317, 362-415) */
 } pl_option;
 
 /* 1 when a lattice can be built for these dimensions, else 0.
@@ -167,6 +171,12 @@ int pl_debug_simplex(pl_handle h, const float *positions, short *rem0, short *ra
 /* Keys of the vertices of the last build, M*pd shorts to device memory, in vertex-index order
  * (HashTableCPU::getKeys(), src/PermutohedralLatticeCPU.h:154; the order is not the reference's). */
 int pl_debug_keys(pl_handle h, short *keys);
+
+/* Values of the vertices as the last pl_filter / pl_apply left them, M*vd floats (doubles for a
+ * lattice of doubles) to device memory, rows in the vertex order of pl_debug_keys: after the blur,
+ * or after the stage PL_OPT_STOP_AFTER names (HashTableCPU::getValues(),
+ * src/PermutohedralLatticeCPU.h:157, read after splat :322-326 or blur :362-415). */
+int pl_debug_values(pl_handle h, void *values);
 
 /* Vertex index (0..M-1) and weight of each point's simplex vertices of the last build: vertex[(pd+1)*N], weight[(pd+1)*N], laid out [r][n]; device pointers.  The replay
  * matrix of src/PermutohedralLatticeCPU.h:187-191, 314-317. */

@@ -225,6 +225,36 @@ def lattice_filter(input_image, reference_image, bilateral=True, theta_alpha=1.0
     return out
 
 
+def _softmax(z):
+    z = np.asarray(z, np.float64)
+    z = z - z.max(axis=-1, keepdims=True)
+    e = np.exp(z)
+    return (e / e.sum(axis=-1, keepdims=True)).astype(np.float32)
+
+
+def mean_field(logits, guide, iterations=5, theta_alpha=80.0, theta_beta=13.0, theta_gamma=3.0,
+               upstream=None, op=None):
+    """CPU twin of permutohedral_lattice_amd.crf.MeanField, for checking it: Q <- softmax(logits +
+    bilateral(Q) + spatial(Q)) `iterations` times on channels-last arrays [B, s_1..s_k, C], every
+    message a fresh lattice_filter call as the reference's op would make it; with `upstream` also
+    the reverse pass, bilateral_reverse(upstream) + spatial_reverse(upstream).  `op`: the
+    lattice_filter to use (default this module's; pass reference().lattice_filter for the
+    reference's own header).  -> (Q, reverse or None)"""
+    op = op or lattice_filter
+    logits = np.ascontiguousarray(logits, np.float32)
+    guide = np.ascontiguousarray(guide, np.float32)
+
+    def messages(q, reverse):
+        return (op(q, guide, True, theta_alpha, theta_beta, theta_gamma, reverse)
+                + op(q, guide, False, theta_alpha, theta_beta, theta_gamma, reverse))
+
+    q = _softmax(logits)
+    for _ in range(iterations):
+        q = _softmax(logits.astype(np.float64) + messages(q, False))
+    rev = None if upstream is None else messages(np.ascontiguousarray(upstream, np.float32), True)
+    return q, rev
+
+
 # ---------------------------------------------------------------------------------------------
 # The reference's own CPU header behind C entry points (present only after `make -C oracle ref`)
 # ---------------------------------------------------------------------------------------------

@@ -24,12 +24,13 @@ PL_ETOOLARGE = -7
 PL_OPT_NORMALIZE, PL_OPT_PROFILE, PL_OPT_TABLE_CELLS, PL_OPT_XCD_AWARE, PL_OPT_PAIR_BLUR = 1, 2, 3, 4, 5
 PL_OPT_GUESS_GRID = 6
 PL_OPT_MERGE_TILES = 7
+PL_OPT_STOP_AFTER = 8
 
 # every symbol include/permutohedral_lattice.h declares
 EXPORTS = (
     "pl_supported", "pl_strerror", "pl_last_hip_error", "pl_create", "pl_destroy", "pl_filter",
     "pl_filter_static", "pl_build", "pl_apply", "pl_set_point_grid", "pl_get_point_grid", "pl_num_vertices", "pl_set_option", "pl_stage_ms", "pl_debug_simplex",
-    "pl_debug_keys", "pl_debug_replay", "pl_compute_positions", "pl_filter_image", "pl_build_image",
+    "pl_debug_keys", "pl_debug_values", "pl_debug_replay", "pl_compute_positions", "pl_filter_image", "pl_build_image",
     "pl_filter_begin", "pl_filter_image_begin", "pl_filter_end", "pl_lattice_filter_op",
     "pl_set_op_concurrency",
     "pl_create_f64", "pl_filter_f64", "pl_build_f64", "pl_apply_f64", "pl_debug_simplex_f64",
@@ -73,6 +74,7 @@ def _load():
     lib.pl_stage_ms.argtypes = [vp, C.POINTER(cf)]
     lib.pl_debug_simplex.argtypes = [vp, vp, vp, vp, vp, vp]
     lib.pl_debug_keys.argtypes = [vp, vp]
+    lib.pl_debug_values.argtypes = [vp, vp]
     lib.pl_debug_replay.argtypes = [vp, vp, vp]
     lib.pl_compute_positions.argtypes = [vp, vp, ci, ci, ci, C.POINTER(ci), cf, cf, vp]
     lib.pl_filter_image.argtypes = [vp, vp, vp, vp, ci, ci, C.POINTER(ci), cf, cf, ci]
@@ -276,6 +278,12 @@ class PermutohedralLattice:
         keys = torch.empty((self.num_vertices, self.pd), dtype=torch.int16, device="cuda")
         _check(_lib.pl_debug_keys(self._h, C.c_void_p(keys.data_ptr())), "pl_debug_keys")
         return keys
+
+    def debug_values(self):
+        """-> vertex values [M, vd] as the last filter/apply left them (rows as in debug_keys)."""
+        v = torch.empty((self.num_vertices, self.vd), dtype=self.dtype, device="cuda")
+        _check(_lib.pl_debug_values(self._h, C.c_void_p(v.data_ptr())), "pl_debug_values")
+        return v
 
     def debug_replay(self):
         """-> (vertex [pd+1, N] i32, weight [pd+1, N] f32) of the last apply/filter."""

@@ -121,6 +121,8 @@ struct pl_lattice {
     bool values_zeroed = false;        // values[0] rows of all vertices are zero
     bool values_splatted = false;      // values[0] already holds the splat of the pending apply
     bool normalize = true;
+    int stop_after = 0;                // PL_OPT_STOP_AFTER: 1 = an apply ends behind the splat, 2 = behind the blur
+    int current_values = 0;            // which of values[] the last apply left the vertex values in
     bool profile = false;
     bool xcd_aware = true;
     bool merge_tiles = true;      // option: workgroups merge their keys in LDS when the points are a grid
@@ -364,6 +366,8 @@ int enqueue_apply_f64(pl_lattice *h, double *output, const double *input, int re
     h->values_splatted = false;
     h->mark(EV_SPLAT);
     int cur = 0;
+    h->current_values = 0;
+    if (h->stop_after == 1) return PL_OK;
     for (int step = 0; step <= pd;) {
         const int axis = reverse ? pd - step : step;
         uint64_t *reset = (!h->table_clean && step == 0) ? h->cell_keys : nullptr;
@@ -395,6 +399,8 @@ int enqueue_apply_f64(pl_lattice *h, double *output, const double *input, int re
         cur = 1 - cur;
     }
     h->mark(EV_BLUR);
+    h->current_values = cur;
+    if (h->stop_after == 2) return PL_OK;
     PL_HIP(plk::slice_f64(pd, vd, h->map, h->replay, h->weights64,
                           h->replay_holds_cells ? h->cell_vertex : nullptr, values[cur], output,
                           h->normalize ? 1 : 0, h->stream));
@@ -427,6 +433,8 @@ int enqueue_apply(pl_lattice *h, void *output_any, const void *input_any, int re
     h->values_splatted = false;
     h->mark(EV_SPLAT);
     int cur = 0;
+    h->current_values = 0;
+    if (h->stop_after == 1) return PL_OK;
     for (int step = 0; step <= pd;) {
         // axes 0..pd, or pd..0 for the reverse pass; two per launch while two are left
         const int axis = reverse ? pd - step : step;
@@ -460,6 +468,8 @@ int enqueue_apply(pl_lattice *h, void *output_any, const void *input_any, int re
         cur = 1 - cur;
     }
     h->mark(EV_BLUR);
+    h->current_values = cur;
+    if (h->stop_after == 2) return PL_OK;
     PL_HIP(plk::slice(pd, vd, h->map, h->replay,
                       h->replay_holds_cells ? h->cell_vertex : nullptr, h->values[cur], output,
                       h->normalize ? 1 : 0, h->stream));
@@ -656,6 +666,10 @@ int pl_set_option(pl_handle h, int option, long value) {
             return PL_OK;
         case PL_OPT_MERGE_TILES:
             h->merge_tiles = value != 0;
+            return PL_OK;
+        case PL_OPT_STOP_AFTER:
+            if (value < 0 || value > 2) return PL_EINVAL;
+            h->stop_after = (int)value;
             return PL_OK;
         case PL_OPT_TABLE_CELLS:
             if (value < 0 || (value & (value - 1)) != 0) return PL_EINVAL;
@@ -993,6 +1007,16 @@ int pl_debug_keys(pl_handle h, short *keys) {
     if (!h || !keys) return PL_EINVAL;
     if (!h->built || !h->verified) return PL_ESTATE;
     PL_HIP(plk::export_keys(h->pd, h->vertex_keys, h->M, keys, h->stream));
+    return PL_OK;
+}
+
+int pl_debug_values(pl_handle h, void *values) {
+    if (!h || !values) return PL_EINVAL;
+    if (!h->built || !h->verified) return PL_ESTATE;
+    if (h->M == 0) return PL_OK;
+    PL_HIP(hipMemcpyAsync(values, h->values[h->current_values],
+                          h->value_size() * (size_t)h->M * (size_t)h->vd, hipMemcpyDeviceToDevice,
+                          h->stream));
     return PL_OK;
 }
 
