@@ -34,19 +34,322 @@ def algorithmic_bytes(n, m, pd, vd):
     }
 
 
-def measured_traffic(kernel_name, side):
+def kernel_source_hash():
+    """Short hash of the sources the HIP library is built from: what a counter measurement is
+    stamped with, so that a figure taken from an older build shows as stale."""
+    import hashlib
+    h = hashlib.sha256()
+    csrc = os.path.join(ROOT, "permutohedral_lattice_amd", "csrc")
+    for name in sorted(os.listdir(csrc)):
+        if name.endswith((".hip", ".h", ".cpp")) and not name.startswith("bilateral_filter_cli"):
+            h.update(name.encode())
+            h.update(open(os.path.join(csrc, name), "rb").read())
+    return h.hexdigest()[:12]
+
+
+def measured_traffic(kernel_name, grid_threads, stem="bench_bilateral_1024_pd5_vd4"):
     """HBM bytes per launch of a kernel (read + written) as rocprofv3's FETCH_SIZE / WRITE_SIZE gave
     them for this workload, scaled by the copy calibration; the summary under profiles/ holds the
-    commands.  None when there is no measurement for this kernel and size."""
-    path = os.path.join(ROOT, "profiles", "bench_bilateral_%d_pd5_vd4_hbm_traffic.json" % side)
+    commands.  -> (bytes or None, stamp) where stamp says which build of the kernels the counters
+    were taken on and whether that is the build running now."""
+    path = os.path.join(ROOT, "profiles", stem + "_hbm_traffic.json")
     try:
-        table = json.load(open(path))["per_kernel_bytes"]
+        record = json.load(open(path))
+        table = record["per_kernel_bytes"]
     except (OSError, ValueError, KeyError):
-        return None
-    key = "%s@%d" % (kernel_name, side * side)
+        return None, None
+    now = kernel_source_hash()
+    stamp = {"measured_on_sources": record.get("kernel_source_hash"), "running_sources": now,
+             "stale": record.get("kernel_source_hash") != now}
+    key = "%s@%d" % (kernel_name, grid_threads)
     if key not in table:
+        return None, stamp
+    return int(sum(table[key])), stamp
+
+
+def kernel_names(pd, vd):
+    """The kernels a filter() call of a grid of points runs for these dimensions, by stage."""
+    fused = vd <= 4
+    d1 = pd + 1
+    if fused:
+        blur = "k_blur3_row<%d, float>" % vd if pd == 2 else "k_blur2_row<%d, float>" % vd
+        slice_k = "k_slice_point<%d, %d>" % (vd, d1)
+    else:
+        blur = "k_blur2_element<float>"
+        slice_k = "k_slice_point<%d, 0>" % vd if vd <= 8 else "k_slice_channels<%d>" % d1
+    width = 16 if vd <= 16 else (32 if vd <= 32 else 64)
+    return {"build": "k_build_tile<%d, %d, float>" % (pd, vd if fused else 0),
+            "splat": "k_splat_dpp<%d, %d>" % (vd, d1) if fused else "k_splat_channels<%d>" % width,
+            "blur_axis": blur, "slice": slice_k}
+
+
+def stage_report(lat, call, n, pd, vd, samples=5, fused_splat=True):
+    """Per-stage milliseconds of `call()` (one filter or apply on `lat`) from HIP events on the
+    lattice's stream, and the stage that takes longest with its share of the HBM roofline."""
+    import permutohedral_lattice_amd as pla
+    lat.set_option(pla.PL_OPT_PROFILE, 1)
+    rows = []
+    for _ in range(samples):
+        call()
+        rows.append(lat.stage_ms())
+    lat.set_option(pla.PL_OPT_PROFILE, 0)
+    stages = {k: statistics.mean(r[k] for r in rows) for k in rows[0]}
+    stages["blur_axis"] = stages["blur"] / (pd + 1)
+    m = lat.num_vertices
+    alg = algorithmic_bytes(n, m, pd, vd)
+    if vd <= 4 and fused_splat:
+        alg["build"] += alg["splat"]      # filter() splats inside the build kernel
+    names = kernel_names(pd, vd)
+    candidates = [k for k in ("build", "splat", "slice") if stages[k] > 0.0]
+    dominant = max(candidates, key=lambda k: stages[k])
+    if stages["blur"] > stages[dominant]:
+        dominant = "blur_axis"
+    gbs = alg[dominant] / (stages[dominant] * 1e-3) / 1e9
+    return stages, {"kernel": names[dominant], "launch_ms": round(stages[dominant], 5),
+                    "algorithmic_bytes_per_launch": alg[dominant], "achieved_GBs": round(gbs, 1),
+                    "frac": round(gbs / HBM_PEAK_GBS, 5)}
+
+
+def parity(got, want):
+    import numpy as np
+    got, want = np.asarray(got, np.float64), np.asarray(want, np.float64)
+    return {"max_abs": float(np.abs(got - want).max()),
+            "rel_l2": float(np.linalg.norm(got - want) / max(np.linalg.norm(want), 1e-30))}
+
+
+def timed(fn, warmup, reps):
+    import torch
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(reps):
+        fn()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / reps
+
+
+def run_configs(args, pla, synth, with_cpu):
+    """Every BASELINE configuration at its full size: time per filter() call (what one call moves
+    against the HBM roofline), the kernel that takes longest with its own roofline share, and the
+    outputs against the CPU reference on the same arrays."""
+    import numpy as np
+    import torch
+    from permutohedral_lattice_amd.crf import MeanField
+    cpu = None
+    if with_cpu:
+        import oracle
+        cpu = oracle.reference()
+    out = {}
+
+    def dev(a):
+        return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+    # Parity is taken against the oracle with one vertex per distinct key, which is what the library
+    # builds.  The reference's own header enters a key a second time at some doublings of its hash
+    # index (its lookup starts from a cell computed before the growth); those few vertices split
+    # their values, and under a normalisation by small weights the outputs around them move by more
+    # than the tolerance.  The figures against the reference's build are printed beside, as they are.
+    def both(got, port, ref_out):
+        rec = {"parity_vs_cpu": port(got)}
+        if ref_out is not None:
+            rec["against_reference_build_with_its_duplicate_vertices"] = ref_out(got)
+        return rec
+
+    def one_filter(name, what, pd, vd, grid, pos, val, reps):
+        n = pos.shape[0]
+        lat = pla.PermutohedralLattice(pd, vd, n)
+        lat.set_point_grid(grid)
+        d_pos, d_val = dev(pos), dev(val)
+        d_out = torch.empty_like(d_val)
+        seconds = timed(lambda: lat.filter(d_out, d_val, d_pos, False), 3 if n < (1 << 22) else 1, reps)
+        m = lat.num_vertices
+        stages, dominant = stage_report(lat, lambda: lat.filter(d_out, d_val, d_pos, False), n, pd, vd,
+                                        samples=5 if n < (1 << 22) else 3)
+        alg = algorithmic_bytes(n, m, pd, vd)["filter"]
+        rec = {"workload": what, "points": n, "pd": pd, "vd": vd, "num_vertices": m,
+               "us_per_filter": round(seconds * 1e6, 1), "Mpoints_per_s": round(n / seconds / 1e6, 1),
+               "algorithmic_bytes_per_filter": alg,
+               "frac_of_hbm_peak": round(alg / seconds / 1e9 / HBM_PEAK_GBS, 5),
+               "merged_tiles": bool(lat.info(pla.PL_INFO_BUILD_MERGED)),
+               "dominant_kernel": dominant,
+               "stage_ms": {k: round(v, 5) for k, v in stages.items()}}
+        if with_cpu:
+            lat.filter(d_out, d_val, d_pos, False)
+            torch.cuda.synchronize()
+            got = d_out.cpu().numpy()
+            t0 = time.perf_counter()
+            want = oracle.Lattice(pd, vd, n).filter(val, pos, False)
+            rec["cpu_seconds_per_filter"] = round(time.perf_counter() - t0, 4)
+            rec.update(both(got, lambda g: parity(g, want),
+                            (lambda g: parity(g, cpu.filter(pd, vd, val, pos, False)[0])) if cpu else None))
+        lat.close()
+        out[name] = rec
+
+    # cfg1: 512 x 512 RGB bilateral
+    img = synth.blob_image(512, 512, seed=0xC0FFEE + 1)
+    one_filter("cfg1", "bilateral RGB 512x512, pd=5 vd=4, theta 8/0.125, one filter() forward", 5, 4,
+               (512, 512), synth.bilateral_positions(img, 8.0, 0.125), img.reshape(-1, 3), 20)
+    # cfg2: 1024 x 1024 spatial-only Gaussian
+    one_filter("cfg2", "spatial-only 1024x1024 grey, pd=2 vd=2, theta 8, one filter() forward", 2, 2,
+               (1024, 1024), synth.spatial_positions((1024, 1024), 8.0),
+               synth.uniform_image((1 << 20, 1), 0xC0FFEE + 2), 20)
+
+    # cfg3: batch 4 grey under an RGB guide, forward + reverse, through the op
+    batch, side = 4, 1024
+    guide = np.stack([synth.blob_image(side, side, seed=0xC0FFEE + 30 + i) for i in range(batch)])
+    inp = synth.uniform_image((batch, side, side, 1), 0xC0FFEE + 3)
+    grad = synth.normal_image((batch, side, side, 1), 0xC0FFEE + 4)
+    d_guide, d_inp, d_grad = dev(guide), dev(inp), dev(grad)
+    res = {}
+
+    def cfg3_step():
+        res["f"] = pla._lattice_filter_raw(d_inp, d_guide, True, 8.0, 0.125, 1.0, False)
+        res["r"] = pla._lattice_filter_raw(d_grad, d_guide, True, 8.0, 0.125, 1.0, True)
+
+    seconds = timed(cfg3_step, 2, 5)
+    n = side * side
+    lat = pla.PermutohedralLattice(5, 2, n)
+    d_out1 = torch.empty((n, 1), dtype=torch.float32, device="cuda")
+    call = lambda: lat.filter_image(d_out1, d_inp[0].view(n, 1), d_guide[0].view(n, 3), (side, side), 8.0, 0.125)
+    call()
+    m = lat.num_vertices
+    stages, dominant = stage_report(lat, call, n, 5, 2)
+    # the op builds its features inside the first kernel: the reference image is read, not positions
+    alg = 4 * n * (3 + 2) + m * (2 * 5 + 4 * 2 * (2 * 6 + 2))
+    rec = {"workload": "greyscale under an RGB guide, batch 4, 1024x1024, pd=5 vd=2, theta 8/0.125: the op "
+                       "forward on the input, then reverse on an N(0,1) upstream gradient (8 filters per step)",
+           "points": n * batch, "pd": 5, "vd": 2, "num_vertices_item0": m,
+           "ms_per_step": round(seconds * 1e3, 4), "us_per_filter": round(seconds * 1e6 / (2 * batch), 1),
+           "Mpoints_per_s": round(2 * batch * n / seconds / 1e6, 1),
+           "algorithmic_bytes_per_filter": alg,
+           "frac_of_hbm_peak": round(2 * batch * alg / seconds / 1e9 / HBM_PEAK_GBS, 5),
+           "dominant_kernel": dominant, "stage_ms": {k: round(v, 5) for k, v in stages.items()}}
+    lat.close()
+    if with_cpu:
+        cfg3_step()
+        torch.cuda.synchronize()
+        got_f, got_r = res["f"].cpu().numpy(), res["r"].cpu().numpy()
+
+        def against(op):
+            return {"forward": parity(got_f, op(inp, guide, True, 8.0, 0.125, 1.0, False)),
+                    "reverse": parity(got_r, op(grad, guide, True, 8.0, 0.125, 1.0, True))}
+
+        t0 = time.perf_counter()
+        rec["parity_vs_cpu"] = against(oracle.lattice_filter)
+        rec["cpu_seconds_per_step"] = round(time.perf_counter() - t0, 3)
+        if cpu is not None:
+            rec["against_reference_build_with_its_duplicate_vertices"] = against(cpu.lattice_filter)
+    out["cfg3"] = rec
+    del d_guide, d_inp, d_grad, res
+
+    # cfg4: 128 x 256 x 256 volume
+    vol = synth.ellipsoid_volume(128, 256, 256, seed=0xC0FFEE + 4)
+    one_filter("cfg4", "volumetric bilateral 128x256x256, pd=4 vd=2, theta 5/0.1, one filter() forward", 4, 2,
+               (128, 256, 256), synth.bilateral_positions(vol, 5.0, 0.1), vol.reshape(-1, 1), 3)
+    del vol
+
+    # cfg5: dense-CRF mean field, 512 x 512, batch 2, 21 classes, five iterations + reverse pass
+    batch, side, classes = 2, 512, 21
+    guide = np.stack([synth.blob_image(side, side, seed=0xC0FFEE + 50 + b) * 255.0
+                      for b in range(batch)]).astype(np.float32)
+    logits = synth.normal_image((batch, side, side, classes), 0xC0FFEE + 5)
+    upstream = synth.normal_image((batch, side, side, classes), 0xC0FFEE + 6)
+    d_guide, d_logits, d_up = dev(guide), dev(logits), dev(upstream)
+    mf = MeanField(d_guide, classes)
+    res = {}
+
+    def cfg5_step():
+        mf.rebuild(d_guide)                       # four builds: two lattices per item
+        res["q"] = mf.infer(d_logits, 5)          # 20 applies
+        res["rev"] = mf.reverse(d_up)             # 4 reversed applies
+
+    seconds = timed(cfg5_step, 2, 5)
+    n = side * side
+    calls = batch * 2 * 6
+    m_bi, m_sp = mf.bilateral[0].num_vertices, mf.spatial[0].num_vertices
+    q0 = torch.softmax(d_logits[0].view(n, classes), dim=-1)
+    msg = torch.empty_like(q0)
+    st_bi, dom_bi = stage_report(mf.bilateral[0], lambda: mf.bilateral[0].apply(msg, q0, False), n, 5,
+                                 classes + 1, fused_splat=False)
+    st_sp, dom_sp = stage_report(mf.spatial[0], lambda: mf.spatial[0].apply(msg, q0, False), n, 2,
+                                 classes + 1, fused_splat=False)
+    # an apply moves what a filter moves less the positions and the keys (the lattice is there)
+    def apply_bytes(m, pd, vd):
+        return 4 * n * 2 * (vd - 1) + m * 4 * vd * (2 * (pd + 1) + 2)
+    alg = batch * 6 * (apply_bytes(m_bi, 5, classes + 1) + apply_bytes(m_sp, 2, classes + 1))
+    rec = {"workload": "dense-CRF mean field, 512x512, batch 2, 21 classes (vd=22): five iterations of "
+                       "softmax(logits + bilateral(Q; 80, 13) + spatial(Q; 3)) and the reverse pass of both "
+                       "filters on an N(0,1) upstream; two lattices per item built once per step (4 builds), "
+                       "24 applies",
+           "points": n * batch, "num_vertices_item0": {"bilateral_pd5": m_bi, "spatial_pd2": m_sp},
+           "ms_per_step": round(seconds * 1e3, 4), "filter_calls_per_step": calls,
+           "us_per_filter": round(seconds * 1e6 / calls, 1),
+           "Mpoints_per_s": round(calls * n / seconds / 1e6, 1),
+           "algorithmic_bytes_per_step": alg,
+           "frac_of_hbm_peak": round(alg / seconds / 1e9 / HBM_PEAK_GBS, 5),
+           "dominant_kernel": {"bilateral_apply": dom_bi, "spatial_apply": dom_sp},
+           "stage_ms": {"bilateral_apply": {k: round(v, 5) for k, v in st_bi.items()},
+                        "spatial_apply": {k: round(v, 5) for k, v in st_sp.items()}}}
+    if with_cpu:
+        cfg5_step()
+        torch.cuda.synchronize()
+        got_q, got_rev = res["q"].cpu().numpy(), res["rev"].cpu().numpy()
+
+        def against(op):
+            want_q, want_rev = oracle.mean_field(logits, guide, 5, upstream=upstream, op=op)
+            return {"Q": parity(got_q, want_q), "reverse": parity(got_rev, want_rev)}
+
+        t0 = time.perf_counter()
+        rec["parity_vs_cpu"] = against(None)
+        rec["cpu_seconds_per_step"] = round(time.perf_counter() - t0, 3)
+        if cpu is not None:
+            rec["against_reference_build_with_its_duplicate_vertices"] = against(cpu.lattice_filter)
+    mf.close()
+    out["cfg5"] = rec
+    return out
+
+
+def run_real_image(args, pla, with_cpu):
+    """The reference's own 800 x 1200 photograph (Images/input.bmp of the reference tree, kept as a
+    test fixture), theta 8/0.125 as its tests filter it: what an image that is not smooth costs and
+    whether the build that merges tiles in LDS holds on it."""
+    import numpy as np
+    import torch
+    path = os.path.join(ROOT, "tests", "golden", "reference_images.npz")
+    if not os.path.exists(path):
         return None
-    return int(sum(table[key]))
+    rgb = (np.load(path)["input"].astype(np.float32) / np.float32(255.0))
+    h, w = rgb.shape[:2]
+    n = h * w
+    d_img = torch.from_numpy(np.ascontiguousarray(rgb.reshape(n, 3))).cuda()
+    d_out = torch.empty_like(d_img)
+    lat = pla.PermutohedralLattice(5, 4, n)
+    call = lambda: lat.filter_image(d_out, d_img, d_img, (h, w), 8.0, 0.125, False)
+    seconds = timed(call, 3, 20)
+    m = lat.num_vertices
+    stages, dominant = stage_report(lat, call, n, 5, 4)
+    alg = 4 * n * (3 + 2 * 3) + m * (2 * 5 + 4 * 4 * (2 * 6 + 2))
+    rec = {"workload": "the reference's 800x1200 photograph under itself, pd=5 vd=4, theta 8/0.125, "
+                       "filter_image() forward", "points": n, "num_vertices": m,
+           "us_per_filter": round(seconds * 1e6, 1), "Mpoints_per_s": round(n / seconds / 1e6, 1),
+           "merged_tiles": bool(lat.info(pla.PL_INFO_BUILD_MERGED)),
+           "algorithmic_bytes_per_filter": alg,
+           "frac_of_hbm_peak": round(alg / seconds / 1e9 / HBM_PEAK_GBS, 5),
+           "dominant_kernel": dominant, "stage_ms": {k: round(v, 5) for k, v in stages.items()}}
+    if with_cpu:
+        import oracle
+        cpu = oracle.reference()
+        call()
+        torch.cuda.synchronize()
+        got = d_out.cpu().numpy().reshape((1,) + rgb.shape)
+        rec["parity_vs_cpu"] = parity(got, oracle.lattice_filter(rgb[None], rgb[None], True, 8.0, 0.125, 1.0, False))
+        if cpu is not None:
+            rec["against_reference_build_with_its_duplicate_vertices"] = parity(
+                got, cpu.lattice_filter(rgb[None], rgb[None], True, 8.0, 0.125, 1.0, False))
+    lat.close()
+    return rec
+
 
 
 def run_side_legs(args, pla, synth, lat, step, img, d_pos, d_val, d_grad, out_f, out_r, side, batch):
@@ -174,6 +477,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--size", type=int, default=1024, help="image side (default 1024)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and parity legs")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="skip the leg that runs every BASELINE configuration at full size")
     ap.add_argument("--headline-only", action="store_true",
                     help="only the timed steps and the per-stage timing (what a rocprofv3 run of "
                          "this file should see): no side legs, no CPU baseline")
@@ -266,9 +571,10 @@ def main():
     achieved = alg[dominant] / (per_launch_ms[dominant] * 1e-3) / 1e9
     kernel_name = {"build": "k_build_tile<5, 4, float>" if fused else "k_build_tile<5, 0, float>", "splat": "k_splat_dpp<4, 6>",
                    "blur_axis": "k_blur2_row<4, float>", "slice": "k_slice_point<4, 6>"}[dominant]
+    traffic, traffic_stamp = measured_traffic(kernel_name, n)
     roofline = {"bound": "hbm", "kernel": kernel_name, "achieved": round(achieved, 2),
                 "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 5),
-                "traffic": measured_traffic(kernel_name, side),
+                "traffic": traffic, "traffic_from": traffic_stamp,
                 "algorithmic_bytes_per_launch": alg[dominant],
                 "launch_ms": round(per_launch_ms[dominant], 5)}
     gpu_kernel_ms = sum(stages[k] for k in ("clear", "build", "ids", "neighbours", "fill", "splat",
@@ -317,6 +623,10 @@ def main():
                        "value": round(pixels_per_step / (double_ms * 1e-3) / 1e6, 3)},
         })
 
+    if side_legs and not args.no_configs:
+        result["configs"] = run_configs(args, pla, synth, not args.no_cpu)
+        result["real_image"] = run_real_image(args, pla, not args.no_cpu)
+
     if not args.no_cpu and not args.headline_only:
         import oracle
         ref = oracle.reference()
@@ -345,12 +655,13 @@ def main():
         lat.filter(out_f, d_val, d_pos, False)
         lat.filter(out_r, d_grad, d_pos, True)
         torch.cuda.synchronize()
-        parity = {}
-        for name, got, want in (("forward", out_f.cpu().numpy(), outs[0]),
-                                ("reverse", out_r.cpu().numpy(), outs[1])):
-            parity[name] = {"max_abs": float(np.abs(got - want).max()),
-                            "rel_l2": float(np.linalg.norm(got - want) / np.linalg.norm(want))}
-        result["parity_vs_cpu"] = parity
+        got_f, got_r = out_f.cpu().numpy(), out_r.cpu().numpy()
+        result["parity_vs_cpu"] = {
+            "forward": parity(got_f, oracle.Lattice(pd, vd, n).filter(val, pos, False)),
+            "reverse": parity(got_r, oracle.Lattice(pd, vd, n).filter(grad, pos, True))}
+        if ref is not None:
+            result["against_reference_build_with_its_duplicate_vertices"] = {
+                "forward": parity(got_f, outs[0]), "reverse": parity(got_r, outs[1])}
 
     print(json.dumps(result))
 

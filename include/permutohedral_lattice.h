@@ -152,6 +152,16 @@ int pl_num_vertices(pl_handle h, int *num_vertices);
 
 int pl_set_option(pl_handle h, int option, long value);
 
+/* What the handle's last build did (for benchmarks and tests): */
+typedef enum pl_info {
+    PL_INFO_BUILD_MERGED = 1,  /* 1 when the last build merged its tiles' keys in LDS (PL_OPT_MERGE_TILES), 0
+                                  when every wavefront went to the table itself (no grid, or a tile with
+                                  too many distinct keys switched merging off for a while) */
+    PL_INFO_TABLE_CELLS = 2,   /* hash cells the last build used */
+    PL_INFO_SCRATCH_BYTES = 3  /* device memory the handle holds for its tables and per-point rows */
+} pl_info;
+int pl_get_info(pl_handle h, int what, long *value);
+
 /* Milliseconds of the kernels of the last pl_build and pl_apply (or pl_filter) with
  * PL_OPT_PROFILE on, from HIP events on the lattice's stream: ms[0] table clear, ms[1] build
  * (embed + simplex + hash insertion), ms[2] vertex numbering, ms[3] neighbour table, ms[4] value

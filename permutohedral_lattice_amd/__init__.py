@@ -25,11 +25,12 @@ PL_OPT_NORMALIZE, PL_OPT_PROFILE, PL_OPT_TABLE_CELLS, PL_OPT_XCD_AWARE, PL_OPT_P
 PL_OPT_GUESS_GRID = 6
 PL_OPT_MERGE_TILES = 7
 PL_OPT_STOP_AFTER = 8
+PL_INFO_BUILD_MERGED, PL_INFO_TABLE_CELLS, PL_INFO_SCRATCH_BYTES = 1, 2, 3
 
 # every symbol include/permutohedral_lattice.h declares
 EXPORTS = (
     "pl_supported", "pl_strerror", "pl_last_hip_error", "pl_create", "pl_destroy", "pl_filter",
-    "pl_filter_static", "pl_build", "pl_apply", "pl_set_point_grid", "pl_get_point_grid", "pl_num_vertices", "pl_set_option", "pl_stage_ms", "pl_debug_simplex",
+    "pl_filter_static", "pl_build", "pl_apply", "pl_set_point_grid", "pl_get_point_grid", "pl_num_vertices", "pl_set_option", "pl_get_info", "pl_stage_ms", "pl_debug_simplex",
     "pl_debug_keys", "pl_debug_values", "pl_debug_replay", "pl_compute_positions", "pl_filter_image", "pl_build_image",
     "pl_filter_begin", "pl_filter_image_begin", "pl_filter_end", "pl_lattice_filter_op",
     "pl_set_op_concurrency",
@@ -71,6 +72,7 @@ def _load():
     lib.pl_get_point_grid.argtypes = [vp, C.POINTER(ci), C.POINTER(ci)]
     lib.pl_num_vertices.argtypes = [vp, C.POINTER(ci)]
     lib.pl_set_option.argtypes = [vp, ci, C.c_long]
+    lib.pl_get_info.argtypes = [vp, ci, C.POINTER(C.c_long)]
     lib.pl_stage_ms.argtypes = [vp, C.POINTER(cf)]
     lib.pl_debug_simplex.argtypes = [vp, vp, vp, vp, vp, vp]
     lib.pl_debug_keys.argtypes = [vp, vp]
@@ -251,6 +253,11 @@ class PermutohedralLattice:
         _check(_lib.pl_set_option(self._h, option, int(value)), "pl_set_option")
         if option == PL_OPT_NORMALIZE:
             self._normalize = bool(value)
+
+    def info(self, what):
+        v = C.c_long()
+        _check(_lib.pl_get_info(self._h, int(what), C.byref(v)), "pl_get_info")
+        return v.value
 
     def stage_ms(self):
         ms = (C.c_float * 8)()

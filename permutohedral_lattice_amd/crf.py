@@ -24,25 +24,32 @@ class MeanField:
     def __init__(self, guide, n_classes, theta_alpha=80.0, theta_beta=13.0, theta_gamma=3.0):
         if guide.dim() < 3:
             raise ValueError("guide must be [batch, spatial..., channels]")
-        self.guide = guide.contiguous()
         self.batch = int(guide.shape[0])
         self.sdims = [int(s) for s in guide.shape[1:-1]]
         self.n = 1
         for s in self.sdims:
             self.n *= s
         self.n_classes = int(n_classes)
+        self.thetas = (float(theta_alpha), float(theta_beta), float(theta_gamma))
         rc, k = int(guide.shape[-1]), len(self.sdims)
-        self.bilateral, self.spatial = [], []
-        for b in range(self.batch):
-            bi = PermutohedralLattice(k + rc, self.n_classes + 1, self.n)
-            bi.build_image(self.guide[b].reshape(self.n, rc), self.sdims, theta_alpha, theta_beta)
-            sp = PermutohedralLattice(k, self.n_classes + 1, self.n)
-            sp.build_image(None, self.sdims, theta_gamma)
-            self.bilateral.append(bi)
-            self.spatial.append(sp)
+        self.bilateral = [PermutohedralLattice(k + rc, self.n_classes + 1, self.n)
+                          for _ in range(self.batch)]
+        self.spatial = [PermutohedralLattice(k, self.n_classes + 1, self.n)
+                        for _ in range(self.batch)]
         shape = (self.batch, self.n, self.n_classes)
         self._msg_bi = torch.empty(shape, dtype=torch.float32, device=guide.device)
         self._msg_sp = torch.empty(shape, dtype=torch.float32, device=guide.device)
+        self.rebuild(guide)
+
+    def rebuild(self, guide):
+        """Build the lattices again for another batch of guide images of the same shape."""
+        self.guide = guide.contiguous()
+        rc = int(guide.shape[-1])
+        theta_alpha, theta_beta, theta_gamma = self.thetas
+        for b in range(self.batch):
+            self.bilateral[b].build_image(self.guide[b].reshape(self.n, rc), self.sdims,
+                                          theta_alpha, theta_beta)
+            self.spatial[b].build_image(None, self.sdims, theta_gamma)
 
     def messages(self, q, reverse=False):
         """bilateral(q) + spatial(q) for ``q [B, ..., n_classes]`` (any spatial shape of N points)."""

@@ -979,6 +979,26 @@ int pl_num_vertices(pl_handle h, int *num_vertices) {
     return PL_OK;
 }
 
+int pl_get_info(pl_handle h, int what, long *value) {
+    if (!h || !value) return PL_EINVAL;
+    switch (what) {
+        case PL_INFO_BUILD_MERGED: *value = h->last_build_merged ? 1 : 0; return PL_OK;
+        case PL_INFO_TABLE_CELLS: *value = (long)h->n_cells; return PL_OK;
+        case PL_INFO_SCRATCH_BYTES: {
+            const size_t mv = plk::max_vertices_for(h->n_cells_alloc);
+            size_t b = (size_t)h->n_cells_alloc * (sizeof(uint64_t) + sizeof(int)) +
+                       mv * (sizeof(uint64_t) + sizeof(int) + 2 * h->value_size() * h->vd +
+                             sizeof(int2) * (size_t)(h->pd + 1));
+            if (h->cell_values) b += h->value_size() * (size_t)h->n_cells_alloc * h->vd;
+            b += h->replay_capacity * (sizeof(plk::ReplayEntry) + sizeof(uint4) +
+                                       (h->f64 ? sizeof(double) : 0));
+            *value = (long)b;
+            return PL_OK;
+        }
+        default: return PL_EINVAL;
+    }
+}
+
 int pl_stage_ms(pl_handle h, float ms[8]) {
     if (!h || !ms) return PL_EINVAL;
     if (!h->profile) return PL_ESTATE;
