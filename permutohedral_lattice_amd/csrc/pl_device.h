@@ -42,7 +42,9 @@ struct KeyCodec {
     static constexpr int kMaxQ = kBias - 2;
     static constexpr uint64_t kFieldMask = (1ull << kBits) - 1ull;
 
-    __device__ static uint64_t pack(const int (&q)[PD], int r) {
+    template <int N>
+    __device__ static uint64_t pack(const int (&q)[N], int r) {
+        static_assert(N >= PD, "one q per stored coordinate");
         uint64_t k = (uint64_t)(uint32_t)r << 60;
 #pragma unroll
         for (int i = 0; i < PD; ++i) k |= (uint64_t)(uint32_t)(q[i] + kBias) << (i * kBits);
@@ -316,6 +318,31 @@ template <int PD, typename T>
 __device__ __forceinline__ void vertex_q(const Simplex<PD, T> &s, int r, int (&q)[PD]) {
 #pragma unroll
     for (int i = 0; i < PD; ++i) q[i] = s.q[i] - ((s.rank[i] > PD - r) ? 1 : 0);
+}
+
+// The packed keys of all pd+1 vertices of a simplex.  From vertex r-1 to vertex r exactly one
+// coordinate drops by one step, the one of rank pd-r+1 (the ranks are a permutation of 0..pd), so
+// a key follows from the one before it: its field of that coordinate (if it is one of the pd that
+// are stored) one lower, its remainder one higher.  No field can borrow from the next: a simplex
+// in key range has every biased field at least 1 after the step (simplex_in_key_range).  Same
+// bits as KeyCodec<PD>::pack(vertex_q(s, r), r).
+template <int PD, typename T>
+__device__ __forceinline__ void vertex_keys_of(const Simplex<PD, T> &s, uint64_t (&key)[PD + 1]) {
+    constexpr int kBits = KeyCodec<PD>::kBits;
+    key[0] = KeyCodec<PD>::pack(s.q, 0);
+#pragma unroll
+    for (int r = 1; r <= PD; ++r) {
+        uint32_t step_lo = 0, step_hi = 0;
+#pragma unroll
+        for (int i = 0; i < PD; ++i) {
+            const bool drops = s.rank[i] == PD - r + 1;
+            if (i * kBits < 32)
+                step_lo = drops ? (1u << ((i * kBits) & 31)) : step_lo;
+            else
+                step_hi = drops ? (1u << ((i * kBits - 32) & 31)) : step_hi;
+        }
+        key[r] = key[r - 1] - (((uint64_t)step_hi << 32) | step_lo) + (1ull << 60);
+    }
 }
 
 template <int PD, typename T>

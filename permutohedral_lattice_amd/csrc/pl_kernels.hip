@@ -222,13 +222,10 @@ __global__ __launch_bounds__(kBlock) void k_build(PointFeatures features, PointM
     // wavefronts a CU holds)
     unsigned leaders[(D1 + 4) / 5] = {};
     auto leader_of = [&](int r) { return (int)((leaders[r / 5] >> (6 * (r % 5))) & 63u); };
+    vertex_keys_of<PD>(s, key);
 #pragma unroll
-    for (int r = 0; r < D1; ++r) {
-        int q[PD];
-        vertex_q<PD>(s, r, q);
-        key[r] = KeyCodec<PD>::pack(q, r);
+    for (int r = 0; r < D1; ++r)
         leaders[r / 5] |= (unsigned)wave_leader_of_equal(key[r], active, lane) << (6 * (r % 5));
-    }
 
     // Insertion of a lane's pd+1 keys proceeds in rounds over all of them at once, so that the
     // loads and compare-and-swaps of one round are in flight together: a round loads the current
@@ -421,11 +418,9 @@ __global__ __launch_bounds__(kBlock) void k_build_tile(PointFeatures features, P
     {
         uint64_t key[D1];
         unsigned open = 0;
+        vertex_keys_of<PD>(s, key);
 #pragma unroll
         for (int r = 0; r < D1; ++r) {
-            int q[PD];
-            vertex_q<PD>(s, r, q);
-            key[r] = KeyCodec<PD>::pack(q, r);
             const int leader = wave_leader_of_equal(key[r], active, lane, kSmallGroup, small[r]);
             leaders[r / 5] |= (unsigned)leader << (6 * (r % 5));
             if (active && leader == lane) open |= 1u << r;
@@ -644,14 +639,27 @@ __global__ __launch_bounds__(64) void k_number_vertices(CreatedLists lists, int 
     const unsigned b = xcd_contiguous_block(blockIdx.x, gridDim.x, 1);
     const int lane = threadIdx.x;
     const unsigned chunk = b / kBlocksPerChunk;
-    // vertices of the workgroups before this one: whole chunks, then the rest one by one
-    int before = 0;
-    for (unsigned i = lane; i < chunk; i += 64) before += lists.chunk_count[i];
+    const size_t list = (size_t)b * (kBlock * D1);
+    // Everything the pass reads that does not depend on something else it reads is asked for at
+    // once, without branches (an index out of range reads element 0 and is dropped afterwards):
+    // the sums of the chunks before this workgroup's, the counts of the workgroups before it in
+    // its chunk, its own count, and the first 64 entries of its list whether it has that many or
+    // not (the list's memory is there).  With a load behind each condition the pass waited for
+    // five memory round trips in a row; now for two, the entries and then their rows of sums.
     static_assert(kBlocksPerChunk == 64, "one lane per workgroup of the chunk");
-    if (chunk * kBlocksPerChunk + lane < b) before += lists.block_count[chunk * kBlocksPerChunk + lane];
+    const bool has_chunk = (unsigned)lane < chunk;
+    int before = lists.chunk_count[has_chunk ? lane : 0];
+    const unsigned sibling = chunk * kBlocksPerChunk + lane;
+    int sibling_count = lists.block_count[sibling < b ? sibling : b];
+    const int count = lists.block_count[b];
+    uint4 first_entry = lists.entries[list + lane];
+    asm volatile("" : "+v"(before), "+v"(sibling_count), "+v"(first_entry.x), "+v"(first_entry.y),
+                 "+v"(first_entry.z));
+    before = has_chunk ? before : 0;
+    for (unsigned i = lane + 64; i < chunk; i += 64) before += lists.chunk_count[i];
+    before += sibling < b ? sibling_count : 0;
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) before += __shfl_xor(before, off);
-    const int count = lists.block_count[b];
     const int max_vertices = vertices.max_vertices;
 
     if (b == gridDim.x - 1) {
@@ -666,9 +674,8 @@ __global__ __launch_bounds__(64) void k_number_vertices(CreatedLists lists, int 
         for (unsigned i = lane; i < n_chunks; i += 64) next_chunk_count[i] = 0;
     }
 
-    const size_t list = (size_t)b * (kBlock * D1);
     for (int i = lane; i < count; i += 64) {
-        const uint4 entry = lists.entries[list + i];
+        const uint4 entry = i < 64 ? first_entry : lists.entries[list + i];
         const int cell = (int)entry.z;
         const int v = before + i;
         if (v < max_vertices) {
