@@ -99,7 +99,7 @@ struct pl_lattice {
     plk::ReplayEntry *replay = nullptr;
     // what each workgroup of the build created (see plk::CreatedLists); the chunk counts exist
     // twice and alternate between builds like the counters
-    uint4 *created_entries = nullptr;      // [n_blocks*256*(pd+1)]
+    uint4 *created_entries = nullptr;      // [n_blocks * list_stride()]
     int *block_count = nullptr;            // [n_blocks]
     int *chunk_count = nullptr;            // [2][n_chunks]
     size_t n_chunks = 0;
@@ -115,6 +115,15 @@ struct pl_lattice {
 
     int M = 0;
     int last_M = -1;
+    // how the last build numbered its vertices (plk::Counters): segments, and the fullest one
+    int n_segments = 0, max_segment = 0;
+    int last_n_segments = 0, last_max_segment = -1;
+    bool one_segment = false;          // the last build overflowed a segment of the largest table
+    // A merging build numbers its vertices itself unless that costs more than it saves: when it
+    // has many thousands of workgroups (they draw their numbers one after the other), or when
+    // the last such build of these points held so many rows of sums for vertices of other
+    // workgroups that adding them afterwards, an atomic each, outweighs the numbering pass.
+    bool numbering_pass_pays = false;
     bool built = false;                // a build has been enqueued and, if verified, fitted
     bool verified = false;             // its status has been read on the host
     bool replay_holds_cells = false;
@@ -166,12 +175,26 @@ struct pl_lattice {
     int max_vertices() const { return (int)plk::max_vertices_for(n_cells); }
     // what the grids of the kernels over the vertices are sized for: the count when the host
     // knows it, else the previous build's with a margin (the kernels cover any count)
+    // (every XCD walks the segments of its eighth of the image, or its eighth of the numbers:
+    // segments as full as the fullest, each with a block that is partly used, cover them all)
     int launch_vertices() const {
         const int mv = max_vertices();
-        if (built && verified) return M < mv ? M : mv;
+        auto walked = [](long long m, int segments, long long fullest) {
+            return (segments > 1 ? segments * fullest : m) + 256ll * (segments > 8 ? segments : 8);
+        };
+        if (built && verified) {
+            const long long m = walked(M, n_segments, max_segment);
+            return m < mv ? (int)m : mv;
+        }
         if (last_M <= 0) return mv;
-        const long long guess = (long long)last_M + last_M / 8 + 1024;
+        const long long last = walked(last_M, last_n_segments, last_max_segment);
+        const long long guess = last + last / 8 + 1024;
         return guess < mv ? (int)guess : mv;
+    }
+    int list_stride() const { return plk::created_list_stride(pd, f64); }
+    plk::CreatedLists lists(int set) const {
+        return plk::CreatedLists{created_entries, block_count, chunk_count + (size_t)set * n_chunks,
+                                 list_stride()};
     }
 };
 
@@ -222,7 +245,8 @@ int ensure_replay(pl_lattice *h) {
     h->replay_capacity = 0;
     h->n_chunks = (h->map.n_blocks + plk::kBlocksPerChunk - 1) / plk::kBlocksPerChunk + 1;
     h->replay = (plk::ReplayEntry *)h->dmalloc(sizeof(plk::ReplayEntry) * (want ? want : 1));
-    h->created_entries = (uint4 *)h->dmalloc(sizeof(uint4) * (want ? want : 1));
+    const size_t entries = (size_t)h->map.n_blocks * (size_t)h->list_stride();
+    h->created_entries = (uint4 *)h->dmalloc(sizeof(uint4) * (entries ? entries : 1));
     h->block_count = (int *)h->dmalloc(sizeof(int) * (h->map.n_blocks ? h->map.n_blocks : 1));
     h->chunk_count = (int *)h->dmalloc(sizeof(int) * 2 * h->n_chunks);
     if (h->f64) h->weights64 = (double *)h->dmalloc(sizeof(double) * (want ? want : 1));
@@ -271,8 +295,13 @@ int enqueue_build(pl_lattice *h, const plk::PointFeatures &features, const doubl
     h->last_build_merged = merge;
     // (a lattice of doubles splats in its build only in the merging kernel)
     const bool fused = splat_input && plk::build_can_splat(h->vd) && (!h->f64 || merge);
+    // (a build for one filter: a lattice built to be applied many times is numbered by the
+    // numbering pass, in the order of the image tiles, which the passes over the vertices walk
+    // a few per cent faster than the order in which the workgroups happened to finish)
+    const bool numbers_in_build =
+        merge && fused && h->map.n_blocks <= 8192u && !h->numbering_pass_pays;
     const size_t floats_per_value = h->f64 ? 2 : 1;
-    if (fused && !h->cell_values_clean) {
+    if (fused && !numbers_in_build && !h->cell_values_clean) {
         PL_HIP(plk::fill_zero(h->cell_values, (size_t)h->n_cells_alloc * h->vd * floats_per_value,
                               h->stream));
         h->cell_values_clean = true;
@@ -289,8 +318,13 @@ int enqueue_build(pl_lattice *h, const plk::PointFeatures &features, const doubl
     h->counter_set = 1 - previous_set;
     const plk::VertexTables vertices{h->cell_vertex, h->vertex_keys, h->vertex_cell, h->neighbours,
                                      h->max_vertices()};
-    const plk::CreatedLists lists{h->created_entries, h->block_count,
-                                  h->chunk_count + (size_t)h->counter_set * h->n_chunks};
+    const plk::CreatedLists lists = h->lists(h->counter_set);
+    // the merging build numbers its vertices itself and reports to the host
+    const plk::InBuildNumbering numbering{
+        h->cell_vertex, h->vertex_keys, h->vertex_cell, h->neighbours, h->max_vertices(),
+        h->values[0], h->f64 ? 2 * h->vd : h->vd,
+        !numbers_in_build ? 0 : (h->one_segment ? 1 : plk::segments_for((uint32_t)h->max_vertices()))};
+    h->one_segment = false;
     // keys go to the part of the table that belongs to their band of rows when the points are
     // known to be a grid (and feature 0 then runs with its slowest extent)
     plk::RegionSource regions{};
@@ -311,7 +345,8 @@ int enqueue_build(pl_lattice *h, const plk::PointFeatures &features, const doubl
     if (h->f64) {
         const plk::Points64 points{positions64, h->weights64, h->scale64};
         PL_HIP(plk::build_f64(h->pd, points, h->map, h->cell_keys, cells, h->counters(), h->replay,
-                              h->xcd_aware ? 1 : 0, lists, regions, merge, fused ? h->vd : 0,
+                              h->xcd_aware ? 1 : 0, lists, regions, merge ? &numbering : nullptr,
+                              fused ? h->vd : 0,
                               static_cast<const double *>(splat_input),
                               h->normalize ? h->vd - 1 : h->vd,
                               reinterpret_cast<double *>(h->cell_values), h->stream));
@@ -320,20 +355,28 @@ int enqueue_build(pl_lattice *h, const plk::PointFeatures &features, const doubl
                           h->replay, h->xcd_aware ? 1 : 0, fused ? h->vd : 0,
                           static_cast<const float *>(splat_input),
                           h->normalize ? h->vd - 1 : h->vd, h->cell_values, lists,
-                          regions, merge, h->stream));
+                          regions, merge ? &numbering : nullptr, h->stream));
     }
     h->mark(EV_BUILD);
-    // the numbering pass zeroes the vertices' value rows: a row of vd doubles is 2*vd zero floats
-    PL_HIP(plk::number_vertices(h->pd, h->map, lists,
-                                h->chunk_count + (size_t)previous_set * h->n_chunks,
-                                (unsigned)h->n_chunks, vertices,
-                                h->values[0], h->f64 ? 2 * h->vd : h->vd,
-                                fused ? h->cell_values : nullptr, h->counters(),
-                                h->d_counters + previous_set, h->h_status, h->stream));
-    if (!h->status_on_device) PL_HIP(hipEventRecord(h->status_written, h->stream));
+    if (!numbers_in_build) {
+        // the numbering pass zeroes the vertices' value rows: a row of vd doubles is 2*vd zero floats
+        PL_HIP(plk::number_vertices(h->pd, h->map, lists,
+                                    h->chunk_count + (size_t)previous_set * h->n_chunks,
+                                    (unsigned)h->n_chunks, vertices,
+                                    h->values[0], h->f64 ? 2 * h->vd : h->vd,
+                                    fused ? h->cell_values : nullptr, h->counters(),
+                                    h->d_counters + previous_set, h->h_status, h->stream));
+    }
+    if (!numbers_in_build && !h->status_on_device) PL_HIP(hipEventRecord(h->status_written, h->stream));
     h->mark(EV_IDS);
+    // (the rows a build that numbered its vertices listed for vertices of other workgroups join
+    // the value table here, and its counts reach the host from here)
     PL_HIP(plk::neighbours(h->pd, vertices, h->counters(), h->cell_keys, cells,
-                           h->launch_vertices(), h->stream));
+                           h->launch_vertices(), numbers_in_build && fused ? &lists : nullptr,
+                           h->map.n_blocks, h->values[0], h->vd, h->f64,
+                           numbers_in_build ? h->counters() : nullptr,
+                           h->d_counters + previous_set, h->h_status, h->stream));
+    if (numbers_in_build && !h->status_on_device) PL_HIP(hipEventRecord(h->status_written, h->stream));
     h->mark(EV_NBR);
     h->replay_holds_cells = true;
     h->values_zeroed = !fused;
@@ -493,6 +536,8 @@ int verify_build(pl_lattice *h, uint32_t *retry_cells) {
     }
     const int flags = status.flags;
     const int m = status.num_vertices;
+    h->last_n_segments = status.n_segments;
+    h->last_max_segment = status.max_segment;
     if (flags & plk::kFlagKeyRange) {
         // (the build may also have overflowed the table, and then rows of sums of the vertices
         // beyond its capacity are still where the fused splat put them)
@@ -516,12 +561,28 @@ int verify_build(pl_lattice *h, uint32_t *retry_cells) {
         h->built = false;
         h->table_clean = false;  // keys beyond the numbered vertices may remain
         h->cell_values_clean = false;
-        if (h->n_cells >= h->max_cells) return PL_EOVERFLOW;  // cannot happen: max_cells holds every vertex
+        if (h->n_cells >= h->max_cells) {
+            // the largest table holds every vertex, but a segment of it may not hold all that
+            // one part of the image creates: once more with the numbers in one run
+            if (status.n_segments <= 1 || (uint32_t)m > plk::max_vertices_for(h->n_cells))
+                return PL_EOVERFLOW;   // (cannot happen)
+            h->one_segment = true;
+            *retry_cells = h->n_cells;
+            return PL_EOVERFLOW;
+        }
         *retry_cells = (h->n_cells > h->max_cells / 4) ? h->max_cells : h->n_cells * 4;
         return PL_EOVERFLOW;
     }
     h->M = m;
     h->last_M = m;
+    h->n_segments = status.n_segments;
+    h->max_segment = status.max_segment;
+    // (in ns, as measured on 1024x1024 and 512x512 images: a row added afterwards takes 0.03 of
+    // the atomic unit's time; the numbering pass 1.5 per workgroup of the build and 0.02 per
+    // vertex, and the build 1500 longer with all its rows going out as atomics)
+    if (status.n_segments != 0 &&
+        0.03 * status.foreign_rows > 1.5 * h->map.n_blocks + 0.02 * m + 1500.0)
+        h->numbering_pass_pays = true;
     h->verified = true;
     if (h->last_build_merged) h->tiles_backoff = 32;
     return PL_OK;
@@ -696,6 +757,7 @@ int pl_set_point_grid(pl_handle h, int n_dims, const int *dims) {
     h->built = false;
     h->grid_given = n_dims > 0;
     h->map = plk::make_point_map(h->N, n_dims, dims);
+    h->numbering_pass_pays = false;
     return ensure_replay(h);
 }
 
@@ -754,6 +816,7 @@ int guess_point_grid(pl_lattice *h, const float *positions) {
     }
     if (dims[0] < 2) return PL_OK;
     h->map = plk::make_point_map(h->N, n_dims, dims);
+    h->numbering_pass_pays = false;
     return ensure_replay(h);
 }
 
@@ -1023,10 +1086,30 @@ int pl_debug_simplex(pl_handle h, const float *positions, short *rem0, short *ra
     return PL_OK;
 }
 
+// The debug exports count the vertices densely, whatever numbers the build gave them: read how
+// many each segment holds (these calls are for tests; they wait for the stream).
+static int vertex_numbers(pl_lattice *h, plk::VertexNumbers *numbers) {
+    plk::Counters counters;
+    PL_HIP(hipMemcpyAsync(&counters, h->counters(), sizeof(counters), hipMemcpyDeviceToHost,
+                          h->stream));
+    PL_HIP(hipStreamSynchronize(h->stream));
+    numbers->n_segments = counters.n_segments;
+    numbers->stride = plk::segment_stride((uint32_t)h->max_vertices(), counters.n_segments);
+    numbers->before[0] = 0;
+    for (int k = 0; k < plk::kMaxSegments; ++k)
+        numbers->before[k + 1] =
+            numbers->before[k] + (k < counters.n_segments ? counters.segment_count[k].n : 0u);
+    numbers->total = counters.n_segments ? numbers->before[plk::kMaxSegments] : (unsigned)h->M;
+    return numbers->total == (unsigned)h->M ? PL_OK : PL_ESTATE;
+}
+
 int pl_debug_keys(pl_handle h, short *keys) {
     if (!h || !keys) return PL_EINVAL;
     if (!h->built || !h->verified) return PL_ESTATE;
-    PL_HIP(plk::export_keys(h->pd, h->vertex_keys, h->M, keys, h->stream));
+    plk::VertexNumbers numbers;
+    const int rc = vertex_numbers(h, &numbers);
+    if (rc != PL_OK) return rc;
+    PL_HIP(plk::export_keys(h->pd, h->vertex_keys, numbers, keys, h->stream));
     return PL_OK;
 }
 
@@ -1034,9 +1117,11 @@ int pl_debug_values(pl_handle h, void *values) {
     if (!h || !values) return PL_EINVAL;
     if (!h->built || !h->verified) return PL_ESTATE;
     if (h->M == 0) return PL_OK;
-    PL_HIP(hipMemcpyAsync(values, h->values[h->current_values],
-                          h->value_size() * (size_t)h->M * (size_t)h->vd, hipMemcpyDeviceToDevice,
-                          h->stream));
+    plk::VertexNumbers numbers;
+    const int rc = vertex_numbers(h, &numbers);
+    if (rc != PL_OK) return rc;
+    PL_HIP(plk::export_values(h->values[h->current_values], h->f64 ? 2 * h->vd : h->vd, numbers,
+                              static_cast<float *>(values), h->stream));
     return PL_OK;
 }
 
@@ -1044,9 +1129,12 @@ int pl_debug_replay(pl_handle h, int *vertex, float *weight) {
     if (!h) return PL_EINVAL;
     if (h->f64) return PL_EINVAL;   // a lattice of doubles: use the *_f64 entry points
     if (!h->built || !h->verified) return PL_ESTATE;
+    plk::VertexNumbers numbers;
+    const int rc = vertex_numbers(h, &numbers);
+    if (rc != PL_OK) return rc;
     PL_HIP(plk::export_replay(h->pd, h->map, h->replay,
-                              h->replay_holds_cells ? h->cell_vertex : nullptr, vertex, weight,
-                              h->stream));
+                              h->replay_holds_cells ? h->cell_vertex : nullptr, numbers, vertex,
+                              weight, h->stream));
     return PL_OK;
 }
 

@@ -440,36 +440,60 @@ __device__ __forceinline__ int wave_leader_of_equal(T x, bool active, int lane, 
         const uint64_t same = lanes_equal(x, lane_value(x, first)) & among;
         if (lane_in(same)) leader = first;
         remaining &= ~same;
-        if (__builtin_popcountll(same) <= small_size) small |= same;
+        if ((int)__builtin_popcountll(same) <= small_size) small |= same;
     }
     return leader;
 }
 
-__device__ __forceinline__ int vertex_count(const Counters *counters, int max_vertices) {
-    const uint32_t m = counters->vertices;
-    return m < (uint32_t)max_vertices ? (int)m : max_vertices;
+// What a build counts in, as the build after next must find it
+__device__ __forceinline__ void reset_counters(Counters *c) {
+    c->vertices = 0;
+    c->flags = 0;
+    for (int k = 0; k < kMaxSegments; ++k) c->segment_count[k].n = 0;   // (n_segments: set by every build)
+    c->foreign_rows_sampled.n = 0;
 }
 
-// The vertex count is only known on the device, so kernels over the vertices are launched for an
-// estimate (the count of the lattice's previous build, with a margin) and every workgroup walks
-// the blocks of 256 items in strides of the grid: a launch for the most vertices the table can
-// hold would spend more time dispatching empty workgroups than the passes spend working.
-// Workgroup b runs on XCD b % 8 and each XCD has its own L2, so the blocks are dealt out such
-// that every XCD gets one contiguous eighth of the items (the grid is a multiple of 8): with
-// vertex numbers that follow the image, the vertices a workgroup gathers from are then mostly
-// ones its own XCD works on.
-struct ItemBlocks {
-    unsigned n_active, chunk, k;
-    __device__ explicit ItemBlocks(size_t n_items)
-        : n_active((unsigned)((n_items + kBlock - 1) / kBlock)), chunk((n_active + 7u) / 8u),
-          k(blockIdx.x) {}
-    __device__ bool next(unsigned &block) {
-        while (k < 8u * chunk) {
-            block = (k & 7u) * chunk + (k >> 3);
-            k += gridDim.x;
-            if (block < n_active) return true;
+// The passes over the vertices.  The vertex counts are only known on the device, so these kernels
+// are launched for an estimate (the counts of the lattice's previous build, with a margin) and
+// every workgroup walks blocks of 256 items in strides: a launch for the most vertices the table
+// can hold would spend more time dispatching empty workgroups than the passes spend working.
+// Workgroup b runs on XCD b % 8 and each XCD has its own L2, so XCD x walks the vertices of the
+// eighth x of the image (the grid is a multiple of 8): the segments that XCD's workgroups
+// numbered, when the build numbered them (Counters::n_segments != 0); else the x-th eighth of
+// the numbers 0 .. vertices-1, which follow the image too.  What a workgroup gathers from is then
+// mostly what its own XCD works on.
+struct SegmentWalk {
+    unsigned first, count;     // the run of numbers this XCD walks
+    unsigned cursor, step;     // next block among the blocks of that run, stride
+    // grid_blocks: workgroups of the grid that walk (a multiple of 8), workgroup: index among them
+    __device__ SegmentWalk(const Counters *counters, int max_vertices, unsigned workgroup,
+                           unsigned grid_blocks) {
+        const unsigned xcd = workgroup % kXcds;
+        const Counters::PaddedCount mine = counters->segment_count[xcd];
+        if (mine.n_segments == (int)kXcds) {
+            const unsigned stride = segment_stride((uint32_t)max_vertices, mine.n_segments);
+            first = xcd * stride;
+            count = mine.n < stride ? mine.n : stride;
+        } else {
+            // (one run: after the numbering pass every line holds the total, after a build
+            // with one segment the first)
+            const unsigned all = mine.n_segments == 1 ? counters->segment_count[0].n : mine.n;
+            const unsigned m = all < (unsigned)max_vertices ? all : (unsigned)max_vertices;
+            const unsigned per_xcd = ((m + kBlock - 1) / kBlock + kXcds - 1) / kXcds * kBlock;
+            first = xcd * per_xcd;
+            count = m > first ? (m - first < per_xcd ? m - first : per_xcd) : 0u;
         }
-        return false;
+        cursor = workgroup / kXcds;
+        step = grid_blocks / kXcds;
+    }
+    // This workgroup's next block b of 256 items, a vertex being items_per_vertex items, in a
+    // pass that visits every block `visits` times
+    __device__ bool next(unsigned items_per_vertex, unsigned visits, unsigned &b) {
+        const unsigned n = (unsigned)(((size_t)count * items_per_vertex + kBlock - 1) / kBlock) * visits;
+        if (cursor >= n) return false;
+        b = cursor;
+        cursor += step;
+        return true;
     }
 };
 

@@ -19,21 +19,56 @@ enum : int {
     kFlagTileFull = 4,    // a workgroup of the merging build has more distinct keys than its LDS table holds
 };
 
-// Device-side state of one build.  Kernels after the numbering pass read the vertex count from
-// here, so the host never has to wait for it between launches.
+// Device-side state of one build.  Kernels after the build read the vertex counts from here, so
+// the host never has to wait for them between launches.
+//
+// Vertex numbers.  The merging build can number its vertices itself: a workgroup draws a run of
+// numbers for the vertices it created from the counter of its segment (one atomic per workgroup;
+// the segment is the eighth of the image the workgroup lies in, which one XCD builds and later
+// walks), and segment x owns the numbers from x * segment_stride(max_vertices, 8) on: eight dense
+// runs in the order in which the workgroups of an eighth got there, n_segments == 8.  A small
+// table has one segment.  An atomic on one address takes about 50 ns and the next one waits for
+// it, so this is for builds of a few thousand workgroups.  Otherwise the numbering is left to
+// number_vertices, which gives the numbers 0 .. vertices-1 (n_segments == 0).
+constexpr int kMaxSegments = 8;
 struct Counters {
-    unsigned int vertices;   // set by the numbering pass (may exceed what the table can hold)
+    unsigned int vertices;   // total (may exceed what the table can hold)
     int flags;
     // how the build spread its keys over the table (KeyRegions in pl_device.h), written by the
     // build for the passes that look keys up after it: they must not read the caller's positions
     // again, which only have to stay valid until the build has run
     float region_lo, region_per_unit;
+    int n_segments;
+    // (a counter per 128 bytes: atomics on one line queue up in one memory channel, whatever
+    // address in the line they name.  Each line also says how the vertices are numbered, and
+    // after the numbering pass every line holds the total: a pass over the vertices learns what
+    // its XCD walks from one line.)
+    struct alignas(128) PaddedCount {
+        unsigned int n;
+        int n_segments;
+    };
+    PaddedCount segment_count[kMaxSegments];
+    // rows of sums for vertices of other workgroups (CreatedLists), counted by every eighth
+    // workgroup of a build that numbers its vertices
+    PaddedCount foreign_rows_sampled;
 };
+constexpr unsigned kForeignSampling = 8;
+__host__ __device__ inline uint32_t segment_stride(uint32_t max_vertices, int n_segments) {
+    return max_vertices / (uint32_t)(n_segments > 0 ? n_segments : 1);
+}
+// Segments a merging build that numbers its vertices uses with a table for max_vertices: none
+// smaller than 2048 numbers (a workgroup can create 512 vertices).
+inline int segments_for(uint32_t max_vertices) {
+    return max_vertices / (uint32_t)kMaxSegments < 2048u ? 1 : kMaxSegments;
+}
 
-// What the numbering pass writes to pinned host memory about the build.
+// What the build (or the numbering pass) writes to pinned host memory about the build.
 struct HostStatus {
     int num_vertices;
     int flags;
+    int max_segment;   // vertices in the fullest segment (num_vertices when there are none)
+    int n_segments;
+    int foreign_rows;  // CreatedLists rows of a build that numbered its vertices (an estimate)
 };
 
 // Per-vertex and per-cell tables of a lattice (all sized by the hash table): vertex v has key
@@ -76,15 +111,44 @@ struct SpatialDims {
     int v[kMaxSpatialDims];
 };
 
-// What the build's workgroups created, for the numbering pass: workgroup b (in the build's
-// virtual order) lists its block_count[b] new vertices from entry b*256*(pd+1) on, one uint4
-// each: (key low word, key high word, hash cell, 0).  chunk_count[c] is the sum over the
-// kBlocksPerChunk workgroups of chunk c and must be zero before the build.
+// Per-workgroup lists, `stride` uint4 per workgroup of the build (in the build's virtual order).
+// A build that leaves the numbering to number_vertices lists what it created: workgroup b has
+// block_count[b] new vertices, one uint4 each: (key low word, key high word, hash cell, 0);
+// chunk_count[c] is the sum over the kBlocksPerChunk workgroups of chunk c and must be zero
+// before the build.
+// A merging build that numbers its vertices itself lists, when it splats, the rows of sums it
+// holds for vertices that another workgroup created (their numbers are not known yet):
+// block_count[b] of them, the rows (four values each) from the start of the workgroup's part and
+// their hash cells, as ints, behind kTileSlots rows.  neighbours() adds them to the value table.
 constexpr int kBlocksPerChunk = 64;
+constexpr int kTileSlots = 512;    // LDS slots of a workgroup of the merging build
 struct CreatedLists {
     uint4 *entries;
     int *block_count;
     int *chunk_count;
+    int stride;
+};
+// uint4 a workgroup's part must hold: its 256 * (pd+1) possible vertices, or kTileSlots rows of
+// four values and as many cells
+inline int created_list_stride(int pd, bool f64) {
+    const int vertices = 256 * (pd + 1);
+    const int rows = kTileSlots * (f64 ? 2 : 1) + kTileSlots / 4;
+    return vertices > rows ? vertices : rows;
+}
+
+// What the merging build needs to number its vertices: the per-vertex tables and the value table
+// (rows of value_words floats: the rows of the vertices a workgroup created receive its sums when
+// the build splats, zeros when not).  n_segments == 0: it does not number them but lists them and
+// adds its sums to the rows of the hash cells, like the plain build, and number_vertices follows.
+struct InBuildNumbering {
+    int *cell_vertex;
+    uint64_t *vertex_keys;
+    int *vertex_cell;
+    int2 *neighbours;
+    int max_vertices;
+    void *values;
+    int value_words;
+    int n_segments;       // 0, 1 or 8 (segments_for)
 };
 
 // Where the feature vector of a point comes from: the row of a positions array, or, with
@@ -136,20 +200,24 @@ hipError_t clear_table(uint64_t *cell_keys, uint32_t n_cells, hipStream_t s);
 // splat_vd != 0 (allowed when build_can_splat(vd)): the kernel also splats `input`
 // (in_channels per point) into cell_values[cell*vd ..], rows addressed by hash cell;
 // number_vertices then moves them into the dense value table.
+// numbering != nullptr: the merging build (the points are a grid).  With numbering->n_segments
+// != 0 it numbers its vertices itself (Counters, CreatedLists, InBuildNumbering): no
+// number_vertices follows it, cell_values is not used, and neighbours() must be given the lists
+// when the build splatted.
 bool build_can_splat(int vd);
 hipError_t build(int pd, const PointFeatures &features, const PointMap &map, const ScaleFactor &scale,
                  uint64_t *cell_keys, uint32_t n_cells, Counters *counters, ReplayEntry *replay,
                  int xcd_aware, int splat_vd, const float *input,
                  int in_channels, float *cell_values, const CreatedLists &created_lists,
-                 const RegionSource &regions, bool merge_in_workgroup, hipStream_t s);
+                 const RegionSource &regions, const InBuildNumbering *numbering, hipStream_t s);
 
 // The build for double values: the same kernel on points.positions with points.scale; replay[]
 // receives the cells (and the weights rounded to float), points.weights[r*T+t] the weights.
 hipError_t build_f64(int pd, const Points64 &points, const PointMap &map, uint64_t *cell_keys,
                      uint32_t n_cells, Counters *counters, ReplayEntry *replay, int xcd_aware,
                      const CreatedLists &created_lists, const RegionSource &regions,
-                     bool merge_in_workgroup, int splat_vd, const double *input, int in_channels,
-                     double *cell_values, hipStream_t s);
+                     const InBuildNumbering *numbering, int splat_vd, const double *input,
+                     int in_channels, double *cell_values, hipStream_t s);
 
 // Dense vertex numbers in the order of the build's workgroups (same map as the build):
 // cell_vertex[cell] := v, vertex_keys[v] := key, vertex_cell[v] := cell,
@@ -167,9 +235,17 @@ hipError_t number_vertices(int pd, const PointMap &map, const CreatedLists &list
 // launch_vertices (here and below): the vertex count the grid is sized for; any count is
 // covered, a wrong estimate only costs time.
 // Keys are looked for where the build put them: counters->region_* as the build left them.
+// foreign_rows != nullptr (after a merging build that numbered its vertices and splatted): the
+// launch also adds the rows the build's n_lists workgroups listed to `values` (rows of vd floats
+// or doubles).
+// report != nullptr (after a merging build that numbered its vertices): the launch also sums the
+// segments' counts in *report (the build's counters, == counters), copies them and the flags to
+// *host_status and zeroes *next_counters, as number_vertices does otherwise.
 hipError_t neighbours(int pd, const VertexTables &vertices, const Counters *counters,
                       const uint64_t *cell_keys, uint32_t n_cells, int launch_vertices,
-                      hipStream_t s);
+                      const CreatedLists *foreign_rows, unsigned n_lists, void *values, int vd,
+                      bool values_are_double, Counters *report, Counters *next_counters,
+                      HostStatus *host_status, hipStream_t s);
 
 hipError_t fill_zero(float *p, size_t n, hipStream_t s);
 
@@ -213,12 +289,35 @@ hipError_t slice(int pd, int vd, const PointMap &map, const ReplayEntry *replay,
 hipError_t debug_simplex(int pd, const float *positions, int N, const ScaleFactor &scale,
                          short *rem0, short *rank, short *keys, float *barycentric, hipStream_t s);
 
-hipError_t export_keys(int pd, const uint64_t *vertex_keys, int M, short *keys, hipStream_t s);
+// How the debug exports count the vertices: densely, segment after segment.  before[k]: vertices
+// in the segments below k; total: all of them.
+struct VertexNumbers {
+    int n_segments;      // 0: the numbers are dense already
+    unsigned stride;
+    unsigned before[kMaxSegments + 1];
+    unsigned total;
+    __host__ __device__ unsigned dense_of(unsigned v) const {
+        if (n_segments == 0) return v;
+        const unsigned k = v / stride;
+        return before[k] + (v - k * stride);
+    }
+    __host__ __device__ unsigned vertex_of(unsigned dense) const {
+        if (n_segments == 0) return dense;
+        unsigned k = 0;
+        while (k + 1 < (unsigned)n_segments && dense >= before[k + 1]) ++k;
+        return k * stride + (dense - before[k]);
+    }
+};
+hipError_t export_keys(int pd, const uint64_t *vertex_keys, const VertexNumbers &numbers, short *keys,
+                       hipStream_t s);
+// out[d * words ..] := the row of the d-th vertex (rows of `words` floats)
+hipError_t export_values(const float *values, int words, const VertexNumbers &numbers, float *out,
+                         hipStream_t s);
 
 // replay arrays in point order: vertex[r*N+n], weight[r*N+n]; cell_vertex != nullptr when
 // the replay rows still hold hash cells
 hipError_t export_replay(int pd, const PointMap &map, const ReplayEntry *replay,
-                         const int *cell_vertex, int *vertex,
+                         const int *cell_vertex, const VertexNumbers &numbers, int *vertex,
                          float *weight, hipStream_t s);
 
 // The value passes for double values (pl_kernels_f64.hip): as splat, blur_axis, slice,

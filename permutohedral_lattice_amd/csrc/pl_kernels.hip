@@ -16,6 +16,8 @@
 //
 // Packed key.  Every coordinate of lattice vertex with remainder r is (pd+1)*q_i + r, so a key is
 // (r, q_0..q_{pd-1}): r in bits 60..63, q_i biased into a field of B = min(16, 60/pd) bits.
+#include <type_traits>
+
 #include "pl_kernels.h"
 #include "pl_device.h"
 
@@ -24,6 +26,12 @@ namespace plk {
 namespace {
 
 using namespace device;
+
+// A vertex's row of values, moved as one vector when its size is a power of two
+template <int VD, typename S = float>
+struct alignas(VD == 3 ? sizeof(S) : sizeof(S) * VD) ValueRow {
+    S c[VD];
+};
 
 template <int PD>
 __device__ __forceinline__ void load_position(const float *positions, int n, float (&pos)[PD]) {
@@ -289,7 +297,7 @@ __global__ __launch_bounds__(kBlock) void k_build(PointFeatures features, PointM
         int base = 0;
         if (lane == 0 && total) base = atomicAdd(&group_created, total);
         base = __builtin_amdgcn_readfirstlane(base);
-        const size_t list = (size_t)vblock * (kBlock * D1);
+        const size_t list = (size_t)vblock * (size_t)created_lists.stride;
 #pragma unroll
         for (int r = 0; r < D1; ++r) {
             if ((created >> r) & 1u) {
@@ -353,7 +361,7 @@ __global__ __launch_bounds__(kBlock) void k_build(PointFeatures features, PointM
 // in the table in HBM by one thread, and its row goes out with one request.  A workgroup whose
 // distinct keys do not fit the LDS table raises kFlagTileFull and the host repeats the build with
 // k_build (and uses it for a while).  Three barriers; every thread reaches each of them.
-constexpr int kTileSlots = 2 * kBlock;    // LDS slots per workgroup (at most 6 * kBlock keys exist)
+static_assert(kTileSlots == 2 * kBlock, "a thread places at most two slots in the table");
 constexpr int kTileProbeLimit = 48;
 
 template <int PD, int SPLAT_VD, typename T = float>
@@ -364,22 +372,31 @@ __global__ __launch_bounds__(kBlock) void k_build_tile(PointFeatures features, P
                                                         int xcd_aware, const void *__restrict__ input_any,
                                                         int in_channels, void *cell_values_any,
                                                         CreatedLists created_lists,
-                                                        Points64 points64, RegionSource region_source) {
+                                                        Points64 points64, RegionSource region_source,
+                                                        InBuildNumbering numbering) {
     constexpr bool kDouble = sizeof(T) == sizeof(double);
     constexpr int D1 = PD + 1;
     constexpr int VD = SPLAT_VD ? SPLAT_VD : 2;
     constexpr int P = (VD == 2 && !kDouble) ? 2 : 4;      // values per LDS row of sums
     const T *__restrict__ input = static_cast<const T *>(input_any);
-    T *cell_values = static_cast<T *>(cell_values_any);
     __shared__ uint64_t slot_key[kTileSlots];
     __shared__ int slot_cell[kTileSlots];
     __shared__ T slot_sum[SPLAT_VD ? kTileSlots * P : 1];
+    // the slots in use, in the order their keys arrived: the last phases walk these, not all slots
+    __shared__ unsigned short occupied[kTileSlots];
+    __shared__ int n_occupied;
+    // which of the vertices this workgroup created a slot's key is (kNotCreated: none of them)
+    __shared__ unsigned short slot_rank[kTileSlots];
+    constexpr unsigned short kNotCreated = 0xffffu;
     __shared__ int group_created;
     const int tid = threadIdx.x;
     for (int i = tid; i < kTileSlots; i += kBlock) slot_key[i] = kEmptyCell;
     if (SPLAT_VD)
         for (int i = tid; i < kTileSlots * P; i += kBlock) slot_sum[i] = (T)0;
-    if (tid == 0) group_created = 0;
+    if (tid == 0) {
+        n_occupied = 0;
+        group_created = 0;
+    }
 
     const unsigned vblock = xcd_contiguous_block(blockIdx.x, gridDim.x, xcd_aware);
     const size_t t = (size_t)vblock * kBlock + tid;   // slot in the replay arrays
@@ -434,10 +451,14 @@ __global__ __launch_bounds__(kBlock) void k_build_tile(PointFeatures features, P
                     const uint64_t seen =
                         atomicCAS((unsigned long long *)&slot_key[slot[r]],
                                   (unsigned long long)kEmptyCell, (unsigned long long)key[r]);
-                    if (seen == kEmptyCell || seen == key[r])
+                    if (seen == kEmptyCell || seen == key[r]) {
                         open &= ~(1u << r);
-                    else
+                        // the slot was empty: it joins the list of slots in use
+                        if (seen == kEmptyCell)
+                            occupied[atomicAdd(&n_occupied, 1)] = (unsigned short)slot[r];
+                    } else {
                         slot[r] = (slot[r] + 1) & (kTileSlots - 1);
+                    }
                 }
             }
             any_open = open != 0;
@@ -499,15 +520,20 @@ __global__ __launch_bounds__(kBlock) void k_build_tile(PointFeatures features, P
     }
     __syncthreads();        // the keys and sums of all four wavefronts are in the LDS table
 
-    // Every occupied slot goes to the table in HBM: thread i takes slots i and i + kBlock, in
-    // rounds over both as in k_build.
-    constexpr int H = kTileSlots / kBlock;
+    // Every slot in use goes to the table in HBM: thread i takes the i-th of them (and the
+    // (i + kBlock)-th when a tile has that many, in rounds over both as in k_build).  A tile of an
+    // image has about a hundred, so two of the four wavefronts have nothing to do here.
     const KeyRegions regions = key_regions(region_source);
     if (blockIdx.x == 0 && tid == 0) {
         counters->region_lo = regions.lo;
         counters->region_per_unit = regions.per_unit;
     }
-    {
+    const int n_in_use = n_occupied;
+    // numbering.n_segments != 0: the workgroups number their vertices themselves; else they list
+    // them for the numbering pass and add all their sums to the rows of the hash cells
+    const bool numbers_here = numbering.n_segments != 0;
+    auto place_in_table = [&](auto slots_per_thread) {
+        constexpr int H = decltype(slots_per_thread)::value;
         // A round looks at the pair of cells a key has come to (one 16-byte load), takes the key's
         // cell if it is there, else swaps the key into the pair's first empty cell, else moves on
         // to the next pair.  A swap lost to another key looks at the same pair again: each turn
@@ -516,10 +542,13 @@ __global__ __launch_bounds__(kBlock) void k_build_tile(PointFeatures features, P
         uint32_t cell[H], pair_index[H];
         ulonglong2 seen[H];
         unsigned open = 0, created = 0;
+        int in_slot[H];
 #pragma unroll
         for (int h = 0; h < H; ++h) {
-            key[h] = slot_key[tid + h * kBlock];
-            if (key[h] != kEmptyCell) open |= 1u << h;
+            const bool has = tid + h * kBlock < n_in_use;
+            in_slot[h] = has ? (int)occupied[tid + h * kBlock] : 0;
+            key[h] = has ? slot_key[in_slot[h]] : kEmptyCell;
+            if (has) open |= 1u << h;
             cell[h] = cell_of_key<PD>(key[h], mask, regions);
             pair_index[h] = 0;
         }
@@ -569,7 +598,8 @@ __global__ __launch_bounds__(kBlock) void k_build_tile(PointFeatures features, P
         if (any_open) atomicOr(&counters->flags, kFlagTableFull);
 #pragma unroll
         for (int h = 0; h < H; ++h)
-            slot_cell[tid + h * kBlock] = (open >> h) & 1u ? -1 : (int)cell[h];
+            if (tid + h * kBlock < n_in_use)
+                slot_cell[in_slot[h]] = (open >> h) & 1u ? -1 : (int)cell[h];
 
         // the vertices this workgroup created, as in k_build
         int offset[H];
@@ -584,37 +614,155 @@ __global__ __launch_bounds__(kBlock) void k_build_tile(PointFeatures features, P
         int base = 0;
         if (lane == 0 && total) base = atomicAdd(&group_created, total);
         base = __builtin_amdgcn_readfirstlane(base);
-        const size_t list = (size_t)vblock * (kBlock * D1);
 #pragma unroll
-        for (int h = 0; h < H; ++h) {
-            if ((created >> h) & 1u) {
-                created_lists.entries[list + base + offset[h]] =
-                    make_uint4((uint32_t)key[h], (uint32_t)(key[h] >> 32), cell[h], 0u);
+        for (int h = 0; h < H; ++h)
+            if (tid + h * kBlock < n_in_use)
+                slot_rank[in_slot[h]] =
+                    (created >> h) & 1u ? (unsigned short)(base + offset[h]) : kNotCreated;
+        if (!numbers_here) {
+            // (for the numbering pass: what this workgroup created, as in k_build)
+            const size_t list = (size_t)vblock * (size_t)created_lists.stride;
+#pragma unroll
+            for (int h = 0; h < H; ++h) {
+                if ((created >> h) & 1u) {
+                    created_lists.entries[list + base + offset[h]] =
+                        make_uint4((uint32_t)key[h], (uint32_t)(key[h] >> 32), cell[h], 0u);
+                }
             }
         }
+    };
+    if ((tid & ~63) < n_in_use) {
+        if (n_in_use <= kBlock)
+            place_in_table(std::integral_constant<int, 1>{});
+        else
+            place_in_table(std::integral_constant<int, kTileSlots / kBlock>{});
     }
-    __syncthreads();        // every slot's cell is known, and so is the number of vertices created
-    if (tid == 0) {
-        const int sum = group_created;
-        created_lists.block_count[vblock] = sum;
-        if (sum) atomicAdd(&created_lists.chunk_count[vblock / kBlocksPerChunk], sum);
-    }
-    if (SPLAT_VD) {
-        // rows of sums: P consecutive lanes per slot, one request per row
-#pragma unroll
-        for (int i = 0; i < kTileSlots * P / kBlock; ++i) {
-            const int sl = i * (kBlock / P) + tid / P;
-            const int channel = tid % P;
-            const int cell = slot_cell[sl];
-            if (slot_key[sl] != kEmptyCell && cell >= 0 && channel < VD)
-                atomicAdd(cell_values + (size_t)cell * VD + channel, slot_sum[sl * P + channel]);
+    __syncthreads();        // every slot's cell is known
+
+    if (!numbers_here) {
+        // The numbering pass follows: it needs the length of the workgroup's list, and moves the
+        // rows of sums from the hash cells to the vertices.
+        if (tid == 0) {
+            const int sum = group_created;
+            created_lists.block_count[vblock] = sum;
+            if (sum) atomicAdd(&created_lists.chunk_count[vblock / kBlocksPerChunk], sum);
         }
+        if (SPLAT_VD) {
+            // rows of sums: P consecutive lanes per slot in use, one request per row
+            T *cell_values = static_cast<T *>(cell_values_any);
+            const int channel = tid % P;
+            for (int i = tid / P; i < n_in_use; i += kBlock / P) {
+                const int sl = (int)occupied[i];
+                const int cell = slot_cell[sl];
+                if (cell >= 0 && channel < VD)
+                    atomicAdd(cell_values + (size_t)cell * VD + channel, slot_sum[sl * P + channel]);
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < D1; ++r) {
+            const int c = slot[r] >= 0 ? slot_cell[slot[r]] : -1;
+            replay[(size_t)r * n_slots + t] = ReplayEntry{c, valid ? (float)s.weight[r] : 0.0f};
+            if constexpr (kDouble) points64.weights[(size_t)r * n_slots + t] = valid ? s.weight[r] : 0.0;
+        }
+        return;
     }
+
+    // Numbers for the vertices this workgroup created: a run of its segment's, drawn with one
+    // atomic (the segment is the eighth of the image the workgroup lies in, which is the XCD it
+    // runs on when the workgroups are dealt out that way; a small table has one segment).  The
+    // atomic takes a microsecond or more to come back -- a segment's workgroups all add to one
+    // address -- so only the first wavefront waits for it: the others end behind their replay rows
+    // and leave their places to the wavefronts of the next workgroup.
+    const unsigned stride = segment_stride((uint32_t)numbering.max_vertices, numbering.n_segments);
+    unsigned segment = 0;
+    if (numbering.n_segments == (int)kXcds)
+        segment = xcd_aware ? (blockIdx.x % kXcds) : (unsigned)(((size_t)vblock * kXcds) / gridDim.x);
+    const unsigned count = (unsigned)group_created;
+    unsigned first = 0;
+    if (tid == 0 && count) first = atomicAdd(&counters->segment_count[segment].n, count);
 #pragma unroll
     for (int r = 0; r < D1; ++r) {
         const int c = slot[r] >= 0 ? slot_cell[slot[r]] : -1;
         replay[(size_t)r * n_slots + t] = ReplayEntry{c, valid ? (float)s.weight[r] : 0.0f};
         if constexpr (kDouble) points64.weights[(size_t)r * n_slots + t] = valid ? s.weight[r] : 0.0;
+    }
+    if (blockIdx.x == 0 && tid < kMaxSegments) {
+        counters->n_segments = numbering.n_segments;
+        counters->segment_count[tid].n_segments = numbering.n_segments;
+    }
+    if (tid >= 64) return;
+
+    // Per slot in use: a vertex this workgroup created gets its number, its entries in the
+    // per-vertex tables and its row of the value table (the tile's sums, or zeros when the build
+    // does not splat; other workgroups' sums for it are added by neighbours()); the sums for a
+    // vertex that another workgroup created go to this workgroup's list.
+    first = (unsigned)__builtin_amdgcn_readfirstlane((int)first);
+    // (a run that leaves the segment: the host repeats the build with a larger table; what is
+    // enqueued behind this build walks the segment's numbers, so those still get vertices)
+    if (lane == 0 && first + count > stride) atomicOr(&counters->flags, kFlagTableFull);
+    T *values = static_cast<T *>(numbering.values);
+    const int numbers_from = (int)(segment * stride);
+    uint4 *part = created_lists.entries + (size_t)vblock * (size_t)created_lists.stride;
+    T *foreign_rows = reinterpret_cast<T *>(part);
+    int *foreign_cells = reinterpret_cast<int *>(part + kTileSlots * (kDouble ? 2 : 1));
+    int n_foreign = 0;
+    for (int i0 = 0; i0 < n_in_use; i0 += 64) {
+        const int i = i0 + lane;
+        const bool has = i < n_in_use;
+        const int sl = has ? (int)occupied[i] : 0;
+        const int cell = has ? slot_cell[sl] : -1;
+        const unsigned short rank = slot_rank[sl];
+        const bool mine = cell >= 0 && rank != kNotCreated;
+        const bool foreign = SPLAT_VD != 0 && cell >= 0 && rank == kNotCreated;
+        T row[4] = {(T)0, (T)0, (T)0, (T)0};
+        if (SPLAT_VD) {
+#pragma unroll
+            for (int j = 0; j < P; ++j) row[j] = slot_sum[sl * P + j];
+        }
+        if (mine) {
+            // (a number beyond the segment is not given out: what runs until the host repeats
+            // the build must find a valid one)
+            const bool fits = first + rank < stride;
+            const int v = fits ? numbers_from + (int)(first + rank) : 0;
+            numbering.cell_vertex[cell] = v;
+            if (fits) {
+                numbering.vertex_keys[v] = slot_key[sl];
+                numbering.vertex_cell[v] = cell;
+#pragma unroll
+                for (int a = 0; a < D1; ++a)
+                    numbering.neighbours[(size_t)a * numbering.max_vertices + v] = make_int2(-1, -1);
+                if (SPLAT_VD) {
+                    if constexpr (VD == 4 || (VD == 2 && !kDouble)) {
+                        reinterpret_cast<ValueRow<VD, T> *>(values)[v] =
+                            *reinterpret_cast<const ValueRow<VD, T> *>(row);
+                    } else {
+#pragma unroll
+                        for (int j = 0; j < VD; ++j) values[(size_t)v * VD + j] = row[j];
+                    }
+                } else {
+                    float *words = static_cast<float *>(numbering.values);
+                    for (int j = 0; j < numbering.value_words; ++j)
+                        words[(size_t)v * numbering.value_words + j] = 0.0f;
+                }
+            }
+        }
+        if (SPLAT_VD) {
+            const uint64_t b = wave_ballot(foreign);
+            const int offset = n_foreign + (int)__builtin_amdgcn_mbcnt_hi(
+                                               (uint32_t)(b >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)b, 0u));
+            n_foreign += (int)__builtin_popcountll(b);
+            if (foreign) {
+                foreign_cells[offset] = cell;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) foreign_rows[(size_t)offset * 4 + j] = row[j];
+            }
+        }
+    }
+    if (lane == 0) {
+        created_lists.block_count[vblock] = n_foreign;
+        // (how many such rows there are in all tells the host whether numbering here pays)
+        if ((blockIdx.x / kXcds) % kForeignSampling == 0 && n_foreign)
+            atomicAdd(&counters->foreign_rows_sampled.n, (unsigned)n_foreign);
     }
 }
 
@@ -639,7 +787,7 @@ __global__ __launch_bounds__(64) void k_number_vertices(CreatedLists lists, int 
     const unsigned b = xcd_contiguous_block(blockIdx.x, gridDim.x, 1);
     const int lane = threadIdx.x;
     const unsigned chunk = b / kBlocksPerChunk;
-    const size_t list = (size_t)b * (kBlock * D1);
+    const size_t list = (size_t)b * (size_t)lists.stride;
     // Everything the pass reads that does not depend on something else it reads is asked for at
     // once, without branches (an index out of range reads element 0 and is dropped afterwards):
     // the sums of the chunks before this workgroup's, the counts of the workgroups before it in
@@ -666,10 +814,17 @@ __global__ __launch_bounds__(64) void k_number_vertices(CreatedLists lists, int 
         if (lane == 0) {
             const uint32_t m = (uint32_t)(before + count);
             counters->vertices = m;
+            counters->n_segments = 0;
+            for (int k = 0; k < kMaxSegments; ++k) {
+                counters->segment_count[k].n = m;
+                counters->segment_count[k].n_segments = 0;
+            }
             host_status->num_vertices = (int)m;
             host_status->flags = counters->flags | (m > (uint32_t)max_vertices ? kFlagTableFull : 0);
-            next_counters->vertices = 0;
-            next_counters->flags = 0;
+            host_status->max_segment = (int)m;
+            host_status->n_segments = 0;
+            host_status->foreign_rows = 0;
+            reset_counters(next_counters);
         }
         for (unsigned i = lane; i < n_chunks; i += 64) next_chunk_count[i] = 0;
     }
@@ -722,22 +877,76 @@ __global__ __launch_bounds__(64) void k_number_vertices(CreatedLists lists, int 
 // vertices follow each other.  u is the + neighbour of v exactly when v is the - neighbour of u:
 // one lookup fills out[a][v].x and out[a][u].y (all entries start as -1).
 // ------------------------------------------------------------------------------------------------
+// After a merging build that numbered its vertices and splatted, the launch also adds the rows of
+// sums that the build's workgroups hold for vertices other workgroups created (ForeignRows) to the
+// value table, now that every vertex has its number: its first foreign_blocks workgroups (a
+// multiple of 8, or 0) take four workgroups' lists each, one per wavefront, a row per group of
+// four lanes.  S: the value type.
+template <typename S>
+__device__ __forceinline__ void add_foreign_rows(const CreatedLists &lists, unsigned n_lists,
+                                                 unsigned group, int vd,
+                                                 const int *__restrict__ cell_vertex, S *values) {
+    const unsigned list = group * (kBlock / 64) + (threadIdx.x >> 6);
+    if (list >= n_lists) return;
+    const int lane = threadIdx.x & 63;
+    const int n = lists.block_count[list];
+    const uint4 *part = lists.entries + (size_t)list * (size_t)lists.stride;
+    const S *rows = reinterpret_cast<const S *>(part);
+    const int *cells = reinterpret_cast<const int *>(part + kTileSlots * (sizeof(S) / sizeof(float)));
+    const int channel = lane & 3;
+    // (what bounds this is the atomic unit, a request per row: asking for all rows of the four
+    // lists at once instead of sixteen rows at a time per list made it slower)
+    for (int e = lane >> 2; e < n; e += 16) {
+        const int v = cell_vertex[cells[e]];
+        if (channel < vd) atomicAdd(values + (size_t)v * vd + channel, rows[(size_t)e * 4 + channel]);
+    }
+}
+
 template <int PD>
 __global__ __launch_bounds__(kBlock) void k_neighbours(VertexTables vertices,
                                                         const Counters *counters,
                                                         const uint64_t *__restrict__ cell_keys,
-                                                        uint32_t mask) {
+                                                        uint32_t mask, unsigned foreign_blocks,
+                                                        CreatedLists lists, unsigned n_lists,
+                                                        void *values, int vd, int values_are_double,
+                                                        Counters *report, Counters *next_counters,
+                                                        HostStatus *host_status) {
     constexpr int D1 = PD + 1;
+    // After a merging build nothing has told the host yet how the build went: the segments' counts
+    // are summed here, and what the next build will count in is cleared.
+    if (report && blockIdx.x == gridDim.x - 1 && threadIdx.x == 0) {
+        unsigned total = 0, fullest = 0;
+        const int n_segments = report->n_segments;
+        for (int k = 0; k < n_segments; ++k) {
+            const unsigned c = report->segment_count[k].n;
+            total += c;
+            fullest = c > fullest ? c : fullest;
+        }
+        report->vertices = total;
+        host_status->num_vertices = (int)total;
+        host_status->flags = report->flags;
+        host_status->max_segment = (int)fullest;
+        host_status->n_segments = n_segments;
+        host_status->foreign_rows = (int)(report->foreign_rows_sampled.n * kForeignSampling);
+        reset_counters(next_counters);
+    }
+    if (blockIdx.x < foreign_blocks) {
+        const unsigned group = xcd_contiguous_block(blockIdx.x, foreign_blocks, 1);
+        if (values_are_double)
+            add_foreign_rows(lists, n_lists, group, vd, vertices.cell_vertex, static_cast<double *>(values));
+        else
+            add_foreign_rows(lists, n_lists, group, vd, vertices.cell_vertex, static_cast<float *>(values));
+        return;
+    }
     const KeyRegions regions{counters->region_lo, counters->region_per_unit};
     const int max_vertices = vertices.max_vertices;
-    const int M = vertex_count(counters, max_vertices);
-    const unsigned runs = (unsigned)((M + kBlock - 1) / kBlock);
-    ItemBlocks blocks((size_t)runs * D1 * kBlock);
+    SegmentWalk walk(counters, max_vertices, blockIdx.x - foreign_blocks, gridDim.x - foreign_blocks);
     unsigned ib;
-    while (blocks.next(ib)) {
+    while (walk.next(1u, D1, ib)) {
     const int a = (int)(ib % D1);
-    const int v = (int)(ib / D1) * kBlock + (int)threadIdx.x;
-    if (v >= M) continue;
+    const unsigned i = (ib / D1) * kBlock + threadIdx.x;
+    if (i >= walk.count) continue;
+    const int v = (int)(walk.first + i);
 
     int q[PD], r;
     KeyCodec<PD>::unpack(vertices.vertex_keys[v], q, r);
@@ -1092,12 +1301,12 @@ __global__ __launch_bounds__(kBlock) void k_blur_element(const Counters *counter
                                                           const int2 *__restrict__ nbr,
                                                           uint64_t *reset_cell_keys,
                                                           const int *__restrict__ vertex_cell) {
-    const int M = vertex_count(counters, max_vertices);
-    ItemBlocks blocks((size_t)M * vd);
+    SegmentWalk walk(counters, max_vertices, blockIdx.x, gridDim.x);
     unsigned eb;
-    while (blocks.next(eb)) {
-        const size_t e = (size_t)eb * kBlock + threadIdx.x;
-        if (e >= (size_t)M * vd) continue;
+    while (walk.next((unsigned)vd, 1u, eb)) {
+        const size_t i = (size_t)eb * kBlock + threadIdx.x;
+        if (i >= (size_t)walk.count * vd) continue;
+        const size_t e = (size_t)walk.first * vd + i;
         const int v = (int)(e / (size_t)vd);
         const int j = (int)(e - (size_t)v * vd);
         const int2 nb = nbr[v];
@@ -1122,12 +1331,12 @@ __global__ __launch_bounds__(kBlock) void k_blur2_element(const Counters *counte
                                                            const int2 *__restrict__ nbr_b,
                                                            uint64_t *reset_cell_keys,
                                                            const int *__restrict__ vertex_cell) {
-    const int M = vertex_count(counters, max_vertices);
-    ItemBlocks blocks((size_t)M * vd);
+    SegmentWalk walk(counters, max_vertices, blockIdx.x, gridDim.x);
     unsigned eb;
-    while (blocks.next(eb)) {
-        const size_t e = (size_t)eb * kBlock + threadIdx.x;
-        if (e >= (size_t)M * vd) continue;
+    while (walk.next((unsigned)vd, 1u, eb)) {
+        const size_t i = (size_t)eb * kBlock + threadIdx.x;
+        if (i >= (size_t)walk.count * vd) continue;
+        const size_t e = (size_t)walk.first * vd + i;
         const int v = (int)(e / (size_t)vd);
         const int j = (int)(e - (size_t)v * vd);
         int u[9];
@@ -1144,11 +1353,6 @@ __global__ __launch_bounds__(kBlock) void k_blur2_element(const Counters *counte
 // vertex numbers that follow the image the rows a thread gathers are near each other, and a
 // quarter of the memory instructions moves the same bytes (34 -> 25 us for the three launches
 // of pd = 5, vd = 4).  Same arithmetic per channel, same results.
-template <int VD, typename S = float>
-struct alignas(VD == 3 ? sizeof(S) : sizeof(S) * VD) ValueRow {
-    S c[VD];
-};
-
 template <int VD, typename S = float>
 __device__ __forceinline__ ValueRow<VD, S> blur_rows(const ValueRow<VD, S> &a, const ValueRow<VD, S> &self,
                                                   const ValueRow<VD, S> &b) {
@@ -1187,12 +1391,12 @@ __global__ __launch_bounds__(kBlock) void k_blur_row(const Counters *counters, i
                                                       const int2 *__restrict__ nbr,
                                                       uint64_t *reset_cell_keys,
                                                       const int *__restrict__ vertex_cell) {
-    const int M = vertex_count(counters, max_vertices);
-    ItemBlocks blocks((size_t)M);
+    SegmentWalk walk(counters, max_vertices, blockIdx.x, gridDim.x);
     unsigned vb;
-    while (blocks.next(vb)) {
-        const int v = (int)(vb * kBlock + threadIdx.x);
-        if (v >= M) continue;
+    while (walk.next(1u, 1u, vb)) {
+        const unsigned i = vb * kBlock + threadIdx.x;
+        if (i >= walk.count) continue;
+        const int v = (int)(walk.first + i);
         const int2 nb = nbr[v];
         const int u[3] = {nb.x, v, nb.y};
         ValueRow<VD, S> row[3];
@@ -1210,12 +1414,12 @@ __global__ __launch_bounds__(kBlock) void k_blur2_row(const Counters *counters, 
                                                        const int2 *__restrict__ nbr_b,
                                                        uint64_t *reset_cell_keys,
                                                        const int *__restrict__ vertex_cell) {
-    const int M = vertex_count(counters, max_vertices);
-    ItemBlocks blocks((size_t)M);
+    SegmentWalk walk(counters, max_vertices, blockIdx.x, gridDim.x);
     unsigned vb;
-    while (blocks.next(vb)) {
-        const int v = (int)(vb * kBlock + threadIdx.x);
-        if (v >= M) continue;
+    while (walk.next(1u, 1u, vb)) {
+        const unsigned i = vb * kBlock + threadIdx.x;
+        if (i >= walk.count) continue;
+        const int v = (int)(walk.first + i);
         // level 1: the vertex's neighbours along both axes; level 2: the a-neighbours of its
         // b-neighbours; level 3: nine rows
         int u[9];
@@ -1272,12 +1476,12 @@ __global__ __launch_bounds__(kBlock) void k_blur3_row(const Counters *counters, 
                                                        const int2 *__restrict__ nbr_c,
                                                        uint64_t *reset_cell_keys,
                                                        const int *__restrict__ vertex_cell) {
-    const int M = vertex_count(counters, max_vertices);
-    ItemBlocks blocks((size_t)M);
+    SegmentWalk walk(counters, max_vertices, blockIdx.x, gridDim.x);
     unsigned vb;
-    while (blocks.next(vb)) {
-        const int v = (int)(vb * kBlock + threadIdx.x);
-        if (v >= M) continue;
+    while (walk.next(1u, 1u, vb)) {
+        const unsigned i = vb * kBlock + threadIdx.x;
+        if (i >= walk.count) continue;
+        const int v = (int)(walk.first + i);
         int u[27];
         three_axis_sources(nbr_a, nbr_b, nbr_c, v, u);
         ValueRow<VD, S> row[27];
@@ -1501,15 +1705,24 @@ __global__ __launch_bounds__(kBlock) void k_debug_simplex(const float *__restric
     }
 }
 
+// The debug exports count the vertices densely, segment after segment (VertexNumbers).
 template <int PD>
 __global__ __launch_bounds__(kBlock) void k_export_keys(const uint64_t *__restrict__ vertex_keys,
-                                                         int M, short *keys) {
-    const int v = blockIdx.x * kBlock + threadIdx.x;
-    if (v >= M) return;
+                                                         VertexNumbers numbers, short *keys) {
+    const unsigned d = blockIdx.x * kBlock + threadIdx.x;
+    if (d >= numbers.total) return;
     int q[PD], r;
-    KeyCodec<PD>::unpack(vertex_keys[v], q, r);
+    KeyCodec<PD>::unpack(vertex_keys[numbers.vertex_of(d)], q, r);
 #pragma unroll
-    for (int i = 0; i < PD; ++i) keys[(size_t)v * PD + i] = (short)(q[i] * (PD + 1) + r);
+    for (int i = 0; i < PD; ++i) keys[(size_t)d * PD + i] = (short)(q[i] * (PD + 1) + r);
+}
+
+__global__ __launch_bounds__(kBlock) void k_export_values(const float *__restrict__ values, int words,
+                                                           VertexNumbers numbers, float *out) {
+    const size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x;
+    if (i >= (size_t)numbers.total * words) return;
+    const unsigned d = (unsigned)(i / words);
+    out[i] = values[(size_t)numbers.vertex_of(d) * words + (i - (size_t)d * words)];
 }
 
 // replay arrays from thread order to point order: out[r*N + n]; cells are translated to vertex
@@ -1517,6 +1730,7 @@ __global__ __launch_bounds__(kBlock) void k_export_keys(const uint64_t *__restri
 __global__ __launch_bounds__(kBlock) void k_export_replay(int d1, PointMap map,
                                                            const ReplayEntry *__restrict__ replay,
                                                            const int *__restrict__ cell_vertex,
+                                                           VertexNumbers numbers,
                                                            int *vertex, float *weight) {
     const size_t t = (size_t)blockIdx.x * kBlock + threadIdx.x;
     const size_t T = (size_t)gridDim.x * kBlock;
@@ -1527,7 +1741,7 @@ __global__ __launch_bounds__(kBlock) void k_export_replay(int d1, PointMap map,
         if (vertex) {
             int v = e.index;
             if (cell_vertex && v >= 0) v = cell_vertex[v];
-            vertex[(size_t)r * map.N + n] = v;
+            vertex[(size_t)r * map.N + n] = v >= 0 ? (int)numbers.dense_of((unsigned)v) : v;
         }
         if (weight) weight[(size_t)r * map.N + n] = e.weight;
     }
@@ -1635,15 +1849,18 @@ hipError_t build(int pd, const PointFeatures &features, const PointMap &map, con
                  uint64_t *cell_keys, uint32_t n_cells, Counters *counters, ReplayEntry *replay,
                  int xcd_aware, int splat_vd, const float *input,
                  int in_channels, float *cell_values, const CreatedLists &created_lists,
-                 const RegionSource &regions, bool merge_in_workgroup, hipStream_t s) {
+                 const RegionSource &regions, const InBuildNumbering *numbering, hipStream_t s) {
     if (map.n_blocks == 0) return hipSuccess;
+    const bool merge_in_workgroup = numbering != nullptr;
+    const InBuildNumbering in_build = numbering ? *numbering : InBuildNumbering{};
 #define PLK_BUILD_ARGS                                                                             \
     dim3(map.n_blocks), dim3(kBlock), 0, s, features, map, scale, cell_keys, n_cells - 1u,         \
         counters, replay, xcd_aware, (const void *)input, in_channels, (void *)cell_values,        \
         created_lists, Points64{}, regions
 #define PLK_BUILD(SPLAT_VD)                                                                        \
     if (merge_in_workgroup)                                                                        \
-        PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_build_tile<PD, SPLAT_VD>), PLK_BUILD_ARGS))      \
+        PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_build_tile<PD, SPLAT_VD>), PLK_BUILD_ARGS,       \
+                                               in_build))                                          \
     else                                                                                           \
         PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_build<PD, SPLAT_VD>), PLK_BUILD_ARGS))
     switch (splat_vd) {
@@ -1661,16 +1878,19 @@ hipError_t build(int pd, const PointFeatures &features, const PointMap &map, con
 hipError_t build_f64(int pd, const Points64 &points, const PointMap &map, uint64_t *cell_keys,
                      uint32_t n_cells, Counters *counters, ReplayEntry *replay, int xcd_aware,
                      const CreatedLists &created_lists, const RegionSource &regions,
-                     bool merge_in_workgroup, int splat_vd, const double *input, int in_channels,
-                     double *cell_values, hipStream_t s) {
+                     const InBuildNumbering *numbering, int splat_vd, const double *input,
+                     int in_channels, double *cell_values, hipStream_t s) {
     if (map.n_blocks == 0) return hipSuccess;
+    const bool merge_in_workgroup = numbering != nullptr;
+    const InBuildNumbering in_build = numbering ? *numbering : InBuildNumbering{};
     if (splat_vd && !merge_in_workgroup) return hipErrorInvalidValue;
 #define PLK_BUILD_ARGS                                                                             \
     dim3(map.n_blocks), dim3(kBlock), 0, s, PointFeatures{}, map, ScaleFactor{}, cell_keys,        \
         n_cells - 1u, counters, replay, xcd_aware, (const void *)input, in_channels,               \
         (void *)cell_values, created_lists, points, regions
 #define PLK_BUILD(SPLAT_VD)                                                                        \
-    PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_build_tile<PD, SPLAT_VD, double>), PLK_BUILD_ARGS))
+    PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_build_tile<PD, SPLAT_VD, double>), PLK_BUILD_ARGS,  \
+                                           in_build))
     if (merge_in_workgroup) {
         switch (splat_vd) {
             case 0: PLK_BUILD(0); break;
@@ -1701,12 +1921,20 @@ hipError_t number_vertices(int pd, const PointMap &map, const CreatedLists &list
 
 hipError_t neighbours(int pd, const VertexTables &vertices, const Counters *counters,
                       const uint64_t *cell_keys, uint32_t n_cells, int launch_vertices,
-                      hipStream_t s) {
+                      const CreatedLists *foreign_rows, unsigned n_lists, void *values, int vd,
+                      bool values_are_double, Counters *report, Counters *next_counters,
+                      HostStatus *host_status, hipStream_t s) {
     if (vertices.max_vertices <= 0) return hipErrorInvalidValue;
-    const size_t items = (size_t)(pd + 1) * ((size_t)launch_vertices + kBlock);
-    PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_neighbours<PD>), dim3(vertex_blocks(items)),
+    const size_t items = (size_t)(pd + 1) * (size_t)launch_vertices;
+    const unsigned foreign_blocks =
+        foreign_rows ? (blocks_for(n_lists, kBlock / 64) + kXcds - 1u) / kXcds * kXcds : 0u;
+    PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_neighbours<PD>),
+                                           dim3(foreign_blocks + vertex_blocks(items)),
                                            dim3(kBlock), 0, s, vertices, counters, cell_keys,
-                                           n_cells - 1u));
+                                           n_cells - 1u, foreign_blocks,
+                                           foreign_rows ? *foreign_rows : CreatedLists{}, n_lists,
+                                           values, vd, values_are_double ? 1 : 0, report,
+                                           next_counters, host_status));
     return hipGetLastError();
 }
 
@@ -1945,19 +2173,30 @@ hipError_t debug_simplex(int pd, const float *positions, int N, const ScaleFacto
     return hipGetLastError();
 }
 
-hipError_t export_keys(int pd, const uint64_t *vertex_keys, int M, short *keys, hipStream_t s) {
-    if (M <= 0) return hipSuccess;
+hipError_t export_keys(int pd, const uint64_t *vertex_keys, const VertexNumbers &numbers, short *keys,
+                       hipStream_t s) {
+    const unsigned M = numbers.total;
+    if (M == 0) return hipSuccess;
     PLK_DISPATCH_PD(pd, hipLaunchKernelGGL(k_export_keys<PD>, dim3(blocks_for((size_t)M)),
-                                           dim3(kBlock), 0, s, vertex_keys, M, keys));
+                                           dim3(kBlock), 0, s, vertex_keys, numbers, keys));
+    return hipGetLastError();
+}
+
+hipError_t export_values(const float *values, int words, const VertexNumbers &numbers, float *out,
+                         hipStream_t s) {
+    const size_t n = (size_t)numbers.total * words;
+    if (n == 0) return hipSuccess;
+    hipLaunchKernelGGL(k_export_values, dim3(blocks_for(n)), dim3(kBlock), 0, s, values, words,
+                       numbers, out);
     return hipGetLastError();
 }
 
 hipError_t export_replay(int pd, const PointMap &map, const ReplayEntry *replay,
-                         const int *cell_vertex, int *vertex,
+                         const int *cell_vertex, const VertexNumbers &numbers, int *vertex,
                          float *weight, hipStream_t s) {
     if (map.n_blocks == 0) return hipSuccess;
     hipLaunchKernelGGL(k_export_replay, dim3(map.n_blocks), dim3(kBlock), 0, s, pd + 1, map,
-                       replay, cell_vertex, vertex, weight);
+                       replay, cell_vertex, numbers, vertex, weight);
     return hipGetLastError();
 }
 
