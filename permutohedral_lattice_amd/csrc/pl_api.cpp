@@ -93,6 +93,14 @@ struct pl_lattice {
     uint32_t max_cells = 0;            // enough for N*(pd+1) vertices
     long forced_cells = 0;
     bool table_clean = false;          // every cell of [0, n_cells) is empty
+    // Keys of two words (plk::Key128), for coordinates that do not fit the packed key (pd >= 5):
+    // a build that meets such a coordinate is repeated with them, and so are the next
+    // wide_backoff builds of this lattice (doubled every time it happens again, up to 1024)
+    // before the packed key is tried again.  The key arrays are then twice as large.
+    bool wide_keys = false;            // the last build (and the arrays) use them
+    bool wide_alloc = false;           // cell_keys, vertex_keys and the lists have room for them
+    int wide_for = 0, wide_backoff = 32;
+    bool may_widen = true;             // (not in the static scratch of pl_filter_static: no room)
 
     // per-point arrays, (pd+1) rows of map.n_blocks*256 entries in thread order
     plk::PointMap map{};
@@ -104,6 +112,7 @@ struct pl_lattice {
     int *chunk_count = nullptr;            // [2][n_chunks]
     size_t n_chunks = 0;
     size_t replay_capacity = 0;
+    bool lists_wide = false;               // created_entries has room for two entries per vertex
 
     plk::Counters *d_counters = nullptr;   // two sets, used by alternate builds
     int counter_set = 0;                   // the set of the last build
@@ -191,7 +200,7 @@ struct pl_lattice {
         const long long guess = last + last / 8 + 1024;
         return guess < mv ? (int)guess : mv;
     }
-    int list_stride() const { return plk::created_list_stride(pd, f64); }
+    int list_stride() const { return plk::created_list_stride(pd, f64) * (lists_wide ? 2 : 1); }
     plk::CreatedLists lists(int set) const {
         return plk::CreatedLists{created_entries, block_count, chunk_count + (size_t)set * n_chunks,
                                  list_stride()};
@@ -200,8 +209,9 @@ struct pl_lattice {
 
 namespace {
 
-int ensure_table(pl_lattice *h, uint32_t cells) {
-    if (cells <= h->n_cells_alloc) return PL_OK;
+int ensure_table(pl_lattice *h, uint32_t cells, bool wide) {
+    if (cells <= h->n_cells_alloc && (!wide || h->wide_alloc)) return PL_OK;
+    if (cells < h->n_cells_alloc) cells = h->n_cells_alloc;
     // the old arrays may still be read by work in flight
     PL_HIP(hipStreamSynchronize(h->stream));
     h->dfree(h->cell_keys);
@@ -216,9 +226,10 @@ int ensure_table(pl_lattice *h, uint32_t cells) {
     h->table_clean = false;
     h->cell_values_clean = false;
     const size_t mv = plk::max_vertices_for(cells);
-    h->cell_keys = (uint64_t *)h->dmalloc(sizeof(uint64_t) * (size_t)cells);
+    const size_t key_words = wide || h->wide_alloc ? 2 : 1;
+    h->cell_keys = (uint64_t *)h->dmalloc(sizeof(uint64_t) * key_words * (size_t)cells);
     h->cell_vertex = (int *)h->dmalloc(sizeof(int) * (size_t)cells);
-    h->vertex_keys = (uint64_t *)h->dmalloc(sizeof(uint64_t) * mv);
+    h->vertex_keys = (uint64_t *)h->dmalloc(sizeof(uint64_t) * key_words * mv);
     h->vertex_cell = (int *)h->dmalloc(sizeof(int) * mv);
     h->values[0] = (float *)h->dmalloc(h->value_size() * mv * (size_t)h->vd);
     h->values[1] = (float *)h->dmalloc(h->value_size() * mv * (size_t)h->vd);
@@ -230,12 +241,14 @@ int ensure_table(pl_lattice *h, uint32_t cells) {
         !h->values[1] || !h->neighbours || (fused_splat && !h->cell_values))
         return PL_ENOMEM;
     h->n_cells_alloc = cells;
+    h->wide_alloc = key_words == 2;
     return PL_OK;
 }
 
-int ensure_replay(pl_lattice *h) {
+int ensure_replay(pl_lattice *h, bool wide) {
     const size_t want = (size_t)h->map.n_blocks * 256 * (size_t)(h->pd + 1);
-    if (want <= h->replay_capacity && h->replay) return PL_OK;
+    if (want <= h->replay_capacity && h->replay && (!wide || h->lists_wide)) return PL_OK;
+    h->lists_wide = h->lists_wide || wide;
     PL_HIP(hipStreamSynchronize(h->stream));
     h->dfree(h->replay);
     h->dfree(h->weights64);
@@ -283,15 +296,20 @@ uint32_t initial_cells(const pl_lattice *h) {
 // A lattice for double values takes its positions from positions64 and never splats in the build.
 int enqueue_build(pl_lattice *h, const plk::PointFeatures &features, const double *positions64,
                   uint32_t cells, const void *splat_input) {
-    int rc = ensure_table(h, cells);
+    // keys of two words while a build that needed them is recent (the plain build only)
+    const bool wide = h->wide_for > 0;
+    if (h->wide_for > 0) h->wide_for -= 1;
+    if (wide != h->wide_keys) h->table_clean = false;   // (cells of another width)
+    h->wide_keys = wide;
+    int rc = ensure_table(h, cells, wide);
     if (rc != PL_OK) return rc;
     // the per-point arrays follow the point map; an allocation that failed when the map was set
     // is made up for here
-    rc = ensure_replay(h);
+    rc = ensure_replay(h, wide);
     if (rc != PL_OK) return rc;
     // tiles of an image share most of their vertices among their four wavefronts
-    const bool merge = h->merge_tiles && h->tiles_off_for == 0 && h->map.mode != 0;
-    if (h->tiles_off_for > 0) h->tiles_off_for -= 1;
+    const bool merge = h->merge_tiles && h->tiles_off_for == 0 && h->map.mode != 0 && !wide;
+    if (h->tiles_off_for > 0 && !wide) h->tiles_off_for -= 1;
     h->last_build_merged = merge;
     // (a lattice of doubles splats in its build only in the merging kernel)
     const bool fused = splat_input && plk::build_can_splat(h->vd) && (!h->f64 || merge);
@@ -308,7 +326,7 @@ int enqueue_build(pl_lattice *h, const plk::PointFeatures &features, const doubl
     }
     h->mark(EV_T0);
     if (!h->table_clean || cells != h->n_cells) {
-        PL_HIP(plk::clear_table(h->cell_keys, cells, h->stream));
+        PL_HIP(plk::clear_table(h->cell_keys, wide ? 2 * cells : cells, h->stream));
     }
     h->table_clean = false;
     h->n_cells = cells;
@@ -349,13 +367,13 @@ int enqueue_build(pl_lattice *h, const plk::PointFeatures &features, const doubl
                               fused ? h->vd : 0,
                               static_cast<const double *>(splat_input),
                               h->normalize ? h->vd - 1 : h->vd,
-                              reinterpret_cast<double *>(h->cell_values), h->stream));
+                              reinterpret_cast<double *>(h->cell_values), wide, h->stream));
     } else {
         PL_HIP(plk::build(h->pd, features, h->map, h->scale, h->cell_keys, cells, h->counters(),
                           h->replay, h->xcd_aware ? 1 : 0, fused ? h->vd : 0,
                           static_cast<const float *>(splat_input),
                           h->normalize ? h->vd - 1 : h->vd, h->cell_values, lists,
-                          regions, merge ? &numbering : nullptr, h->stream));
+                          regions, merge ? &numbering : nullptr, wide, h->stream));
     }
     h->mark(EV_BUILD);
     if (!numbers_in_build) {
@@ -365,7 +383,7 @@ int enqueue_build(pl_lattice *h, const plk::PointFeatures &features, const doubl
                                     (unsigned)h->n_chunks, vertices,
                                     h->values[0], h->f64 ? 2 * h->vd : h->vd,
                                     fused ? h->cell_values : nullptr, h->counters(),
-                                    h->d_counters + previous_set, h->h_status, h->stream));
+                                    h->d_counters + previous_set, h->h_status, wide, h->stream));
     }
     if (!numbers_in_build && !h->status_on_device) PL_HIP(hipEventRecord(h->status_written, h->stream));
     h->mark(EV_IDS);
@@ -375,7 +393,7 @@ int enqueue_build(pl_lattice *h, const plk::PointFeatures &features, const doubl
                            h->launch_vertices(), numbers_in_build && fused ? &lists : nullptr,
                            h->map.n_blocks, h->values[0], h->vd, h->f64,
                            numbers_in_build ? h->counters() : nullptr,
-                           h->d_counters + previous_set, h->h_status, h->stream));
+                           h->d_counters + previous_set, h->h_status, wide, h->stream));
     if (numbers_in_build && !h->status_on_device) PL_HIP(hipEventRecord(h->status_written, h->stream));
     h->mark(EV_NBR);
     h->replay_holds_cells = true;
@@ -413,7 +431,7 @@ int enqueue_apply_f64(pl_lattice *h, double *output, const double *input, int re
     if (h->stop_after == 1) return PL_OK;
     for (int step = 0; step <= pd;) {
         const int axis = reverse ? pd - step : step;
-        uint64_t *reset = (!h->table_clean && step == 0) ? h->cell_keys : nullptr;
+        uint64_t *reset = (!h->table_clean && step == 0 && !h->wide_keys) ? h->cell_keys : nullptr;
         const int left = pd + 1 - step;
         // (three axes in one launch pay only when they are all there is: pd = 2; otherwise 27 row
         // gathers per vertex cost more than the launch they save)
@@ -482,7 +500,7 @@ int enqueue_apply(pl_lattice *h, void *output_any, const void *input_any, int re
         // axes 0..pd, or pd..0 for the reverse pass; two per launch while two are left
         const int axis = reverse ? pd - step : step;
         // the first blur after a build also empties the vertices' hash cells
-        uint64_t *reset = (!h->table_clean && step == 0) ? h->cell_keys : nullptr;
+        uint64_t *reset = (!h->table_clean && step == 0 && !h->wide_keys) ? h->cell_keys : nullptr;
         const int left = pd + 1 - step;
         // (three axes in one launch pay only when they are all there is: pd = 2; otherwise 27 row
         // gathers per vertex cost more than the launch they save)
@@ -544,6 +562,14 @@ int verify_build(pl_lattice *h, uint32_t *retry_cells) {
         h->built = false;
         h->table_clean = false;
         h->cell_values_clean = false;
+        // A coordinate that does not fit the packed key: once more with keys of two words, which
+        // hold every short (and so do the next builds of this lattice, for a while).  With those
+        // the coordinate is beyond the reference's own keys.
+        if (!h->wide_keys && h->may_widen && plk::key_field_bits(h->pd) < 16) {
+            h->wide_for = h->wide_backoff;
+            h->wide_backoff = h->wide_backoff >= 512 ? 1024 : h->wide_backoff * 2;
+            *retry_cells = h->n_cells;
+        }
         return PL_EOVERFLOW;
     }
     if (flags & plk::kFlagTileFull) {
@@ -647,7 +673,7 @@ static int create_lattice(int pd, int vd, int N, bool f64, pl_stream stream, con
 
     int rc = PL_OK;
     if (hip_failed(hipGetDevice(&h->device))) rc = PL_EHIP;
-    if (rc == PL_OK) rc = ensure_replay(h);
+    if (rc == PL_OK) rc = ensure_replay(h, false);
     if (rc == PL_OK) {
         h->d_counters = (plk::Counters *)h->dmalloc(2 * sizeof(plk::Counters));
         if (!h->d_counters) rc = PL_ENOMEM;
@@ -758,7 +784,7 @@ int pl_set_point_grid(pl_handle h, int n_dims, const int *dims) {
     h->grid_given = n_dims > 0;
     h->map = plk::make_point_map(h->N, n_dims, dims);
     h->numbering_pass_pays = false;
-    return ensure_replay(h);
+    return ensure_replay(h, false);
 }
 
 int pl_get_point_grid(pl_handle h, int *n_dims, int dims[3]) {
@@ -817,7 +843,7 @@ int guess_point_grid(pl_lattice *h, const float *positions) {
     if (dims[0] < 2) return PL_OK;
     h->map = plk::make_point_map(h->N, n_dims, dims);
     h->numbering_pass_pays = false;
-    return ensure_replay(h);
+    return ensure_replay(h, false);
 }
 
 // Checks the arguments of the *_image entry points, sets the grid hint and describes the features.
@@ -1109,7 +1135,7 @@ int pl_debug_keys(pl_handle h, short *keys) {
     plk::VertexNumbers numbers;
     const int rc = vertex_numbers(h, &numbers);
     if (rc != PL_OK) return rc;
-    PL_HIP(plk::export_keys(h->pd, h->vertex_keys, numbers, keys, h->stream));
+    PL_HIP(plk::export_keys(h->pd, h->vertex_keys, numbers, keys, h->wide_keys, h->stream));
     return PL_OK;
 }
 
@@ -1528,9 +1554,10 @@ extern "C" int pl_filter_static(int pd, int vd, int N, float *output, const floa
     h->max_cells = pow2_at_least(rows * 2 < 4096 ? 4096 : rows * 2);
     h->forced_cells = (long)h->max_cells;
     h->guess_grid = false;   // (looking for a grid in the positions would allocate and wait)
+    h->may_widen = false;    // (keys of two words would need the arrays allocated again)
     h->map = plk::make_point_map(N, 0, nullptr);
     h->status_on_device = true;
-    rc = ensure_replay(h);
+    rc = ensure_replay(h, false);
     if (rc != PL_OK) return rc;
     h->d_counters = (plk::Counters *)h->dmalloc(2 * sizeof(plk::Counters));
     h->h_status = (plk::HostStatus *)h->dmalloc(sizeof(plk::HostStatus));

@@ -67,6 +67,40 @@ __device__ __forceinline__ uint32_t hash_key(uint64_t k) {
     return x;
 }
 
+// Wide keys.  The packed 64-bit key leaves pd >= 5 less than the 16 bits per coordinate that the
+// reference's keys have (short key[pd], src/PermutohedralLatticeCPU.h:297-304): a lattice whose
+// coordinates do not fit is built again with keys of two words, 16 bits per field (15 for pd = 8,
+// whose fields need 13), r in the top four bits of the second word.  A biased field is never all
+// ones and r is at most 8, so neither word of a key is all ones, the mark of an empty word.
+struct Key128 {
+    uint64_t a, b;
+};
+__device__ __forceinline__ bool operator==(const Key128 &x, const Key128 &y) {
+    return x.a == y.a && x.b == y.b;
+}
+template <int PD>
+struct WideCodec {
+    static constexpr int kBits = (124 / PD) > 16 ? 16 : (124 / PD);
+    static constexpr int kBias = 1 << (kBits - 1);
+    template <int N>
+    __device__ static Key128 pack(const int (&q)[N], int r) {
+        static_assert(N >= PD, "one q per stored coordinate");
+        unsigned __int128 k = (unsigned __int128)(unsigned)r << 124;
+#pragma unroll
+        for (int i = 0; i < PD; ++i) k |= (unsigned __int128)(uint32_t)(q[i] + kBias) << (i * kBits);
+        return Key128{(uint64_t)k, (uint64_t)(k >> 64)};
+    }
+    __device__ static void unpack(const Key128 &key, int (&q)[PD], int &r) {
+        const unsigned __int128 k = ((unsigned __int128)key.b << 64) | key.a;
+        r = (int)(key.b >> 60);
+#pragma unroll
+        for (int i = 0; i < PD; ++i)
+            q[i] = (int)((uint32_t)(k >> (i * kBits)) & ((1u << kBits) - 1u)) - kBias;
+    }
+};
+__device__ __forceinline__ uint32_t hash_key(const Key128 &k) {
+    return hash_key(k.a ^ (k.b * 0x9E3779B97F4A7C15ull) ^ (k.b >> 31));
+}
 // Keys spread over the table by where they lie along feature 0.  Every XCD has an L2 of its own,
 // and the kernels deal their work out so that an XCD handles one band of image rows (one
 // contiguous eighth of the tiles, of the vertices): if a vertex's cell is taken from the eighth of
@@ -354,6 +388,27 @@ __device__ __forceinline__ bool simplex_in_key_range(const Simplex<PD, T> &s) {
     return ok;
 }
 
+// Every coordinate of every vertex of the simplex is a short, as the reference's keys are
+// (q_i - 1 is the lowest a vertex takes, and the remainder is at most pd)
+template <int PD, typename T>
+__device__ __forceinline__ bool simplex_in_short_range(const Simplex<PD, T> &s) {
+    bool ok = true;
+#pragma unroll
+    for (int i = 0; i < PD; ++i)
+        ok = ok && ((s.q[i] - 1) * (PD + 1) >= -32768) && (s.q[i] * (PD + 1) + PD <= 32767) &&
+             s.q[i] > -40000 && s.q[i] < 40000;
+    return ok;
+}
+template <int PD, typename T>
+__device__ __forceinline__ void wide_keys_of(const Simplex<PD, T> &s, Key128 (&key)[PD + 1]) {
+#pragma unroll
+    for (int r = 0; r <= PD; ++r) {
+        int q[PD];
+        vertex_q<PD>(s, r, q);
+        key[r] = WideCodec<PD>::pack(q, r);
+    }
+}
+
 // ------------------------------------------------------------------------------------------------
 // Which point a thread works on.  Points that are neighbours in the image share lattice vertices,
 // and every duplicate that meets inside one wavefront is merged before it reaches memory, so a
@@ -410,6 +465,13 @@ __device__ __forceinline__ uint64_t lane_value(uint64_t x, int lane) {
     const uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)x, lane);
     const uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(x >> 32), lane);
     return ((uint64_t)hi << 32) | lo;
+}
+
+__device__ __forceinline__ Key128 lane_value(const Key128 &x, int lane) {
+    return Key128{lane_value(x.a, lane), lane_value(x.b, lane)};
+}
+__device__ __forceinline__ uint64_t lanes_equal(const Key128 &x, const Key128 &k) {
+    return lanes_equal(x.a, k.a) & lanes_equal(x.b, k.b);
 }
 
 // Lanes that hold the same value of `x` elect the lowest of them as leader.  Returns the leader's
@@ -549,6 +611,16 @@ __device__ __forceinline__ double wave_sums_to_quads_f64(bool member, const doub
     }
     return x;
 }
+
+// (keys of two words exist for the dimensions whose packed key has fields of less than 16 bits)
+#define PLK_DISPATCH_WIDE_PD(pd, CALL)            \
+    switch (pd) {                                 \
+        case 5: { constexpr int PD = 5; CALL; } break; \
+        case 6: { constexpr int PD = 6; CALL; } break; \
+        case 7: { constexpr int PD = 7; CALL; } break; \
+        case 8: { constexpr int PD = 8; CALL; } break; \
+        default: return hipErrorInvalidValue;     \
+    }
 
 #define PLK_DISPATCH_PD(pd, CALL)                 \
     switch (pd) {                                 \

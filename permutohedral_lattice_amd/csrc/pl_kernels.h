@@ -15,7 +15,8 @@ constexpr uint32_t kMaxCells = 1u << 28;   // cells are addressed by 32-bit byte
 // bits of Counters::flags
 enum : int {
     kFlagTableFull = 1,   // a probe sequence wrapped, or more vertices were created than the table may hold
-    kFlagKeyRange = 2,    // a lattice coordinate does not fit its field of the packed key
+    kFlagKeyRange = 2,    // a lattice coordinate does not fit its field of the key (packed key: the build
+                          // is repeated with keys of two words; those: it is no short)
     kFlagTileFull = 4,    // a workgroup of the merging build has more distinct keys than its LDS table holds
 };
 
@@ -204,12 +205,17 @@ hipError_t clear_table(uint64_t *cell_keys, uint32_t n_cells, hipStream_t s);
 // != 0 it numbers its vertices itself (Counters, CreatedLists, InBuildNumbering): no
 // number_vertices follows it, cell_values is not used, and neighbours() must be given the lists
 // when the build splatted.
+// wide_keys (pd >= 5, plain build only): keys of two words, for lattices whose coordinates do not
+// fit the packed key but are shorts, as the reference's keys are: cell_keys then holds two words
+// per cell (both all ones when empty), the lists two entries per vertex, and number_vertices,
+// neighbours and export_keys must be told.
 bool build_can_splat(int vd);
 hipError_t build(int pd, const PointFeatures &features, const PointMap &map, const ScaleFactor &scale,
                  uint64_t *cell_keys, uint32_t n_cells, Counters *counters, ReplayEntry *replay,
                  int xcd_aware, int splat_vd, const float *input,
                  int in_channels, float *cell_values, const CreatedLists &created_lists,
-                 const RegionSource &regions, const InBuildNumbering *numbering, hipStream_t s);
+                 const RegionSource &regions, const InBuildNumbering *numbering, bool wide_keys,
+                 hipStream_t s);
 
 // The build for double values: the same kernel on points.positions with points.scale; replay[]
 // receives the cells (and the weights rounded to float), points.weights[r*T+t] the weights.
@@ -217,7 +223,7 @@ hipError_t build_f64(int pd, const Points64 &points, const PointMap &map, uint64
                      uint32_t n_cells, Counters *counters, ReplayEntry *replay, int xcd_aware,
                      const CreatedLists &created_lists, const RegionSource &regions,
                      const InBuildNumbering *numbering, int splat_vd, const double *input,
-                     int in_channels, double *cell_values, hipStream_t s);
+                     int in_channels, double *cell_values, bool wide_keys, hipStream_t s);
 
 // Dense vertex numbers in the order of the build's workgroups (same map as the build):
 // cell_vertex[cell] := v, vertex_keys[v] := key, vertex_cell[v] := cell,
@@ -228,7 +234,7 @@ hipError_t build_f64(int pd, const Points64 &points, const PointMap &map, uint64
 hipError_t number_vertices(int pd, const PointMap &map, const CreatedLists &lists,
                            int *next_chunk_count, unsigned n_chunks, const VertexTables &vertices,
                            float *values, int vd, float *cell_values, Counters *counters, Counters *next_counters,
-                           HostStatus *host_status, hipStream_t s);
+                           HostStatus *host_status, bool wide_keys, hipStream_t s);
 
 // neighbours[a*max_vertices+v] := vertex indices of v's two neighbours along blur axis a, for v
 // below the vertex count; entries of absent neighbours keep their -1.
@@ -245,7 +251,7 @@ hipError_t neighbours(int pd, const VertexTables &vertices, const Counters *coun
                       const uint64_t *cell_keys, uint32_t n_cells, int launch_vertices,
                       const CreatedLists *foreign_rows, unsigned n_lists, void *values, int vd,
                       bool values_are_double, Counters *report, Counters *next_counters,
-                      HostStatus *host_status, hipStream_t s);
+                      HostStatus *host_status, bool wide_keys, hipStream_t s);
 
 hipError_t fill_zero(float *p, size_t n, hipStream_t s);
 
@@ -309,7 +315,7 @@ struct VertexNumbers {
     }
 };
 hipError_t export_keys(int pd, const uint64_t *vertex_keys, const VertexNumbers &numbers, short *keys,
-                       hipStream_t s);
+                       bool wide_keys, hipStream_t s);
 // out[d * words ..] := the row of the d-th vertex (rows of `words` floats)
 hipError_t export_values(const float *values, int words, const VertexNumbers &numbers, float *out,
                          hipStream_t s);

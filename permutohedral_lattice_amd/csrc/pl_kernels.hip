@@ -173,7 +173,10 @@ __device__ __forceinline__ uint64_t *cell_at(uint64_t *cell_keys, uint32_t cell)
 
 // T = double (SPLAT_VD == 0 only): positions, scale factors and the weights written are those of
 // `points64`; the replay rows then carry the cells only.
-template <int PD, int SPLAT_VD, typename T = float>
+// WIDE: keys of two words (Key128) in cells of two words; one cell per probe step, plain hashing.
+// A cell is claimed by swapping the first word in; its second word follows with a store, and a
+// lane that finds the first word of its key with the second still missing looks again.
+template <int PD, int SPLAT_VD, typename T = float, bool WIDE = false>
 __global__ __launch_bounds__(kBlock) void k_build(PointFeatures features, PointMap map,
                                                    ScaleFactor scale, uint64_t *cell_keys,
                                                    uint32_t mask, Counters *counters,
@@ -218,19 +221,23 @@ __global__ __launch_bounds__(kBlock) void k_build(PointFeatures features, PointM
     // and ranks they come from (twice as many registers) across it instead: have them now.
 #pragma unroll
     for (int r = 0; r < D1; ++r) asm volatile("" : "+v"(s.weight[r]));
-    const bool in_range = simplex_in_key_range<PD>(s);
+    const bool in_range = WIDE ? simplex_in_short_range<PD>(s) : simplex_in_key_range<PD>(s);
     if (valid && !in_range) atomicOr(&counters->flags, kFlagKeyRange);
     const bool active = valid && in_range;
 
     // Wavefront-level deduplication: each distinct key of the wavefront is inserted by one lane
     // (the lowest that holds it) and its cell is broadcast to the others.  Only leaders touch the
     // table.
-    uint64_t key[D1];
+    using Key = std::conditional_t<WIDE, Key128, uint64_t>;
+    Key key[D1];
     // (leader lanes are kept five to a register, six bits each: registers decide how many
     // wavefronts a CU holds)
     unsigned leaders[(D1 + 4) / 5] = {};
     auto leader_of = [&](int r) { return (int)((leaders[r / 5] >> (6 * (r % 5))) & 63u); };
-    vertex_keys_of<PD>(s, key);
+    if constexpr (WIDE)
+        wide_keys_of<PD>(s, key);
+    else
+        vertex_keys_of<PD>(s, key);
 #pragma unroll
     for (int r = 0; r < D1; ++r)
         leaders[r / 5] |= (unsigned)wave_leader_of_equal(key[r], active, lane) << (6 * (r % 5));
@@ -246,15 +253,70 @@ __global__ __launch_bounds__(kBlock) void k_build(PointFeatures features, PointM
         counters->region_per_unit = regions.per_unit;
     }
     uint32_t cell[D1];
-    uint64_t seen[D1];
     unsigned open = 0;      // bit r: this lane still has to place key r
     unsigned created = 0;   // bit r: this lane's swap made the vertex of rank r
 #pragma unroll
-    for (int r = 0; r < D1; ++r) {
+    for (int r = 0; r < D1; ++r)
         if (active && leader_of(r) == lane) open |= 1u << r;
-        cell[r] = cell_of_key<PD>(key[r], mask, regions);
-    }
     bool any_open = open != 0;
+    if constexpr (WIDE) {
+        // Rounds as below.  Words are read past the first-level cache: a second word may arrive
+        // while this lane waits for it.  A lane waits at most kWideWaits rounds in all for
+        // second words (the owner stores it right behind its swap), then reports a full table.
+        constexpr int kWideWaits = 1 << 16;
+        uint64_t *words = cell_keys;   // cell c: words 2c (first) and 2c+1 (second)
+        int waits = 0;
+#pragma unroll
+        for (int r = 0; r < D1; ++r) cell[r] = hash_key(key[r]) & mask;
+        for (uint32_t probe = 0; any_open && probe <= mask + 2u;) {
+            uint64_t first[D1], second[D1];
+#pragma unroll
+            for (int r = 0; r < D1; ++r) {
+                if ((open >> r) & 1u) {
+                    first[r] = __hip_atomic_load(words + 2 * (size_t)cell[r], __ATOMIC_RELAXED,
+                                                 __HIP_MEMORY_SCOPE_AGENT);
+                    second[r] = __hip_atomic_load(words + 2 * (size_t)cell[r] + 1, __ATOMIC_RELAXED,
+                                                  __HIP_MEMORY_SCOPE_AGENT);
+                }
+            }
+            bool swapped[D1];
+#pragma unroll
+            for (int r = 0; r < D1; ++r) {
+                swapped[r] = false;
+                if (((open >> r) & 1u) && first[r] == kEmptyCell) {
+                    first[r] = atomicCAS((unsigned long long *)(words + 2 * (size_t)cell[r]),
+                                         (unsigned long long)kEmptyCell, (unsigned long long)key[r].a);
+                    swapped[r] = first[r] == kEmptyCell;
+                    second[r] = kEmptyCell;   // (of a cell that another lane took meanwhile: look again)
+                }
+            }
+            bool stepped = false, waited = false;
+#pragma unroll
+            for (int r = 0; r < D1; ++r) {
+                if (!((open >> r) & 1u)) continue;
+                if (swapped[r]) {
+                    __hip_atomic_store(words + 2 * (size_t)cell[r] + 1, key[r].b, __ATOMIC_RELAXED,
+                                       __HIP_MEMORY_SCOPE_AGENT);
+                    created |= 1u << r;
+                    open &= ~(1u << r);
+                } else if (first[r] == key[r].a && second[r] == key[r].b) {
+                    open &= ~(1u << r);           // already there
+                } else if (first[r] == key[r].a && second[r] == kEmptyCell) {
+                    waited = true;                // its second word is on its way, or it is our key's
+                } else {
+                    cell[r] = (cell[r] + 1u) & mask;
+                    stepped = true;
+                }
+            }
+            any_open = open != 0;
+            if (stepped) ++probe;
+            if (waited && ++waits > kWideWaits) break;
+        }
+    }
+    uint64_t seen[D1];
+    if constexpr (!WIDE) {
+#pragma unroll
+    for (int r = 0; r < D1; ++r) cell[r] = cell_of_key<PD>(key[r], mask, regions);
     for (uint32_t probe = 0; any_open && probe <= mask + 2u; ++probe) {
 #pragma unroll
         for (int r = 0; r < D1; ++r)
@@ -276,6 +338,7 @@ __global__ __launch_bounds__(kBlock) void k_build(PointFeatures features, PointM
             }
         }
         any_open = open != 0;
+    }
     }
     if (any_open) atomicOr(&counters->flags, kFlagTableFull);
 
@@ -301,8 +364,16 @@ __global__ __launch_bounds__(kBlock) void k_build(PointFeatures features, PointM
 #pragma unroll
         for (int r = 0; r < D1; ++r) {
             if ((created >> r) & 1u) {
-                created_lists.entries[list + base + offset[r]] =
-                    make_uint4((uint32_t)key[r], (uint32_t)(key[r] >> 32), cell[r], 0u);
+                if constexpr (WIDE) {
+                    // (two entries per vertex: the key, then the cell)
+                    uint4 *entry = created_lists.entries + list + 2 * (size_t)(base + offset[r]);
+                    entry[0] = make_uint4((uint32_t)key[r].a, (uint32_t)(key[r].a >> 32),
+                                          (uint32_t)key[r].b, (uint32_t)(key[r].b >> 32));
+                    entry[1] = make_uint4(cell[r], 0u, 0u, 0u);
+                } else {
+                    created_lists.entries[list + base + offset[r]] =
+                        make_uint4((uint32_t)key[r], (uint32_t)(key[r] >> 32), cell[r], 0u);
+                }
             }
         }
         if (lane == 0 && atomicAdd(&waves_done, 1) == kBlock / 64 - 1) {
@@ -775,7 +846,9 @@ __global__ __launch_bounds__(kBlock) void k_build_tile(PointFeatures features, P
 // from cell_values, which the fused build+splat filled, or zeroed), and (-1, -1) for all its
 // neighbour entries.  The last wavefront knows the total: it publishes it to the device counters
 // and to host-visible memory and clears what the next build will count in.
-template <int D1>
+// WIDE: the build had keys of two words: two entries per vertex (key, then cell), and
+// vertex_keys holds two words per vertex.
+template <int D1, bool WIDE = false>
 __global__ __launch_bounds__(64) void k_number_vertices(CreatedLists lists, int *next_chunk_count,
                                                         unsigned n_chunks,
                                                         VertexTables vertices, float *values, int vd,
@@ -800,7 +873,7 @@ __global__ __launch_bounds__(64) void k_number_vertices(CreatedLists lists, int 
     const unsigned sibling = chunk * kBlocksPerChunk + lane;
     int sibling_count = lists.block_count[sibling < b ? sibling : b];
     const int count = lists.block_count[b];
-    uint4 first_entry = lists.entries[list + lane];
+    uint4 first_entry = lists.entries[list + (WIDE ? 2 * lane + 1 : lane)];
     asm volatile("" : "+v"(before), "+v"(sibling_count), "+v"(first_entry.x), "+v"(first_entry.y),
                  "+v"(first_entry.z));
     before = has_chunk ? before : 0;
@@ -830,12 +903,16 @@ __global__ __launch_bounds__(64) void k_number_vertices(CreatedLists lists, int 
     }
 
     for (int i = lane; i < count; i += 64) {
-        const uint4 entry = i < 64 ? first_entry : lists.entries[list + i];
-        const int cell = (int)entry.z;
+        const uint4 entry =
+            i < 64 ? first_entry : lists.entries[list + (WIDE ? 2 * (size_t)i + 1 : (size_t)i)];
+        const int cell = WIDE ? (int)entry.x : (int)entry.z;
         const int v = before + i;
         if (v < max_vertices) {
             vertices.cell_vertex[cell] = v;
-            vertices.vertex_keys[v] = ((uint64_t)entry.y << 32) | entry.x;
+            if constexpr (WIDE)
+                reinterpret_cast<uint4 *>(vertices.vertex_keys)[v] = lists.entries[list + 2 * (size_t)i];
+            else
+                vertices.vertex_keys[v] = ((uint64_t)entry.y << 32) | entry.x;
             vertices.vertex_cell[v] = cell;
             if (cell_values && vd == 4) {
                 float4 *from = reinterpret_cast<float4 *>(cell_values) + cell;
@@ -902,7 +979,8 @@ __device__ __forceinline__ void add_foreign_rows(const CreatedLists &lists, unsi
     }
 }
 
-template <int PD>
+// WIDE: keys and cells of two words (see k_build), one cell per probe step, plain hashing.
+template <int PD, bool WIDE = false>
 __global__ __launch_bounds__(kBlock) void k_neighbours(VertexTables vertices,
                                                         const Counters *counters,
                                                         const uint64_t *__restrict__ cell_keys,
@@ -949,7 +1027,12 @@ __global__ __launch_bounds__(kBlock) void k_neighbours(VertexTables vertices,
     const int v = (int)(walk.first + i);
 
     int q[PD], r;
-    KeyCodec<PD>::unpack(vertices.vertex_keys[v], q, r);
+    if constexpr (WIDE) {
+        const ulonglong2 k = reinterpret_cast<const ulonglong2 *>(vertices.vertex_keys)[v];
+        WideCodec<PD>::unpack(Key128{k.x, k.y}, q, r);
+    } else {
+        KeyCodec<PD>::unpack(vertices.vertex_keys[v], q, r);
+    }
     int qp[PD];
     const bool wrap_up = (r == PD);
 #pragma unroll
@@ -957,10 +1040,23 @@ __global__ __launch_bounds__(kBlock) void k_neighbours(VertexTables vertices,
         const bool on_axis = (i == a);
         qp[i] = q[i] + (wrap_up ? (on_axis ? 0 : 1) : (on_axis ? -1 : 0));
     }
-    const uint64_t want = KeyCodec<PD>::pack(qp, wrap_up ? 0 : r + 1);
-    uint32_t h = cell_of_key<PD>(want, mask, regions);
     int u = -1;
-    for (uint32_t index = 0; index <= (mask >> 1) + 1u; ++index) {
+    if constexpr (WIDE) {
+        const Key128 want = WideCodec<PD>::pack(qp, wrap_up ? 0 : r + 1);
+        uint32_t h = hash_key(want) & mask;
+        for (uint32_t index = 0; index <= mask; ++index) {
+            const ulonglong2 cur = reinterpret_cast<const ulonglong2 *>(cell_keys)[h];
+            if (cur.x == want.a && cur.y == want.b) {
+                u = vertices.cell_vertex[h];
+                break;
+            }
+            if (cur.x == kEmptyCell) break;
+            h = (h + 1u) & mask;
+        }
+    }
+    const uint64_t want = WIDE ? 0ull : KeyCodec<PD>::pack(qp, wrap_up ? 0 : r + 1);
+    uint32_t h = WIDE ? 0u : cell_of_key<PD>(want, mask, regions);
+    for (uint32_t index = 0; !WIDE && index <= (mask >> 1) + 1u; ++index) {
         const ulonglong2 cur = *reinterpret_cast<const ulonglong2 *>(cell_keys + h);
         if (cur.x == want || (cur.x != kEmptyCell && cur.y == want)) {
             u = vertices.cell_vertex[cur.x == want ? h : h + 1u];
@@ -1706,13 +1802,18 @@ __global__ __launch_bounds__(kBlock) void k_debug_simplex(const float *__restric
 }
 
 // The debug exports count the vertices densely, segment after segment (VertexNumbers).
-template <int PD>
+template <int PD, bool WIDE>
 __global__ __launch_bounds__(kBlock) void k_export_keys(const uint64_t *__restrict__ vertex_keys,
                                                          VertexNumbers numbers, short *keys) {
     const unsigned d = blockIdx.x * kBlock + threadIdx.x;
     if (d >= numbers.total) return;
     int q[PD], r;
-    KeyCodec<PD>::unpack(vertex_keys[numbers.vertex_of(d)], q, r);
+    if constexpr (WIDE) {
+        const ulonglong2 k = reinterpret_cast<const ulonglong2 *>(vertex_keys)[numbers.vertex_of(d)];
+        WideCodec<PD>::unpack(Key128{k.x, k.y}, q, r);
+    } else {
+        KeyCodec<PD>::unpack(vertex_keys[numbers.vertex_of(d)], q, r);
+    }
 #pragma unroll
     for (int i = 0; i < PD; ++i) keys[(size_t)d * PD + i] = (short)(q[i] * (PD + 1) + r);
 }
@@ -1849,8 +1950,10 @@ hipError_t build(int pd, const PointFeatures &features, const PointMap &map, con
                  uint64_t *cell_keys, uint32_t n_cells, Counters *counters, ReplayEntry *replay,
                  int xcd_aware, int splat_vd, const float *input,
                  int in_channels, float *cell_values, const CreatedLists &created_lists,
-                 const RegionSource &regions, const InBuildNumbering *numbering, hipStream_t s) {
+                 const RegionSource &regions, const InBuildNumbering *numbering, bool wide_keys,
+                 hipStream_t s) {
     if (map.n_blocks == 0) return hipSuccess;
+    if (wide_keys && numbering) return hipErrorInvalidValue;
     const bool merge_in_workgroup = numbering != nullptr;
     const InBuildNumbering in_build = numbering ? *numbering : InBuildNumbering{};
 #define PLK_BUILD_ARGS                                                                             \
@@ -1861,6 +1964,9 @@ hipError_t build(int pd, const PointFeatures &features, const PointMap &map, con
     if (merge_in_workgroup)                                                                        \
         PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_build_tile<PD, SPLAT_VD>), PLK_BUILD_ARGS,       \
                                                in_build))                                          \
+    else if (wide_keys)                                                                            \
+        PLK_DISPATCH_WIDE_PD(pd, hipLaunchKernelGGL((k_build<PD, SPLAT_VD, float, true>),          \
+                                                    PLK_BUILD_ARGS))                               \
     else                                                                                           \
         PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_build<PD, SPLAT_VD>), PLK_BUILD_ARGS))
     switch (splat_vd) {
@@ -1879,8 +1985,9 @@ hipError_t build_f64(int pd, const Points64 &points, const PointMap &map, uint64
                      uint32_t n_cells, Counters *counters, ReplayEntry *replay, int xcd_aware,
                      const CreatedLists &created_lists, const RegionSource &regions,
                      const InBuildNumbering *numbering, int splat_vd, const double *input,
-                     int in_channels, double *cell_values, hipStream_t s) {
+                     int in_channels, double *cell_values, bool wide_keys, hipStream_t s) {
     if (map.n_blocks == 0) return hipSuccess;
+    if (wide_keys && numbering) return hipErrorInvalidValue;
     const bool merge_in_workgroup = numbering != nullptr;
     const InBuildNumbering in_build = numbering ? *numbering : InBuildNumbering{};
     if (splat_vd && !merge_in_workgroup) return hipErrorInvalidValue;
@@ -1899,6 +2006,8 @@ hipError_t build_f64(int pd, const Points64 &points, const PointMap &map, uint64
             case 4: PLK_BUILD(4); break;
             default: return hipErrorInvalidValue;
         }
+    } else if (wide_keys) {
+        PLK_DISPATCH_WIDE_PD(pd, hipLaunchKernelGGL((k_build<PD, 0, double, true>), PLK_BUILD_ARGS))
     } else {
         PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_build<PD, 0, double>), PLK_BUILD_ARGS))
     }
@@ -1911,11 +2020,19 @@ hipError_t number_vertices(int pd, const PointMap &map, const CreatedLists &list
                            int *next_chunk_count, unsigned n_chunks, const VertexTables &vertices,
                            float *values,
                            int vd, float *cell_values, Counters *counters, Counters *next_counters,
-                           HostStatus *host_status, hipStream_t s) {
+                           HostStatus *host_status, bool wide_keys, hipStream_t s) {
     if (map.n_blocks == 0) return hipErrorInvalidValue;
-    PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_number_vertices<PD + 1>), dim3(map.n_blocks), dim3(64),
-                                           0, s, lists, next_chunk_count, n_chunks, vertices, values, vd,
-                                           cell_values, counters, next_counters, host_status));
+    if (wide_keys) {
+        PLK_DISPATCH_WIDE_PD(pd, hipLaunchKernelGGL((k_number_vertices<PD + 1, true>), dim3(map.n_blocks),
+                                               dim3(64), 0, s, lists, next_chunk_count, n_chunks,
+                                               vertices, values, vd, cell_values, counters,
+                                               next_counters, host_status));
+    } else {
+        PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_number_vertices<PD + 1>), dim3(map.n_blocks),
+                                               dim3(64), 0, s, lists, next_chunk_count, n_chunks,
+                                               vertices, values, vd, cell_values, counters,
+                                               next_counters, host_status));
+    }
     return hipGetLastError();
 }
 
@@ -1923,18 +2040,25 @@ hipError_t neighbours(int pd, const VertexTables &vertices, const Counters *coun
                       const uint64_t *cell_keys, uint32_t n_cells, int launch_vertices,
                       const CreatedLists *foreign_rows, unsigned n_lists, void *values, int vd,
                       bool values_are_double, Counters *report, Counters *next_counters,
-                      HostStatus *host_status, hipStream_t s) {
+                      HostStatus *host_status, bool wide_keys, hipStream_t s) {
     if (vertices.max_vertices <= 0) return hipErrorInvalidValue;
     const size_t items = (size_t)(pd + 1) * (size_t)launch_vertices;
     const unsigned foreign_blocks =
         foreign_rows ? (blocks_for(n_lists, kBlock / 64) + kXcds - 1u) / kXcds * kXcds : 0u;
-    PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_neighbours<PD>),
-                                           dim3(foreign_blocks + vertex_blocks(items)),
-                                           dim3(kBlock), 0, s, vertices, counters, cell_keys,
-                                           n_cells - 1u, foreign_blocks,
-                                           foreign_rows ? *foreign_rows : CreatedLists{}, n_lists,
-                                           values, vd, values_are_double ? 1 : 0, report,
-                                           next_counters, host_status));
+#define PLK_NEIGHBOURS(WIDE, DISPATCH)                                                             \
+    DISPATCH(pd, hipLaunchKernelGGL((k_neighbours<PD, WIDE>),                                      \
+                                           dim3(foreign_blocks + vertex_blocks(items)),            \
+                                           dim3(kBlock), 0, s, vertices, counters, cell_keys,      \
+                                           n_cells - 1u, foreign_blocks,                           \
+                                           foreign_rows ? *foreign_rows : CreatedLists{}, n_lists, \
+                                           values, vd, values_are_double ? 1 : 0, report,          \
+                                           next_counters, host_status))
+    if (wide_keys) {
+        PLK_NEIGHBOURS(true, PLK_DISPATCH_WIDE_PD);
+    } else {
+        PLK_NEIGHBOURS(false, PLK_DISPATCH_PD);
+    }
+#undef PLK_NEIGHBOURS
     return hipGetLastError();
 }
 
@@ -2174,11 +2298,16 @@ hipError_t debug_simplex(int pd, const float *positions, int N, const ScaleFacto
 }
 
 hipError_t export_keys(int pd, const uint64_t *vertex_keys, const VertexNumbers &numbers, short *keys,
-                       hipStream_t s) {
+                       bool wide_keys, hipStream_t s) {
     const unsigned M = numbers.total;
     if (M == 0) return hipSuccess;
-    PLK_DISPATCH_PD(pd, hipLaunchKernelGGL(k_export_keys<PD>, dim3(blocks_for((size_t)M)),
-                                           dim3(kBlock), 0, s, vertex_keys, numbers, keys));
+    if (wide_keys) {
+        PLK_DISPATCH_WIDE_PD(pd, hipLaunchKernelGGL((k_export_keys<PD, true>), dim3(blocks_for((size_t)M)),
+                                               dim3(kBlock), 0, s, vertex_keys, numbers, keys));
+    } else {
+        PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_export_keys<PD, false>), dim3(blocks_for((size_t)M)),
+                                               dim3(kBlock), 0, s, vertex_keys, numbers, keys));
+    }
     return hipGetLastError();
 }
 

@@ -209,3 +209,22 @@ def test_key_range_overflow_is_reported():
     lat.filter(out, dev(np.ones((n, 1))), dev(pos), False)
     torch.cuda.synchronize()
     assert np.abs(host(out) - 1.0).max() <= F64_TOL
+
+
+def test_coordinates_within_the_reference_short_keys_are_filtered_in_double():
+    """Lattice coordinates beyond the packed key's 12 bits (pd = 5) but within the reference's
+    short keys (src/PermutohedralLatticeCPU.h:297-304): keys of two words, same lattice and
+    outputs as the CPU path for T = double."""
+    rng = np.random.default_rng(205)
+    n, pd = 2500, 5
+    pos = rng.uniform(0.0, 1.0, (n, pd))
+    pos[:, 0] = rng.uniform(0.0, 7500.0, n)
+    pos[: n // 2, 1:] = pos[n // 2 : 2 * (n // 2), 1:]
+    pos[: n // 2, 0] = pos[n // 2 : 2 * (n // 2), 0] + rng.uniform(0.0, 0.3, n // 2)
+    val = rng.uniform(0, 1, (n, 2))
+    cpu = oracle.Lattice(pd, 3, n, dtype=np.float64)
+    want = cpu.filter(val, pos)
+    got, lat = gpu_filter(pd, 3, pos, val)
+    assert lat.num_vertices == cpu.num_vertices
+    assert (sorted_keys(host(lat.debug_keys()))[0] == sorted_keys(cpu.keys())[0]).all()
+    assert np.abs(got - want).max() <= F64_TOL

@@ -436,7 +436,8 @@ def test_all_points_in_one_simplex_collide_on_every_vertex():
 
 
 def test_coordinates_beyond_the_packed_key_range_are_reported():
-    """pd=5 packs 12 bits per coordinate; positions far outside must fail loudly, not wrap."""
+    """Lattice coordinates beyond a short, where the reference's own keys wrap, must fail loudly
+    (pd=5 packs 12 bits per coordinate and goes to keys of two words first)."""
     n = 256
     pos = np.full((n, 5), 1.0, np.float32)
     pos[7, 0] = 30000.0
@@ -452,6 +453,38 @@ def test_coordinates_beyond_the_packed_key_range_are_reported():
     got, _ = gpu_filter(4, 2, pos4, val)
     check_integers(4, pos4)
     assert_float_parity(got, oracle.Lattice(4, 2, n).filter(val, pos4))
+
+
+@pytest.mark.parametrize("pd,reach", [(5, 7500.0), (6, 6400.0), (8, 5000.0)])
+def test_coordinates_within_the_reference_short_keys_are_filtered(pd, reach):
+    """The reference's keys are shorts at every pd (src/PermutohedralLatticeCPU.h:297-304); the
+    packed 64-bit key has 12, 10 and 7 bits per coordinate at pd = 5, 6, 8.  Lattice coordinates
+    beyond those but within a short are filtered with keys of two words: same vertex count, same
+    keys, same outputs as the CPU path; and the handle goes on working for positions near zero."""
+    rng = np.random.default_rng(100 + pd)
+    n = 3000
+    pos = rng.uniform(0.0, 1.0, (n, pd)).astype(np.float32)
+    pos[:, 0] = rng.uniform(0.0, reach, n).astype(np.float32)      # far out along one feature
+    pos[: n // 2, 1:] = pos[n // 2 : 2 * (n // 2), 1:]              # and vertices that are shared
+    pos[: n // 2, 0] = pos[n // 2 : 2 * (n // 2), 0] + rng.uniform(0.0, 0.3, n // 2).astype(np.float32)
+    o = oracle.dump_simplex(pos)
+    coords = o["keys"].astype(np.int64)
+    beyond_packed = (1 << (min(16, 60 // pd) - 1)) * (pd + 1)
+    assert np.abs(coords).max() > beyond_packed and np.abs(o["rem0"].astype(np.int64)).max() < 32000
+    val = rng.uniform(0, 1, (n, 2)).astype(np.float32)
+    cpu = oracle.Lattice(pd, 3, n)
+    want = cpu.filter(val, pos)
+    got, lat = gpu_filter(pd, 3, pos, val)
+    assert lat.num_vertices == cpu.num_vertices
+    assert (sorted_keys(host(lat.debug_keys()))[0] == sorted_keys(cpu.keys())[0]).all()
+    assert_float_parity(got, want)
+    got_r, _ = gpu_filter(pd, 3, pos, val, reverse=True, lattice=lat)
+    assert_float_parity(got_r, oracle.Lattice(pd, 3, n).filter(val, pos, reverse=True))
+    near = rng.uniform(0.0, 4.0, (n, pd)).astype(np.float32)
+    got_n, _ = gpu_filter(pd, 3, near, val, lattice=lat)
+    cpu_n = oracle.Lattice(pd, 3, n)
+    assert_float_parity(got_n, cpu_n.filter(val, near))
+    assert lat.num_vertices == cpu_n.num_vertices
 
 
 def test_handle_filters_correctly_after_a_refused_call_that_also_overflowed_its_table():
