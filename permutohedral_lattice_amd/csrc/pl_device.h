@@ -227,12 +227,15 @@ __device__ __forceinline__ void enclosing_simplex(const float (&pos)[PD], const 
     int qsum = 0;
 #pragma unroll
     for (int i = 0; i < D1; ++i) {
+        // (The reference rounds between ceil(v) and floor(v) times pd+1.  The ceiling is the
+        // floor plus one unless v is whole, and then both of its candidates are the same point:
+        // one step above the floor's multiple decides the same, without a second rounding.)
         const float v = (float)((double)el[i] * inv_d1);
-        const float cu = ceilf(v), fl = floorf(v);
-        const float above = cu * (float)D1, below = fl * (float)D1;
+        const float fl = floorf(v);
+        const float below = fl * (float)D1, above = below + (float)D1;
         const bool up = (above - el[i]) < (el[i] - below);
         rem[i] = up ? above : below;
-        s.q[i] = (int)(up ? cu : fl);
+        s.q[i] = (int)fl + (up ? 1 : 0);
         qsum += s.q[i];
     }
 
@@ -474,6 +477,25 @@ __device__ __forceinline__ uint64_t lanes_equal(const Key128 &x, const Key128 &k
     return lanes_equal(x.a, k.a) & lanes_equal(x.b, k.b);
 }
 
+// x := value (the same in all lanes) in the lanes of `lanes`, which must be among the executing
+// ones.  One v_mov under a narrowed exec mask: as `lanes ? value : x` the compiler spends a move of
+// the value into a vector register and a select.
+__device__ __forceinline__ void set_in_lanes(int &x, uint64_t lanes, int value) {
+    uint64_t saved;
+    asm volatile(
+        "s_mov_b64 %1, exec\n\t"
+        "s_mov_b64 exec, %2\n\t"
+        "v_mov_b32 %0, %3\n\t"
+        "s_mov_b64 exec, %1"
+        : "+v"(x), "=&s"(saved)
+        : "s"(lanes), "s"(value));
+}
+// Lanes in a mask, counted in 32-bit halves (the count of 64 bits is carried as a 64-bit number,
+// and a comparison with it then runs on the vector unit)
+__device__ __forceinline__ int lanes_in(uint64_t mask) {
+    return __builtin_popcount((uint32_t)mask) + __builtin_popcount((uint32_t)(mask >> 32));
+}
+
 // Lanes that hold the same value of `x` elect the lowest of them as leader.  Returns the leader's
 // lane; inactive lanes get their own.  One iteration per distinct value in the wavefront, each a
 // v_readlane of the first unassigned lane's value, a compare and a ballot.
@@ -485,7 +507,7 @@ __device__ __forceinline__ int wave_leader_of_equal(T x, bool active, int lane) 
     while (remaining) {
         const int first = __builtin_ctzll(remaining);
         const uint64_t same = lanes_equal(x, lane_value(x, first)) & among;
-        if (lane_in(same)) leader = first;
+        set_in_lanes(leader, same, first);
         remaining &= ~same;
     }
     return leader;
@@ -500,9 +522,9 @@ __device__ __forceinline__ int wave_leader_of_equal(T x, bool active, int lane, 
     while (remaining) {
         const int first = __builtin_ctzll(remaining);
         const uint64_t same = lanes_equal(x, lane_value(x, first)) & among;
-        if (lane_in(same)) leader = first;
+        set_in_lanes(leader, same, first);
         remaining &= ~same;
-        if ((int)__builtin_popcountll(same) <= small_size) small |= same;
+        if (lanes_in(same) <= small_size) small |= same;
     }
     return leader;
 }

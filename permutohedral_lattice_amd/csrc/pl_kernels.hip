@@ -512,6 +512,8 @@ __global__ __launch_bounds__(kBlock) void k_build_tile(PointFeatures features, P
             const int leader = wave_leader_of_equal(key[r], active, lane, kSmallGroup, small[r]);
             leaders[r / 5] |= (unsigned)leader << (6 * (r % 5));
             if (active && leader == lane) open |= 1u << r;
+            // (a cheaper hash -- three 24-bit multiplies instead of three 32-bit ones -- spread the
+            // keys of a tile worse and cost 9 us of probing for the 1 us it saved)
             slot[r] = (int)((hash_key(key[r]) >> 20) & (kTileSlots - 1));
         }
         bool any_open = open != 0;
@@ -572,6 +574,8 @@ __global__ __launch_bounds__(kBlock) void k_build_tile(PointFeatures features, P
                 }
             } else {
                 const QuadTerms quad = quad_terms<VD>(term, lane);
+                // (one group per turn: two side by side, to overlap their chains of cross-lane
+                // additions, cost more for the odd group out than they gain)
                 while (remaining) {
                     const int first = __builtin_ctzll(remaining);
                     const uint64_t group = lanes_equal(leader, first) & among;
