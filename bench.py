@@ -482,6 +482,10 @@ def main():
     ap.add_argument("--headline-only", action="store_true",
                     help="only the timed steps and the per-stage timing (what a rocprofv3 run of "
                          "this file should see): no side legs, no CPU baseline")
+    ap.add_argument("--configs-only", action="store_true",
+                    help="only the leg that runs every BASELINE configuration at full size, without "
+                         "the CPU reference (what a rocprofv3 run for the kernels of those "
+                         "configurations should see); prints that leg's record")
     ap.add_argument("--calibrate-copy-mib", type=int, default=0,
                     help="only run device-to-device copies of this many MiB (a kernel of known "
                          "traffic, for scaling rocprofv3's FETCH_SIZE / WRITE_SIZE) and exit")
@@ -506,6 +510,9 @@ def main():
         torch.cuda.synchronize()
         print(json.dumps({"calibration": "5 x dst.copy_(src), float32", "bytes_read_per_copy": nbytes,
                           "bytes_written_per_copy": nbytes}))
+        return
+    if args.configs_only:
+        print(json.dumps({"configs": run_configs(args, pla, synth, False)}))
         return
     side = args.size
     n, pd, vd = side * side, 5, 4
