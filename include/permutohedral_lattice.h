@@ -67,10 +67,16 @@ typedef enum pl_option {
                                the keys and sums of its tile in LDS before they go to the hash table;
                                0: every wavefront goes to the table itself (same results; for
                                measuring the difference) */
-    PL_OPT_STOP_AFTER = 8   /* 0 (default): a filter or apply runs to the end.  1: it ends behind the
+    PL_OPT_STOP_AFTER = 8,  /* 0 (default): a filter or apply runs to the end.  1: it ends behind the
                                splat, 2: behind the blur; the output is then not written and
                                pl_debug_values gives the vertex values of that stage (for checking the
                                stages one by one against src/PermutohedralLatticeCPU.h:306-317, 362-415) */
+    PL_OPT_ORDER_POINTS = 9 /* 1 (default): points that are a plain list (no grid given or found, at
+                               least 4096 of them) are worked on in an order in which neighbours in
+                               space are neighbours in the list, found anew by every build from the
+                               first two features, so that the workgroups of the build can merge their
+                               keys as for an image (PL_OPT_MERGE_TILES); 0: in the order of the list
+                               (same results up to the order of float additions) */
 } pl_option;
 
 /* 1 when a lattice can be built for these dimensions, else 0.
@@ -158,7 +164,10 @@ typedef enum pl_info {
                                   when every wavefront went to the table itself (no grid, or a tile with
                                   too many distinct keys switched merging off for a while) */
     PL_INFO_TABLE_CELLS = 2,   /* hash cells the last build used */
-    PL_INFO_SCRATCH_BYTES = 3  /* device memory the handle holds for its tables and per-point rows */
+    PL_INFO_SCRATCH_BYTES = 3, /* device memory the handle holds for its tables and per-point rows */
+    PL_INFO_FOREIGN_ROWS = 4   /* when the last build numbered its vertices itself: how many rows of sums
+                                  its workgroups held for vertices that other workgroups created (an
+                                  estimate from every eighth workgroup); else -1 */
 } pl_info;
 int pl_get_info(pl_handle h, int what, long *value);
 

@@ -25,7 +25,8 @@ PL_OPT_NORMALIZE, PL_OPT_PROFILE, PL_OPT_TABLE_CELLS, PL_OPT_XCD_AWARE, PL_OPT_P
 PL_OPT_GUESS_GRID = 6
 PL_OPT_MERGE_TILES = 7
 PL_OPT_STOP_AFTER = 8
-PL_INFO_BUILD_MERGED, PL_INFO_TABLE_CELLS, PL_INFO_SCRATCH_BYTES = 1, 2, 3
+PL_OPT_ORDER_POINTS = 9
+PL_INFO_BUILD_MERGED, PL_INFO_TABLE_CELLS, PL_INFO_SCRATCH_BYTES, PL_INFO_FOREIGN_ROWS = 1, 2, 3, 4
 
 # every symbol include/permutohedral_lattice.h declares
 EXPORTS = (

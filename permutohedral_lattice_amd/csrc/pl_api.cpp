@@ -133,6 +133,7 @@ struct pl_lattice {
     // the last such build of these points held so many rows of sums for vertices of other
     // workgroups that adding them afterwards, an atomic each, outweighs the numbering pass.
     bool numbering_pass_pays = false;
+    long foreign_rows = -1;            // of the last build (an estimate from a sample); -1: it listed none
     bool built = false;                // a build has been enqueued and, if verified, fitted
     bool verified = false;             // its status has been read on the host
     bool replay_holds_cells = false;
@@ -157,6 +158,14 @@ struct pl_lattice {
     bool guess_grid = true;
     bool grid_guessed = false;             // a guess has been made (whatever came out)
     plk::GridGuess *d_guess = nullptr;
+    // A plain list of points (no grid given or found) is worked on in an order in which
+    // neighbours in space are neighbours in the list (plk::order_by_locality), made anew by every
+    // build, so that the merging build serves it too
+    bool order_points = true;              // option
+    int *point_order = nullptr;            // [N]
+    unsigned *locality_words = nullptr;    // boxes, range of feature 0, counts and firsts of the bins
+    uint2 *bin_rank = nullptr;             // [N]
+    int order_capacity = 0;
     hipEvent_t ev[EV_COUNT] = {};
     bool ev_recorded[EV_COUNT] = {};
 
@@ -271,6 +280,38 @@ int ensure_replay(pl_lattice *h, bool wide) {
     return PL_OK;
 }
 
+// The arrays of the ordering pass for a plain list of N points
+plk::LocalityScratch locality_scratch(const pl_lattice *h) {
+    const unsigned max_bins = plk::locality_bins_for(h->N);
+    plk::LocalityScratch scratch{};
+    constexpr size_t box_words = 4 * plk::kLocalityBoxRows;
+    scratch.partial_boxes = reinterpret_cast<float4 *>(h->locality_words);
+    scratch.range0 = reinterpret_cast<float *>(h->locality_words + box_words);
+    scratch.bin_count = h->locality_words + box_words + 4;
+    scratch.bin_first = h->locality_words + box_words + 4 + max_bins;
+    scratch.bin_rank = h->bin_rank;
+    scratch.max_bins = max_bins;
+    return scratch;
+}
+
+int ensure_order(pl_lattice *h) {
+    if (h->point_order && h->order_capacity >= h->N) return PL_OK;
+    PL_HIP(hipStreamSynchronize(h->stream));
+    h->dfree(h->point_order);
+    h->dfree(h->locality_words);
+    h->dfree(h->bin_rank);
+    h->order_capacity = 0;
+    const size_t words = 4 * plk::kLocalityBoxRows + 4 + 2 * (size_t)plk::locality_bins_for(h->N);
+    h->point_order = (int *)h->dmalloc(sizeof(int) * (size_t)h->N);
+    h->locality_words = (unsigned *)h->dmalloc(sizeof(unsigned) * words);
+    h->bin_rank = (uint2 *)h->dmalloc(sizeof(uint2) * (size_t)h->N);
+    if (!h->point_order || !h->locality_words || !h->bin_rank) return PL_ENOMEM;
+    // (the pass leaves its counts zero for the next call)
+    PL_HIP(plk::fill_zero(reinterpret_cast<float *>(h->locality_words), words, h->stream));
+    h->order_capacity = h->N;
+    return PL_OK;
+}
+
 uint32_t initial_cells(const pl_lattice *h) {
     uint64_t want;
     if (h->forced_cells > 0) {
@@ -308,8 +349,20 @@ int enqueue_build(pl_lattice *h, const plk::PointFeatures &features, const doubl
     rc = ensure_replay(h, wide);
     if (rc != PL_OK) return rc;
     // tiles of an image share most of their vertices among their four wavefronts
-    const bool merge = h->merge_tiles && h->tiles_off_for == 0 && h->map.mode != 0 && !wide;
+    const bool merge_allowed = h->merge_tiles && h->tiles_off_for == 0 && !wide;
     if (h->tiles_off_for > 0 && !wide) h->tiles_off_for -= 1;
+    // a plain list is put in an order that gives its workgroups such tiles
+    if (h->map.mode <= 1) {
+        const bool ordered = merge_allowed && h->order_points && h->N >= 4096 &&
+                             (positions64 || features.positions);
+        if (ordered) {
+            rc = ensure_order(h);
+            if (rc != PL_OK) return rc;
+        }
+        h->map.mode = ordered ? 1 : 0;
+        h->map.order = ordered ? h->point_order : nullptr;
+    }
+    const bool merge = merge_allowed && h->map.mode != 0;
     h->last_build_merged = merge;
     // (a lattice of doubles splats in its build only in the merging kernel)
     const bool fused = splat_input && plk::build_can_splat(h->vd) && (!h->f64 || merge);
@@ -325,6 +378,10 @@ int enqueue_build(pl_lattice *h, const plk::PointFeatures &features, const doubl
         h->cell_values_clean = true;
     }
     h->mark(EV_T0);
+    if (h->map.mode == 1)
+        PL_HIP(plk::order_by_locality(h->f64 ? nullptr : features.positions,
+                                      h->f64 ? positions64 : nullptr, h->N, h->pd,
+                                      locality_scratch(h), h->point_order, h->stream));
     if (!h->table_clean || cells != h->n_cells) {
         PL_HIP(plk::clear_table(h->cell_keys, wide ? 2 * cells : cells, h->stream));
     }
@@ -352,6 +409,8 @@ int enqueue_build(pl_lattice *h, const plk::PointFeatures &features, const doubl
     regions.scale0 = h->f64 ? (float)h->scale64.v[0] : h->scale.v[0];
     regions.positions = h->f64 ? nullptr : features.positions;
     regions.positions64 = h->f64 ? positions64 : nullptr;
+    // (in the order of a list feature 0 grows with the workgroups as it does down an image)
+    regions.range0 = h->map.mode == 1 ? locality_scratch(h).range0 : nullptr;
     if (!h->f64 && !features.positions) {
         if (features.n_spatial_dims > 0) {
             regions.first = 0.0f;
@@ -606,6 +665,7 @@ int verify_build(pl_lattice *h, uint32_t *retry_cells) {
     // (in ns, as measured on 1024x1024 and 512x512 images: a row added afterwards takes 0.03 of
     // the atomic unit's time; the numbering pass 1.5 per workgroup of the build and 0.02 per
     // vertex, and the build 1500 longer with all its rows going out as atomics)
+    h->foreign_rows = status.n_segments != 0 ? (long)status.foreign_rows : -1;
     if (status.n_segments != 0 &&
         0.03 * status.foreign_rows > 1.5 * h->map.n_blocks + 0.02 * m + 1500.0)
         h->numbering_pass_pays = true;
@@ -722,6 +782,9 @@ int pl_destroy(pl_handle h) {
     h->dfree(h->chunk_count);
     h->dfree(h->d_counters);
     h->dfree(h->d_guess);
+    h->dfree(h->point_order);
+    h->dfree(h->locality_words);
+    h->dfree(h->bin_rank);
     if (h->h_status) (void)hipHostFree(h->h_status);
     if (h->status_written) (void)hipEventDestroy(h->status_written);
     for (int i = 0; i < EV_COUNT; ++i)
@@ -753,6 +816,9 @@ int pl_set_option(pl_handle h, int option, long value) {
             return PL_OK;
         case PL_OPT_MERGE_TILES:
             h->merge_tiles = value != 0;
+            return PL_OK;
+        case PL_OPT_ORDER_POINTS:
+            h->order_points = value != 0;
             return PL_OK;
         case PL_OPT_STOP_AFTER:
             if (value < 0 || value > 2) return PL_EINVAL;
@@ -789,7 +855,7 @@ int pl_set_point_grid(pl_handle h, int n_dims, const int *dims) {
 
 int pl_get_point_grid(pl_handle h, int *n_dims, int dims[3]) {
     if (!h || !n_dims || !dims) return PL_EINVAL;
-    *n_dims = h->map.mode == 0 ? 0 : h->map.mode;
+    *n_dims = h->map.mode <= 1 ? 0 : h->map.mode;
     for (int i = 0; i < 3; ++i) dims[i] = 0;
     if (h->map.mode == 2) {
         dims[0] = h->map.dims[1];
@@ -1073,6 +1139,7 @@ int pl_get_info(pl_handle h, int what, long *value) {
     switch (what) {
         case PL_INFO_BUILD_MERGED: *value = h->last_build_merged ? 1 : 0; return PL_OK;
         case PL_INFO_TABLE_CELLS: *value = (long)h->n_cells; return PL_OK;
+        case PL_INFO_FOREIGN_ROWS: *value = h->foreign_rows; return PL_OK;
         case PL_INFO_SCRATCH_BYTES: {
             const size_t mv = plk::max_vertices_for(h->n_cells_alloc);
             size_t b = (size_t)h->n_cells_alloc * (sizeof(uint64_t) + sizeof(int)) +
@@ -1081,6 +1148,10 @@ int pl_get_info(pl_handle h, int what, long *value) {
             if (h->cell_values) b += h->value_size() * (size_t)h->n_cells_alloc * h->vd;
             b += h->replay_capacity * (sizeof(plk::ReplayEntry) + sizeof(uint4) +
                                        (h->f64 ? sizeof(double) : 0));
+            if (h->point_order)
+                b += (size_t)h->order_capacity * (sizeof(int) + sizeof(uint2)) +
+                     sizeof(unsigned) * (4 * plk::kLocalityBoxRows + 4 +
+                                         2 * (size_t)plk::locality_bins_for(h->order_capacity));
             *value = (long)b;
             return PL_OK;
         }
@@ -1555,6 +1626,7 @@ extern "C" int pl_filter_static(int pd, int vd, int N, float *output, const floa
     h->forced_cells = (long)h->max_cells;
     h->guess_grid = false;   // (looking for a grid in the positions would allocate and wait)
     h->may_widen = false;    // (keys of two words would need the arrays allocated again)
+    h->order_points = false; // (no room for the arrays of the ordering pass)
     h->map = plk::make_point_map(N, 0, nullptr);
     h->status_on_device = true;
     rc = ensure_replay(h, false);

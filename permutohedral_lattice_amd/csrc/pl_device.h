@@ -120,7 +120,10 @@ __device__ __forceinline__ KeyRegions key_regions(const RegionSource &src) {
     KeyRegions regions{0.0f, 0.0f};
     if (!src.enabled || src.N < 2) return regions;
     float a = src.first, b = src.last;
-    if (src.positions) {
+    if (src.range0) {
+        a = src.range0[0];
+        b = src.range0[1];
+    } else if (src.positions) {
         a = src.positions[0];
         b = src.positions[(size_t)(src.N - 1) * src.pd];
     } else if (src.positions64) {
@@ -422,9 +425,12 @@ __device__ __forceinline__ void wide_keys_of(const Simplex<PD, T> &s, Key128 (&k
 // Per-point scratch (the replay arrays) is stored in thread order, so it stays coalesced.
 // ------------------------------------------------------------------------------------------------
 __device__ __forceinline__ int point_of_thread(const PointMap &m, unsigned vblock, unsigned tid) {
-    if (m.mode == 0) {
+    if (m.mode <= 1) {
         const size_t n = (size_t)vblock * kBlock + tid;
-        return n < (size_t)m.N ? (int)n : -1;
+        if (n >= (size_t)m.N) return -1;
+        if (m.mode == 0) return (int)n;
+        const int p = m.order[n];
+        return (unsigned)p < (unsigned)m.N ? p : -1;
     }
     const unsigned wave = tid >> 6, lane = tid & 63;
     const unsigned tiles_yx = (unsigned)m.tiles[1] * (unsigned)m.tiles[2];

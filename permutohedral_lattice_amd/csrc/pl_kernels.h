@@ -166,10 +166,12 @@ struct PointFeatures {
 // How threads are laid over the points (see point_of_thread in pl_kernels.hip).
 struct PointMap {
     int N;
-    int mode;        // 0: 256 consecutive points per workgroup; 2: 16x16 tiles; 3: 4x8x8 tiles
+    int mode;        // 0: 256 consecutive points per workgroup; 1: 256 consecutive entries of
+                     // `order`; 2: 16x16 tiles; 3: 4x8x8 tiles
     int dims[3];     // grid extents, slowest first (leading extents folded into dims[0])
     int tiles[3];    // workgroup tiles along each extent
     unsigned n_blocks;
+    const int *order;   // mode 1: the points, neighbours in space next to each other (order_by_locality)
 };
 
 // Where feature 0 of the first and of the last point can be read (one of the two pointers, or
@@ -178,6 +180,7 @@ struct PointMap {
 struct RegionSource {
     const float *positions;
     const double *positions64;
+    const float *range0;   // or: the smallest and the largest feature 0 of all points, in device memory
     float first, last;
     float scale0;          // scale factor of feature 0
     int N, pd;
@@ -362,6 +365,29 @@ struct GridGuess {
     int mismatch;
 };
 hipError_t guess_grid(const float *positions, int N, int pd, GridGuess *guess, hipStream_t s);
+
+// A plain list of points, put in an order in which neighbours in space are neighbours in the
+// list, so that 256 consecutive points share lattice vertices as the pixels of an image tile do
+// and the merging build works for them as well.  The points are binned by their first two
+// features: square bins, sized to hold about 64 points if these lay evenly in their bounding box,
+// numbered so that 2x2 bins are consecutive, each next to the one before it, and feature 0 grows
+// with the number.  Four launches:
+// bounding boxes, count (every point draws its rank in its bin), scan of the counts, scatter.
+// The order inside a bin is whatever the atomics gave; it only orders the work.
+// bin_count must be zero before the first call; every call leaves it so.
+constexpr int kLocalityBoxRows = 1024;
+struct LocalityScratch {
+    float4 *partial_boxes; // [kLocalityBoxRows] the boxes of as many shares of the points
+    float *range0;         // [4] smallest and largest feature 0, then (a word) the bins in use
+    unsigned *bin_count;   // [max_bins], 16-byte aligned
+    unsigned *bin_first;   // [max_bins], 16-byte aligned
+    uint2 *bin_rank;       // [N] bin of the point, its rank there
+    unsigned max_bins;     // a multiple of four
+};
+inline unsigned locality_bins_for(int N) { return ((unsigned)N / 32u + 1024u) & ~3u; }
+// positions or positions64 (the other null); order: N entries
+hipError_t order_by_locality(const float *positions, const double *positions64, int N, int pd,
+                             const LocalityScratch &scratch, int *order, hipStream_t s);
 
 hipError_t compute_positions(const float *reference, float *positions, int N, int n_ref_channels,
                              int n_spatial_dims, const SpatialDims &dims, float spatial_std,
