@@ -359,14 +359,23 @@ def run_side_legs(args, pla, synth, lat, step, img, d_pos, d_val, d_grad, out_f,
 
     # the same without the grid hint (a caller of filter() that only has N points): once with the
     # library left to find the image in the positions, once with the points as a plain list
+    # (and the plain list with its points in no order at all, and that list taken in the order it
+    # comes in instead of the order of space the library puts it in)
     plain = {}
-    for name, guess in (("grid_found_by_the_library", 1), ("plain_list", 0)):
+    shuffle = torch.randperm(lat.N, device="cuda", generator=torch.Generator("cuda").manual_seed(5))
+    s_pos, s_val, s_grad = (t[shuffle].contiguous() for t in (d_pos, d_val, d_grad))
+    for name, guess, ordered, (l_pos, l_val, l_grad) in (
+            ("grid_found_by_the_library", 1, 1, (d_pos, d_val, d_grad)),
+            ("plain_list", 0, 1, (d_pos, d_val, d_grad)),
+            ("plain_list_shuffled", 0, 1, (s_pos, s_val, s_grad)),
+            ("plain_list_shuffled_in_list_order", 0, 0, (s_pos, s_val, s_grad))):
         other = pla.PermutohedralLattice(lat.pd, lat.vd, lat.N)
         other.set_option(pla.PL_OPT_GUESS_GRID, guess)
+        other.set_option(pla.PL_OPT_ORDER_POINTS, ordered)
 
         def other_step():
-            other.filter(out_f, d_val, d_pos, False)
-            other.filter(out_r, d_grad, d_pos, True)
+            other.filter(out_f, l_val, l_pos, False)
+            other.filter(out_r, l_grad, l_pos, True)
 
         for _ in range(2):
             other_step()

@@ -162,7 +162,7 @@ struct pl_lattice {
     // neighbours in space are neighbours in the list (plk::order_by_locality), made anew by every
     // build, so that the merging build serves it too
     bool order_points = true;              // option
-    int *point_order = nullptr;            // [N]
+    int *point_order = nullptr;            // [256 * locality_tiles_for(N)]
     unsigned *locality_words = nullptr;    // boxes, range of feature 0, counts and firsts of the bins
     uint2 *bin_rank = nullptr;             // [N]
     int order_capacity = 0;
@@ -189,6 +189,10 @@ struct pl_lattice {
         if (profile && ev[which]) ev_recorded[which] = hipEventRecord(ev[which], stream) == hipSuccess;
     }
     plk::Counters *counters() { return d_counters + counter_set; }
+    // workgroups of the build that hold points (of an ordered list: about; the rest end at once)
+    unsigned working_blocks() const {
+        return map.mode == 1 ? (unsigned)(((size_t)N + 255) / 256) : map.n_blocks;
+    }
     size_t value_size() const { return f64 ? sizeof(double) : sizeof(float); }
     int max_vertices() const { return (int)plk::max_vertices_for(n_cells); }
     // what the grids of the kernels over the vertices are sized for: the count when the host
@@ -291,6 +295,8 @@ plk::LocalityScratch locality_scratch(const pl_lattice *h) {
     scratch.bin_first = h->locality_words + box_words + 4 + max_bins;
     scratch.bin_rank = h->bin_rank;
     scratch.max_bins = max_bins;
+    scratch.n_tiles = h->locality_words + box_words + 3;
+    scratch.max_tiles = plk::locality_tiles_for(h->N);
     return scratch;
 }
 
@@ -302,7 +308,7 @@ int ensure_order(pl_lattice *h) {
     h->dfree(h->bin_rank);
     h->order_capacity = 0;
     const size_t words = 4 * plk::kLocalityBoxRows + 4 + 2 * (size_t)plk::locality_bins_for(h->N);
-    h->point_order = (int *)h->dmalloc(sizeof(int) * (size_t)h->N);
+    h->point_order = (int *)h->dmalloc(sizeof(int) * 256 * (size_t)plk::locality_tiles_for(h->N));
     h->locality_words = (unsigned *)h->dmalloc(sizeof(unsigned) * words);
     h->bin_rank = (uint2 *)h->dmalloc(sizeof(uint2) * (size_t)h->N);
     if (!h->point_order || !h->locality_words || !h->bin_rank) return PL_ENOMEM;
@@ -344,10 +350,6 @@ int enqueue_build(pl_lattice *h, const plk::PointFeatures &features, const doubl
     h->wide_keys = wide;
     int rc = ensure_table(h, cells, wide);
     if (rc != PL_OK) return rc;
-    // the per-point arrays follow the point map; an allocation that failed when the map was set
-    // is made up for here
-    rc = ensure_replay(h, wide);
-    if (rc != PL_OK) return rc;
     // tiles of an image share most of their vertices among their four wavefronts
     const bool merge_allowed = h->merge_tiles && h->tiles_off_for == 0 && !wide;
     if (h->tiles_off_for > 0 && !wide) h->tiles_off_for -= 1;
@@ -361,16 +363,24 @@ int enqueue_build(pl_lattice *h, const plk::PointFeatures &features, const doubl
         }
         h->map.mode = ordered ? 1 : 0;
         h->map.order = ordered ? h->point_order : nullptr;
+        h->map.n_tiles = ordered ? locality_scratch(h).n_tiles : nullptr;
+        // (an ordered list may leave places empty: room for a quarter more than the points fill)
+        h->map.n_blocks = ordered ? plk::locality_tiles_for(h->N)
+                                  : (unsigned)(((size_t)h->N + 255) / 256);
     }
     const bool merge = merge_allowed && h->map.mode != 0;
     h->last_build_merged = merge;
+    // the per-point arrays follow the point map; an allocation that failed when the map was set
+    // is made up for here
+    rc = ensure_replay(h, wide);
+    if (rc != PL_OK) return rc;
     // (a lattice of doubles splats in its build only in the merging kernel)
     const bool fused = splat_input && plk::build_can_splat(h->vd) && (!h->f64 || merge);
     // (a build for one filter: a lattice built to be applied many times is numbered by the
     // numbering pass, in the order of the image tiles, which the passes over the vertices walk
     // a few per cent faster than the order in which the workgroups happened to finish)
     const bool numbers_in_build =
-        merge && fused && h->map.n_blocks <= 8192u && !h->numbering_pass_pays;
+        merge && fused && h->working_blocks() <= 8192u && !h->numbering_pass_pays;
     const size_t floats_per_value = h->f64 ? 2 : 1;
     if (fused && !numbers_in_build && !h->cell_values_clean) {
         PL_HIP(plk::fill_zero(h->cell_values, (size_t)h->n_cells_alloc * h->vd * floats_per_value,
@@ -667,7 +677,7 @@ int verify_build(pl_lattice *h, uint32_t *retry_cells) {
     // vertex, and the build 1500 longer with all its rows going out as atomics)
     h->foreign_rows = status.n_segments != 0 ? (long)status.foreign_rows : -1;
     if (status.n_segments != 0 &&
-        0.03 * status.foreign_rows > 1.5 * h->map.n_blocks + 0.02 * m + 1500.0)
+        0.03 * status.foreign_rows > 1.5 * h->working_blocks() + 0.02 * m + 1500.0)
         h->numbering_pass_pays = true;
     h->verified = true;
     if (h->last_build_merged) h->tiles_backoff = 32;

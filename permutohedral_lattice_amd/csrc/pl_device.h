@@ -425,11 +425,13 @@ __device__ __forceinline__ void wide_keys_of(const Simplex<PD, T> &s, Key128 (&k
 // Per-point scratch (the replay arrays) is stored in thread order, so it stays coalesced.
 // ------------------------------------------------------------------------------------------------
 __device__ __forceinline__ int point_of_thread(const PointMap &m, unsigned vblock, unsigned tid) {
-    if (m.mode <= 1) {
+    if (m.mode == 0) {
         const size_t n = (size_t)vblock * kBlock + tid;
-        if (n >= (size_t)m.N) return -1;
-        if (m.mode == 0) return (int)n;
-        const int p = m.order[n];
+        return n < (size_t)m.N ? (int)n : -1;
+    }
+    if (m.mode == 1) {
+        if (vblock >= *m.n_tiles || vblock >= m.n_blocks) return -1;
+        const int p = m.order[(size_t)vblock * kBlock + tid];
         return (unsigned)p < (unsigned)m.N ? p : -1;
     }
     const unsigned wave = tid >> 6, lane = tid & 63;
@@ -450,6 +452,24 @@ __device__ __forceinline__ int point_of_thread(const PointMap &m, unsigned vbloc
     }
     if (z >= (unsigned)m.dims[0] || y >= (unsigned)m.dims[1] || x >= (unsigned)m.dims[2]) return -1;
     return (int)(((size_t)z * m.dims[1] + y) * m.dims[2] + x);
+}
+
+// The share of the points this workgroup takes (vblock; each XCD a contiguous range of shares when
+// xcd_aware), false when it has none: the workgroups behind the last that holds points of an
+// ordered list.  Those keep their own number as vblock, so that every workgroup of the grid has
+// one of its own.
+__device__ __forceinline__ bool block_of_points(const PointMap &m, int xcd_aware, unsigned &vblock) {
+    unsigned nb = gridDim.x;
+    if (m.mode == 1) {
+        const unsigned tiles = *m.n_tiles;
+        nb = tiles < nb ? tiles : nb;
+        if (blockIdx.x >= nb) {
+            vblock = blockIdx.x;
+            return false;
+        }
+    }
+    vblock = xcd_contiguous_block(blockIdx.x, nb, xcd_aware);
+    return true;
 }
 
 // Mask of the lanes whose predicate holds (the compare result itself, no detour through 0/1)

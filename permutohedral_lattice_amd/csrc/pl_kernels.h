@@ -171,7 +171,11 @@ struct PointMap {
     int dims[3];     // grid extents, slowest first (leading extents folded into dims[0])
     int tiles[3];    // workgroup tiles along each extent
     unsigned n_blocks;
-    const int *order;   // mode 1: the points, neighbours in space next to each other (order_by_locality)
+    // mode 1 (order_by_locality): n_blocks * 256 entries, the points with neighbours in space next
+    // to each other, -1 where a place is left empty; and how many of the workgroups have any
+    // (in device memory: the launch is enqueued before the order is known)
+    const int *order;
+    const unsigned *n_tiles;
 };
 
 // Where feature 0 of the first and of the last point can be read (one of the two pointers, or
@@ -369,10 +373,14 @@ hipError_t guess_grid(const float *positions, int N, int pd, GridGuess *guess, h
 // A plain list of points, put in an order in which neighbours in space are neighbours in the
 // list, so that 256 consecutive points share lattice vertices as the pixels of an image tile do
 // and the merging build works for them as well.  The points are binned by their first two
-// features: square bins, sized to hold about 64 points if these lay evenly in their bounding box,
+// features: square bins, sized to hold about 56 points if these lay evenly in their bounding box,
 // numbered so that 2x2 bins are consecutive, each next to the one before it, and feature 0 grows
-// with the number.  Four launches:
-// bounding boxes, count (every point draws its rank in its bin), scan of the counts, scatter.
+// with the number.  When the points lie evenly enough (an image or a regular grid given as a
+// list), every bin starts a wavefront of its own: a bin is then a wavefront's 64 points as 8x8
+// pixels are, at the price of the places left empty; that is done when it takes at most
+// max_tiles workgroups (a quarter more than the points fill).  Otherwise the bins follow each
+// other without gaps and a wavefront takes parts of two.  Four launches: bounding boxes, count
+// (every point draws its rank in its bin), scan of the counts, scatter.
 // The order inside a bin is whatever the atomics gave; it only orders the work.
 // bin_count must be zero before the first call; every call leaves it so.
 constexpr int kLocalityBoxRows = 1024;
@@ -383,9 +391,15 @@ struct LocalityScratch {
     unsigned *bin_first;   // [max_bins], 16-byte aligned
     uint2 *bin_rank;       // [N] bin of the point, its rank there
     unsigned max_bins;     // a multiple of four
+    unsigned *n_tiles;     // out: workgroups of 256 places that hold points
+    unsigned max_tiles;    // order has 256 * max_tiles entries
 };
+inline unsigned locality_tiles_for(int N) {
+    const unsigned waves = ((unsigned)N + 63u) / 64u;
+    return (waves + waves / 4u + 3u) / 4u + 1u;
+}
 inline unsigned locality_bins_for(int N) { return ((unsigned)N / 32u + 1024u) & ~3u; }
-// positions or positions64 (the other null); order: N entries
+// positions or positions64 (the other null); order: 256 * scratch.max_tiles entries
 hipError_t order_by_locality(const float *positions, const double *positions64, int N, int pd,
                              const LocalityScratch &scratch, int *order, hipStream_t s);
 

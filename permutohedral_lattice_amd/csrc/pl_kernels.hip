@@ -450,6 +450,12 @@ __global__ __launch_bounds__(kBlock) void k_build_tile(PointFeatures features, P
     constexpr int VD = SPLAT_VD ? SPLAT_VD : 2;
     constexpr int P = (VD == 2 && !kDouble) ? 2 : 4;      // values per LDS row of sums
     const T *__restrict__ input = static_cast<const T *>(input_any);
+    unsigned vblock;
+    if (!block_of_points(map, xcd_aware, vblock)) {
+        // (no points: nothing created, no rows of sums for the passes that walk the lists)
+        if (threadIdx.x == 0) created_lists.block_count[vblock] = 0;
+        return;
+    }
     __shared__ uint64_t slot_key[kTileSlots];
     __shared__ int slot_cell[kTileSlots];
     __shared__ T slot_sum[SPLAT_VD ? kTileSlots * P : 1];
@@ -469,7 +475,6 @@ __global__ __launch_bounds__(kBlock) void k_build_tile(PointFeatures features, P
         group_created = 0;
     }
 
-    const unsigned vblock = xcd_contiguous_block(blockIdx.x, gridDim.x, xcd_aware);
     const size_t t = (size_t)vblock * kBlock + tid;   // slot in the replay arrays
     const size_t n_slots = (size_t)gridDim.x * kBlock;
     const int n = point_of_thread(map, vblock, tid);
@@ -1104,7 +1109,8 @@ __global__ __launch_bounds__(kBlock) void k_splat_dpp(PointMap map,
                                                        float *values, int xcd_aware) {
     static_assert(VD >= 2 && VD <= 4, "register splat handles 2..4 channels");
     constexpr int P = VD == 2 ? 2 : 4;   // lanes per vertex row in the final atomic
-    const unsigned vblock = xcd_contiguous_block(blockIdx.x, gridDim.x, xcd_aware);
+    unsigned vblock;
+    if (!block_of_points(map, xcd_aware, vblock)) return;
     const size_t t = (size_t)vblock * kBlock + threadIdx.x;
     const size_t T = (size_t)gridDim.x * kBlock;
     const int n = point_of_thread(map, vblock, threadIdx.x);
@@ -1166,7 +1172,8 @@ __global__ __launch_bounds__(kBlock) void k_splat_dpp_blocks(int vd, PointMap ma
                                                               int in_channels, ReplayEntry *replay,
                                                               const int *__restrict__ cell_vertex,
                                                               float *values, int xcd_aware) {
-    const unsigned vblock = xcd_contiguous_block(blockIdx.x, gridDim.x, xcd_aware);
+    unsigned vblock;
+    if (!block_of_points(map, xcd_aware, vblock)) return;
     const size_t t = (size_t)vblock * kBlock + threadIdx.x;
     const size_t T = (size_t)gridDim.x * kBlock;
     const int n = point_of_thread(map, vblock, threadIdx.x);
@@ -1240,7 +1247,8 @@ __global__ __launch_bounds__(kBlock) void k_splat_channels(int d1, int vd, Point
     // thousand points there are too few wavefronts to hide the latencies of this serial code
     // unless the corners are spread over several of them; each pays for putting the rows into LDS.
     constexpr int kCorners = 2;
-    const unsigned vblock = xcd_contiguous_block(blockIdx.x, gridDim.x, xcd_aware);
+    unsigned vblock;
+    if (!block_of_points(map, xcd_aware, vblock)) return;
     const size_t t = (size_t)vblock * kBlock + threadIdx.x;
     const size_t T = (size_t)gridDim.x * kBlock;
     const int n = point_of_thread(map, vblock, threadIdx.x);
@@ -1609,7 +1617,8 @@ __global__ __launch_bounds__(kBlock) void k_slice_point(int d1, PointMap map,
                                                          float *__restrict__ output, int normalize) {
     // each XCD takes one contiguous range of the tiles: the value rows it gathers (vertex numbers
     // follow the tiles) are then in its own L2 and not in all eight
-    const unsigned vblock = xcd_contiguous_block(blockIdx.x, gridDim.x, 1);
+    unsigned vblock;
+    if (!block_of_points(map, 1, vblock)) return;
     const size_t t = (size_t)vblock * kBlock + threadIdx.x;
     const size_t T = (size_t)gridDim.x * kBlock;
     const int n = point_of_thread(map, vblock, threadIdx.x);
@@ -1672,7 +1681,8 @@ __global__ __launch_bounds__(kBlock) void k_slice_rows_f64(PointMap map,
                                                             const double *__restrict__ values,
                                                             double *__restrict__ output,
                                                             int normalize) {
-    const unsigned vblock = xcd_contiguous_block(blockIdx.x, gridDim.x, 1);
+    unsigned vblock;
+    if (!block_of_points(map, 1, vblock)) return;
     const size_t t = (size_t)vblock * kBlock + threadIdx.x;
     const size_t T = (size_t)gridDim.x * kBlock;
     const int n = point_of_thread(map, vblock, threadIdx.x);
@@ -1730,7 +1740,8 @@ __global__ __launch_bounds__(kBlock) void k_slice_channels(int vd, PointMap map,
     const unsigned slot = item / runs;
     if (slot >= kBlock) return;
     const int j0 = kSliceRun * (int)(item - slot * runs);
-    const unsigned vblock = xcd_contiguous_block(blockIdx.x, gridDim.x, 1);   // as in k_slice_point
+    unsigned vblock;   // as in k_slice_point
+    if (!block_of_points(map, 1, vblock)) return;
     const size_t t = (size_t)vblock * kBlock + slot;
     const int n = point_of_thread(map, vblock, slot);
     if (n < 0) return;
@@ -1959,6 +1970,8 @@ hipError_t build(int pd, const PointFeatures &features, const PointMap &map, con
     if (map.n_blocks == 0) return hipSuccess;
     if (wide_keys && numbering) return hipErrorInvalidValue;
     const bool merge_in_workgroup = numbering != nullptr;
+    // (only the merging kernel knows of workgroups without points, as an ordered list has them)
+    if (map.mode == 1 && (!merge_in_workgroup || !map.order || !map.n_tiles)) return hipErrorInvalidValue;
     const InBuildNumbering in_build = numbering ? *numbering : InBuildNumbering{};
 #define PLK_BUILD_ARGS                                                                             \
     dim3(map.n_blocks), dim3(kBlock), 0, s, features, map, scale, cell_keys, n_cells - 1u,         \
@@ -1993,6 +2006,7 @@ hipError_t build_f64(int pd, const Points64 &points, const PointMap &map, uint64
     if (map.n_blocks == 0) return hipSuccess;
     if (wide_keys && numbering) return hipErrorInvalidValue;
     const bool merge_in_workgroup = numbering != nullptr;
+    if (map.mode == 1 && (!merge_in_workgroup || !map.order || !map.n_tiles)) return hipErrorInvalidValue;
     const InBuildNumbering in_build = numbering ? *numbering : InBuildNumbering{};
     if (splat_vd && !merge_in_workgroup) return hipErrorInvalidValue;
 #define PLK_BUILD_ARGS                                                                             \

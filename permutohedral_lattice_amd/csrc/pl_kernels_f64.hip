@@ -35,7 +35,8 @@ __global__ __launch_bounds__(kBlock) void k_splat_f64(int vd, PointMap map,
                                                        const double *__restrict__ weights,
                                                        const int *__restrict__ cell_vertex,
                                                        double *values, int xcd_aware) {
-    const unsigned vblock = xcd_contiguous_block(blockIdx.x, gridDim.x, xcd_aware);
+    unsigned vblock;
+    if (!block_of_points(map, xcd_aware, vblock)) return;
     const size_t t = (size_t)vblock * kBlock + threadIdx.x;
     const size_t n_slots = (size_t)gridDim.x * kBlock;
     const int n = point_of_thread(map, vblock, threadIdx.x);
@@ -101,7 +102,8 @@ __global__ __launch_bounds__(kBlock) void k_slice_point_f64(int vd, PointMap map
                                                              int normalize) {
     constexpr int kMaxChannels = 8;
     // each XCD takes one contiguous range of the tiles, whose vertices' rows are then in its L2
-    const unsigned vblock = xcd_contiguous_block(blockIdx.x, gridDim.x, 1);
+    unsigned vblock;
+    if (!block_of_points(map, 1, vblock)) return;
     const size_t t = (size_t)vblock * kBlock + threadIdx.x;
     const size_t n_slots = (size_t)gridDim.x * kBlock;
     const int n = point_of_thread(map, vblock, threadIdx.x);
@@ -156,7 +158,8 @@ __global__ __launch_bounds__(kBlock) void k_slice_f64(int vd, PointMap map,
                                                        double *__restrict__ output, int normalize) {
     const int out_channels = normalize ? vd - 1 : vd;
     // each XCD takes one contiguous range of the tiles, whose vertices' rows are then in its L2
-    const unsigned vblock = xcd_contiguous_block(blockIdx.x, gridDim.x, 1);
+    unsigned vblock;
+    if (!block_of_points(map, 1, vblock)) return;
     const size_t t = (size_t)vblock * kBlock + threadIdx.x;
     const size_t n_slots = (size_t)gridDim.x * kBlock;
     const int n = point_of_thread(map, vblock, threadIdx.x);

@@ -24,11 +24,14 @@ constexpr int kScanBlock = 1024;
 // four words instead: some ten thousand atomics on one cache line, one after the other, 0.4 ms.)
 constexpr int kBoxBlocks = kLocalityBoxRows;
 constexpr float kNoValue = -3.4e38f;
-// What is left to gain: a wavefront's 64 points start anywhere in a bin, so they lie in parts of
-// two bins, and share fewer vertices than the 8x8 pixels of an image tile do.  (The build of a
-// 1024x1024 image given as a list: 85 us; with every bin exactly a wavefront's, 60 us.  Bins of 16
-// points along a Hilbert curve changed nothing: a wavefront then takes parts of two small bins
-// plus four whole ones, and the count and the scan of four times the bins cost 10 us more.)
+// A bin is meant to be a wavefront's share: when every bin starts a wavefront of its own, the 64
+// lanes hold points of one bin as they hold 8x8 pixels of an image, and share as many vertices.
+// (The build of a 1024x1024 image given as a list, bins following each other without gaps, so
+// that a wavefront takes parts of two: 85 us; every bin a wavefront: 60 us.  Bins of 16 points
+// along a Hilbert curve, without gaps, changed nothing: a wavefront then takes parts of two small
+// bins plus four whole ones, and the count and the scan of four times the bins cost 10 us more.)
+// Points in a regular pattern fill bins of this size with at most 64 each: 7 or 8 rows of 7 or 8.
+constexpr float kPointsPerBin = 56.0f;
 
 __device__ __forceinline__ float wave_max(float x) {
 #pragma unroll
@@ -85,13 +88,13 @@ __device__ __forceinline__ LocalityBins locality_bins(const float4 *partial_boxe
     const float r0 = hi0 - lo0, r1 = hi1 - lo1;
     // (a box with a NaN or an infinity in it: one bin, the order of the list)
     if (!(r0 >= 0.0f && r0 < 3.0e38f && r1 >= 0.0f && r1 < 3.0e38f)) return b;
-    // the side of a square bin that holds 64 points if they are spread evenly over the box (over
-    // its longer side if it is a line)
+    // the side of a square bin that holds kPointsPerBin points if they are spread evenly over the
+    // box (over its longer side if it is a line)
     float side;
     if (r0 > 0.0f && r1 > 0.0f && r0 * r1 > 0.0f) {
-        side = sqrtf(r0 * (r1 * 64.0f / (float)N));
+        side = sqrtf(r0 * (r1 * kPointsPerBin / (float)N));
     } else {
-        side = fmaxf(r0, r1) * 64.0f / (float)N;
+        side = fmaxf(r0, r1) * kPointsPerBin / (float)N;
     }
     if (!(side > 0.0f)) return b;
     for (int turn = 0; turn < 256; ++turn) {
@@ -131,11 +134,17 @@ __device__ __forceinline__ void first_two_features(const T *__restrict__ positio
     p1 = pd >= 2 ? (float)row[1] : 0.0f;
 }
 
-// The box of every kBoxBlocks-th run of 256 points, one row of partial_boxes per workgroup
+// The box of every kBoxBlocks-th run of 256 points, one row of partial_boxes per workgroup; and
+// every place of the order set to "no point"
 template <typename T>
 __global__ __launch_bounds__(kBlock) void k_locality_box(const T *__restrict__ positions, int N, int pd,
-                                                          float4 *partial_boxes) {
+                                                          float4 *partial_boxes, int *__restrict__ order,
+                                                          size_t order_entries) {
     __shared__ float4 wave_part[kBlock / 64];
+    // (the places of the order that the scatter will leave empty)
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < order_entries;
+         i += (size_t)gridDim.x * kBlock)
+        order[i] = -1;
     float4 v{kNoValue, kNoValue, kNoValue, kNoValue};
 #pragma unroll 4
     for (size_t n = (size_t)blockIdx.x * kBlock + threadIdx.x; n < (size_t)N;
@@ -152,17 +161,25 @@ __global__ __launch_bounds__(kBlock) void k_locality_box(const T *__restrict__ p
 }
 
 // Every point draws its rank in its bin.  The lanes of a wavefront that share a bin (in a list
-// that has any order at all, most of them) draw their ranks with one atomic.
+// that has any order at all, most of them) draw their ranks with one atomic.  A thread takes
+// kCountPoints points, 256 apart, so that their loads and their atomics are in flight together.
+constexpr int kCountPoints = 2;
 template <typename T>
 __global__ __launch_bounds__(kBlock) void k_locality_count(const T *__restrict__ positions, int N, int pd,
                                                             LocalityScratch scratch) {
-    const size_t n = (size_t)blockIdx.x * kBlock + threadIdx.x;
-    const bool valid = n < (size_t)N;
     const int lane = threadIdx.x & 63;
     __shared__ float4 wave_part[kBlock / 64];
-    // (the loads of the point are on their way while the boxes are folded)
-    float p0 = 0.0f, p1 = 0.0f;
-    if (valid) first_two_features(positions, (int)n, pd, p0, p1);
+    // (the loads of the points are on their way while the boxes are folded)
+    size_t n[kCountPoints];
+    bool valid[kCountPoints];
+    float p0[kCountPoints], p1[kCountPoints];
+#pragma unroll
+    for (int k = 0; k < kCountPoints; ++k) {
+        n[k] = ((size_t)blockIdx.x * kCountPoints + k) * kBlock + threadIdx.x;
+        valid[k] = n[k] < (size_t)N;
+        p0[k] = p1[k] = 0.0f;
+        if (valid[k]) first_two_features(positions, (int)n[k], pd, p0[k], p1[k]);
+    }
     const LocalityBins bins = locality_bins(scratch.partial_boxes, wave_part, N, pd, scratch.max_bins);
     if (blockIdx.x == 0 && threadIdx.x == 0) {
         // what the scan needs of them
@@ -170,35 +187,51 @@ __global__ __launch_bounds__(kBlock) void k_locality_count(const T *__restrict__
         scratch.range0[1] = bins.hi0;
         reinterpret_cast<unsigned *>(scratch.range0)[2] = bins.n_bins;
     }
-    const int bin = valid ? (int)bin_of(bins, p0, p1) : 0;
-    // after 16 different bins the lanes that are left draw their ranks one by one
-    uint64_t todo = wave_ballot(valid);
-    int leader = lane;
-    unsigned size = 1, index = 0;
-    for (int turn = 0; todo != 0 && turn < 16; ++turn) {
-        const int first = __builtin_ctzll(todo);
-        const int k = __builtin_amdgcn_readlane(bin, first);
-        const uint64_t same = lanes_equal(bin, k) & todo;
-        if (lane_in(same)) {
-            leader = first;
-            size = (unsigned)__builtin_popcountll(same);
-            index = __builtin_amdgcn_mbcnt_hi((unsigned)(same >> 32),
-                                              __builtin_amdgcn_mbcnt_lo((unsigned)same, 0u));
+    int bin[kCountPoints], leader[kCountPoints];
+    unsigned size[kCountPoints], index[kCountPoints], first_rank[kCountPoints];
+#pragma unroll
+    for (int k = 0; k < kCountPoints; ++k) {
+        bin[k] = valid[k] ? (int)bin_of(bins, p0[k], p1[k]) : 0;
+        // after 16 different bins the lanes that are left draw their ranks one by one
+        uint64_t todo = wave_ballot(valid[k]);
+        leader[k] = lane;
+        size[k] = 1;
+        index[k] = 0;
+        for (int turn = 0; todo != 0 && turn < 16; ++turn) {
+            const int first = __builtin_ctzll(todo);
+            const int b = __builtin_amdgcn_readlane(bin[k], first);
+            const uint64_t same = lanes_equal(bin[k], b) & todo;
+            if (lane_in(same)) {
+                leader[k] = first;
+                size[k] = (unsigned)__builtin_popcountll(same);
+                index[k] = __builtin_amdgcn_mbcnt_hi((unsigned)(same >> 32),
+                                                     __builtin_amdgcn_mbcnt_lo((unsigned)same, 0u));
+            }
+            todo &= ~same;
         }
-        todo &= ~same;
     }
-    unsigned first_rank = 0;
-    if (valid && leader == lane) first_rank = atomicAdd(&scratch.bin_count[bin], size);
-    first_rank = __shfl(first_rank, leader);
-    if (valid) scratch.bin_rank[n] = make_uint2((unsigned)bin, first_rank + index);
+#pragma unroll
+    for (int k = 0; k < kCountPoints; ++k) {
+        first_rank[k] = 0;
+        if (valid[k] && leader[k] == lane) first_rank[k] = atomicAdd(&scratch.bin_count[bin[k]], size[k]);
+    }
+#pragma unroll
+    for (int k = 0; k < kCountPoints; ++k) {
+        first_rank[k] = __shfl(first_rank[k], leader[k]);
+        if (valid[k]) scratch.bin_rank[n[k]] = make_uint2((unsigned)bin[k], first_rank[k] + index[k]);
+    }
 }
 
-// bin_first = the counts before each bin; the counts go back to zero for the next call.
-// One workgroup: every thread takes a run of bins, four at a time (the arrays are as long as
-// max_bins, a multiple of four, and the counts behind the bins in use are zero).
+// bin_first = the place of each bin's first point in the order; the counts go back to zero for
+// the next call.  If giving every bin wavefronts of its own (its count rounded up to 64s) takes no
+// more workgroups than the order has room for, the bins are laid out so; else one behind the
+// other.  One workgroup: every thread takes a run of bins, four at a time (the arrays are as long
+// as max_bins, a multiple of four, and the counts behind the bins in use are zero).
 constexpr unsigned kScanHeld = 8;   // fours of counts a thread holds in registers between its two passes
-__global__ __launch_bounds__(kScanBlock) void k_locality_scan(LocalityScratch scratch) {
+__device__ __forceinline__ unsigned wavefronts_for(unsigned points) { return (points + 63u) >> 6; }
+__global__ __launch_bounds__(kScanBlock) void k_locality_scan(LocalityScratch scratch, int N) {
     __shared__ unsigned wave_total[kScanBlock / 64];
+    __shared__ unsigned wave_padded[kScanBlock / 64];
     uint4 *__restrict__ count4 = reinterpret_cast<uint4 *>(scratch.bin_count);
     uint4 *__restrict__ first4 = reinterpret_cast<uint4 *>(scratch.bin_first);
     unsigned n_bins = reinterpret_cast<const unsigned *>(scratch.range0)[2];
@@ -207,19 +240,30 @@ __global__ __launch_bounds__(kScanBlock) void k_locality_scan(LocalityScratch sc
     const unsigned per = (n_fours + kScanBlock - 1) / kScanBlock;
     const unsigned begin = threadIdx.x * per;
     const unsigned end = begin + per < n_fours ? begin + per : n_fours;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     uint4 held[kScanHeld];
-    unsigned sum = 0;
+    unsigned points = 0, padded = 0;   // of this thread's bins: points, and wavefronts if each bin has its own
+    auto add = [&](const uint4 &c) {
+        points += (c.x + c.y) + (c.z + c.w);
+        padded += (wavefronts_for(c.x) + wavefronts_for(c.y)) + (wavefronts_for(c.z) + wavefronts_for(c.w));
+    };
 #pragma unroll
     for (unsigned k = 0; k < kScanHeld; ++k) {
         held[k] = begin + k < end ? count4[begin + k] : make_uint4(0u, 0u, 0u, 0u);
-        sum += (held[k].x + held[k].y) + (held[k].z + held[k].w);
+        add(held[k]);
     }
-    for (unsigned i = begin + kScanHeld; i < end; ++i) {
-        const uint4 c = count4[i];
-        sum += (c.x + c.y) + (c.z + c.w);
-    }
+    for (unsigned i = begin + kScanHeld; i < end; ++i) add(count4[i]);
+    // which layout: all the wavefronts of the second must fit
+    unsigned all_padded = padded;
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) all_padded += __shfl_xor(all_padded, d);
+    if (lane == 0) wave_padded[wave] = all_padded;
+    __syncthreads();
+    all_padded = 0;
+    for (int w = 0; w < kScanBlock / 64; ++w) all_padded += wave_padded[w];
+    const bool own_wavefronts = all_padded <= 4u * scratch.max_tiles;
     // the sums before this thread: within the wavefront, then over the wavefronts
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const unsigned sum = own_wavefronts ? padded : points;
     unsigned inclusive = sum;
 #pragma unroll
     for (int d = 1; d < 64; d <<= 1) {
@@ -230,13 +274,15 @@ __global__ __launch_bounds__(kScanBlock) void k_locality_scan(LocalityScratch sc
     __syncthreads();
     unsigned before = inclusive - sum;
     for (int w = 0; w < wave; ++w) before += wave_total[w];
+    if (own_wavefronts) before *= 64u;
+    auto room = [&](unsigned c) { return own_wavefronts ? wavefronts_for(c) * 64u : c; };
     auto place = [&](unsigned i, const uint4 &c) {
         uint4 f;
         f.x = before;
-        f.y = f.x + c.x;
-        f.z = f.y + c.y;
-        f.w = f.z + c.z;
-        before = f.w + c.w;
+        f.y = f.x + room(c.x);
+        f.z = f.y + room(c.y);
+        f.w = f.z + room(c.z);
+        before = f.w + room(c.w);
         first4[i] = f;
         count4[i] = make_uint4(0u, 0u, 0u, 0u);
     };
@@ -244,6 +290,11 @@ __global__ __launch_bounds__(kScanBlock) void k_locality_scan(LocalityScratch sc
     for (unsigned k = 0; k < kScanHeld; ++k)
         if (begin + k < end) place(begin + k, held[k]);
     for (unsigned i = begin + kScanHeld; i < end; ++i) place(i, count4[i]);
+    if (threadIdx.x == 0) {
+        const unsigned wavefronts = own_wavefronts ? all_padded : wavefronts_for((unsigned)N);
+        const unsigned tiles = (wavefronts + 3u) / 4u;
+        *scratch.n_tiles = tiles < scratch.max_tiles ? tiles : scratch.max_tiles;
+    }
 }
 
 __global__ __launch_bounds__(kBlock) void k_locality_scatter(LocalityScratch scratch, int N,
@@ -252,8 +303,8 @@ __global__ __launch_bounds__(kBlock) void k_locality_scatter(LocalityScratch scr
     if (n >= (size_t)N) return;
     const uint2 br = scratch.bin_rank[n];
     const unsigned place = scratch.bin_first[br.x] + br.y;
-    // (ranks come from atomics on counts that started at zero, so place < N)
-    if (place < (unsigned)N) order[place] = (int)n;
+    // (ranks come from atomics on counts that started at zero, so the place is the point's own)
+    if ((size_t)place < (size_t)scratch.max_tiles * kBlock) order[place] = (int)n;
 }
 
 template <typename T>
@@ -261,9 +312,10 @@ hipError_t order_points(const T *positions, int N, int pd, const LocalityScratch
                         hipStream_t s) {
     const unsigned blocks = (unsigned)(((size_t)N + kBlock - 1) / kBlock);
     hipLaunchKernelGGL((k_locality_box<T>), dim3(kBoxBlocks), dim3(kBlock), 0, s, positions, N, pd,
-                       scratch.partial_boxes);
-    hipLaunchKernelGGL((k_locality_count<T>), dim3(blocks), dim3(kBlock), 0, s, positions, N, pd, scratch);
-    hipLaunchKernelGGL(k_locality_scan, dim3(1), dim3(kScanBlock), 0, s, scratch);
+                       scratch.partial_boxes, order, (size_t)scratch.max_tiles * kBlock);
+    const unsigned count_blocks = (blocks + kCountPoints - 1) / kCountPoints;
+    hipLaunchKernelGGL((k_locality_count<T>), dim3(count_blocks), dim3(kBlock), 0, s, positions, N, pd, scratch);
+    hipLaunchKernelGGL(k_locality_scan, dim3(1), dim3(kScanBlock), 0, s, scratch, N);
     hipLaunchKernelGGL(k_locality_scatter, dim3(blocks), dim3(kBlock), 0, s, scratch, N, order);
     return hipGetLastError();
 }
@@ -274,7 +326,8 @@ hipError_t order_by_locality(const float *positions, const double *positions64, 
                              const LocalityScratch &scratch, int *order, hipStream_t s) {
     if (N <= 0) return hipSuccess;
     if (!scratch.partial_boxes || !scratch.range0 || !scratch.bin_count || !scratch.bin_first ||
-        !scratch.bin_rank || !order || scratch.max_bins < 4u || scratch.max_bins % 4u != 0u ||
+        !scratch.bin_rank || !order || !scratch.n_tiles || scratch.max_bins < 4u ||
+        (size_t)scratch.max_tiles * kBlock < (size_t)N || scratch.max_bins % 4u != 0u ||
         (reinterpret_cast<uintptr_t>(scratch.bin_count) | reinterpret_cast<uintptr_t>(scratch.bin_first)) % 16u != 0u ||
         pd < 1)
         return hipErrorInvalidValue;
