@@ -24,7 +24,8 @@ typedef enum pl_status {
     PL_EINVAL = -1,       /* null pointer, negative size, bad option */
     PL_EUNSUPPORTED = -2, /* (pd, vd) outside what the kernels are built for */
     PL_ENOMEM = -3,       /* allocator returned NULL */
-    PL_EOVERFLOW = -4,    /* sizes do not fit int32, or lattice coordinates do not fit the packed key */
+    PL_EOVERFLOW = -4,    /* sizes do not fit int32, or lattice coordinates do not fit a short (the range of
+                             the reference's keys; pl_filter_static: do not fit the packed 64-bit key) */
     PL_EHIP = -5,         /* a HIP runtime call failed; pl_last_hip_error() has the code */
     PL_ESTATE = -6,       /* pl_apply before pl_build, and the like */
     PL_ETOOLARGE = -7     /* pl_filter_static: the lattice does not fit the library's static scratch */
