@@ -352,9 +352,8 @@ def run_real_image(args, pla, with_cpu):
 
 
 
-def run_side_legs(args, pla, synth, lat, step, img, d_pos, d_val, d_grad, out_f, out_r, side, batch):
-    """The legs beside the headline: no grid hint, lattice reuse, the op's boundary, a batch."""
-    import numpy as np
+def run_plain_legs(args, pla, lat, d_pos, d_val, d_grad, out_f, out_r):
+    """The headline step on handles that were given no grid -> {leg: ms per step}"""
     import torch
 
     # the same without the grid hint (a caller of filter() that only has N points): once with the
@@ -369,6 +368,8 @@ def run_side_legs(args, pla, synth, lat, step, img, d_pos, d_val, d_grad, out_f,
             ("plain_list", 0, 1, (d_pos, d_val, d_grad)),
             ("plain_list_shuffled", 0, 1, (s_pos, s_val, s_grad)),
             ("plain_list_shuffled_in_list_order", 0, 0, (s_pos, s_val, s_grad))):
+        if args.plain_legs and name not in args.plain_legs.split(","):
+            continue
         other = pla.PermutohedralLattice(lat.pd, lat.vd, lat.N)
         other.set_option(pla.PL_OPT_GUESS_GRID, guess)
         other.set_option(pla.PL_OPT_ORDER_POINTS, ordered)
@@ -386,7 +387,15 @@ def run_side_legs(args, pla, synth, lat, step, img, d_pos, d_val, d_grad, out_f,
         torch.cuda.synchronize()
         plain[name] = 1e3 * (time.perf_counter() - t0) / args.steps
         other.close()
-    plain_ms = plain
+    return plain
+
+
+def run_side_legs(args, pla, synth, lat, step, img, d_pos, d_val, d_grad, out_f, out_r, side, batch):
+    """The legs beside the headline: no grid hint, lattice reuse, the op's boundary, a batch."""
+    import numpy as np
+    import torch
+
+    plain_ms = run_plain_legs(args, pla, lat, d_pos, d_val, d_grad, out_f, out_r)
 
     # build once, apply forward and reverse (what a caller that keeps the lattice gets)
     lat.build(d_pos)
@@ -491,6 +500,10 @@ def main():
     ap.add_argument("--headline-only", action="store_true",
                     help="only the timed steps and the per-stage timing (what a rocprofv3 run of "
                          "this file should see): no side legs, no CPU baseline")
+    ap.add_argument("--plain-only", action="store_true",
+                    help="only the legs without a grid hint (for profiling the ordering of plain lists)")
+    ap.add_argument("--plain-legs", default="",
+                    help="with --plain-only: the legs to run, comma-separated (default: all)")
     ap.add_argument("--configs-only", action="store_true",
                     help="only the leg that runs every BASELINE configuration at full size, without "
                          "the CPU reference (what a rocprofv3 run for the kernels of those "
@@ -556,6 +569,10 @@ def main():
     pixels_per_step = 2 * n
     value = pixels_per_step / (ms_per_step * 1e-3) / 1e6
 
+    if args.plain_only:
+        plain = run_plain_legs(args, pla, lat, d_pos, d_val, d_grad, out_f, out_r)
+        print(json.dumps({"no_grid_hint_ms_per_step": {k: round(v, 4) for k, v in plain.items()}}))
+        return
     side_legs = not args.headline_only
     plain_ms, reuse_ms, double_ms = {}, 0.0, 0.0
     op_ms, batch_ms, batch = {}, {}, 4
