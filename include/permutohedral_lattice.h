@@ -75,7 +75,7 @@ typedef enum pl_option {
     PL_OPT_ORDER_POINTS = 9 /* 1 (default): points that are a plain list (no grid given or found, at
                                least 4096 of them) are worked on in an order in which neighbours in
                                space are neighbours in the list, found anew by every build from the
-                               first two features, so that the workgroups of the build can merge their
+                               first two or three features, so that the workgroups of the build can merge their
                                keys as for an image (PL_OPT_MERGE_TILES); 0: in the order of the list
                                (same results up to the order of float additions) */
 } pl_option;

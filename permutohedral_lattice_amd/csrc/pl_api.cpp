@@ -288,7 +288,7 @@ int ensure_replay(pl_lattice *h, bool wide) {
 plk::LocalityScratch locality_scratch(const pl_lattice *h) {
     const unsigned max_bins = plk::locality_bins_for(h->N);
     plk::LocalityScratch scratch{};
-    constexpr size_t box_words = 4 * plk::kLocalityBoxRows;
+    constexpr size_t box_words = 8 * plk::kLocalityBoxRows;
     scratch.partial_boxes = reinterpret_cast<float4 *>(h->locality_words);
     scratch.range0 = reinterpret_cast<float *>(h->locality_words + box_words);
     scratch.bin_count = h->locality_words + box_words + 4;
@@ -297,6 +297,8 @@ plk::LocalityScratch locality_scratch(const pl_lattice *h) {
     scratch.max_bins = max_bins;
     scratch.n_tiles = h->locality_words + box_words + 3;
     scratch.max_tiles = plk::locality_tiles_for(h->N);
+    scratch.chunk_sums = h->locality_words + box_words + 4 + 2 * (size_t)max_bins;
+    scratch.chunk_first = scratch.chunk_sums + 2 * (size_t)plk::locality_scan_chunks(max_bins);
     return scratch;
 }
 
@@ -307,7 +309,9 @@ int ensure_order(pl_lattice *h) {
     h->dfree(h->locality_words);
     h->dfree(h->bin_rank);
     h->order_capacity = 0;
-    const size_t words = 4 * plk::kLocalityBoxRows + 4 + 2 * (size_t)plk::locality_bins_for(h->N);
+    const unsigned max_bins = plk::locality_bins_for(h->N);
+    const size_t words = 8 * plk::kLocalityBoxRows + 4 + 2 * (size_t)max_bins +
+                         3 * (size_t)plk::locality_scan_chunks(max_bins) + 1;
     h->point_order = (int *)h->dmalloc(sizeof(int) * 256 * (size_t)plk::locality_tiles_for(h->N));
     h->locality_words = (unsigned *)h->dmalloc(sizeof(unsigned) * words);
     h->bin_rank = (uint2 *)h->dmalloc(sizeof(uint2) * (size_t)h->N);
@@ -1160,7 +1164,7 @@ int pl_get_info(pl_handle h, int what, long *value) {
                                        (h->f64 ? sizeof(double) : 0));
             if (h->point_order)
                 b += (size_t)h->order_capacity * (sizeof(int) + sizeof(uint2)) +
-                     sizeof(unsigned) * (4 * plk::kLocalityBoxRows + 4 +
+                     sizeof(unsigned) * (8 * plk::kLocalityBoxRows + 8 +
                                          2 * (size_t)plk::locality_bins_for(h->order_capacity));
             *value = (long)b;
             return PL_OK;

@@ -373,7 +373,8 @@ hipError_t guess_grid(const float *positions, int N, int pd, GridGuess *guess, h
 // A plain list of points, put in an order in which neighbours in space are neighbours in the
 // list, so that 256 consecutive points share lattice vertices as the pixels of an image tile do
 // and the merging build works for them as well.  The points are binned by their first two
-// features: square bins, sized to hold about 56 points if these lay evenly in their bounding box,
+// features, and by the third when its extent compares with theirs (the points of a volume):
+// square or cubic bins, sized to hold about 56 points if these lay evenly in their bounding box,
 // numbered so that 2x2 bins are consecutive, each next to the one before it, and feature 0 grows
 // with the number.  When the points lie evenly enough (an image or a regular grid given as a
 // list), every bin starts a wavefront of its own: a bin is then a wavefront's 64 points as 8x8
@@ -383,9 +384,9 @@ hipError_t guess_grid(const float *positions, int N, int pd, GridGuess *guess, h
 // (every point draws its rank in its bin), scan of the counts, scatter.
 // The order inside a bin is whatever the atomics gave; it only orders the work.
 // bin_count must be zero before the first call; every call leaves it so.
-constexpr int kLocalityBoxRows = 1024;
+constexpr int kLocalityBoxRows = 512;
 struct LocalityScratch {
-    float4 *partial_boxes; // [kLocalityBoxRows] the boxes of as many shares of the points
+    float4 *partial_boxes; // [2 * kLocalityBoxRows] the boxes of as many shares of the points
     float *range0;         // [4] smallest and largest feature 0, then (a word) the bins in use
     unsigned *bin_count;   // [max_bins], 16-byte aligned
     unsigned *bin_first;   // [max_bins], 16-byte aligned
@@ -393,7 +394,11 @@ struct LocalityScratch {
     unsigned max_bins;     // a multiple of four
     unsigned *n_tiles;     // out: workgroups of 256 places that hold points
     unsigned max_tiles;    // order has 256 * max_tiles entries
+    // for the scan of many bins by many workgroups, each a chunk of 4096 bins:
+    unsigned *chunk_sums;  // [2 * locality_scan_chunks(max_bins)]
+    unsigned *chunk_first; // [locality_scan_chunks(max_bins) + 1]
 };
+inline unsigned locality_scan_chunks(unsigned max_bins) { return (max_bins / 4u + 1023u) / 1024u; }
 inline unsigned locality_tiles_for(int N) {
     const unsigned waves = ((unsigned)N + 63u) / 64u;
     return (waves + waves / 4u + 3u) / 4u + 1u;

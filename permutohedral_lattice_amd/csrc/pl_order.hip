@@ -17,13 +17,19 @@ namespace {
 using namespace device;
 
 constexpr int kScanBlock = 1024;
+// more bins than this (lists of more than two million points) are scanned by many workgroups
+constexpr unsigned kOneWorkgroupScans = 65536;
 
-// The bounding box of the first two features is found in two steps: kBoxBlocks workgroups each
-// write the box of their share of the points (largest feature 0, largest -feature 0, the same of
-// feature 1), and every workgroup that needs the box folds those rows itself.  (Atomic maxima on
-// four words instead: some ten thousand atomics on one cache line, one after the other, 0.4 ms.)
+// The bounding box of the first three features is found in two steps: kBoxBlocks workgroups each
+// write the box of their share of the points (per feature the largest value and the largest
+// negated value), and every workgroup that needs the box folds those rows itself.  (Atomic maxima
+// on a few words instead: some ten thousand atomics on one cache line, one after the other, 0.4 ms.)
 constexpr int kBoxBlocks = kLocalityBoxRows;
 constexpr float kNoValue = -3.4e38f;
+constexpr int kBoxFeatures = 3;
+struct Box {
+    float hi[kBoxFeatures], neg_lo[kBoxFeatures];
+};
 // A bin is meant to be a wavefront's share: when every bin starts a wavefront of its own, the 64
 // lanes hold points of one bin as they hold 8x8 pixels of an image, and share as many vertices.
 // (The build of a 1024x1024 image given as a list, bins following each other without gaps, so
@@ -32,6 +38,10 @@ constexpr float kNoValue = -3.4e38f;
 // bins plus four whole ones, and the count and the scan of four times the bins cost 10 us more.)
 // Points in a regular pattern fill bins of this size with at most 64 each: 7 or 8 rows of 7 or 8.
 constexpr float kPointsPerBin = 56.0f;
+// The third feature takes part when its extent is at least this fraction of the larger of the
+// first two: the depth of a volume does, the first colour channel of an image under a wide colour
+// kernel does not (its few bins would only cut the tiles of the image in layers).
+constexpr float kThirdFeatureExtent = 0.125f;
 
 __device__ __forceinline__ float wave_max(float x) {
 #pragma unroll
@@ -39,72 +49,98 @@ __device__ __forceinline__ float wave_max(float x) {
     return x;
 }
 
-// The largest of each component over the workgroup, in every thread.
-// (fmaxf drops NaNs.)
-__device__ __forceinline__ float4 block_max(float4 v, float4 *wave_part) {
-    v.x = wave_max(v.x);
-    v.y = wave_max(v.y);
-    v.z = wave_max(v.z);
-    v.w = wave_max(v.w);
+__device__ __forceinline__ void widen(Box &b, const Box &o) {
+#pragma unroll
+    for (int f = 0; f < kBoxFeatures; ++f) {
+        b.hi[f] = fmaxf(b.hi[f], o.hi[f]);
+        b.neg_lo[f] = fmaxf(b.neg_lo[f], o.neg_lo[f]);
+    }
+}
+__device__ __forceinline__ Box empty_box() {
+    Box b;
+#pragma unroll
+    for (int f = 0; f < kBoxFeatures; ++f) b.hi[f] = b.neg_lo[f] = kNoValue;
+    return b;
+}
+// The rows of partial_boxes: two float4 each
+__device__ __forceinline__ Box load_box(const float4 *rows, int i) {
+    const float4 a = rows[2 * i], c = rows[2 * i + 1];
+    return Box{{a.x, a.z, c.x}, {a.y, a.w, c.y}};
+}
+__device__ __forceinline__ void store_box(float4 *rows, int i, const Box &b) {
+    rows[2 * i] = make_float4(b.hi[0], b.neg_lo[0], b.hi[1], b.neg_lo[1]);
+    rows[2 * i + 1] = make_float4(b.hi[2], b.neg_lo[2], 0.0f, 0.0f);
+}
+
+// The box of the boxes of all threads of the workgroup, in every thread.  (fmaxf drops NaNs.)
+__device__ __forceinline__ Box block_box(Box v, Box *wave_part) {
+#pragma unroll
+    for (int f = 0; f < kBoxFeatures; ++f) {
+        v.hi[f] = wave_max(v.hi[f]);
+        v.neg_lo[f] = wave_max(v.neg_lo[f]);
+    }
     const int wave = threadIdx.x >> 6, n_waves = (blockDim.x + 63) >> 6;
     if ((threadIdx.x & 63) == 0) wave_part[wave] = v;
     __syncthreads();
-    float4 all = wave_part[0];
-    for (int w = 1; w < n_waves; ++w) {
-        const float4 o = wave_part[w];
-        all.x = fmaxf(all.x, o.x);
-        all.y = fmaxf(all.y, o.y);
-        all.z = fmaxf(all.z, o.z);
-        all.w = fmaxf(all.w, o.w);
-    }
+    Box all = wave_part[0];
+    for (int w = 1; w < n_waves; ++w) widen(all, wave_part[w]);
     return all;
 }
 
 // The bins for the box; the same in every thread of every kernel of one call.
 struct LocalityBins {
-    float lo0, lo1, per_unit;   // bin along feature i = (feature i - lo_i) * per_unit
-    int n0, n1;                 // bins along the two features
-    unsigned n_bins;            // numbers in use: pairs of bins along each feature stay together
+    float lo[kBoxFeatures], per_unit;   // bin along feature i = (feature i - lo_i) * per_unit
+    int n[kBoxFeatures];                // bins along the features (1 along one that takes no part)
+    unsigned n_bins;                    // numbers in use: 2x2 bins along the first two features stay together
     float hi0;
 };
-__device__ __forceinline__ LocalityBins locality_bins(const float4 *partial_boxes, float4 *wave_part,
+__device__ __forceinline__ uint64_t bin_numbers(int n0, int n1, int n2) {
+    return (uint64_t)((n0 + 1) >> 1) * (uint64_t)((n1 + 1) >> 1) * 4u * (uint64_t)n2;
+}
+__device__ __forceinline__ LocalityBins locality_bins(const float4 *partial_boxes, Box *wave_part,
                                                       int N, int pd, unsigned max_bins) {
-    float4 mine{kNoValue, kNoValue, kNoValue, kNoValue};
-    for (int i = threadIdx.x; i < kBoxBlocks; i += blockDim.x) {
-        const float4 o = partial_boxes[i];
-        mine.x = fmaxf(mine.x, o.x);
-        mine.y = fmaxf(mine.y, o.y);
-        mine.z = fmaxf(mine.z, o.z);
-        mine.w = fmaxf(mine.w, o.w);
+    Box mine = empty_box();
+    for (int i = threadIdx.x; i < kBoxBlocks; i += blockDim.x) widen(mine, load_box(partial_boxes, i));
+    const Box box = block_box(mine, wave_part);
+    LocalityBins b{{0.0f, 0.0f, 0.0f}, 0.0f, {1, 1, 1}, 4u, 0.0f};
+    float r[kBoxFeatures];
+#pragma unroll
+    for (int f = 0; f < kBoxFeatures; ++f) {
+        const bool there = f < pd;
+        b.lo[f] = there ? -box.neg_lo[f] : 0.0f;
+        r[f] = there ? box.hi[f] + box.neg_lo[f] : 0.0f;
     }
-    const float4 box = block_max(mine, wave_part);
-    LocalityBins b{0.0f, 0.0f, 0.0f, 1, 1, 4u, 0.0f};
-    const float hi0 = box.x, lo0 = -box.y;
-    const float hi1 = pd >= 2 ? box.z : 0.0f;
-    const float lo1 = pd >= 2 ? -box.w : 0.0f;
-    b.lo0 = lo0;
-    b.lo1 = lo1;
-    b.hi0 = hi0;
-    const float r0 = hi0 - lo0, r1 = hi1 - lo1;
+    b.hi0 = box.hi[0];
     // (a box with a NaN or an infinity in it: one bin, the order of the list)
-    if (!(r0 >= 0.0f && r0 < 3.0e38f && r1 >= 0.0f && r1 < 3.0e38f)) return b;
-    // the side of a square bin that holds kPointsPerBin points if they are spread evenly over the
-    // box (over its longer side if it is a line)
+#pragma unroll
+    for (int f = 0; f < kBoxFeatures; ++f)
+        if (!(r[f] >= 0.0f && r[f] < 3.0e38f)) return b;
+    const float flat = fmaxf(r[0], r[1]);
+    const bool third = r[2] > 0.0f && r[2] >= kThirdFeatureExtent * flat;
+    if (!third) r[2] = 0.0f;
+    // the side of a square (cubic) bin that holds kPointsPerBin points if they are spread evenly
+    // over the box (over its longer side if it is a line)
+    const float per_point = kPointsPerBin / (float)N;
     float side;
-    if (r0 > 0.0f && r1 > 0.0f && r0 * r1 > 0.0f) {
-        side = sqrtf(r0 * (r1 * kPointsPerBin / (float)N));
+    if (third && r[0] > 0.0f && r[1] > 0.0f) {
+        side = cbrtf(r[0] * r[1] * (r[2] * per_point));
+    } else if (third && flat > 0.0f) {
+        side = sqrtf(flat * (r[2] * per_point));
+    } else if (r[0] > 0.0f && r[1] > 0.0f && r[0] * r[1] > 0.0f) {
+        side = sqrtf(r[0] * (r[1] * per_point));
     } else {
-        side = fmaxf(r0, r1) * kPointsPerBin / (float)N;
+        side = fmaxf(flat, r[2]) * per_point;
     }
     if (!(side > 0.0f)) return b;
     for (int turn = 0; turn < 256; ++turn) {
-        const float f0 = r0 / side + 1.0f, f1 = r1 / side + 1.0f;
-        if (f0 < 1.0e6f && f1 < 1.0e6f) {
-            const int n0 = (int)f0, n1 = (int)f1;
-            const uint64_t numbers = (uint64_t)((n0 + 1) >> 1) * (uint64_t)((n1 + 1) >> 1) * 4u;
+        const float f0 = r[0] / side + 1.0f, f1 = r[1] / side + 1.0f, f2 = r[2] / side + 1.0f;
+        if (f0 < 1.0e6f && f1 < 1.0e6f && f2 < 1.0e6f) {
+            const int n0 = (int)f0, n1 = (int)f1, n2 = (int)f2;
+            const uint64_t numbers = bin_numbers(n0, n1, n2);
             if (numbers <= (uint64_t)max_bins) {
-                b.n0 = n0;
-                b.n1 = n1;
+                b.n[0] = n0;
+                b.n[1] = n1;
+                b.n[2] = n2;
                 b.n_bins = (unsigned)numbers;
                 b.per_unit = 1.0f / side;
                 return b;
@@ -114,50 +150,54 @@ __device__ __forceinline__ LocalityBins locality_bins(const float4 *partial_boxe
     }
     return b;
 }
-__device__ __forceinline__ unsigned bin_of(const LocalityBins &b, float p0, float p1) {
+__device__ __forceinline__ unsigned bin_of(const LocalityBins &b, const float (&p)[kBoxFeatures]) {
     // (fminf and fmaxf drop a NaN operand: such a point lands in bin 0)
-    const int b0 = (int)fminf(fmaxf((p0 - b.lo0) * b.per_unit, 0.0f), (float)(b.n0 - 1));
-    const int b1 = (int)fminf(fmaxf((p1 - b.lo1) * b.per_unit, 0.0f), (float)(b.n1 - 1));
-    const unsigned pair = (unsigned)(b0 >> 1) * (unsigned)((b.n1 + 1) >> 1) + (unsigned)(b1 >> 1);
+    int c[kBoxFeatures];
+#pragma unroll
+    for (int f = 0; f < kBoxFeatures; ++f)
+        c[f] = (int)fminf(fmaxf((p[f] - b.lo[f]) * b.per_unit, 0.0f), (float)(b.n[f] - 1));
+    const unsigned pair = (unsigned)(c[0] >> 1) * (unsigned)((b.n[1] + 1) >> 1) + (unsigned)(c[1] >> 1);
     // The four bins of a 2x2 block in the order down, across, up: each bin touches the one before
     // it, and the last touches the first of the block to its right, so that any 256 consecutive
     // points (a workgroup of the build, wherever its share starts) lie in bins that hang together.
-    const unsigned down = (unsigned)(b0 & 1), across = (unsigned)(b1 & 1);
-    return pair * 4u + (across ? 3u - down : down);
+    // The bins along the third feature follow each other inside each of those.
+    const unsigned down = (unsigned)(c[0] & 1), across = (unsigned)(c[1] & 1);
+    return (pair * 4u + (across ? 3u - down : down)) * (unsigned)b.n[2] + (unsigned)c[2];
 }
 
 template <typename T>
-__device__ __forceinline__ void first_two_features(const T *__restrict__ positions, int n, int pd,
-                                                   float &p0, float &p1) {
-    const T *row = positions + (size_t)n * pd;
-    p0 = (float)row[0];
-    p1 = pd >= 2 ? (float)row[1] : 0.0f;
+__device__ __forceinline__ void first_features(const T *__restrict__ positions, size_t n, int pd,
+                                               float (&p)[kBoxFeatures]) {
+    const T *row = positions + n * (size_t)pd;
+#pragma unroll
+    for (int f = 0; f < kBoxFeatures; ++f) p[f] = f < pd ? (float)row[f] : 0.0f;
 }
 
-// The box of every kBoxBlocks-th run of 256 points, one row of partial_boxes per workgroup; and
+// The box of every kBoxBlocks-th run of 1024 points, one row of partial_boxes per workgroup; and
 // every place of the order set to "no point"
 template <typename T>
-__global__ __launch_bounds__(kBlock) void k_locality_box(const T *__restrict__ positions, int N, int pd,
-                                                          float4 *partial_boxes, int *__restrict__ order,
-                                                          size_t order_entries) {
-    __shared__ float4 wave_part[kBlock / 64];
+__global__ __launch_bounds__(kScanBlock) void k_locality_box(const T *__restrict__ positions, int N, int pd,
+                                                              float4 *partial_boxes, int *__restrict__ order,
+                                                              size_t order_entries) {
+    __shared__ Box wave_part[kScanBlock / 64];
     // (the places of the order that the scatter will leave empty)
-    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < order_entries;
-         i += (size_t)gridDim.x * kBlock)
+    for (size_t i = (size_t)blockIdx.x * kScanBlock + threadIdx.x; i < order_entries;
+         i += (size_t)gridDim.x * kScanBlock)
         order[i] = -1;
-    float4 v{kNoValue, kNoValue, kNoValue, kNoValue};
+    Box v = empty_box();
 #pragma unroll 4
-    for (size_t n = (size_t)blockIdx.x * kBlock + threadIdx.x; n < (size_t)N;
-         n += (size_t)gridDim.x * kBlock) {
-        float p0, p1;
-        first_two_features(positions, (int)n, pd, p0, p1);
-        v.x = fmaxf(v.x, p0);
-        v.y = fmaxf(v.y, -p0);
-        v.z = fmaxf(v.z, p1);
-        v.w = fmaxf(v.w, -p1);
+    for (size_t n = (size_t)blockIdx.x * kScanBlock + threadIdx.x; n < (size_t)N;
+         n += (size_t)gridDim.x * kScanBlock) {
+        float p[kBoxFeatures];
+        first_features(positions, n, pd, p);
+#pragma unroll
+        for (int f = 0; f < kBoxFeatures; ++f) {
+            v.hi[f] = fmaxf(v.hi[f], p[f]);
+            v.neg_lo[f] = fmaxf(v.neg_lo[f], -p[f]);
+        }
     }
-    v = block_max(v, wave_part);
-    if (threadIdx.x == 0) partial_boxes[blockIdx.x] = v;
+    v = block_box(v, wave_part);
+    if (threadIdx.x == 0) store_box(partial_boxes, blockIdx.x, v);
 }
 
 // Every point draws its rank in its bin.  The lanes of a wavefront that share a bin (in a list
@@ -168,22 +208,23 @@ template <typename T>
 __global__ __launch_bounds__(kBlock) void k_locality_count(const T *__restrict__ positions, int N, int pd,
                                                             LocalityScratch scratch) {
     const int lane = threadIdx.x & 63;
-    __shared__ float4 wave_part[kBlock / 64];
+    __shared__ Box wave_part[kBlock / 64];
     // (the loads of the points are on their way while the boxes are folded)
     size_t n[kCountPoints];
     bool valid[kCountPoints];
-    float p0[kCountPoints], p1[kCountPoints];
+    float p[kCountPoints][kBoxFeatures];
 #pragma unroll
     for (int k = 0; k < kCountPoints; ++k) {
         n[k] = ((size_t)blockIdx.x * kCountPoints + k) * kBlock + threadIdx.x;
         valid[k] = n[k] < (size_t)N;
-        p0[k] = p1[k] = 0.0f;
-        if (valid[k]) first_two_features(positions, (int)n[k], pd, p0[k], p1[k]);
+#pragma unroll
+        for (int f = 0; f < kBoxFeatures; ++f) p[k][f] = 0.0f;
+        if (valid[k]) first_features(positions, n[k], pd, p[k]);
     }
     const LocalityBins bins = locality_bins(scratch.partial_boxes, wave_part, N, pd, scratch.max_bins);
     if (blockIdx.x == 0 && threadIdx.x == 0) {
         // what the scan needs of them
-        scratch.range0[0] = bins.lo0;
+        scratch.range0[0] = bins.lo[0];
         scratch.range0[1] = bins.hi0;
         reinterpret_cast<unsigned *>(scratch.range0)[2] = bins.n_bins;
     }
@@ -191,7 +232,7 @@ __global__ __launch_bounds__(kBlock) void k_locality_count(const T *__restrict__
     unsigned size[kCountPoints], index[kCountPoints], first_rank[kCountPoints];
 #pragma unroll
     for (int k = 0; k < kCountPoints; ++k) {
-        bin[k] = valid[k] ? (int)bin_of(bins, p0[k], p1[k]) : 0;
+        bin[k] = valid[k] ? (int)bin_of(bins, p[k]) : 0;
         // after 16 different bins the lanes that are left draw their ranks one by one
         uint64_t todo = wave_ballot(valid[k]);
         leader[k] = lane;
@@ -297,6 +338,114 @@ __global__ __launch_bounds__(kScanBlock) void k_locality_scan(LocalityScratch sc
     }
 }
 
+// The same in three launches, for more bins than one workgroup scans in a few microseconds: every
+// workgroup takes kScanChunk fours of bins (a thread kScanRun of them, next to each other), the
+// first launch leaves each chunk's two sums, one workgroup chooses the layout and turns the chosen
+// sums into the places before each chunk, the third launch places the bins.
+constexpr unsigned kScanRun = 4, kScanChunk = kScanRun * kBlock;
+__device__ __forceinline__ void chunk_counts(const LocalityScratch &scratch, uint4 (&c)[kScanRun],
+                                             unsigned &points, unsigned &padded) {
+    const uint4 *__restrict__ count4 = reinterpret_cast<const uint4 *>(scratch.bin_count);
+    const unsigned n_fours = scratch.max_bins / 4u;
+    const unsigned begin = blockIdx.x * kScanChunk + threadIdx.x * kScanRun;
+    points = padded = 0;
+#pragma unroll
+    for (unsigned k = 0; k < kScanRun; ++k) {
+        c[k] = begin + k < n_fours ? count4[begin + k] : make_uint4(0u, 0u, 0u, 0u);
+        points += (c[k].x + c[k].y) + (c[k].z + c[k].w);
+        padded += (wavefronts_for(c[k].x) + wavefronts_for(c[k].y)) +
+                  (wavefronts_for(c[k].z) + wavefronts_for(c[k].w));
+    }
+}
+__global__ __launch_bounds__(kBlock) void k_locality_chunk_sums(LocalityScratch scratch) {
+    __shared__ unsigned part[2][kBlock / 64];
+    uint4 c[kScanRun];
+    unsigned points, padded;
+    chunk_counts(scratch, c, points, padded);
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) {
+        points += __shfl_xor(points, d);
+        padded += __shfl_xor(padded, d);
+    }
+    if ((threadIdx.x & 63) == 0) {
+        part[0][threadIdx.x >> 6] = points;
+        part[1][threadIdx.x >> 6] = padded;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        unsigned a = 0, b = 0;
+        for (int w = 0; w < kBlock / 64; ++w) {
+            a += part[0][w];
+            b += part[1][w];
+        }
+        scratch.chunk_sums[2 * blockIdx.x] = a;
+        scratch.chunk_sums[2 * blockIdx.x + 1] = b;
+    }
+}
+// (one wavefront: the chunks are few)
+__global__ __launch_bounds__(64) void k_locality_chunk_places(LocalityScratch scratch, int N, unsigned n_chunks) {
+    unsigned all_padded = 0;
+    for (unsigned i = threadIdx.x; i < n_chunks; i += 64) all_padded += scratch.chunk_sums[2 * i + 1];
+#pragma unroll
+    for (int d = 32; d >= 1; d >>= 1) all_padded += __shfl_xor(all_padded, d);
+    const bool own_wavefronts = all_padded <= 4u * scratch.max_tiles;
+    unsigned before = 0;
+    for (unsigned i0 = 0; i0 < n_chunks; i0 += 64) {
+        const unsigned i = i0 + threadIdx.x;
+        const unsigned sum = i < n_chunks ? scratch.chunk_sums[2 * i + (own_wavefronts ? 1 : 0)] : 0u;
+        unsigned inclusive = sum;
+#pragma unroll
+        for (int d = 1; d < 64; d <<= 1) {
+            const unsigned other = __shfl_up(inclusive, d);
+            if ((int)threadIdx.x >= d) inclusive += other;
+        }
+        if (i < n_chunks) scratch.chunk_first[i] = (before + inclusive - sum) * (own_wavefronts ? 64u : 1u);
+        before += __shfl(inclusive, 63);
+    }
+    if (threadIdx.x == 0) {
+        scratch.chunk_first[n_chunks] = own_wavefronts ? 1u : 0u;
+        const unsigned wavefronts = own_wavefronts ? all_padded : wavefronts_for((unsigned)N);
+        const unsigned tiles = (wavefronts + 3u) / 4u;
+        *scratch.n_tiles = tiles < scratch.max_tiles ? tiles : scratch.max_tiles;
+    }
+}
+__global__ __launch_bounds__(kBlock) void k_locality_chunk_scan(LocalityScratch scratch, unsigned n_chunks) {
+    __shared__ unsigned wave_total[kBlock / 64];
+    uint4 *__restrict__ count4 = reinterpret_cast<uint4 *>(scratch.bin_count);
+    uint4 *__restrict__ first4 = reinterpret_cast<uint4 *>(scratch.bin_first);
+    const unsigned n_fours = scratch.max_bins / 4u;
+    const unsigned begin = blockIdx.x * kScanChunk + threadIdx.x * kScanRun;
+    const bool own_wavefronts = scratch.chunk_first[n_chunks] != 0u;
+    uint4 c[kScanRun];
+    unsigned points, padded;
+    chunk_counts(scratch, c, points, padded);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const unsigned sum = own_wavefronts ? padded * 64u : points;
+    unsigned inclusive = sum;
+#pragma unroll
+    for (int d = 1; d < 64; d <<= 1) {
+        const unsigned other = __shfl_up(inclusive, d);
+        if (lane >= d) inclusive += other;
+    }
+    if (lane == 63) wave_total[wave] = inclusive;
+    __syncthreads();
+    unsigned before = scratch.chunk_first[blockIdx.x] + inclusive - sum;
+    for (int w = 0; w < wave; ++w) before += wave_total[w];
+    auto room = [&](unsigned n) { return own_wavefronts ? wavefronts_for(n) * 64u : n; };
+#pragma unroll
+    for (unsigned k = 0; k < kScanRun; ++k) {
+        if (begin + k >= n_fours) break;
+        uint4 f;
+        f.x = before;
+        f.y = f.x + room(c[k].x);
+        f.z = f.y + room(c[k].y);
+        f.w = f.z + room(c[k].z);
+        before = f.w + room(c[k].w);
+        first4[begin + k] = f;
+        count4[begin + k] = make_uint4(0u, 0u, 0u, 0u);
+    }
+}
+
 __global__ __launch_bounds__(kBlock) void k_locality_scatter(LocalityScratch scratch, int N,
                                                               int *__restrict__ order) {
     const size_t n = (size_t)blockIdx.x * kBlock + threadIdx.x;
@@ -311,11 +460,19 @@ template <typename T>
 hipError_t order_points(const T *positions, int N, int pd, const LocalityScratch &scratch, int *order,
                         hipStream_t s) {
     const unsigned blocks = (unsigned)(((size_t)N + kBlock - 1) / kBlock);
-    hipLaunchKernelGGL((k_locality_box<T>), dim3(kBoxBlocks), dim3(kBlock), 0, s, positions, N, pd,
+    hipLaunchKernelGGL((k_locality_box<T>), dim3(kBoxBlocks), dim3(kScanBlock), 0, s, positions, N, pd,
                        scratch.partial_boxes, order, (size_t)scratch.max_tiles * kBlock);
     const unsigned count_blocks = (blocks + kCountPoints - 1) / kCountPoints;
     hipLaunchKernelGGL((k_locality_count<T>), dim3(count_blocks), dim3(kBlock), 0, s, positions, N, pd, scratch);
-    hipLaunchKernelGGL(k_locality_scan, dim3(1), dim3(kScanBlock), 0, s, scratch, N);
+    if (scratch.max_bins <= kOneWorkgroupScans) {
+        hipLaunchKernelGGL(k_locality_scan, dim3(1), dim3(kScanBlock), 0, s, scratch, N);
+    } else {
+        // (over all max_bins: the counts behind the bins in use are zero)
+        const unsigned n_chunks = locality_scan_chunks(scratch.max_bins);
+        hipLaunchKernelGGL(k_locality_chunk_sums, dim3(n_chunks), dim3(kBlock), 0, s, scratch);
+        hipLaunchKernelGGL(k_locality_chunk_places, dim3(1), dim3(64), 0, s, scratch, N, n_chunks);
+        hipLaunchKernelGGL(k_locality_chunk_scan, dim3(n_chunks), dim3(kBlock), 0, s, scratch, n_chunks);
+    }
     hipLaunchKernelGGL(k_locality_scatter, dim3(blocks), dim3(kBlock), 0, s, scratch, N, order);
     return hipGetLastError();
 }
@@ -326,7 +483,8 @@ hipError_t order_by_locality(const float *positions, const double *positions64, 
                              const LocalityScratch &scratch, int *order, hipStream_t s) {
     if (N <= 0) return hipSuccess;
     if (!scratch.partial_boxes || !scratch.range0 || !scratch.bin_count || !scratch.bin_first ||
-        !scratch.bin_rank || !order || !scratch.n_tiles || scratch.max_bins < 4u ||
+        !scratch.bin_rank || !order || !scratch.n_tiles || !scratch.chunk_sums || !scratch.chunk_first ||
+        scratch.max_bins < 4u ||
         (size_t)scratch.max_tiles * kBlock < (size_t)N || scratch.max_bins % 4u != 0u ||
         (reinterpret_cast<uintptr_t>(scratch.bin_count) | reinterpret_cast<uintptr_t>(scratch.bin_first)) % 16u != 0u ||
         pd < 1)

@@ -38,6 +38,11 @@ def point_lists():
                                rng.uniform(0, 1, (n, 1)))
     cases["cloud_in_clumps"] = (4, 3, (rng.normal(0, 1, (n, 4)) + rng.integers(0, 3, (n, 1)) * 30.0),
                                 rng.uniform(0, 1, (n, 2)))
+    vol = synth.ellipsoid_volume(24, 40, 48, seed=7)
+    vpos = synth.bilateral_positions(vol, 5.0, 0.1)
+    shuffle3 = rng.permutation(vpos.shape[0])
+    cases["volume_as_a_list"] = (4, 2, vpos, vol.reshape(-1, 1))
+    cases["volume_with_its_voxels_shuffled"] = (4, 2, vpos[shuffle3], vol.reshape(-1, 1)[shuffle3])
     cases["points_on_a_line"] = (1, 2, rng.uniform(-50, 50, (5000, 1)), rng.uniform(0, 1, (5000, 1)))
     flat = rng.uniform(0, 30, (9000, 2))
     flat[:, 1] = 7.25                      # (no extent along the second feature)
@@ -157,4 +162,38 @@ def test_list_of_doubles():
             assert np.abs(host(out) - want).max() <= 1e-12
         assert (sorted_keys(host(lat.debug_keys()))[0] == sorted_keys(cpu.keys())[0]).all()
         assert lat.info(pla.PL_INFO_BUILD_MERGED) == ordered
+        lat.close()
+
+
+def test_large_lists_against_the_grid():
+    """More points than one workgroup scans the bins of (the scan then runs in three launches): a
+    volume of 2.6 million voxels as a grid, as a list in its own order and as a shuffled list must
+    give the same lattice and, point by point, the same outputs."""
+    dims, pd, vd = (128, 160, 128), 4, 2
+    n = int(np.prod(dims))
+    vol = synth.ellipsoid_volume(*dims, seed=11)
+    pos = synth.bilateral_positions(vol, 5.0, 0.1)
+    val = vol.reshape(-1, 1).astype(np.float32)
+    d_pos, d_val = dev(pos), dev(val)
+    out = torch.empty((n, vd - 1), dtype=torch.float32, device="cuda")
+    grid = pla.PermutohedralLattice(pd, vd, n)
+    grid.set_point_grid(dims)
+    grid.filter(out, d_val, d_pos, False)
+    torch.cuda.synchronize()
+    want, m = out.clone(), grid.num_vertices
+    want_keys = sorted_keys(host(grid.debug_keys()))[0]
+    grid.close()
+    shuffle = torch.randperm(n, device="cuda", generator=torch.Generator("cuda").manual_seed(3))
+    for l_pos, l_val, l_want in ((d_pos, d_val, want),
+                                 (d_pos[shuffle].contiguous(), d_val[shuffle].contiguous(), want[shuffle])):
+        lat = pla.PermutohedralLattice(pd, vd, n)
+        lat.set_option(pla.PL_OPT_GUESS_GRID, 0)
+        for _ in range(2):
+            out.fill_(float("nan"))
+            lat.filter(out, l_val, l_pos, False)
+            torch.cuda.synchronize()
+            assert lat.info(pla.PL_INFO_BUILD_MERGED) == 1
+            assert lat.num_vertices == m
+            assert float((out - l_want).abs().max()) <= 2e-5
+        assert (sorted_keys(host(lat.debug_keys()))[0] == want_keys).all()
         lat.close()
