@@ -173,21 +173,21 @@ __device__ __forceinline__ void first_features(const T *__restrict__ positions, 
     for (int f = 0; f < kBoxFeatures; ++f) p[f] = f < pd ? (float)row[f] : 0.0f;
 }
 
-// The box of every kBoxBlocks-th run of 1024 points, one row of partial_boxes per workgroup; and
-// every place of the order set to "no point"
-template <typename T>
-__global__ __launch_bounds__(kScanBlock) void k_locality_box(const T *__restrict__ positions, int N, int pd,
-                                                              float4 *partial_boxes, int *__restrict__ order,
-                                                              size_t order_entries) {
-    __shared__ Box wave_part[kScanBlock / 64];
+// The box of every kBoxBlocks-th run of THREADS points, one row of partial_boxes per workgroup;
+// and every place of the order set to "no point"
+template <typename T, int THREADS>
+__global__ __launch_bounds__(THREADS) void k_locality_box(const T *__restrict__ positions, int N, int pd,
+                                                           float4 *partial_boxes, int *__restrict__ order,
+                                                           size_t order_entries) {
+    __shared__ Box wave_part[THREADS / 64];
     // (the places of the order that the scatter will leave empty)
-    for (size_t i = (size_t)blockIdx.x * kScanBlock + threadIdx.x; i < order_entries;
-         i += (size_t)gridDim.x * kScanBlock)
+    for (size_t i = (size_t)blockIdx.x * THREADS + threadIdx.x; i < order_entries;
+         i += (size_t)gridDim.x * THREADS)
         order[i] = -1;
     Box v = empty_box();
 #pragma unroll 4
-    for (size_t n = (size_t)blockIdx.x * kScanBlock + threadIdx.x; n < (size_t)N;
-         n += (size_t)gridDim.x * kScanBlock) {
+    for (size_t n = (size_t)blockIdx.x * THREADS + threadIdx.x; n < (size_t)N;
+         n += (size_t)gridDim.x * THREADS) {
         float p[kBoxFeatures];
         first_features(positions, n, pd, p);
 #pragma unroll
@@ -460,8 +460,16 @@ template <typename T>
 hipError_t order_points(const T *positions, int N, int pd, const LocalityScratch &scratch, int *order,
                         hipStream_t s) {
     const unsigned blocks = (unsigned)(((size_t)N + kBlock - 1) / kBlock);
-    hipLaunchKernelGGL((k_locality_box<T>), dim3(kBoxBlocks), dim3(kScanBlock), 0, s, positions, N, pd,
-                       scratch.partial_boxes, order, (size_t)scratch.max_tiles * kBlock);
+    // (a thread takes four points or a few more: workgroups of 1024 threads for the longest lists)
+    if ((size_t)N > (size_t)4 * kBoxBlocks * 512)
+        hipLaunchKernelGGL((k_locality_box<T, 1024>), dim3(kBoxBlocks), dim3(1024), 0, s, positions, N, pd,
+                           scratch.partial_boxes, order, (size_t)scratch.max_tiles * kBlock);
+    else if ((size_t)N > (size_t)4 * kBoxBlocks * 256)
+        hipLaunchKernelGGL((k_locality_box<T, 512>), dim3(kBoxBlocks), dim3(512), 0, s, positions, N, pd,
+                           scratch.partial_boxes, order, (size_t)scratch.max_tiles * kBlock);
+    else
+        hipLaunchKernelGGL((k_locality_box<T, 256>), dim3(kBoxBlocks), dim3(256), 0, s, positions, N, pd,
+                           scratch.partial_boxes, order, (size_t)scratch.max_tiles * kBlock);
     const unsigned count_blocks = (blocks + kCountPoints - 1) / kCountPoints;
     hipLaunchKernelGGL((k_locality_count<T>), dim3(count_blocks), dim3(kBlock), 0, s, positions, N, pd, scratch);
     if (scratch.max_bins <= kOneWorkgroupScans) {
