@@ -121,11 +121,13 @@ def test_op_on_a_side_stream_is_ordered_with_that_stream():
     close(z.cpu().numpy(), want)
 
 
-def test_apply_can_be_captured_in_a_graph_and_replayed():
+@pytest.mark.parametrize("points", ["grid", "list"])
+def test_apply_can_be_captured_in_a_graph_and_replayed(points):
     """pl_apply only launches kernels on the lattice's stream (no allocation, no wait, no memset),
     so a caller may capture it in a HIP graph: the mean-field loop of a dense CRF replays the same
     splat/blur/slice sequence many times.  Every replay is checked against the eager result, with
-    eager work and synchronisations in between."""
+    eager work and synchronisations in between.  (list: the points as a plain list, which the
+    build puts in the order of space; the kernels of the apply then read that order.)"""
     h = w = 96
     n, vd = h * w, 6
     guide = synth.blob_image(h, w, seed=60) * 255.0
@@ -135,8 +137,12 @@ def test_apply_can_be_captured_in_a_graph_and_replayed():
     d_pos = dev(pos)
     torch.cuda.synchronize()
     with torch.cuda.stream(s):
-        lat.set_point_grid((h, w))
+        if points == "grid":
+            lat.set_point_grid((h, w))
+        else:
+            lat.set_option(pla.PL_OPT_GUESS_GRID, 0)
         lat.build(d_pos)
+        assert lat.info(pla.PL_INFO_BUILD_MERGED) == 1
         static_in = torch.zeros((n, vd - 1), dtype=torch.float32, device="cuda")
         static_out = torch.zeros_like(static_in)
         lat.apply(static_out, static_in, False)      # warm-up outside the capture
