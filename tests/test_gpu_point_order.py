@@ -197,3 +197,29 @@ def test_large_lists_against_the_grid():
             assert float((out - l_want).abs().max()) <= 2e-5
         assert (sorted_keys(host(lat.debug_keys()))[0] == want_keys).all()
         lat.close()
+
+
+@pytest.mark.parametrize("pd,vd,n", [(1, 2, 4096), (2, 3, 4097), (3, 4, 5000), (4, 2, 4100), (5, 3, 6000),
+                                     (6, 2, 4500), (7, 2, 4200), (8, 3, 4300), (5, 9, 5200), (3, 22, 4800)])
+def test_lists_just_long_enough_to_be_ordered(pd, vd, n):
+    """Every pd, few and many channels, lengths around the 4096 points from which a list is
+    ordered (ragged last workgroups, bins with a handful of points)."""
+    rng = np.random.default_rng(100 * pd + vd)
+    pos = (rng.uniform(0, 1, (n, pd)) * rng.uniform(2, 12, pd)).astype(np.float32)
+    val = rng.uniform(0, 1, (n, vd - 1)).astype(np.float32)
+    cpu = oracle.Lattice(pd, vd, n)
+    want = cpu.filter(val, pos)
+    lat = pla.PermutohedralLattice(pd, vd, n)
+    lat.set_option(pla.PL_OPT_GUESS_GRID, 0)
+    out = torch.empty((n, vd - 1), dtype=torch.float32, device="cuda")
+    for _ in range(2):
+        lat.filter(out, dev(val), dev(pos), False)
+        torch.cuda.synchronize()
+        check_against_oracle(lat, cpu, pos, out, want)
+    lat.build(dev(pos))
+    lat.apply(out, dev(val), True)
+    torch.cuda.synchronize()
+    want_reverse = oracle.Lattice(pd, vd, n).filter(val, pos, True)
+    assert np.abs(host(out) - want_reverse).max() <= MAX_ABS_TOL
+    assert rel_l2(host(out), want_reverse) <= REL_L2_TOL
+    lat.close()
