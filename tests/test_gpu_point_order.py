@@ -162,7 +162,30 @@ def test_list_of_doubles():
             assert np.abs(host(out) - want).max() <= 1e-12
         assert (sorted_keys(host(lat.debug_keys()))[0] == sorted_keys(cpu.keys())[0]).all()
         assert lat.info(pla.PL_INFO_BUILD_MERGED) == ordered
+        # built once and applied (the splat and the slice of doubles read the order as well)
+        lat.build(dev(pos64))
+        lat.apply(out, dev(val64), True)
+        torch.cuda.synchronize()
+        want_reverse = oracle.Lattice(pd, vd, n, dtype=np.float64).filter(val64, pos64, True)
+        assert np.abs(host(out) - want_reverse).max() <= 1e-12
         lat.close()
+
+
+def test_list_of_doubles_with_many_channels():
+    pd, vd, n = 3, 7, 6000
+    rng = np.random.default_rng(77)
+    pos = rng.uniform(0, 9, (n, pd))
+    val = rng.uniform(0, 1, (n, vd - 1))
+    cpu = oracle.Lattice(pd, vd, n, dtype=np.float64)
+    want = cpu.filter(val, pos)
+    lat = pla.PermutohedralLattice(pd, vd, n, dtype=torch.float64)
+    out = torch.empty((n, vd - 1), dtype=torch.float64, device="cuda")
+    lat.filter(out, dev(val), dev(pos), False)
+    torch.cuda.synchronize()
+    assert lat.num_vertices == cpu.num_vertices
+    assert lat.info(pla.PL_INFO_BUILD_MERGED) == 1
+    assert np.abs(host(out) - want).max() <= 1e-12
+    lat.close()
 
 
 def test_large_lists_against_the_grid():
