@@ -374,7 +374,7 @@ hipError_t guess_grid(const float *positions, int N, int pd, GridGuess *guess, h
 // list, so that 256 consecutive points share lattice vertices as the pixels of an image tile do
 // and the merging build works for them as well.  The points are binned by their first two
 // features, and by the third when its extent compares with theirs (the points of a volume):
-// square or cubic bins, sized to hold about 56 points if these lay evenly in their bounding box,
+// square or cubic bins, sized to hold about 60 points if these lay evenly in their bounding box,
 // numbered so that 2x2 bins are consecutive, each next to the one before it, and feature 0 grows
 // with the number.  When the points lie evenly enough (an image or a regular grid given as a
 // list), every bin starts a wavefront of its own: a bin is then a wavefront's 64 points as 8x8
