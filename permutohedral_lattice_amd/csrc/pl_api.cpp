@@ -1162,10 +1162,13 @@ int pl_get_info(pl_handle h, int what, long *value) {
             if (h->cell_values) b += h->value_size() * (size_t)h->n_cells_alloc * h->vd;
             b += h->replay_capacity * (sizeof(plk::ReplayEntry) + sizeof(uint4) +
                                        (h->f64 ? sizeof(double) : 0));
-            if (h->point_order)
-                b += (size_t)h->order_capacity * (sizeof(int) + sizeof(uint2)) +
-                     sizeof(unsigned) * (8 * plk::kLocalityBoxRows + 8 +
-                                         2 * (size_t)plk::locality_bins_for(h->order_capacity));
+            if (h->point_order) {
+                const unsigned max_bins = plk::locality_bins_for(h->order_capacity);
+                b += sizeof(int) * 256 * (size_t)plk::locality_tiles_for(h->order_capacity) +
+                     sizeof(uint2) * (size_t)h->order_capacity +
+                     sizeof(unsigned) * (8 * plk::kLocalityBoxRows + 5 + 2 * (size_t)max_bins +
+                                         3 * (size_t)plk::locality_scan_chunks(max_bins));
+            }
             *value = (long)b;
             return PL_OK;
         }
