@@ -163,7 +163,7 @@ struct pl_lattice {
     // build, so that the merging build serves it too
     bool order_points = true;              // option
     int *point_order = nullptr;            // [256 * locality_tiles_for(N)]
-    unsigned *locality_words = nullptr;    // boxes, range of feature 0, counts and firsts of the bins
+    unsigned *locality_words = nullptr;    // the bins, range of feature 0, counts and firsts of the bins
     uint2 *bin_rank = nullptr;             // [N]
     int order_capacity = 0;
     hipEvent_t ev[EV_COUNT] = {};
@@ -288,16 +288,18 @@ int ensure_replay(pl_lattice *h, bool wide) {
 plk::LocalityScratch locality_scratch(const pl_lattice *h) {
     const unsigned max_bins = plk::locality_bins_for(h->N);
     plk::LocalityScratch scratch{};
-    constexpr size_t box_words = 8 * plk::kLocalityBoxRows;
-    scratch.partial_boxes = reinterpret_cast<float4 *>(h->locality_words);
-    scratch.range0 = reinterpret_cast<float *>(h->locality_words + box_words);
-    scratch.bin_count = h->locality_words + box_words + 4;
-    scratch.bin_first = h->locality_words + box_words + 4 + max_bins;
+    // (32 words ahead of the arrays: the record of the bins, the range, the number of tiles)
+    constexpr size_t head_words = 32;
+    static_assert(plk::kLocalityBinsBytes <= 16 * sizeof(unsigned), "the record fits its place");
+    scratch.bins = h->locality_words;
+    scratch.range0 = reinterpret_cast<float *>(h->locality_words + 16);
+    scratch.n_tiles = h->locality_words + 20;
+    scratch.bin_count = h->locality_words + head_words;
+    scratch.bin_first = h->locality_words + head_words + max_bins;
     scratch.bin_rank = h->bin_rank;
     scratch.max_bins = max_bins;
-    scratch.n_tiles = h->locality_words + box_words + 3;
     scratch.max_tiles = plk::locality_tiles_for(h->N);
-    scratch.chunk_sums = h->locality_words + box_words + 4 + 2 * (size_t)max_bins;
+    scratch.chunk_sums = h->locality_words + head_words + 2 * (size_t)max_bins;
     scratch.chunk_first = scratch.chunk_sums + 2 * (size_t)plk::locality_scan_chunks(max_bins);
     return scratch;
 }
@@ -310,8 +312,7 @@ int ensure_order(pl_lattice *h) {
     h->dfree(h->bin_rank);
     h->order_capacity = 0;
     const unsigned max_bins = plk::locality_bins_for(h->N);
-    const size_t words = 8 * plk::kLocalityBoxRows + 4 + 2 * (size_t)max_bins +
-                         3 * (size_t)plk::locality_scan_chunks(max_bins) + 1;
+    const size_t words = 32 + 2 * (size_t)max_bins + 3 * (size_t)plk::locality_scan_chunks(max_bins) + 1;
     h->point_order = (int *)h->dmalloc(sizeof(int) * 256 * (size_t)plk::locality_tiles_for(h->N));
     h->locality_words = (unsigned *)h->dmalloc(sizeof(unsigned) * words);
     h->bin_rank = (uint2 *)h->dmalloc(sizeof(uint2) * (size_t)h->N);
@@ -1166,7 +1167,7 @@ int pl_get_info(pl_handle h, int what, long *value) {
                 const unsigned max_bins = plk::locality_bins_for(h->order_capacity);
                 b += sizeof(int) * 256 * (size_t)plk::locality_tiles_for(h->order_capacity) +
                      sizeof(uint2) * (size_t)h->order_capacity +
-                     sizeof(unsigned) * (8 * plk::kLocalityBoxRows + 5 + 2 * (size_t)max_bins +
+                     sizeof(unsigned) * (33 + 2 * (size_t)max_bins +
                                          3 * (size_t)plk::locality_scan_chunks(max_bins));
             }
             *value = (long)b;

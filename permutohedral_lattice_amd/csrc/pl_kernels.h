@@ -380,14 +380,15 @@ hipError_t guess_grid(const float *positions, int N, int pd, GridGuess *guess, h
 // list), every bin starts a wavefront of its own: a bin is then a wavefront's 64 points as 8x8
 // pixels are, at the price of the places left empty; that is done when it takes at most
 // max_tiles workgroups (a quarter more than the points fill).  Otherwise the bins follow each
-// other without gaps and a wavefront takes parts of two.  Four launches: bounding boxes, count
-// (every point draws its rank in its bin), scan of the counts, scatter.
+// other without gaps and a wavefront takes parts of two.  Four launches: the bins (from the
+// bounding box of a sample of the points), count (every point draws its rank in its bin), scan of
+// the counts, scatter.
 // The order inside a bin is whatever the atomics gave; it only orders the work.
 // bin_count must be zero before the first call; every call leaves it so.
-constexpr int kLocalityBoxRows = 512;
+constexpr size_t kLocalityBinsBytes = 64;
 struct LocalityScratch {
-    float4 *partial_boxes; // [2 * kLocalityBoxRows] the boxes of as many shares of the points
-    float *range0;         // [4] smallest and largest feature 0, then (a word) the bins in use
+    void *bins;            // [kLocalityBinsBytes] the bins of this call, from its first kernel to the others
+    float *range0;         // [2] smallest and largest feature 0 (of the sampled points)
     unsigned *bin_count;   // [max_bins], 16-byte aligned
     unsigned *bin_first;   // [max_bins], 16-byte aligned
     uint2 *bin_rank;       // [N] bin of the point, its rank there

@@ -20,11 +20,18 @@ constexpr int kScanBlock = 1024;
 // more bins than this (lists of more than two million points) are scanned by many workgroups
 constexpr unsigned kOneWorkgroupScans = 65536;
 
-// The bounding box of the first three features is found in two steps: kBoxBlocks workgroups each
-// write the box of their share of the points (per feature the largest value and the largest
-// negated value), and every workgroup that needs the box folds those rows itself.  (Atomic maxima
-// on a few words instead: some ten thousand atomics on one cache line, one after the other, 0.4 ms.)
-constexpr int kBoxBlocks = kLocalityBoxRows;
+// The bins are laid over the bounding box of the first three features of a sample of the points
+// (kBoxSamples of them, in runs of kSampleRun at places a multiplicative hash picks, so that no
+// pattern of the list falls between them; single points all over the list cost 16 us, most of it
+// address translation: every sample in a page of its own): one small workgroup finds it and
+// leaves the bins for the other kernels.
+// Points outside the sample's box land in the bins at its edge; a far outlier no longer
+// stretches the bins of all the others.  (A pass over all points cost 7 us for a million points
+// and 41 us for 8.4 million, and its 512 partial boxes had to be folded by every workgroup that
+// needed them; atomic maxima on a few words instead were some ten thousand atomics on one cache
+// line, one after the other, 0.4 ms.)
+constexpr int kBoxSamples = 4096;
+constexpr unsigned kSampleRun = 16;
 constexpr float kNoValue = -3.4e38f;
 constexpr int kBoxFeatures = 3;
 struct Box {
@@ -64,16 +71,6 @@ __device__ __forceinline__ Box empty_box() {
     for (int f = 0; f < kBoxFeatures; ++f) b.hi[f] = b.neg_lo[f] = kNoValue;
     return b;
 }
-// The rows of partial_boxes: two float4 each
-__device__ __forceinline__ Box load_box(const float4 *rows, int i) {
-    const float4 a = rows[2 * i], c = rows[2 * i + 1];
-    return Box{{a.x, a.z, c.x}, {a.y, a.w, c.y}};
-}
-__device__ __forceinline__ void store_box(float4 *rows, int i, const Box &b) {
-    rows[2 * i] = make_float4(b.hi[0], b.neg_lo[0], b.hi[1], b.neg_lo[1]);
-    rows[2 * i + 1] = make_float4(b.hi[2], b.neg_lo[2], 0.0f, 0.0f);
-}
-
 // The box of the boxes of all threads of the workgroup, in every thread.  (fmaxf drops NaNs.)
 __device__ __forceinline__ Box block_box(Box v, Box *wave_part) {
 #pragma unroll
@@ -96,14 +93,14 @@ struct LocalityBins {
     unsigned n_bins;                    // numbers in use: 2x2 bins along the first two features stay together
     float hi0;
 };
+static_assert(sizeof(LocalityBins) <= kLocalityBinsBytes, "the record the kernels pass the bins in");
+__device__ __forceinline__ LocalityBins *bins_record(const LocalityScratch &scratch) {
+    return static_cast<LocalityBins *>(scratch.bins);
+}
 __device__ __forceinline__ uint64_t bin_numbers(int n0, int n1, int n2) {
     return (uint64_t)((n0 + 1) >> 1) * (uint64_t)((n1 + 1) >> 1) * 4u * (uint64_t)n2;
 }
-__device__ __forceinline__ LocalityBins locality_bins(const float4 *partial_boxes, Box *wave_part,
-                                                      int N, int pd, unsigned max_bins) {
-    Box mine = empty_box();
-    for (int i = threadIdx.x; i < kBoxBlocks; i += blockDim.x) widen(mine, load_box(partial_boxes, i));
-    const Box box = block_box(mine, wave_part);
+__device__ __forceinline__ LocalityBins bins_over(const Box &box, int N, int pd, unsigned max_bins) {
     LocalityBins b{{0.0f, 0.0f, 0.0f}, 0.0f, {1, 1, 1}, 4u, 0.0f};
     float r[kBoxFeatures];
 #pragma unroll
@@ -175,43 +172,59 @@ __device__ __forceinline__ void first_features(const T *__restrict__ positions, 
     for (int f = 0; f < kBoxFeatures; ++f) p[f] = f < pd ? (float)row[f] : 0.0f;
 }
 
-// The box of every kBoxBlocks-th run of THREADS points, one row of partial_boxes per workgroup;
-// and every place of the order set to "no point"
-template <typename T, int THREADS>
-__global__ __launch_bounds__(THREADS) void k_locality_box(const T *__restrict__ positions, int N, int pd,
-                                                           float4 *partial_boxes, int *__restrict__ order,
-                                                           size_t order_entries) {
-    __shared__ Box wave_part[THREADS / 64];
-    // (the places of the order that the scatter will leave empty)
-    for (size_t i = (size_t)blockIdx.x * THREADS + threadIdx.x; i < order_entries;
-         i += (size_t)gridDim.x * THREADS)
-        order[i] = -1;
+// The bins for this list: the box of the sampled points, the bins over it, left in memory for the
+// kernels that follow (one workgroup)
+template <typename T>
+__global__ __launch_bounds__(kScanBlock) void k_locality_bins(const T *__restrict__ positions, int N, int pd,
+                                                               LocalityScratch scratch) {
+    __shared__ Box wave_part[kScanBlock / 64];
+    // (all the loads first, none behind a branch: a sample past the end reads the last point)
+    constexpr int kPerThread = kBoxSamples / kScanBlock;
+    float p[kPerThread][kBoxFeatures];
+#pragma unroll
+    for (int k = 0; k < kPerThread; ++k) {
+        const unsigned sample = (unsigned)(k * kScanBlock) + threadIdx.x;
+        // (every point when there are no more than samples)
+        const unsigned run = sample / kSampleRun, in_run = sample % kSampleRun;
+        unsigned n = N <= kBoxSamples
+                         ? sample
+                         : (unsigned)((((uint64_t)run * 0x9E3779B97F4A7C15ull) >> 32) * (uint64_t)(unsigned)N >> 32) + in_run;
+        n = n < (unsigned)N ? n : (unsigned)N - 1u;
+        first_features(positions, (size_t)n, pd, p[k]);
+    }
     Box v = empty_box();
-#pragma unroll 4
-    for (size_t n = (size_t)blockIdx.x * THREADS + threadIdx.x; n < (size_t)N;
-         n += (size_t)gridDim.x * THREADS) {
-        float p[kBoxFeatures];
-        first_features(positions, n, pd, p);
+#pragma unroll
+    for (int k = 0; k < kPerThread; ++k) {
 #pragma unroll
         for (int f = 0; f < kBoxFeatures; ++f) {
-            v.hi[f] = fmaxf(v.hi[f], p[f]);
-            v.neg_lo[f] = fmaxf(v.neg_lo[f], -p[f]);
+            v.hi[f] = fmaxf(v.hi[f], p[k][f]);
+            v.neg_lo[f] = fmaxf(v.neg_lo[f], -p[k][f]);
         }
     }
     v = block_box(v, wave_part);
-    if (threadIdx.x == 0) store_box(partial_boxes, blockIdx.x, v);
+    if (threadIdx.x == 0) {
+        const LocalityBins bins = bins_over(v, N, pd, scratch.max_bins);
+        *bins_record(scratch) = bins;
+        scratch.range0[0] = bins.lo[0];
+        scratch.range0[1] = bins.hi0;
+    }
 }
 
 // Every point draws its rank in its bin.  The lanes of a wavefront that share a bin (in a list
 // that has any order at all, most of them) draw their ranks with one atomic.  A thread takes
 // kCountPoints points, 256 apart, so that their loads and their atomics are in flight together.
+// (Also: every place of the order set to "no point".)
 constexpr int kCountPoints = 2;
 template <typename T>
 __global__ __launch_bounds__(kBlock) void k_locality_count(const T *__restrict__ positions, int N, int pd,
-                                                            LocalityScratch scratch) {
+                                                            LocalityScratch scratch, int *__restrict__ order,
+                                                            size_t order_entries) {
     const int lane = threadIdx.x & 63;
-    __shared__ Box wave_part[kBlock / 64];
-    // (the loads of the points are on their way while the boxes are folded)
+    // (the places of the order that the scatter will leave empty)
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < order_entries;
+         i += (size_t)gridDim.x * kBlock)
+        order[i] = -1;
+    const LocalityBins bins = *bins_record(scratch);
     size_t n[kCountPoints];
     bool valid[kCountPoints];
     float p[kCountPoints][kBoxFeatures];
@@ -222,13 +235,6 @@ __global__ __launch_bounds__(kBlock) void k_locality_count(const T *__restrict__
 #pragma unroll
         for (int f = 0; f < kBoxFeatures; ++f) p[k][f] = 0.0f;
         if (valid[k]) first_features(positions, n[k], pd, p[k]);
-    }
-    const LocalityBins bins = locality_bins(scratch.partial_boxes, wave_part, N, pd, scratch.max_bins);
-    if (blockIdx.x == 0 && threadIdx.x == 0) {
-        // what the scan needs of them
-        scratch.range0[0] = bins.lo[0];
-        scratch.range0[1] = bins.hi0;
-        reinterpret_cast<unsigned *>(scratch.range0)[2] = bins.n_bins;
     }
     int bin[kCountPoints], leader[kCountPoints];
     unsigned size[kCountPoints], index[kCountPoints], first_rank[kCountPoints];
@@ -277,7 +283,7 @@ __global__ __launch_bounds__(kScanBlock) void k_locality_scan(LocalityScratch sc
     __shared__ unsigned wave_padded[kScanBlock / 64];
     uint4 *__restrict__ count4 = reinterpret_cast<uint4 *>(scratch.bin_count);
     uint4 *__restrict__ first4 = reinterpret_cast<uint4 *>(scratch.bin_first);
-    unsigned n_bins = reinterpret_cast<const unsigned *>(scratch.range0)[2];
+    unsigned n_bins = bins_record(scratch)->n_bins;
     if (n_bins > scratch.max_bins) n_bins = scratch.max_bins;
     const unsigned n_fours = (n_bins + 3u) / 4u;
     const unsigned per = (n_fours + kScanBlock - 1) / kScanBlock;
@@ -462,18 +468,10 @@ template <typename T>
 hipError_t order_points(const T *positions, int N, int pd, const LocalityScratch &scratch, int *order,
                         hipStream_t s) {
     const unsigned blocks = (unsigned)(((size_t)N + kBlock - 1) / kBlock);
-    // (a thread takes four points or a few more: workgroups of 1024 threads for the longest lists)
-    if ((size_t)N > (size_t)4 * kBoxBlocks * 512)
-        hipLaunchKernelGGL((k_locality_box<T, 1024>), dim3(kBoxBlocks), dim3(1024), 0, s, positions, N, pd,
-                           scratch.partial_boxes, order, (size_t)scratch.max_tiles * kBlock);
-    else if ((size_t)N > (size_t)4 * kBoxBlocks * 256)
-        hipLaunchKernelGGL((k_locality_box<T, 512>), dim3(kBoxBlocks), dim3(512), 0, s, positions, N, pd,
-                           scratch.partial_boxes, order, (size_t)scratch.max_tiles * kBlock);
-    else
-        hipLaunchKernelGGL((k_locality_box<T, 256>), dim3(kBoxBlocks), dim3(256), 0, s, positions, N, pd,
-                           scratch.partial_boxes, order, (size_t)scratch.max_tiles * kBlock);
+    hipLaunchKernelGGL((k_locality_bins<T>), dim3(1), dim3(kScanBlock), 0, s, positions, N, pd, scratch);
     const unsigned count_blocks = (blocks + kCountPoints - 1) / kCountPoints;
-    hipLaunchKernelGGL((k_locality_count<T>), dim3(count_blocks), dim3(kBlock), 0, s, positions, N, pd, scratch);
+    hipLaunchKernelGGL((k_locality_count<T>), dim3(count_blocks), dim3(kBlock), 0, s, positions, N, pd, scratch,
+                       order, (size_t)scratch.max_tiles * kBlock);
     if (scratch.max_bins <= kOneWorkgroupScans) {
         hipLaunchKernelGGL(k_locality_scan, dim3(1), dim3(kScanBlock), 0, s, scratch, N);
     } else {
@@ -492,7 +490,7 @@ hipError_t order_points(const T *positions, int N, int pd, const LocalityScratch
 hipError_t order_by_locality(const float *positions, const double *positions64, int N, int pd,
                              const LocalityScratch &scratch, int *order, hipStream_t s) {
     if (N <= 0) return hipSuccess;
-    if (!scratch.partial_boxes || !scratch.range0 || !scratch.bin_count || !scratch.bin_first ||
+    if (!scratch.bins || !scratch.range0 || !scratch.bin_count || !scratch.bin_first ||
         !scratch.bin_rank || !order || !scratch.n_tiles || !scratch.chunk_sums || !scratch.chunk_first ||
         scratch.max_bins < 4u ||
         (size_t)scratch.max_tiles * kBlock < (size_t)N || scratch.max_bins % 4u != 0u ||
