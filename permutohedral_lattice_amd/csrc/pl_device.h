@@ -516,10 +516,13 @@ __device__ __forceinline__ void set_in_lanes(int &x, uint64_t lanes, int value) 
         : "+v"(x), "=&s"(saved)
         : "s"(lanes), "s"(value));
 }
-// Lanes in a mask, counted in 32-bit halves (the count of 64 bits is carried as a 64-bit number,
-// and a comparison with it then runs on the vector unit)
+// Lanes in a mask, as a 32-bit scalar (the compiler's count of 64 bits is carried as a 64-bit
+// number, and a comparison with it then runs on the vector unit; two 32-bit counts and an addition
+// stay on the scalar unit but are three instructions)
 __device__ __forceinline__ int lanes_in(uint64_t mask) {
-    return __builtin_popcount((uint32_t)mask) + __builtin_popcount((uint32_t)(mask >> 32));
+    int n;
+    asm("s_bcnt1_i32_b64 %0, %1" : "=s"(n) : "s"(mask) : "scc");
+    return n;
 }
 
 // Lanes that hold the same value of `x` elect the lowest of them as leader.  Returns the leader's
