@@ -92,3 +92,13 @@ def test_op_and_feature_builder_argument_checks():
     assert lib.pl_compute_positions(None, None, -1, 3, 2, dims, 1.0, 1.0, None) == pla.PL_EINVAL
     assert lib.pl_compute_positions(None, None, 0, 3, 2, dims, 1.0, 1.0, None) == pla.PL_OK
     assert lib.pl_compute_positions(None, None, 64, 3, 2, dims, 1.0, 1.0, None) == pla.PL_EINVAL
+
+
+def test_python_constants_are_the_headers():
+    """Every PL_* enumerator of the header has the same value in the Python mirror."""
+    text = open(os.path.join(ROOT, "include", "permutohedral_lattice.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    found = {name: int(value) for name, value in re.findall(r"\b(PL_[A-Z_0-9]+)\s*=\s*(-?\d+)", text)}
+    assert len(found) >= 20
+    for name, value in found.items():
+        assert getattr(pla, name) == value, name
