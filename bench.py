@@ -37,14 +37,8 @@ def algorithmic_bytes(n, m, pd, vd):
 def kernel_source_hash():
     """Short hash of the sources the HIP library is built from: what a counter measurement is
     stamped with, so that a figure taken from an older build shows as stale."""
-    import hashlib
-    h = hashlib.sha256()
-    csrc = os.path.join(ROOT, "permutohedral_lattice_amd", "csrc")
-    for name in sorted(os.listdir(csrc)):
-        if name.endswith((".hip", ".h", ".cpp")) and not name.startswith("bilateral_filter_cli"):
-            h.update(name.encode())
-            h.update(open(os.path.join(csrc, name), "rb").read())
-    return h.hexdigest()[:12]
+    from permutohedral_lattice_amd.build import source_hash
+    return source_hash()
 
 
 def measured_traffic(kernel_name, grid_threads, stem="bench_bilateral_1024_pd5_vd4"):
@@ -574,6 +568,16 @@ def main():
         print(json.dumps({"no_grid_hint_ms_per_step": {k: round(v, 4) for k, v in plain.items()}}))
         return
     side_legs = not args.headline_only
+    # The legs beside the headline drive entry points whose kernels hand arrays to each other in
+    # layouts this file's helpers assume; a library built from other sources than the ones in the
+    # tree (an experiment left in place) gets the headline only.
+    library_sources, tree_sources = pla.library_source_hash(), kernel_source_hash()
+    side_legs_refused = side_legs and library_sources != tree_sources
+    if side_legs_refused:
+        side_legs = False
+        print("bench.py: the loaded library was built from sources %s, the tree holds %s: headline "
+              "only; rebuild with `python permutohedral_lattice_amd/build.py`"
+              % (library_sources, tree_sources), file=sys.stderr)
     plain_ms, reuse_ms, double_ms = {}, 0.0, 0.0
     op_ms, batch_ms, batch = {}, {}, 4
     if side_legs:
@@ -629,7 +633,11 @@ def main():
                             "frac": round(filter_gbs / HBM_PEAK_GBS, 5)},
         "stage_ms": {k: round(v, 5) for k, v in stages.items()},
         "kernel_ms_per_filter": round(gpu_kernel_ms, 4),
+        "library_sources": library_sources,
     }
+    if side_legs_refused:
+        result["side_legs_refused"] = "library built from sources %s, tree holds %s" % (
+            library_sources, tree_sources)
     if side_legs:
         result.update({
             "no_grid_hint": {"what": "same step on a handle that was given no grid",
@@ -660,7 +668,7 @@ def main():
         result["configs"] = run_configs(args, pla, synth, not args.no_cpu)
         result["real_image"] = run_real_image(args, pla, not args.no_cpu)
 
-    if not args.no_cpu and not args.headline_only:
+    if not args.no_cpu and not args.headline_only and not side_legs_refused:
         import oracle
         ref = oracle.reference()
         cores = 1

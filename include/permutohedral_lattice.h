@@ -90,6 +90,21 @@ const char *pl_strerror(int status);
 int pl_last_hip_error(void);
 
 /*
+ * What this build of the library is, for bindings and harnesses that must not drive a library
+ * whose device-side array layouts differ from the ones they were written for (no handle, no GPU
+ * needed).  The reference has no counterpart: its host and device code are one translation unit.
+ */
+typedef enum pl_library_property {
+    PL_LIB_LAYOUT_VERSION = 1,   /* bumped whenever the layout of an array that one kernel writes and
+                                    another reads changes (replay rows, hash cells, per-vertex tables) */
+    PL_LIB_REPLAY_ROW_BYTES = 2, /* size of one replay row (vertex or cell, barycentric weight) */
+    PL_LIB_SOURCE_HASH = 3       /* first 48 bits of the SHA-256 over the library's source files as its
+                                    build script hashed them (0 when built without the script) */
+} pl_library_property;
+#define PL_LAYOUT_VERSION 3
+int pl_library_info(int what, long long *value);
+
+/*
  * Lattice for (pd, vd, N): pd feature dimensions, vd = value channels + 1 homogeneous, N points.
  * Stands in for PermutohedralLatticeCPU<T>(pd, vd, N) (src/PermutohedralLatticeCPU.h:419) and
  * PermutohedralLatticeGPU<T,pd,vd>(n, allocator, stream) (src/PermutohedralLatticeGPU.cuh:434).
@@ -117,8 +132,11 @@ int pl_filter(pl_handle h, float *output, const float *input, const float *posit
  * process, tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the
  * reference, whose lattice objects allocate in their constructors
  * (src/PermutohedralLatticeGPU.cuh:434-451).  No handle: the lattice lives for the length of the call
- * in a static device array of 64 MiB inside the library (one copy per GPU the library runs on,
- * held until the process ends), and the call makes no hipMalloc, hipFree, hipHostMalloc or event.
+ * in a static device array of 64 MiB inside the library, and the call makes no hipMalloc, hipFree,
+ * hipHostMalloc or event.  The array is part of the library's code object: every process that
+ * loads the library holds 64 MiB of device memory on each GPU it runs kernels of the library on,
+ * until the process ends, whether it ever calls this entry point or not.  `stream` must belong to
+ * the GPU that is current when the call is made (NULL: its default stream), else PL_EINVAL.
  * Limits: N*(pd+1) <= 131072 (e.g. 21845 points at pd = 5) and vd <= 8, float values; beyond them
  * PL_ETOOLARGE.  The hash table is sized for N*(pd+1) vertices, so no input makes it overflow.
  * The points are taken as a plain list (no grid is looked for).  Same results as pl_filter; the

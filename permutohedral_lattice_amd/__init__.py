@@ -27,10 +27,17 @@ PL_OPT_MERGE_TILES = 7
 PL_OPT_STOP_AFTER = 8
 PL_OPT_ORDER_POINTS = 9
 PL_INFO_BUILD_MERGED, PL_INFO_TABLE_CELLS, PL_INFO_SCRATCH_BYTES, PL_INFO_FOREIGN_ROWS = 1, 2, 3, 4
+PL_LIB_LAYOUT_VERSION, PL_LIB_REPLAY_ROW_BYTES, PL_LIB_SOURCE_HASH = 1, 2, 3
+# The device-side array layouts this module (and the tests and benchmarks on top of it) were
+# written for: PL_LAYOUT_VERSION of include/permutohedral_lattice.h and the size of a replay row.
+# A library that reports other values is not driven at all: its kernels would read each other's
+# arrays in a layout this side knows nothing of.
+LAYOUT_VERSION = 3
+REPLAY_ROW_BYTES = 8
 
 # every symbol include/permutohedral_lattice.h declares
 EXPORTS = (
-    "pl_supported", "pl_strerror", "pl_last_hip_error", "pl_create", "pl_destroy", "pl_filter",
+    "pl_supported", "pl_strerror", "pl_last_hip_error", "pl_library_info", "pl_create", "pl_destroy", "pl_filter",
     "pl_filter_static", "pl_build", "pl_apply", "pl_set_point_grid", "pl_get_point_grid", "pl_num_vertices", "pl_set_option", "pl_get_info", "pl_stage_ms", "pl_debug_simplex",
     "pl_debug_keys", "pl_debug_values", "pl_debug_replay", "pl_compute_positions", "pl_filter_image", "pl_build_image",
     "pl_filter_begin", "pl_filter_image_begin", "pl_filter_end", "pl_lattice_filter_op",
@@ -49,16 +56,31 @@ class PermutohedralError(RuntimeError):
         super().__init__("%s: %s" % (where, msg))
 
 
-def _load():
-    if not os.path.exists(LIB_PATH):
+def _library_property(lib, what):
+    v = C.c_longlong()
+    status = lib.pl_library_info(int(what), C.byref(v))
+    if status != PL_OK:
+        raise ImportError("pl_library_info(%d) failed with status %d" % (what, status))
+    return v.value
+
+
+def _load(path=LIB_PATH):
+    if not os.path.exists(path):
         raise ImportError(
             "%s is missing: build it with `python permutohedral_lattice_amd/build.py` "
-            "(there is no CPU fallback)" % LIB_PATH)
-    lib = C.CDLL(LIB_PATH)
+            "(there is no CPU fallback)" % path)
+    lib = C.CDLL(path)
     stale = [name for name in EXPORTS if not hasattr(lib, name)]
     if stale:
         raise ImportError("%s lacks %s: rebuild it with `python permutohedral_lattice_amd/build.py`"
-                          % (LIB_PATH, ", ".join(stale)))
+                          % (path, ", ".join(stale)))
+    lib.pl_library_info.argtypes = [C.c_int, C.POINTER(C.c_longlong)]
+    got = (_library_property(lib, PL_LIB_LAYOUT_VERSION), _library_property(lib, PL_LIB_REPLAY_ROW_BYTES))
+    if got != (LAYOUT_VERSION, REPLAY_ROW_BYTES):
+        raise ImportError(
+            "%s has array layout version %d with replay rows of %d bytes; this module drives version "
+            "%d with rows of %d bytes: rebuild it with `python permutohedral_lattice_amd/build.py`"
+            % (path, got[0], got[1], LAYOUT_VERSION, REPLAY_ROW_BYTES))
     vp, ci, cf = C.c_void_p, C.c_int, C.c_float
     lib.pl_supported.argtypes = [ci, ci]
     lib.pl_strerror.argtypes = [ci]
@@ -136,6 +158,12 @@ def _stream_ptr(stream=None):
 
 def supported(pd, vd):
     return bool(_lib.pl_supported(pd, vd))
+
+
+def library_source_hash():
+    """The hash of its sources the loaded library was built with, as 12 hex digits (what
+    ``build.source_hash()`` gives for the sources it was compiled from)."""
+    return "%012x" % _library_property(_lib, PL_LIB_SOURCE_HASH)
 
 
 class PermutohedralLattice:

@@ -29,6 +29,20 @@ FLAGS = [
 ]
 
 
+def source_hash():
+    """Short hash of the sources the library is built from (every .hip, .h and .cpp under csrc/
+    but the command-line tool): the library reports it (pl_library_info), so that a measurement or
+    a harness can tell which build of the kernels it is talking to."""
+    import hashlib
+    h = hashlib.sha256()
+    csrc = os.path.join(_HERE, "csrc")
+    for name in sorted(os.listdir(csrc)):
+        if name.endswith((".hip", ".h", ".cpp")) and not name.startswith("bilateral_filter_cli"):
+            h.update(name.encode())
+            h.update(open(os.path.join(csrc, name), "rb").read())
+    return h.hexdigest()[:12]
+
+
 def hipcc():
     for cand in (os.environ.get("HIPCC"), "/opt/rocm/bin/hipcc", "hipcc"):
         if cand and (os.path.isabs(cand) and os.path.exists(cand) or not os.path.isabs(cand)):
@@ -37,7 +51,7 @@ def hipcc():
 
 
 def build(verbose=False):
-    cmd = [hipcc()] + FLAGS + SOURCES + ["-o", LIB_PATH]
+    cmd = [hipcc()] + FLAGS + ["-DPL_SOURCE_HASH=0x%sLL" % source_hash()] + SOURCES + ["-o", LIB_PATH]
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)

@@ -127,7 +127,11 @@ struct pl_lattice {
     // how the last build numbered its vertices (plk::Counters): segments, and the fullest one
     int n_segments = 0, max_segment = 0;
     int last_n_segments = 0, last_max_segment = -1;
-    bool one_segment = false;          // the last build overflowed a segment of the largest table
+    // A build at the largest table whose vertices crowd one eighth of the image overflows that
+    // eighth's run of numbers: the call is repeated with the numbers in one run, and so are the
+    // next one_segment_backoff builds of this lattice (doubled every time it happens again, up to
+    // 1024) before eight runs are tried again.
+    int one_segment_for = 0, one_segment_backoff = 32;
     // A merging build numbers its vertices itself unless that costs more than it saves: when it
     // has many thousands of workgroups (they draw their numbers one after the other), or when
     // the last such build of these points held so many rows of sums for vertices of other
@@ -168,6 +172,9 @@ struct pl_lattice {
     int order_capacity = 0;
     hipEvent_t ev[EV_COUNT] = {};
     bool ev_recorded[EV_COUNT] = {};
+    // which of the eight stages pl_stage_ms reports launched a kernel in the last build / apply
+    // (an interval between two events with nothing in between still reads a few microseconds)
+    bool stage_ran[8] = {};
 
     // a filter call that has been enqueued but not yet checked on the host (pl_filter_*_begin)
     struct Pending {
@@ -393,6 +400,10 @@ int enqueue_build(pl_lattice *h, const plk::PointFeatures &features, const doubl
         h->cell_values_clean = true;
     }
     h->mark(EV_T0);
+    h->stage_ran[0] = h->map.mode == 1 || !h->table_clean || cells != h->n_cells;
+    h->stage_ran[1] = true;
+    h->stage_ran[2] = !numbers_in_build;
+    h->stage_ran[3] = true;
     if (h->map.mode == 1)
         PL_HIP(plk::order_by_locality(h->f64 ? nullptr : features.positions,
                                       h->f64 ? positions64 : nullptr, h->N, h->pd,
@@ -413,8 +424,8 @@ int enqueue_build(pl_lattice *h, const plk::PointFeatures &features, const doubl
     const plk::InBuildNumbering numbering{
         h->cell_vertex, h->vertex_keys, h->vertex_cell, h->neighbours, h->max_vertices(),
         h->values[0], h->f64 ? 2 * h->vd : h->vd,
-        !numbers_in_build ? 0 : (h->one_segment ? 1 : plk::segments_for((uint32_t)h->max_vertices()))};
-    h->one_segment = false;
+        !numbers_in_build ? 0 : (h->one_segment_for > 0 ? 1 : plk::segments_for((uint32_t)h->max_vertices()))};
+    if (numbers_in_build && h->one_segment_for > 0) h->one_segment_for -= 1;
     // keys go to the part of the table that belongs to their band of rows when the points are
     // known to be a grid (and feature 0 then runs with its slowest extent)
     plk::RegionSource regions{};
@@ -486,6 +497,10 @@ int enqueue_apply_f64(pl_lattice *h, double *output, const double *input, int re
     double *values[2] = {reinterpret_cast<double *>(h->values[0]),
                          reinterpret_cast<double *>(h->values[1])};
     h->mark(EV_A0);
+    h->stage_ran[4] = !h->values_splatted && !h->values_zeroed;
+    h->stage_ran[5] = !h->values_splatted;
+    h->stage_ran[6] = h->stop_after != 1;
+    h->stage_ran[7] = h->stop_after == 0;
     if (!h->values_splatted) {
         if (!h->values_zeroed)
             PL_HIP(plk::fill_zero(h->values[0], (size_t)mv * vd * 2, h->stream));
@@ -554,6 +569,10 @@ int enqueue_apply(pl_lattice *h, void *output_any, const void *input_any, int re
     const int in_channels = h->normalize ? vd - 1 : vd;
     const int mv = h->max_vertices();
     h->mark(EV_A0);
+    h->stage_ran[4] = !h->values_splatted && !h->values_zeroed;
+    h->stage_ran[5] = !h->values_splatted;
+    h->stage_ran[6] = h->stop_after != 1;
+    h->stage_ran[7] = h->stop_after == 0;
     if (!h->values_splatted) {
         if (!h->values_zeroed) PL_HIP(plk::fill_zero(h->values[0], (size_t)mv * vd, h->stream));
         h->mark(EV_FILL);
@@ -666,7 +685,8 @@ int verify_build(pl_lattice *h, uint32_t *retry_cells) {
             // one part of the image creates: once more with the numbers in one run
             if (status.n_segments <= 1 || (uint32_t)m > plk::max_vertices_for(h->n_cells))
                 return PL_EOVERFLOW;   // (cannot happen)
-            h->one_segment = true;
+            h->one_segment_for = h->one_segment_backoff;
+            h->one_segment_backoff = h->one_segment_backoff >= 512 ? 1024 : h->one_segment_backoff * 2;
             *retry_cells = h->n_cells;
             return PL_EOVERFLOW;
         }
@@ -711,6 +731,19 @@ const char *pl_strerror(int status) {
 }
 
 int pl_last_hip_error(void) { return g_last_hip_error; }
+
+#ifndef PL_SOURCE_HASH
+#define PL_SOURCE_HASH 0
+#endif
+int pl_library_info(int what, long long *value) {
+    if (!value) return PL_EINVAL;
+    switch (what) {
+        case PL_LIB_LAYOUT_VERSION: *value = PL_LAYOUT_VERSION; return PL_OK;
+        case PL_LIB_REPLAY_ROW_BYTES: *value = (long long)sizeof(plk::ReplayEntry); return PL_OK;
+        case PL_LIB_SOURCE_HASH: *value = (long long)(PL_SOURCE_HASH); return PL_OK;
+        default: return PL_EINVAL;
+    }
+}
 
 static int create_lattice(int pd, int vd, int N, bool f64, pl_stream stream, const pl_alloc *alloc,
                           pl_handle *out) {
@@ -865,6 +898,8 @@ int pl_set_point_grid(pl_handle h, int n_dims, const int *dims) {
     h->grid_given = n_dims > 0;
     h->map = plk::make_point_map(h->N, n_dims, dims);
     h->numbering_pass_pays = false;
+    h->one_segment_for = 0;
+    h->one_segment_backoff = 32;
     return ensure_replay(h, false);
 }
 
@@ -924,6 +959,8 @@ int guess_point_grid(pl_lattice *h, const float *positions) {
     if (dims[0] < 2) return PL_OK;
     h->map = plk::make_point_map(h->N, n_dims, dims);
     h->numbering_pass_pays = false;
+    h->one_segment_for = 0;
+    h->one_segment_backoff = 32;
     return ensure_replay(h, false);
 }
 
@@ -1186,7 +1223,7 @@ int pl_stage_ms(pl_handle h, float ms[8]) {
                              {EV_SPLAT, EV_BLUR}, {EV_BLUR, EV_SLICE}};
     for (int i = 0; i < 8; ++i) {
         ms[i] = 0.0f;
-        if (h->ev_recorded[pairs[i][0]] && h->ev_recorded[pairs[i][1]])
+        if (h->stage_ran[i] && h->ev_recorded[pairs[i][0]] && h->ev_recorded[pairs[i][1]])
             PL_HIP(hipEventElapsedTime(&ms[i], h->ev[pairs[i][0]], h->ev[pairs[i][1]]));
     }
     return PL_OK;
@@ -1619,6 +1656,13 @@ extern "C" int pl_filter_static(int pd, int vd, int N, float *output, const floa
     std::lock_guard<std::mutex> lock(g_static_mutex);
     int device = 0;
     PL_HIP(hipGetDevice(&device));
+    // the array's address is that of the current device: a stream of another GPU would run the
+    // kernels there with this one's address (NULL, the default stream, follows the current device)
+    if (stream) {
+        int stream_device = -1;
+        PL_HIP(hipStreamGetDevice((hipStream_t)stream, &stream_device));
+        if (stream_device != device) return PL_EINVAL;
+    }
     StaticLattice *st = nullptr;
     int rc = static_scratch_of(device, &st);
     if (rc != PL_OK) return rc;

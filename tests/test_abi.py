@@ -102,3 +102,58 @@ def test_python_constants_are_the_headers():
     assert len(found) >= 20
     for name, value in found.items():
         assert getattr(pla, name) == value, name
+
+
+def _stub_library(tmp_path, layout_version, row_bytes):
+    """A library with every export of the real one, all doing nothing, that reports the given
+    array layout: what a build of the kernels with another replay-row format would look like to
+    the loader."""
+    import subprocess
+    src = ["int pl_library_info(int what, long long *value) {",
+           "    *value = what == 1 ? %d : (what == 2 ? %d : 0);" % (layout_version, row_bytes),
+           "    return 0;", "}"]
+    for name in pla.EXPORTS:
+        if name == "pl_library_info":
+            continue
+        if name == "pl_strerror":
+            src.append('const char *pl_strerror(int s) { (void)s; return "stub"; }')
+        else:
+            src.append("int %s(void) { return 0; }" % name)
+    c_file = tmp_path / "stub.c"
+    c_file.write_text("\n".join(src) + "\n")
+    so = tmp_path / ("libstub_%d_%d.so" % (layout_version, row_bytes))
+    subprocess.run(["gcc", "-shared", "-fPIC", "-o", str(so), str(c_file)], check=True)
+    return str(so)
+
+
+def test_library_reports_the_layout_the_python_side_drives():
+    assert pla.LAYOUT_VERSION == pla._library_property(pla._lib, pla.PL_LIB_LAYOUT_VERSION)
+    assert pla.REPLAY_ROW_BYTES == pla._library_property(pla._lib, pla.PL_LIB_REPLAY_ROW_BYTES)
+    text = open(os.path.join(ROOT, "include", "permutohedral_lattice.h")).read()
+    assert int(re.search(r"#define PL_LAYOUT_VERSION (\d+)", text).group(1)) == pla.LAYOUT_VERSION
+    v = C.c_longlong()
+    assert pla._lib.pl_library_info(99, C.byref(v)) == pla.PL_EINVAL
+    assert pla._lib.pl_library_info(1, None) == pla.PL_EINVAL
+
+
+def test_library_source_hash_is_that_of_the_sources_in_the_tree():
+    from permutohedral_lattice_amd import build
+    assert pla.library_source_hash() == build.source_hash(), \
+        "the library in the tree was built from other sources: run permutohedral_lattice_amd/build.py"
+
+
+def test_a_library_with_another_array_layout_is_refused(tmp_path):
+    # same layout: loads
+    pla._load(_stub_library(tmp_path, pla.LAYOUT_VERSION, pla.REPLAY_ROW_BYTES))
+    # replay rows of 6 bytes, or another layout version: refused before anything is bound
+    with pytest.raises(ImportError, match="array layout version"):
+        pla._load(_stub_library(tmp_path, pla.LAYOUT_VERSION, 6))
+    with pytest.raises(ImportError, match="array layout version"):
+        pla._load(_stub_library(tmp_path, pla.LAYOUT_VERSION + 1, pla.REPLAY_ROW_BYTES))
+
+
+def test_documented_build_command_lists_every_source():
+    from permutohedral_lattice_amd import build
+    text = open(os.path.join(ROOT, "INTEGRATION.md")).read()
+    for path in build.SOURCES:
+        assert os.path.relpath(path, ROOT) in text, path

@@ -74,3 +74,34 @@ def test_static_filter_at_its_size_limit_and_beyond():
                           torch.empty((64, 8), dtype=torch.float32, device="cuda"),
                           torch.empty((64, 2), dtype=torch.float32, device="cuda"), 2, 9)
     assert e.value.status == pla.PL_ETOOLARGE
+
+
+def test_static_filter_leaves_the_free_device_memory_as_it_was():
+    """hipMemGetInfo before and after: an allocation that crept into the path (and was not given
+    back) would show, and so would one that is given back only later (the figures are read while
+    nothing else runs in this process)."""
+    pos, val = _case(64, 64, 105)
+    n = pos.shape[0]
+    d_pos, d_val = _dev(pos), _dev(val)
+    out = torch.empty((n, 3), dtype=torch.float32, device="cuda")
+    pla.filter_static(out, d_val, d_pos, 5, 4, False)      # (the first call on a device looks the array up)
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info()
+    lowest = free_before
+    for reverse in (False, True, False):
+        pla.filter_static(out, d_val, d_pos, 5, 4, reverse)
+        lowest = min(lowest, torch.cuda.mem_get_info()[0])
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after == free_before and lowest == free_before
+
+
+def test_static_filter_refuses_a_stream_of_another_kind_of_argument():
+    # (one GPU here: a stream of another device cannot be made; the current device's own stream passes)
+    pos, val = _case(32, 32, 106)
+    d_pos, d_val = _dev(pos), _dev(val)
+    out = torch.empty((pos.shape[0], 3), dtype=torch.float32, device="cuda")
+    s = torch.cuda.Stream()
+    with torch.cuda.stream(s):
+        pla.filter_static(out, d_val, d_pos, 5, 4, False, stream=s)
+    want = oracle.Lattice(5, 4, pos.shape[0]).filter(val, pos, False)
+    assert np.abs(out.cpu().numpy() - want).max() <= MAX_ABS_TOL
