@@ -64,6 +64,8 @@ def _load():
         fn("set_reference_growth_quirk").argtypes = [C.c_void_p, C.c_int]
         fn("num_growths").argtypes = [C.c_void_p]
         fn("num_growths").restype = C.c_int
+        fn("growth_keys").argtypes = [C.c_void_p, np.ctypeslib.ndpointer(np.int16, flags="C_CONTIGUOUS")]
+        fn("growth_keys").restype = C.c_int
         fn("num_vertices").argtypes = [C.c_void_p]
         fn("num_vertices").restype = C.c_int
         for name, typ in (("keys", C.c_int16), ("values", ct), ("replay_vertex", C.c_int32),
@@ -147,6 +149,14 @@ class Lattice:
     @property
     def num_growths(self):
         return self._fn("num_growths")(self._h)
+
+    @property
+    def growth_keys(self):
+        """[doublings, pd] int16: the key that was being looked up when the index doubled, per
+        doubling: with the quirk on, the lookups that probed from a stale cell."""
+        out = np.zeros((24, self.pd), np.int16)
+        n = self._fn("growth_keys")(self._h, out)
+        return out[:n].copy()
 
     def __del__(self):
         if getattr(self, "_h", None):
@@ -279,6 +289,8 @@ class _Ref:
                                      C.POINTER(C.c_int), C.c_void_p, C.POINTER(C.c_double)]
             fn("filter_stages").argtypes = [C.c_int, C.c_int, C.c_int, fp, fp, fp, C.c_int,
                                             C.POINTER(C.c_int), C.c_void_p, C.c_void_p, C.c_void_p]
+            fn("filter_replay").argtypes = [C.c_int, C.c_int, C.c_int, fp, fp, fp, C.c_int,
+                                            C.POINTER(C.c_int), C.c_void_p, C.c_void_p, C.c_void_p]
             fn("lattice_filter_op").argtypes = [fp, C.c_void_p, fp, C.c_int, C.c_int, _i32p,
                                                 C.c_int, C.c_int, C.c_int, C.c_float, C.c_float,
                                                 C.c_float, C.c_int]
@@ -351,6 +363,23 @@ class _Ref:
             res["after_splat"] = a[:m.value].copy()
             res["after_blur"] = b[:m.value].copy()
         return res
+
+    def filter_replay(self, pd, vd, inp, positions, reverse=False, dtype=np.float32):
+        """-> dict(output, M, keys [M, pd] in first-touch order, replay_vertex [N, pd+1],
+        replay_weight [N, pd+1]): one filter call and the rows its slice replayed."""
+        inp = np.ascontiguousarray(inp, dtype)
+        n = inp.size // (vd - 1)
+        inp = inp.reshape(n, vd - 1)
+        positions = np.ascontiguousarray(positions, dtype).reshape(n, pd)
+        out = np.empty_like(inp)
+        m = C.c_int()
+        keys = np.empty((n * (pd + 1), pd), np.int16)
+        vertex = np.empty((n, pd + 1), np.int32)
+        weight = np.empty((n, pd + 1), dtype)
+        self._fn("filter_replay", dtype)(pd, vd, n, out, inp, positions, int(reverse), C.byref(m),
+                                         _opt(keys), _opt(vertex), _opt(weight))
+        return dict(output=out, M=m.value, keys=keys[:m.value].copy(), replay_vertex=vertex,
+                    replay_weight=weight)
 
     def lattice_filter(self, input_image, reference_image, bilateral=True, theta_alpha=1.0,
                        theta_beta=1.0, theta_gamma=1.0, reverse=False):

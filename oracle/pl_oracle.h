@@ -78,6 +78,10 @@ void plo_filter_raw(plo_lattice *l, float *output, const float *input_vd,
 void plo_set_reference_growth_quirk(plo_lattice *l, int on);
 /* number of index doublings during the last splat/blur */
 int plo_num_growths(const plo_lattice *l);
+/* the key whose lookup triggered each doubling (the lookups that, in the reference, probe from a
+ * stale cell): out gets pd shorts per doubling, at most PLO_MAX_GROWTHS of them; returns how many */
+#define PLO_MAX_GROWTHS 24
+int plo_growth_keys(const plo_lattice *l, short *out);
 
 int plo_num_vertices(const plo_lattice *l);
 /* keys in first-touch order, M*pd shorts */
@@ -125,6 +129,7 @@ void plo_filter_raw_f64(plo_lattice_f64 *l, double *output, const double *input_
                         const double *positions, int reverse);
 void plo_set_reference_growth_quirk_f64(plo_lattice_f64 *l, int on);
 int plo_num_growths_f64(const plo_lattice_f64 *l);
+int plo_growth_keys_f64(const plo_lattice_f64 *l, short *out);
 int plo_num_vertices_f64(const plo_lattice_f64 *l);
 const short *plo_keys_f64(const plo_lattice_f64 *l);
 const double *plo_values_f64(const plo_lattice_f64 *l);

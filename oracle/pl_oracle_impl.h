@@ -160,6 +160,10 @@ struct PLO_LATTICE {
     int M;
     int n_growths;
     int stale_cell_after_growth;
+    /* the key that was being looked up when the index doubled, per doubling (pd shorts each,
+     * the first PLO_MAX_GROWTHS of them): with the quirk on, the lookups that probed from a
+     * stale cell */
+    short growth_keys[PLO_MAX_GROWTHS * 32];
     int *replay_vertex;      /* N*(pd+1) */
     PLO_T *replay_weight;    /* N*(pd+1) */
     double t_splat, t_blur, t_slice;
@@ -231,6 +235,8 @@ static int PLO_STATIC(vertex_find)(PLO_LATTICE *l, const short *key, int create)
     const int pd = l->pd;
     size_t c = PLO_STATIC(key_hash)(key, pd) % l->n_cells;
     if ((size_t)l->M >= l->n_cells / 2 - 1) {
+        if (l->n_growths < PLO_MAX_GROWTHS)
+            memcpy(l->growth_keys + (size_t)l->n_growths * 32, key, sizeof(short) * (size_t)pd);
         PLO_STATIC(index_grow)(l);
         if (!l->stale_cell_after_growth) c = PLO_STATIC(key_hash)(key, pd) % l->n_cells;
     }
@@ -252,6 +258,12 @@ static int PLO_STATIC(vertex_find)(PLO_LATTICE *l, const short *key, int create)
 
 void PLO_FN(set_reference_growth_quirk)(PLO_LATTICE *l, int on) { l->stale_cell_after_growth = on; }
 int PLO_FN(num_growths)(const PLO_LATTICE *l) { return l->n_growths; }
+int PLO_FN(growth_keys)(const PLO_LATTICE *l, short *out) {
+    const int n = l->n_growths < PLO_MAX_GROWTHS ? l->n_growths : PLO_MAX_GROWTHS;
+    for (int g = 0; g < n; ++g)
+        memcpy(out + (size_t)g * l->pd, l->growth_keys + (size_t)g * 32, sizeof(short) * (size_t)l->pd);
+    return n;
+}
 
 PLO_LATTICE *PLO_FN(create)(int pd, int vd, int N) {
     if (pd < 1 || vd < 2 || N < 0) return NULL;

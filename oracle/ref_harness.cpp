@@ -112,6 +112,29 @@ void filter_stages(int pd, int vd, int N, T *output, const T *input,
     }
 }
 
+// One filter call that also hands out what the slice replays: per point and simplex corner the
+// index of the vertex the splat's lookup returned and its weight (matrix[n*(pd+1)+r], the
+// reference's {offset = vertex*vd, weight}), and the vertex keys in first-touch order.  Where the
+// reference's index doubled and entered a key twice, the list holds that key twice and the rows
+// say which of the two each point was given.
+template <typename T>
+void filter_replay(int pd, int vd, int N, T *output, const T *input, const T *positions,
+                   int reverse, int *num_vertices, short *keys_out, int *replay_vertex,
+                   T *replay_weight) {
+    PermutohedralLatticeCPU<T> lattice(pd, vd, N);
+    lattice.filter(output, input, positions, reverse != 0);
+    const int M = lattice.hashTable.size();
+    if (num_vertices) *num_vertices = M;
+    if (keys_out) {
+        const short *k = lattice.hashTable.getKeys();
+        for (size_t i = 0; i < size_t(M) * pd; ++i) keys_out[i] = k[i];
+    }
+    for (size_t i = 0; i < size_t(N) * (pd + 1); ++i) {
+        if (replay_vertex) replay_vertex[i] = lattice.matrix[i].offset / vd;
+        if (replay_weight) replay_weight[i] = lattice.matrix[i].weight;
+    }
+}
+
 // The op's per-batch-item loop (src/LatticeFilterKernel.cpp:111-179) driven through the
 // reference's own CPU functor bodies (compute_kernel_cpu + PermutohedralLatticeCPU::filter).
 template <typename T>
@@ -165,6 +188,12 @@ int lattice_filter_op(const T *input, const T *reference, T *output, int batch,
                                      double *stage_seconds) {                                      \
         filter_stages<T>(pd, vd, N, output, input, positions, reverse, num_vertices,               \
                          values_after_splat, values_after_blur, stage_seconds);                    \
+    }                                                                                              \
+    void plref_filter_replay##SUFFIX(int pd, int vd, int N, T *output, const T *input,             \
+                                     const T *positions, int reverse, int *num_vertices,           \
+                                     short *keys_out, int *replay_vertex, T *replay_weight) {      \
+        filter_replay<T>(pd, vd, N, output, input, positions, reverse, num_vertices, keys_out,     \
+                         replay_vertex, replay_weight);                                            \
     }                                                                                              \
     int plref_lattice_filter_op##SUFFIX(const T *input, const T *reference, T *output, int batch,  \
                                         int n_spatial_dims, const int *spatial_dims,               \

@@ -49,10 +49,49 @@ def lattice_case(ref, name, pd, vd, positions, values, per_point=True, dtype=np.
                                                        os.path.getsize(path) / 1024))
 
 
+def growth_case(ref, name, side, theta_alpha, theta_beta, seed, noise):
+    """A case whose vertex count makes the reference's hash index double three times.  The lookup
+    that triggers a doubling probes from a stale cell (src/PermutohedralLatticeCPU.h:163-165, :62):
+    it can enter a key a second time or miss a neighbour.  Stored: the image (positions are
+    synth.bilateral_positions of it, values its colours), and from the reference's own build the
+    outputs of both blur orders, the vertex keys in first-touch order (a duplicated key appears
+    twice) and the vertex each replay row names; from the oracle with the quirk reproduced, the
+    key that was being looked up at each doubling."""
+    import hashlib
+    img = synth.blob_image(side, side, seed=seed, noise=noise)
+    positions = synth.bilateral_positions(img, theta_alpha, theta_beta)
+    values = np.ascontiguousarray(img.reshape(-1, 3))
+    fwd = ref.filter_replay(5, 4, values, positions, False)
+    rev = ref.filter_replay(5, 4, values, positions, True)
+    assert fwd["M"] == rev["M"] and np.array_equal(fwd["keys"], rev["keys"])
+    quirk = oracle.Lattice(5, 4, side * side, reference_growth_quirk=True)
+    assert np.array_equal(quirk.filter(values, positions, False), fwd["output"])
+    growth_keys = quirk.growth_keys
+    path = os.path.join(HERE, "%s.npz" % name)
+    np.savez_compressed(
+        path, pd=np.int32(5), vd=np.int32(4), side=np.int32(side),
+        thetas=np.array([theta_alpha, theta_beta], np.float32), image=img.astype(np.float32),
+        positions_sha256=np.frombuffer(hashlib.sha256(positions.tobytes()).digest(), np.uint8),
+        num_vertices=np.int32(fwd["M"]), vertex_keys=fwd["keys"],
+        replay_vertex=fwd["replay_vertex"].astype(np.int32),
+        output_forward=fwd["output"], output_reverse=rev["output"],
+        growth_keys=growth_keys)
+    distinct = len(np.unique(fwd["keys"], axis=0))
+    print("%-28s N=%6d M=%6d distinct=%6d doublings=%d  %7.1f KB" % (
+        name, side * side, fwd["M"], distinct, len(growth_keys), os.path.getsize(path) / 1024))
+
+
 def main():
     ref = oracle.reference()
     if ref is None:
         raise SystemExit("oracle/_ref/libplref.so is missing: run `make -C oracle ref` first")
+
+    # `make_golden.py growth` writes only the case of three doublings (the other fixtures are
+    # reproduced bit for bit by a full run, but their archives would change with the date)
+    growth_only = len(sys.argv) > 1 and sys.argv[1] == "growth"
+    growth_case(ref, "growth_three_doublings_pd5_vd4", 256, 3.0, 0.04, 141, 0.03)
+    if growth_only:
+        return
 
     # scale factors, bit patterns
     factors = {"pd%d" % pd: ref.scale_factor(pd) for pd in range(1, 9)}

@@ -386,3 +386,62 @@ def test_op_uses_theta_gamma_when_not_bilateral():
     direct = oracle.Lattice(2, 3, 1024).filter(img.reshape(-1, 2), pos)
     assert (bits(out.reshape(-1, 2)) == bits(direct)).all()
     assert rel_l2(out, img) > 1e-3
+
+
+# ---------------------------------------------------------------------------------------------
+# three doublings of the reference's index: where its outputs differ from one vertex per key
+# ---------------------------------------------------------------------------------------------
+
+def _growth_fixture():
+    import hashlib
+    from permutohedral_lattice_amd import synth
+    g = load_golden("growth_three_doublings_pd5_vd4")
+    img = g["image"]
+    pos = synth.bilateral_positions(img, float(g["thetas"][0]), float(g["thetas"][1]))
+    assert hashlib.sha256(pos.tobytes()).digest() == g["positions_sha256"].tobytes()
+    return g, pos, np.ascontiguousarray(img.reshape(-1, 3))
+
+
+def test_three_doublings_quirk_mode_is_the_reference_bit_for_bit():
+    g, pos, val = _growth_fixture()
+    n = pos.shape[0]
+    lat = oracle.Lattice(5, 4, n, reference_growth_quirk=True)
+    out = lat.filter(val, pos, False)
+    assert lat.num_growths == 3 and len(g["growth_keys"]) == 3
+    assert lat.num_vertices == int(g["num_vertices"])
+    assert np.array_equal(lat.keys(), g["vertex_keys"])
+    assert np.array_equal(lat.replay()[0].reshape(n, 6), g["replay_vertex"])
+    assert np.array_equal(bits(out), bits(g["output_forward"]))
+    assert np.array_equal(lat.growth_keys, g["growth_keys"])
+    rev = oracle.Lattice(5, 4, n, reference_growth_quirk=True).filter(val, pos, True)
+    assert np.array_equal(bits(rev), bits(g["output_reverse"]))
+
+
+def test_three_doublings_difference_is_confined_to_the_keys_looked_up_at_the_doublings():
+    """One vertex per distinct key (the oracle's default, what the HIP library builds) against the
+    reference's own outputs: bit-equal at every point that has no simplex vertex within one blur
+    step per axis of a key that was being looked up when the index doubled; the duplicated key is
+    one of those; the deviation inside is the documented one (above the 1e-3 tolerance here)."""
+    from growth_quirk import blur_neighbourhood, duplicated_keys, points_touching
+    g, pos, val = _growth_fixture()
+    n = pos.shape[0]
+    dup_keys, n_dup = duplicated_keys(g["vertex_keys"])
+    assert n_dup == 1
+    growth = {k.tobytes() for k in g["growth_keys"]}
+    assert all(k.tobytes() in growth for k in dup_keys)
+    lat = oracle.Lattice(5, 4, n)
+    out = lat.filter(val, pos, False)
+    rev = oracle.Lattice(5, 4, n).filter(val, pos, True)
+    assert lat.num_vertices == int(g["num_vertices"]) - n_dup
+    near = points_touching(oracle.dump_simplex(pos)["keys"], blur_neighbourhood(g["growth_keys"], 5))
+    assert 0 < near.sum() <= 256 * len(g["growth_keys"])          # 543 of 65 536 points
+    # the points whose replay rows name a duplicated vertex are among them
+    dup_vertices = [v for v in range(len(g["vertex_keys"]))
+                    if any((g["vertex_keys"][v] == k).all() for k in dup_keys)]
+    named = np.isin(g["replay_vertex"], dup_vertices).any(axis=1)
+    assert named.any() and not (named & ~near).any()
+    for got, want in ((out, g["output_forward"]), (rev, g["output_reverse"])):
+        assert np.array_equal(bits(got[~near]), bits(want[~near]))
+        d = np.abs(got - want).max(axis=1)
+        assert 1e-3 < d.max() < 5e-3                                # 1.43e-3 both ways
+        assert (d > 1e-4).sum() <= 64 * len(g["growth_keys"])       # 110 forward, 85 reverse
