@@ -72,6 +72,12 @@ typedef enum pl_option {
                                splat, 2: behind the blur; the output is then not written and
                                pl_debug_values gives the vertex values of that stage (for checking the
                                stages one by one against src/PermutohedralLatticeCPU.h:306-317, 362-415) */
+    PL_OPT_VERTEX_LISTS = 10, /* 1 (default): pl_build also writes, per vertex, the list of the (point,
+                               weight) rows that name it, and every pl_apply on that lattice splats
+                               by gathering along those lists (no atomics, the same order of
+                               additions on every call); 0: pl_apply splats as pl_filter does, point
+                               by point with sums per wavefront (same results up to the order of
+                               float additions; for measuring the difference).  Float lattices. */
     PL_OPT_ORDER_POINTS = 9 /* 1 (default): points that are a plain list (no grid given or found, at
                                least 4096 of them) are worked on in an order in which neighbours in
                                space are neighbours in the list, found anew by every build from the

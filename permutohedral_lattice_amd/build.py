@@ -15,7 +15,7 @@ _ROOT = os.path.dirname(_HERE)
 LIB_PATH = os.path.join(_HERE, "libpermutohedral_hip.so")
 
 SOURCES = [os.path.join(_HERE, "csrc", name)
-           for name in ("pl_kernels.hip", "pl_kernels_f64.hip", "pl_order.hip", "pl_api.cpp")]
+           for name in ("pl_kernels.hip", "pl_kernels_f64.hip", "pl_order.hip", "pl_gather.hip", "pl_api.cpp")]
 
 # -ffp-contract=off: the lattice's integer results need unfused IEEE float operations.
 # -munsafe-fp-atomics: float atomicAdd becomes the hardware global_atomic_add_f32.

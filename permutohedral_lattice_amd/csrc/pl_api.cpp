@@ -114,6 +114,14 @@ struct pl_lattice {
     size_t replay_capacity = 0;
     bool lists_wide = false;               // created_entries has room for two entries per vertex
 
+    // A lattice that is built to be applied (pl_build) also gets, per vertex, the list of the
+    // (point, weight) that touch it; pl_apply then splats by gathering (plk::VertexLists)
+    bool vertex_lists = true;              // option
+    plk::VertexLists lists_of_vertices{};
+    size_t lists_for_vertices = 0;         // max_vertices the arrays were allocated for
+    bool lists_valid = false;              // they describe the last build
+    unsigned list_chunks = 0, long_lists = 0;   // of the last build: chunks in all, lists of several
+
     plk::Counters *d_counters = nullptr;   // two sets, used by alternate builds
     int counter_set = 0;                   // the set of the last build
     plk::HostStatus *h_status = nullptr;   // pinned, written by the device
@@ -291,6 +299,45 @@ int ensure_replay(pl_lattice *h, bool wide) {
     return PL_OK;
 }
 
+int ensure_vertex_lists(pl_lattice *h) {
+    const size_t mv = plk::max_vertices_for(h->n_cells_alloc);
+    plk::VertexLists &l = h->lists_of_vertices;
+    if (l.start && h->lists_for_vertices >= mv && l.capacity >= h->replay_capacity) return PL_OK;
+    PL_HIP(hipStreamSynchronize(h->stream));
+    h->dfree(l.start);
+    h->dfree(l.entries);
+    h->dfree(l.count);
+    h->dfree(l.places);
+    h->dfree(l.block_sums);
+    h->dfree(l.chunks.chunk_start);
+    h->dfree(l.chunks.chunk);
+    h->dfree(l.chunks.long_lists);
+    h->dfree(l.chunks.partial_rows);
+    h->lists_for_vertices = 0;
+    l.capacity = 0;
+    const size_t rows = h->replay_capacity ? h->replay_capacity : 1;
+    const size_t max_chunks = plk::vertex_list_max_chunks((int)mv, rows);
+    const size_t max_long = plk::vertex_list_max_long(rows);
+    l.start = (unsigned *)h->dmalloc(sizeof(unsigned) * (mv + 1));
+    l.entries = (plk::ListEntry *)h->dmalloc(sizeof(plk::ListEntry) * rows);
+    l.count = (unsigned *)h->dmalloc(sizeof(unsigned) * (mv + 2));
+    l.places = (unsigned *)h->dmalloc(sizeof(unsigned) * rows);
+    l.block_sums = (unsigned *)h->dmalloc(sizeof(unsigned) * 2 * (plk::vertex_list_scan_blocks((int)mv) + 1));
+    l.chunks.chunk_start = (unsigned *)h->dmalloc(sizeof(unsigned) * (mv + 1));
+    l.chunks.chunk = (plk::ListChunk *)h->dmalloc(sizeof(plk::ListChunk) * max_chunks);
+    l.chunks.long_lists = (unsigned *)h->dmalloc(sizeof(unsigned) * max_long);
+    l.chunks.partial_rows = (float *)h->dmalloc(sizeof(float) * max_chunks * (size_t)h->vd);
+    if (!l.start || !l.entries || !l.count || !l.places || !l.block_sums || !l.chunks.chunk_start ||
+        !l.chunks.chunk || !l.chunks.long_lists || !l.chunks.partial_rows)
+        return PL_ENOMEM;
+    l.chunks.info = l.count + mv;
+    l.chunks.max_chunks = (unsigned)max_chunks;
+    l.chunks.max_long = (unsigned)max_long;
+    h->lists_for_vertices = mv;
+    l.capacity = h->replay_capacity;
+    return PL_OK;
+}
+
 // The arrays of the ordering pass for a plain list of N points
 plk::LocalityScratch locality_scratch(const pl_lattice *h) {
     const unsigned max_bins = plk::locality_bins_for(h->N);
@@ -317,6 +364,15 @@ int ensure_order(pl_lattice *h) {
     h->dfree(h->point_order);
     h->dfree(h->locality_words);
     h->dfree(h->bin_rank);
+    h->dfree(h->lists_of_vertices.start);
+    h->dfree(h->lists_of_vertices.entries);
+    h->dfree(h->lists_of_vertices.count);
+    h->dfree(h->lists_of_vertices.places);
+    h->dfree(h->lists_of_vertices.block_sums);
+    h->dfree(h->lists_of_vertices.chunks.chunk_start);
+    h->dfree(h->lists_of_vertices.chunks.chunk);
+    h->dfree(h->lists_of_vertices.chunks.long_lists);
+    h->dfree(h->lists_of_vertices.chunks.partial_rows);
     h->order_capacity = 0;
     const unsigned max_bins = plk::locality_bins_for(h->N);
     const size_t words = 32 + 2 * (size_t)max_bins + 3 * (size_t)plk::locality_scan_chunks(max_bins) + 1;
@@ -486,6 +542,7 @@ int enqueue_build(pl_lattice *h, const plk::PointFeatures &features, const doubl
     h->values_splatted = fused;
     h->built = true;
     h->verified = false;
+    h->lists_valid = false;
     return PL_OK;
 }
 
@@ -569,11 +626,17 @@ int enqueue_apply(pl_lattice *h, void *output_any, const void *input_any, int re
     const int in_channels = h->normalize ? vd - 1 : vd;
     const int mv = h->max_vertices();
     h->mark(EV_A0);
-    h->stage_ran[4] = !h->values_splatted && !h->values_zeroed;
+    const bool gather = !h->values_splatted && h->lists_valid;
+    h->stage_ran[4] = !h->values_splatted && !h->values_zeroed && !gather;
     h->stage_ran[5] = !h->values_splatted;
     h->stage_ran[6] = h->stop_after != 1;
     h->stage_ran[7] = h->stop_after == 0;
-    if (!h->values_splatted) {
+    if (gather) {
+        // (every vertex's row is written whole: nothing to clear)
+        h->mark(EV_FILL);
+        PL_HIP(plk::splat_gather(vd, h->lists_of_vertices, h->list_chunks, h->long_lists, input,
+                                 in_channels, h->values[0], h->stream));
+    } else if (!h->values_splatted) {
         if (!h->values_zeroed) PL_HIP(plk::fill_zero(h->values[0], (size_t)mv * vd, h->stream));
         h->mark(EV_FILL);
         PL_HIP(plk::splat(pd, vd, h->map, input, in_channels, h->replay,
@@ -790,7 +853,8 @@ static int create_lattice(int pd, int vd, int N, bool f64, pl_stream stream, con
                                                  2 * sizeof(plk::Counters) / sizeof(float), h->stream)))
         rc = PL_EHIP;
     if (rc == PL_OK &&
-        hip_failed(hipHostMalloc((void **)&h->h_status, sizeof(plk::HostStatus), hipHostMallocDefault)))
+        hip_failed(hipHostMalloc((void **)&h->h_status, sizeof(plk::HostStatus) + 2 * sizeof(unsigned),
+                                 hipHostMallocDefault)))
         rc = PL_EHIP;
     if (rc == PL_OK && hip_failed(hipEventCreateWithFlags(&h->status_written, hipEventDisableTiming)))
         rc = PL_EHIP;
@@ -867,6 +931,10 @@ int pl_set_option(pl_handle h, int option, long value) {
             return PL_OK;
         case PL_OPT_ORDER_POINTS:
             h->order_points = value != 0;
+            return PL_OK;
+        case PL_OPT_VERTEX_LISTS:
+            h->vertex_lists = value != 0;
+            if (!h->vertex_lists) h->lists_valid = false;
             return PL_OK;
         case PL_OPT_STOP_AFTER:
             if (value < 0 || value > 2) return PL_EINVAL;
@@ -999,14 +1067,39 @@ int build_lattice(pl_lattice *h, const plk::PointFeatures &features,
         h->built = h->verified = true;
         return PL_OK;
     }
+    // The lattice is there to be applied: per vertex the list of the rows that name it, so that
+    // every apply splats by gathering (float values; a build without a splat numbers its vertices
+    // densely).  The lists are enqueued behind the build, before the host waits for its report.
+    const bool lists = h->vertex_lists && !h->f64 && !h->status_on_device;
     uint32_t cells = initial_cells(h);
     for (;;) {
         int rc = enqueue_build(h, features, positions64, cells, nullptr);
         if (rc != PL_OK) return rc;
+        if (lists) {
+            rc = ensure_vertex_lists(h);
+            if (rc != PL_OK) return rc;
+            PL_HIP(plk::build_vertex_lists(h->pd, h->map, h->replay,
+                                           h->replay_holds_cells ? h->cell_vertex : nullptr,
+                                           h->max_vertices(), h->lists_of_vertices,
+                                           reinterpret_cast<unsigned *>(h->h_status + 1), h->stream));
+            h->replay_holds_cells = false;
+        }
         rc = verify_build(h, &cells);
-        if (rc == PL_OK) return PL_OK;
+        if (rc == PL_OK) break;
         if (!cells) return rc;
     }
+    if (lists && h->n_segments == 0) {
+        // (how many chunks there are, and whether any list has several, sizes every apply's
+        // launches: read once here, where the caller is building and expects to wait)
+        // (the last kernel of the lists wrote them behind the build's status, in pinned memory)
+        PL_HIP(hipStreamSynchronize(h->stream));
+        const volatile unsigned *info = reinterpret_cast<const volatile unsigned *>(h->h_status + 1);
+        const plk::ListChunks &c = h->lists_of_vertices.chunks;
+        h->long_lists = info[0] < c.max_long ? info[0] : c.max_long;
+        h->list_chunks = info[1] < c.max_chunks ? info[1] : c.max_chunks;
+        h->lists_valid = true;
+    }
+    return PL_OK;
 }
 
 // pl_filter in two halves.  begin: build and apply are enqueued together and the call returns.
@@ -1200,6 +1293,12 @@ int pl_get_info(pl_handle h, int what, long *value) {
             if (h->cell_values) b += h->value_size() * (size_t)h->n_cells_alloc * h->vd;
             b += h->replay_capacity * (sizeof(plk::ReplayEntry) + sizeof(uint4) +
                                        (h->f64 ? sizeof(double) : 0));
+            if (h->lists_of_vertices.start)
+                b += sizeof(unsigned) * (3 * h->lists_for_vertices + 5 +
+                                         plk::vertex_list_scan_blocks((int)h->lists_for_vertices) +
+                                         h->lists_of_vertices.chunks.max_long) +
+                     (size_t)h->lists_of_vertices.chunks.max_chunks * (sizeof(plk::ListChunk) + sizeof(float) * h->vd) +
+                     h->lists_of_vertices.capacity * (sizeof(plk::ListEntry) + sizeof(unsigned));
             if (h->point_order) {
                 const unsigned max_bins = plk::locality_bins_for(h->order_capacity);
                 b += sizeof(int) * 256 * (size_t)plk::locality_tiles_for(h->order_capacity) +

@@ -1,0 +1,512 @@
+// The splat of a lattice that is applied many times, as a gather.
+//
+// The reference splats point by point (src/PermutohedralLatticeCPU.h:306-326; its CUDA path with
+// atomics, src/PermutohedralLatticeGPU.cuh:273-333).  The splat kernels of pl_kernels.hip do the
+// same per wavefront: they find, on every call, which of a wavefront's points share a vertex, sum
+// those in registers and add the sums with one atomic request per wavefront and vertex.  For a
+// lattice that is built once and applied many times (pl_build, then pl_apply) none of that changes
+// between the calls, so the build can write the transpose of the replay matrix once: for every
+// vertex the list of (point, weight) that touch it, one run of a single array in vertex order
+// (compressed rows).  The splat is then a gather per vertex: no election, no atomics, no zero fill
+// of the value table, and sums that are added in the same order on every call.
+//
+// Lists differ in length by orders of magnitude (a wide kernel over a flat part of an image gives
+// one vertex ten thousand rows while most have twenty), so the unit of work is a chunk of at most
+// kListChunk rows of one list: a list of one chunk is summed straight into the value table, the
+// chunks of a longer list into partial rows that a second, small launch adds up.
+//
+// This translation unit needs no -ffp-contract=off (nothing here decides an integer), but is
+// compiled with the same flags as the others.
+#include "pl_kernels.h"
+#include "pl_device.h"
+
+namespace plk {
+
+namespace {
+
+using namespace device;
+
+// ------------------------------------------------------------------------------------------------
+// Lists, step 1: every (point, corner) draws its place in its vertex's list.  The lanes of a
+// wavefront that name the same vertex are found as in the splat (one turn per distinct vertex,
+// no memory access in it); then the lowest lane of each group adds the group's size to the
+// vertex's count with one returning atomic -- all of a wavefront's in flight together -- and a
+// lane's place is what came back plus its rank in the group.  Rows that still hold hash cells are
+// translated to vertices and written back, as the first splat after a build does.
+// ------------------------------------------------------------------------------------------------
+template <int D1>
+__global__ __launch_bounds__(kBlock) void k_list_places(PointMap map, ReplayEntry *replay,
+                                                         const int *__restrict__ cell_vertex,
+                                                         unsigned *count, unsigned *places,
+                                                         int max_vertices) {
+    unsigned vblock;
+    if (!block_of_points(map, 1, vblock)) return;
+    const size_t t = (size_t)vblock * kBlock + threadIdx.x;
+    const size_t T = (size_t)gridDim.x * kBlock;
+    const int n = point_of_thread(map, vblock, threadIdx.x);
+    const int lane = threadIdx.x & 63;
+
+    int vertex[D1];
+#pragma unroll
+    for (int r = 0; r < D1; ++r) vertex[r] = n >= 0 ? replay[(size_t)r * T + t].index : -1;
+    if (cell_vertex) {
+#pragma unroll
+        for (int r = 0; r < D1; ++r)
+            if (vertex[r] >= 0) vertex[r] = cell_vertex[vertex[r]];
+#pragma unroll
+        for (int r = 0; r < D1; ++r)
+            if (n >= 0) replay[(size_t)r * T + t].index = vertex[r];
+    }
+    int leader[D1], rank[D1], size[D1];
+#pragma unroll
+    for (int r = 0; r < D1; ++r) {
+        // (a vertex number beyond the table cannot come out of a build that fitted; such a row
+        // would take no part)
+        if ((unsigned)vertex[r] >= (unsigned)max_vertices) vertex[r] = -1;
+        leader[r] = lane;
+        rank[r] = 0;
+        size[r] = 0;
+        uint64_t remaining = wave_ballot(vertex[r] >= 0);
+        while (remaining) {
+            const int first = __builtin_ctzll(remaining);
+            const uint64_t group = lanes_equal(vertex[r], lane_value(vertex[r], first)) & remaining;
+            remaining &= ~group;
+            if (lane_in(group)) {
+                leader[r] = first;
+                rank[r] = (int)__builtin_amdgcn_mbcnt_hi((uint32_t)(group >> 32),
+                                                         __builtin_amdgcn_mbcnt_lo((uint32_t)group, 0u));
+                size[r] = lanes_in(group);
+            }
+        }
+    }
+    unsigned base[D1];
+#pragma unroll
+    for (int r = 0; r < D1; ++r)
+        base[r] = (vertex[r] >= 0 && leader[r] == lane) ? atomicAdd(&count[vertex[r]], (unsigned)size[r]) : 0u;
+#pragma unroll
+    for (int r = 0; r < D1; ++r) {
+        const unsigned b = (unsigned)__shfl((int)base[r], leader[r]);
+        if (vertex[r] >= 0) places[(size_t)r * T + t] = b + (unsigned)rank[r];
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Lists, step 2: where every vertex's list starts, and where its chunks start: exclusive prefix
+// sums over all n vertex numbers of the table (numbers without a vertex count zero) of the counts
+// and of the chunks the counts make, both in one pass of three launches: sums of blocks of
+// kScanItems items; a scan of those by one workgroup; the scan inside each block from its start.
+// The last launch also describes the chunk of every list that has one chunk and names the lists
+// that have several (in the order the atomics give; each of those is summed on its own), whose
+// chunks a small launch describes.  start[n], chunk_start[n]: the totals.
+// ------------------------------------------------------------------------------------------------
+constexpr int kScanPerThread = 8;
+constexpr int kScanItems = kBlock * kScanPerThread;
+
+__host__ __device__ inline unsigned chunks_of(unsigned count) {
+    return (count + (unsigned)kListChunk - 1u) / (unsigned)kListChunk;
+}
+
+// exclusive prefix sums of one pair of values per thread over the workgroup; *total: the sums of all
+__device__ __forceinline__ uint2 block_exclusive_scan(uint2 x, uint2 *total) {
+    __shared__ uint2 wave_sum[kBlock / 64];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    uint2 inclusive = x;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const unsigned a = (unsigned)__shfl_up((int)inclusive.x, off);
+        const unsigned b = (unsigned)__shfl_up((int)inclusive.y, off);
+        if (lane >= off) {
+            inclusive.x += a;
+            inclusive.y += b;
+        }
+    }
+    __syncthreads();   // (wave_sum may still be read by a previous call)
+    if (lane == 63) wave_sum[wave] = inclusive;
+    __syncthreads();
+    uint2 before = make_uint2(0u, 0u), all = make_uint2(0u, 0u);
+#pragma unroll
+    for (int w = 0; w < kBlock / 64; ++w) {
+        const uint2 s = wave_sum[w];
+        before.x += w < wave ? s.x : 0u;
+        before.y += w < wave ? s.y : 0u;
+        all.x += s.x;
+        all.y += s.y;
+    }
+    *total = all;
+    return make_uint2(before.x + inclusive.x - x.x, before.y + inclusive.y - x.y);
+}
+
+// (also zeroes info[0], the number of long lists, which the last launch of the pass counts)
+__global__ __launch_bounds__(kBlock) void k_scan_block_sums(const unsigned *__restrict__ count,
+                                                             unsigned n, uint2 *block_sums,
+                                                             unsigned *info) {
+    if (blockIdx.x == 0 && threadIdx.x == 0) info[0] = 0u;
+    const size_t first = (size_t)blockIdx.x * kScanItems + (size_t)threadIdx.x * kScanPerThread;
+    uint2 sum = make_uint2(0u, 0u);
+#pragma unroll
+    for (int i = 0; i < kScanPerThread; ++i) {
+        const unsigned c = first + i < n ? count[first + i] : 0u;
+        sum.x += c;
+        sum.y += chunks_of(c);
+    }
+    uint2 total;
+    (void)block_exclusive_scan(sum, &total);
+    if (threadIdx.x == 0) block_sums[blockIdx.x] = total;
+}
+
+// block_sums[0 .. n_blocks) := their exclusive prefix sums, block_sums[n_blocks] := the totals
+__global__ __launch_bounds__(kBlock) void k_scan_of_block_sums(uint2 *block_sums, unsigned n_blocks) {
+    uint2 carry = make_uint2(0u, 0u);
+    for (unsigned first = 0; first < n_blocks; first += kBlock) {
+        const unsigned i = first + threadIdx.x;
+        const uint2 x = i < n_blocks ? block_sums[i] : make_uint2(0u, 0u);
+        uint2 total;
+        const uint2 before = block_exclusive_scan(x, &total);
+        if (i < n_blocks) block_sums[i] = make_uint2(carry.x + before.x, carry.y + before.y);
+        carry.x += total.x;
+        carry.y += total.y;
+    }
+    if (threadIdx.x == 0) block_sums[n_blocks] = carry;
+}
+
+__global__ __launch_bounds__(kBlock) void k_scan_starts(const unsigned *__restrict__ count, unsigned n,
+                                                         const uint2 *__restrict__ block_sums,
+                                                         unsigned *start, ListChunks chunks) {
+    const size_t first = (size_t)blockIdx.x * kScanItems + (size_t)threadIdx.x * kScanPerThread;
+    unsigned c[kScanPerThread];
+    uint2 sum = make_uint2(0u, 0u);
+#pragma unroll
+    for (int i = 0; i < kScanPerThread; ++i) {
+        c[i] = first + i < n ? count[first + i] : 0u;
+        sum.x += c[i];
+        sum.y += chunks_of(c[i]);
+    }
+    uint2 total;
+    const uint2 base = block_sums[blockIdx.x];
+    const uint2 before = block_exclusive_scan(sum, &total);
+    unsigned entry = base.x + before.x, chunk = base.y + before.y;
+#pragma unroll
+    for (int i = 0; i < kScanPerThread; ++i) {
+        if (first + i < n) {
+            const unsigned v = (unsigned)(first + i);
+            start[v] = entry;
+            chunks.chunk_start[v] = chunk;
+            const unsigned of_v = chunks_of(c[i]);
+            if (of_v == 1u && chunk < chunks.max_chunks) {
+                chunks.chunk[chunk] = ListChunk{entry, entry + c[i], v, 1u};
+            } else if (of_v > 1u) {
+                const unsigned at = atomicAdd(&chunks.info[0], 1u);
+                if (at < chunks.max_long) chunks.long_lists[at] = v;
+            }
+            entry += c[i];
+            chunk += of_v;
+        }
+    }
+    if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 0) {
+        const uint2 all = block_sums[gridDim.x];
+        start[n] = all.x;
+        chunks.chunk_start[n] = all.y;
+        chunks.info[1] = all.y < chunks.max_chunks ? all.y : chunks.max_chunks;
+    }
+}
+
+// The chunks of the lists that have several: a workgroup per list, a thread per chunk.
+__global__ __launch_bounds__(kBlock) void k_long_list_chunks(const unsigned *__restrict__ start,
+                                                              ListChunks chunks, unsigned *host_info) {
+    const unsigned n_long = chunks.info[0] < chunks.max_long ? chunks.info[0] : chunks.max_long;
+    if (host_info && blockIdx.x == 0 && threadIdx.x == 0) {
+        host_info[0] = chunks.info[0];
+        host_info[1] = chunks.info[1];
+    }
+    for (unsigned i = blockIdx.x; i < n_long; i += gridDim.x) {
+        const unsigned v = chunks.long_lists[i];
+        const unsigned from = chunks.chunk_start[v], to = chunks.chunk_start[v + 1];
+        const unsigned list_from = start[v], list_to = start[v + 1];
+        for (unsigned c = from + threadIdx.x; c < to && c < chunks.max_chunks; c += kBlock) {
+            const unsigned first = list_from + (c - from) * (unsigned)kListChunk;
+            const unsigned last =
+                list_to - first < (unsigned)kListChunk ? list_to : first + (unsigned)kListChunk;
+            chunks.chunk[c] = ListChunk{first, last, v, 0u};
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// Lists, step 3: every (point, corner) writes (point, weight) to its place in its vertex's list.
+// ------------------------------------------------------------------------------------------------
+template <int D1>
+__global__ __launch_bounds__(kBlock) void k_list_fill(PointMap map,
+                                                       const ReplayEntry *__restrict__ replay,
+                                                       const unsigned *__restrict__ places,
+                                                       const unsigned *__restrict__ start,
+                                                       ListEntry *entries, int max_vertices,
+                                                       size_t capacity) {
+    unsigned vblock;
+    if (!block_of_points(map, 1, vblock)) return;
+    const size_t t = (size_t)vblock * kBlock + threadIdx.x;
+    const size_t T = (size_t)gridDim.x * kBlock;
+    const int n = point_of_thread(map, vblock, threadIdx.x);
+    if (n < 0) return;
+    ReplayEntry e[D1];
+    unsigned place[D1], first[D1];
+#pragma unroll
+    for (int r = 0; r < D1; ++r) {
+        e[r] = replay[(size_t)r * T + t];
+        place[r] = places[(size_t)r * T + t];
+    }
+#pragma unroll
+    for (int r = 0; r < D1; ++r)
+        first[r] = start[(unsigned)e[r].index < (unsigned)max_vertices ? e[r].index : 0];
+#pragma unroll
+    for (int r = 0; r < D1; ++r) {
+        const size_t at = (size_t)first[r] + place[r];
+        if ((unsigned)e[r].index < (unsigned)max_vertices && at < capacity)
+            entries[at] = ListEntry{n, e[r].weight};
+    }
+}
+
+// The rows of a chunk and where its sums go: the vertex's row of the value table when the chunk
+// is the whole list, else the chunk's partial row.  One 16-byte load.
+struct ChunkWork {
+    unsigned from, to;     // entries
+    float *row;            // vd floats, or nullptr: no chunk
+};
+__device__ __forceinline__ ChunkWork chunk_work(unsigned c, unsigned n_chunks, const ListChunks &chunks,
+                                                int vd, float *values) {
+    ChunkWork w{0u, 0u, nullptr};
+    if (c >= n_chunks) return w;
+    const uint4 d = reinterpret_cast<const uint4 *>(chunks.chunk)[c];   // {from, to, vertex, whole}
+    w.from = d.x;
+    w.to = d.y;
+    w.row = d.w ? values + (size_t)d.z * vd : chunks.partial_rows + (size_t)c * vd;
+    return w;
+}
+
+// ------------------------------------------------------------------------------------------------
+// The splat as a gather, up to four channels: kLanes lanes per chunk take every kLanes-th of its
+// rows, four each per turn with all their loads in flight (the entries, then the input rows they
+// name, each row one request), and the lanes' sums are added across the group.  The row of every
+// vertex is written whole, so the value table needs no zero fill.
+// ------------------------------------------------------------------------------------------------
+constexpr int kLanes = 8;      // lanes per chunk
+constexpr int kInFlight = 4;   // entries per lane and turn
+
+// An input row of IN floats, read with one request (rows of three floats are only aligned to four
+// bytes, which a 12-byte load allows)
+template <int IN>
+struct alignas(IN == 3 ? 4 : 4 * IN) InputRow {
+    float c[IN];
+};
+
+// IN: channels of an input row, VD - 1 (the last channel of the vertex row is the sum of the bare
+// weights) or VD
+template <int VD, int IN>
+__global__ __launch_bounds__(kBlock) void k_splat_gather(ListChunks chunks,
+                                                          const ListEntry *__restrict__ entries,
+                                                          const float *__restrict__ input,
+                                                          float *values) {
+    static_assert(VD >= 2 && VD <= 4 && (IN == VD || IN == VD - 1), "the rows are gathered in registers");
+    const unsigned n_chunks = chunks.info[1];
+    const unsigned sub = threadIdx.x % kLanes;
+    constexpr unsigned per_block = kBlock / kLanes;
+    // (chunks follow the vertex numbers, which follow the image: every XCD takes one contiguous
+    // range of them, so that the input rows its chunks share stay in its L2)
+    const unsigned first_block = xcd_contiguous_block(blockIdx.x, gridDim.x, 1);
+    for (unsigned c0 = first_block * per_block; c0 < n_chunks; c0 += gridDim.x * per_block) {
+        const ChunkWork work = chunk_work(c0 + threadIdx.x / kLanes, n_chunks, chunks, VD, values);
+        float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        // (the lanes of a chunk leave the loop together: what they exchange below is complete)
+        for (unsigned turn = work.from; turn < work.to; turn += kLanes * kInFlight) {
+            ListEntry e[kInFlight];
+            bool valid[kInFlight];
+#pragma unroll
+            for (int u = 0; u < kInFlight; ++u) {
+                const unsigned i = turn + (unsigned)u * kLanes + sub;
+                valid[u] = i < work.to;
+                e[u] = entries[valid[u] ? i : work.from];
+            }
+            InputRow<IN> x[kInFlight];
+#pragma unroll
+            for (int u = 0; u < kInFlight; ++u)
+                x[u] = reinterpret_cast<const InputRow<IN> *>(input)[e[u].point];
+#pragma unroll
+            for (int u = 0; u < kInFlight; ++u) {
+                const float w = valid[u] ? e[u].weight : 0.0f;
+#pragma unroll
+                for (int j = 0; j < VD; ++j) acc[j] += w * (j < IN ? x[u].c[j] : 1.0f);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < VD; ++j) {
+#pragma unroll
+            for (int off = 1; off < kLanes; off <<= 1) acc[j] += __shfl_xor(acc[j], off);
+        }
+        if (work.row && sub == 0) {
+#pragma unroll
+            for (int j = 0; j < VD; ++j) work.row[j] = acc[j];
+        }
+    }
+}
+
+// Any number of channels: W lanes per chunk (a power of two, 16..64, at least vd unless vd > 64),
+// lane c on channel c.  The lanes read W entries of the list at once, one each, and hand them
+// round; every lane then reads its channel of the rows they name, sixteen loads in flight.
+// Channels past the input are the homogeneous one.
+template <int W>
+__global__ __launch_bounds__(kBlock) void k_splat_gather_channels(ListChunks chunks, int vd,
+                                                                   const ListEntry *__restrict__ entries,
+                                                                   const float *__restrict__ input,
+                                                                   int in_channels, float *values) {
+    const unsigned n_chunks = chunks.info[1];
+    constexpr unsigned per_block = kBlock / W;
+    const int sub = threadIdx.x % W;
+    constexpr int kBatch = 16;
+    const unsigned first_block = xcd_contiguous_block(blockIdx.x, gridDim.x, 1);
+    for (unsigned c0 = first_block * per_block; c0 < n_chunks; c0 += gridDim.x * per_block) {
+        const ChunkWork work = chunk_work(c0 + threadIdx.x / W, n_chunks, chunks, vd, values);
+        for (int ch0 = 0; ch0 < vd; ch0 += W) {
+            const int c = ch0 + sub;
+            float acc = 0.0f;
+            for (unsigned turn = work.from; turn < work.to; turn += W) {
+                const unsigned mine = turn + (unsigned)sub;
+                const ListEntry e = entries[mine < work.to ? mine : work.from];
+                const unsigned here = work.to - turn < (unsigned)W ? work.to - turn : (unsigned)W;
+                for (unsigned k0 = 0; k0 < here; k0 += kBatch) {
+                    float x[kBatch], w[kBatch];
+#pragma unroll
+                    for (int k = 0; k < kBatch; ++k) {
+                        // (entries past the end of the chunk: its first row, weight zero)
+                        const bool in_list = k0 + k < here;
+                        const int src = in_list ? (int)(k0 + k) : 0;
+                        const int p = __shfl(e.point, src, W);
+                        w[k] = in_list ? __shfl(e.weight, src, W) : 0.0f;
+                        x[k] = c < in_channels ? input[(size_t)p * in_channels + c] : 1.0f;
+                    }
+#pragma unroll
+                    for (int k = 0; k < kBatch; ++k) acc += w[k] * x[k];
+                }
+            }
+            if (work.row && c < vd) work.row[c] = acc;
+        }
+    }
+}
+
+// The lists of more than one chunk: the vertex's row := the sum of its chunks' partial rows.  A
+// workgroup per list and block of 32 channels: thread (s, c) adds channel c of every eighth chunk,
+// four loads in flight, and the eight sums are added through LDS (the same order on every call).
+__global__ __launch_bounds__(kBlock) void k_sum_partial_rows(ListChunks chunks, int vd, float *values) {
+    __shared__ float part[kBlock / 32][32];
+    const unsigned n_long = chunks.info[0] < chunks.max_long ? chunks.info[0] : chunks.max_long;
+    const unsigned slot = threadIdx.x >> 5, sub = threadIdx.x & 31;
+    constexpr unsigned kSlots = kBlock / 32;
+    for (unsigned i = blockIdx.x; i < n_long; i += gridDim.x) {
+        const unsigned v = chunks.long_lists[i];
+        const unsigned from = chunks.chunk_start[v], to = chunks.chunk_start[v + 1];
+        for (int c0 = 0; c0 < vd; c0 += 32) {
+            const int c = c0 + (int)sub;
+            float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+            for (unsigned k = from + slot; k < to; k += 4u * kSlots) {
+#pragma unroll
+                for (int u = 0; u < 4; ++u) {
+                    const unsigned ku = k + kSlots * (unsigned)u;
+                    if (ku < to && c < vd) acc[u] += chunks.partial_rows[(size_t)ku * vd + c];
+                }
+            }
+            __syncthreads();   // (part may still be read from the turn before)
+            part[slot][sub] = (acc[0] + acc[1]) + (acc[2] + acc[3]);
+            __syncthreads();
+            if (slot == 0 && c < vd) {
+                float sum = 0.0f;
+#pragma unroll
+                for (unsigned k = 0; k < kSlots; ++k) sum += part[k][sub];
+                values[(size_t)v * vd + c] = sum;
+            }
+        }
+    }
+}
+
+}  // namespace
+
+size_t vertex_list_scan_blocks(int max_vertices) {
+    return ((size_t)max_vertices + kScanItems - 1) / kScanItems;
+}
+size_t vertex_list_max_chunks(int max_vertices, size_t rows) {
+    return (size_t)max_vertices + rows / (size_t)kListChunk + 1;
+}
+size_t vertex_list_max_long(size_t rows) { return rows / (size_t)kListChunk + 1; }
+
+hipError_t build_vertex_lists(int pd, const PointMap &map, ReplayEntry *replay, const int *cell_vertex,
+                              int max_vertices, const VertexLists &lists, unsigned *host_info,
+                              hipStream_t s) {
+    if (max_vertices <= 0) return hipSuccess;
+    hipError_t err = fill_zero(reinterpret_cast<float *>(lists.count), (size_t)max_vertices, s);
+    if (err != hipSuccess) return err;
+    const dim3 block(kBlock);
+    if (map.n_blocks) {
+        const dim3 grid(map.n_blocks);
+        PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_list_places<PD + 1>), grid, block, 0, s, map, replay,
+                                               cell_vertex, lists.count, lists.places, max_vertices));
+    }
+    const unsigned n = (unsigned)max_vertices;
+    const unsigned scan_blocks = (unsigned)vertex_list_scan_blocks(max_vertices);
+    uint2 *block_sums = reinterpret_cast<uint2 *>(lists.block_sums);
+    hipLaunchKernelGGL(k_scan_block_sums, dim3(scan_blocks), block, 0, s, lists.count, n, block_sums,
+                       lists.chunks.info);
+    hipLaunchKernelGGL(k_scan_of_block_sums, dim3(1), block, 0, s, block_sums, scan_blocks);
+    hipLaunchKernelGGL(k_scan_starts, dim3(scan_blocks), block, 0, s, lists.count, n, block_sums,
+                       lists.start, lists.chunks);
+    // (how many lists have several chunks is known on the device only: a grid that covers a
+    // usual number of them, the workgroups walk the rest)
+    const unsigned long_blocks = lists.chunks.max_long < 1024u ? lists.chunks.max_long : 1024u;
+    hipLaunchKernelGGL(k_long_list_chunks, dim3(long_blocks ? long_blocks : 1u), block, 0, s,
+                       lists.start, lists.chunks, host_info);
+    if (map.n_blocks) {
+        const dim3 grid(map.n_blocks);
+        PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_list_fill<PD + 1>), grid, block, 0, s, map, replay,
+                                               lists.places, lists.start, lists.entries, max_vertices,
+                                               lists.capacity));
+    }
+    return hipGetLastError();
+}
+
+hipError_t splat_gather(int vd, const VertexLists &lists, unsigned n_chunks, unsigned n_long,
+                        const float *input, int in_channels, float *values, hipStream_t s) {
+    if (n_chunks == 0) return hipSuccess;
+    const dim3 block(kBlock);
+#define PLK_GATHER(VD)                                                                               \
+    case VD:                                                                                        \
+        if (in_channels == VD)                                                                      \
+            hipLaunchKernelGGL((k_splat_gather<VD, VD>), dim3(blocks_for(n_chunks, kBlock / kLanes)),\
+                               block, 0, s, lists.chunks, lists.entries, input, values);\
+        else if (in_channels == VD - 1)                                                             \
+            hipLaunchKernelGGL((k_splat_gather<VD, VD - 1>),                                         \
+                               dim3(blocks_for(n_chunks, kBlock / kLanes)), block, 0, s,            \
+                               lists.chunks, lists.entries, input, values);            \
+        else                                                                                        \
+            return hipErrorInvalidValue;                                                            \
+        break;
+    switch (vd) {
+        PLK_GATHER(2) PLK_GATHER(3) PLK_GATHER(4)
+        default:
+            if (vd <= 16)
+                hipLaunchKernelGGL(k_splat_gather_channels<16>, dim3(blocks_for(n_chunks, kBlock / 16)),
+                                   block, 0, s, lists.chunks, vd, lists.entries, input,
+                                   in_channels, values);
+            else if (vd <= 32)
+                hipLaunchKernelGGL(k_splat_gather_channels<32>, dim3(blocks_for(n_chunks, kBlock / 32)),
+                                   block, 0, s, lists.chunks, vd, lists.entries, input,
+                                   in_channels, values);
+            else
+                hipLaunchKernelGGL(k_splat_gather_channels<64>, dim3(blocks_for(n_chunks, kBlock / 64)),
+                                   block, 0, s, lists.chunks, vd, lists.entries, input,
+                                   in_channels, values);
+            break;
+    }
+#undef PLK_GATHER
+    if (n_long)
+        hipLaunchKernelGGL(k_sum_partial_rows, dim3(n_long), block, 0, s,
+                           lists.chunks, vd, values);
+    return hipGetLastError();
+}
+
+}  // namespace plk

@@ -269,6 +269,55 @@ hipError_t splat(int pd, int vd, const PointMap &map, const float *input, int in
                  ReplayEntry *replay, const int *cell_vertex, float *values,
                  int xcd_aware, hipStream_t s);
 
+// The transpose of the replay matrix, for lattices that are applied many times (pl_gather.hip):
+// the rows that name vertex v are entries[start[v] .. start[v+1]), each the point and its weight.
+// Vertices must be numbered densely (number_vertices).  The unit of work of the splat that
+// gathers is a chunk of at most kListChunk rows of one list: the chunks of vertex v are
+// chunk_start[v] .. chunk_start[v+1], chunk c is described by chunk[c]; a list of several chunks is
+// summed into the partial rows of its chunks first (partial_rows[c * vd ..]) and is named in
+// long_lists.  info: {long lists, chunks in all}.
+constexpr int kListChunk = 128;
+struct ListEntry {
+    int point;
+    float weight;
+};
+struct alignas(16) ListChunk {
+    unsigned from, to;       // its rows: entries[from .. to)
+    unsigned vertex;
+    unsigned whole;          // 1: the chunk is all of its vertex's list
+};
+struct ListChunks {
+    unsigned *chunk_start;   // [max_vertices + 1]
+    ListChunk *chunk;        // [max_chunks]
+    unsigned *long_lists;    // [max_long]
+    float *partial_rows;     // [max_chunks * vd]
+    unsigned *info;          // [2], the two words behind VertexLists::count
+    unsigned max_chunks, max_long;
+};
+struct VertexLists {
+    unsigned *start;       // [max_vertices + 1]
+    ListEntry *entries;    // [capacity]: one per replay row
+    unsigned *count;       // [max_vertices + 2] scratch of the build of the lists (and info)
+    unsigned *places;      // [capacity] scratch, in the layout of the replay rows
+    unsigned *block_sums;  // [2 * (vertex_list_scan_blocks(max_vertices) + 1)] scratch, 8-byte aligned
+    size_t capacity;
+    ListChunks chunks;
+};
+size_t vertex_list_scan_blocks(int max_vertices);
+size_t vertex_list_max_chunks(int max_vertices, size_t rows);
+size_t vertex_list_max_long(size_t rows);
+// cell_vertex != nullptr: the replay rows still hold hash cells; they are translated and written
+// back.  When the stream has run this, lists.chunks.info holds the numbers splat_gather wants,
+// and so do the two words at host_info (memory the device can write, read by the host).
+hipError_t build_vertex_lists(int pd, const PointMap &map, ReplayEntry *replay, const int *cell_vertex,
+                              int max_vertices, const VertexLists &lists, unsigned *host_info,
+                              hipStream_t s);
+// Stage 3 from the lists: values[v] := sum over v's entries of weight * input row (every vertex's
+// row is written whole; no zero fill needed).  n_chunks, n_long: lists.chunks.info as the build of
+// the lists left it (a second launch adds up the lists of several chunks when there are any).
+hipError_t splat_gather(int vd, const VertexLists &lists, unsigned n_chunks, unsigned n_long,
+                        const float *input, int in_channels, float *values, hipStream_t s);
+
 // Stage 4, one axis: dst[v] = 1/4 src[n1] + 1/2 src[v] + 1/4 src[n2] for v < counters->num_vertices.
 // reset_cell_keys != nullptr: also empty the hash cell of every vertex (vertex_cell[v]).
 hipError_t blur_axis(int vd, const Counters *counters, int max_vertices, const float *src, float *dst,

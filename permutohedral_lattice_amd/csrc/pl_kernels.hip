@@ -517,9 +517,8 @@ __global__ __launch_bounds__(kBlock) void k_build_tile(PointFeatures features, P
             const int leader = wave_leader_of_equal(key[r], active, lane, kSmallGroup, small[r]);
             leaders[r / 5] |= (unsigned)leader << (6 * (r % 5));
             if (active && leader == lane) open |= 1u << r;
-            // (a cheaper hash -- three 24-bit multiplies instead of three 32-bit ones -- spread the
-            // keys of a tile worse and cost 9 us of probing for the 1 us it saved)
-            slot[r] = (int)((hash_key(key[r]) >> 20) & (kTileSlots - 1));
+            static_assert(kTileSlots == 1 << (32 - kTileSlotShift), "the slot is the hash's high bits");
+            slot[r] = (int)(hash_key(key[r]) >> kTileSlotShift);
         }
         bool any_open = open != 0;
         for (int probe = 0; any_open && probe < kTileProbeLimit; ++probe) {
