@@ -264,6 +264,7 @@ def run_configs(args, pla, synth, with_cpu):
     m_bi, m_sp = mf.bilateral[0].num_vertices, mf.spatial[0].num_vertices
     q0 = torch.softmax(d_logits[0].view(n, classes), dim=-1)
     msg = torch.empty_like(q0)
+    torch.cuda.synchronize()      # (the lattices work on streams of their own)
     st_bi, dom_bi = stage_report(mf.bilateral[0], lambda: mf.bilateral[0].apply(msg, q0, False), n, 5,
                                  classes + 1, fused_splat=False)
     st_sp, dom_sp = stage_report(mf.spatial[0], lambda: mf.spatial[0].apply(msg, q0, False), n, 2,

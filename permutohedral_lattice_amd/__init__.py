@@ -27,6 +27,7 @@ PL_OPT_MERGE_TILES = 7
 PL_OPT_STOP_AFTER = 8
 PL_OPT_ORDER_POINTS = 9
 PL_OPT_VERTEX_LISTS = 10
+PL_OPT_NUMBER_SEGMENTS = 11
 PL_INFO_BUILD_MERGED, PL_INFO_TABLE_CELLS, PL_INFO_SCRATCH_BYTES, PL_INFO_FOREIGN_ROWS = 1, 2, 3, 4
 PL_LIB_LAYOUT_VERSION, PL_LIB_REPLAY_ROW_BYTES, PL_LIB_SOURCE_HASH = 1, 2, 3
 # The device-side array layouts this module (and the tests and benchmarks on top of it) were

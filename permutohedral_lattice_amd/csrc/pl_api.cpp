@@ -140,6 +140,7 @@ struct pl_lattice {
     // next one_segment_backoff builds of this lattice (doubled every time it happens again, up to
     // 1024) before eight runs are tried again.
     int one_segment_for = 0, one_segment_backoff = 32;
+    int forced_segments = 0;           // option: 0 = by the size of the build, else 1, 8 or 64
     // A merging build numbers its vertices itself unless that costs more than it saves: when it
     // has many thousands of workgroups (they draw their numbers one after the other), or when
     // the last such build of these points held so many rows of sums for vertices of other
@@ -447,8 +448,7 @@ int enqueue_build(pl_lattice *h, const plk::PointFeatures &features, const doubl
     // (a build for one filter: a lattice built to be applied many times is numbered by the
     // numbering pass, in the order of the image tiles, which the passes over the vertices walk
     // a few per cent faster than the order in which the workgroups happened to finish)
-    const bool numbers_in_build =
-        merge && fused && h->working_blocks() <= 8192u && !h->numbering_pass_pays;
+    const bool numbers_in_build = merge && fused && !h->numbering_pass_pays && h->forced_segments >= 0;
     const size_t floats_per_value = h->f64 ? 2 : 1;
     if (fused && !numbers_in_build && !h->cell_values_clean) {
         PL_HIP(plk::fill_zero(h->cell_values, (size_t)h->n_cells_alloc * h->vd * floats_per_value,
@@ -480,7 +480,8 @@ int enqueue_build(pl_lattice *h, const plk::PointFeatures &features, const doubl
     const plk::InBuildNumbering numbering{
         h->cell_vertex, h->vertex_keys, h->vertex_cell, h->neighbours, h->max_vertices(),
         h->values[0], h->f64 ? 2 * h->vd : h->vd,
-        !numbers_in_build ? 0 : (h->one_segment_for > 0 ? 1 : plk::segments_for((uint32_t)h->max_vertices()))};
+        !numbers_in_build ? 0 : (h->one_segment_for > 0 ? 1 : plk::segments_for((uint32_t)h->max_vertices(),
+                                                                              h->forced_segments == 64 ? 1u << 20 : h->forced_segments == 8 ? 1u : h->working_blocks()))};
     if (numbers_in_build && h->one_segment_for > 0) h->one_segment_for -= 1;
     // keys go to the part of the table that belongs to their band of rows when the points are
     // known to be a grid (and feature 0 then runs with its slowest extent)
@@ -760,12 +761,13 @@ int verify_build(pl_lattice *h, uint32_t *retry_cells) {
     h->last_M = m;
     h->n_segments = status.n_segments;
     h->max_segment = status.max_segment;
-    // (in ns, as measured on 1024x1024 and 512x512 images: a row added afterwards takes 0.03 of
-    // the atomic unit's time; the numbering pass 1.5 per workgroup of the build and 0.02 per
-    // vertex, and the build 1500 longer with all its rows going out as atomics)
+    // (in ns, as measured on 1024x1024 and 512x512 images and a 128x256x256 volume: a row added
+    // afterwards takes 0.037 of the atomic unit's time (1.85 M rows of the volume: 69 us); the
+    // numbering pass 1.25 per workgroup of the build and 0.02 per vertex (the volume's 32 768
+    // workgroups: 41 us), and the build 1500 longer with all its rows going out as atomics)
     h->foreign_rows = status.n_segments != 0 ? (long)status.foreign_rows : -1;
     if (status.n_segments != 0 &&
-        0.03 * status.foreign_rows > 1.5 * h->working_blocks() + 0.02 * m + 1500.0)
+        0.037 * status.foreign_rows > 1.25 * h->working_blocks() + 0.02 * m + 1500.0)
         h->numbering_pass_pays = true;
     h->verified = true;
     if (h->last_build_merged) h->tiles_backoff = 32;
@@ -931,6 +933,10 @@ int pl_set_option(pl_handle h, int option, long value) {
             return PL_OK;
         case PL_OPT_ORDER_POINTS:
             h->order_points = value != 0;
+            return PL_OK;
+        case PL_OPT_NUMBER_SEGMENTS:
+            if (value != 0 && value != 8 && value != 64 && value != -1) return PL_EINVAL;
+            h->forced_segments = (int)value;
             return PL_OK;
         case PL_OPT_VERTEX_LISTS:
             h->vertex_lists = value != 0;

@@ -583,20 +583,36 @@ __device__ __forceinline__ void reset_counters(Counters *c) {
 // the numbers 0 .. vertices-1, which follow the image too.  What a workgroup gathers from is then
 // mostly what its own XCD works on.
 struct SegmentWalk {
-    unsigned first, count;     // the run of numbers this XCD walks
+    unsigned first, count;     // the run of numbers being walked (one of this XCD's)
     unsigned cursor, step;     // next block among the blocks of that run, stride
+    // the runs this XCD walks: the segments run_first .. run_first + runs - 1 (runs == 0: one run
+    // that is no segment, set up by the constructor)
+    const Counters *counters;
+    unsigned run, runs, run_first, stride;
+    __device__ void load_run() {
+        const unsigned n = counters->segment_count[run_first + run].n;
+        first = (run_first + run) * stride;
+        count = n < stride ? n : stride;
+    }
     // grid_blocks: workgroups of the grid that walk (a multiple of 8), workgroup: index among them
-    __device__ SegmentWalk(const Counters *counters, int max_vertices, unsigned workgroup,
-                           unsigned grid_blocks) {
+    __device__ SegmentWalk(const Counters *counters_, int max_vertices, unsigned workgroup,
+                           unsigned grid_blocks)
+        : counters(counters_) {
         const unsigned xcd = workgroup % kXcds;
         const Counters::PaddedCount mine = counters->segment_count[xcd];
-        if (mine.n_segments == (int)kXcds) {
-            const unsigned stride = segment_stride((uint32_t)max_vertices, mine.n_segments);
-            first = xcd * stride;
-            count = mine.n < stride ? mine.n : stride;
+        run = 0;
+        if (mine.n_segments >= (int)kXcds) {
+            // (eight segments: XCD x walks segment x; sixty-four: segments 8x .. 8x + 7)
+            runs = (unsigned)mine.n_segments / kXcds;
+            run_first = xcd * runs;
+            stride = segment_stride((uint32_t)max_vertices, mine.n_segments);
+            load_run();
         } else {
             // (one run: after the numbering pass every line holds the total, after a build
             // with one segment the first)
+            runs = 0;
+            run_first = 0;
+            stride = 0;
             const unsigned all = mine.n_segments == 1 ? counters->segment_count[0].n : mine.n;
             const unsigned m = all < (unsigned)max_vertices ? all : (unsigned)max_vertices;
             const unsigned per_xcd = ((m + kBlock - 1) / kBlock + kXcds - 1) / kXcds * kBlock;
@@ -606,14 +622,22 @@ struct SegmentWalk {
         cursor = workgroup / kXcds;
         step = grid_blocks / kXcds;
     }
-    // This workgroup's next block b of 256 items, a vertex being items_per_vertex items, in a
-    // pass that visits every block `visits` times
+    // This workgroup's next block b of 256 items of the run (first, count), a vertex being
+    // items_per_vertex items, in a pass that visits every block `visits` times
     __device__ bool next(unsigned items_per_vertex, unsigned visits, unsigned &b) {
-        const unsigned n = (unsigned)(((size_t)count * items_per_vertex + kBlock - 1) / kBlock) * visits;
-        if (cursor >= n) return false;
-        b = cursor;
-        cursor += step;
-        return true;
+        for (;;) {
+            const unsigned n =
+                (unsigned)(((size_t)count * items_per_vertex + kBlock - 1) / kBlock) * visits;
+            if (cursor < n) {
+                b = cursor;
+                cursor += step;
+                return true;
+            }
+            if (run + 1 >= runs) return false;
+            cursor -= n;       // (the stride carries over into the XCD's next run)
+            run += 1;
+            load_run();
+        }
     }
 };
 

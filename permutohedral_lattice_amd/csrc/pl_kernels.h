@@ -57,10 +57,12 @@ constexpr unsigned kForeignSampling = 8;
 __host__ __device__ inline uint32_t segment_stride(uint32_t max_vertices, int n_segments) {
     return max_vertices / (uint32_t)(n_segments > 0 ? n_segments : 1);
 }
-// Segments a merging build that numbers its vertices uses with a table for max_vertices: none
-// smaller than 2048 numbers (a workgroup can create 512 vertices).
-inline int segments_for(uint32_t max_vertices) {
-    return max_vertices / (uint32_t)kMaxSegments < 2048u ? 1 : kMaxSegments;
+// Segments a merging build of `workgroups` workgroups that numbers its vertices uses with a table
+// for max_vertices: none smaller than 2048 numbers (a workgroup can create 512 vertices); eight,
+// or sixty-four when a segment of eight would serve more than a thousand workgroups.
+inline int segments_for(uint32_t max_vertices, unsigned workgroups) {
+    if (max_vertices / 8u < 2048u) return 1;
+    return workgroups > 8192u && max_vertices / (uint32_t)kMaxSegments >= 2048u ? kMaxSegments : 8;
 }
 
 // What the build (or the numbering pass) writes to pinned host memory about the build.
@@ -149,7 +151,7 @@ struct InBuildNumbering {
     int max_vertices;
     void *values;
     int value_words;
-    int n_segments;       // 0, 1 or 8 (segments_for)
+    int n_segments;       // 0, 1, 8 or 64 (segments_for)
 };
 
 // Where the feature vector of a point comes from: the row of a positions array, or, with

@@ -754,8 +754,20 @@ __global__ __launch_bounds__(kBlock) void k_build_tile(PointFeatures features, P
     // and leave their places to the wavefronts of the next workgroup.
     const unsigned stride = segment_stride((uint32_t)numbering.max_vertices, numbering.n_segments);
     unsigned segment = 0;
-    if (numbering.n_segments == (int)kXcds)
-        segment = xcd_aware ? (blockIdx.x % kXcds) : (unsigned)(((size_t)vblock * kXcds) / gridDim.x);
+    if (numbering.n_segments >= (int)kXcds) {
+        // the eighth of the image this workgroup lies in and, with sixty-four segments, which
+        // eighth of that (vblock runs through an XCD's share of the workgroups in order)
+        const unsigned parts = (unsigned)numbering.n_segments / kXcds;
+        if (xcd_aware) {
+            const unsigned nb = map.mode == 1 && *map.n_tiles < gridDim.x ? *map.n_tiles : gridDim.x;
+            const unsigned xcd = blockIdx.x % kXcds;
+            const unsigned share = nb / kXcds + (xcd < nb % kXcds ? 1u : 0u);
+            const unsigned index = blockIdx.x / kXcds;
+            segment = xcd * parts + (share ? (unsigned)(((size_t)index * parts) / share) : 0u);
+        } else {
+            segment = (unsigned)(((size_t)vblock * (size_t)numbering.n_segments) / gridDim.x);
+        }
+    }
     const unsigned count = (unsigned)group_created;
     unsigned first = 0;
     if (tid == 0 && count) first = atomicAdd(&counters->segment_count[segment].n, count);

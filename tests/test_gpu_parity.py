@@ -742,3 +742,35 @@ def test_vertex_count_far_from_the_previous_one():
         torch.cuda.synchronize()
         assert_float_parity(host(out), oracle.Lattice(5, 4, n).filter(val, pos, True))
     assert counts[1] > 20 * counts[0]
+
+
+@pytest.mark.parametrize("segments", [8, 64])
+def test_vertex_numbers_drawn_from_eight_or_sixty_four_counters(segments):
+    """A build that numbers its vertices itself, with the numbers of every eighth of the image in
+    one run or in eight (what a build of more than 8192 workgroups uses): same lattice, same
+    outputs; the exports close the gaps between the runs."""
+    side = 384
+    img = synth.blob_image(side, side, seed=31)
+    pos = synth.bilateral_positions(img, 4.0, 0.08)
+    val = np.ascontiguousarray(img.reshape(-1, 3))
+    n = side * side
+    lat = pla.PermutohedralLattice(5, 4, n)
+    lat.set_point_grid((side, side))
+    lat.set_option(pla.PL_OPT_NUMBER_SEGMENTS, segments)
+    lat.set_option(pla.PL_OPT_TABLE_CELLS, 1 << 21)     # (room for 64 runs of 2048 numbers or more)
+    cpu = oracle.Lattice(5, 4, n)
+    for reverse in (False, True):
+        got, _ = gpu_filter(5, 4, pos, val, reverse, lattice=lat)
+        want = oracle.Lattice(5, 4, n).filter(val, pos, reverse) if reverse else cpu.filter(val, pos, False)
+        assert lat.num_vertices == cpu.num_vertices
+        assert_float_parity(got, want)
+    got_keys, _ = sorted_keys(host(lat.debug_keys()))
+    want_keys, _ = sorted_keys(cpu.keys())
+    assert (got_keys == want_keys).all()
+    # replay rows through the keys they point to
+    vertex, weight = lat.debug_replay()
+    keys = host(lat.debug_keys())
+    point_keys = oracle.dump_simplex(pos)["keys"]
+    v = host(vertex)
+    for r in (0, 3, 5):
+        assert (keys[v[r]] == point_keys[:, r, :]).all()
