@@ -385,6 +385,35 @@ def run_plain_legs(args, pla, lat, d_pos, d_val, d_grad, out_f, out_r):
     return plain
 
 
+def run_reuse_leg(args, pla, lat, d_pos, d_val, d_grad, out_f, out_r):
+    """Build once, apply forward and reverse (what a caller that keeps the lattice gets): with the
+    per-vertex lists pl_build writes (the applies splat by gathering) and without them (the applies
+    splat as filter() does).  -> {mode: {build_ms, ms_per_step}}"""
+    import torch
+    out = {}
+    for name, lists in (("without_vertex_lists", 0), ("with_vertex_lists", 1)):
+        lat.set_option(pla.PL_OPT_VERTEX_LISTS, lists)
+        for _ in range(2):
+            lat.build(d_pos)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(5):
+            lat.build(d_pos)
+        torch.cuda.synchronize()
+        build_ms = 1e3 * (time.perf_counter() - t0) / 5
+        for _ in range(2):
+            lat.apply(out_f, d_val, False)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(args.steps):
+            lat.apply(out_f, d_val, False)
+            lat.apply(out_r, d_grad, True)
+        torch.cuda.synchronize()
+        out[name] = {"build_ms": round(build_ms, 4),
+                     "ms_per_step": round(1e3 * (time.perf_counter() - t0) / args.steps, 4)}
+    return out
+
+
 def run_side_legs(args, pla, synth, lat, step, img, d_pos, d_val, d_grad, out_f, out_r, side, batch):
     """The legs beside the headline: no grid hint, lattice reuse, the op's boundary, a batch."""
     import numpy as np
@@ -392,15 +421,7 @@ def run_side_legs(args, pla, synth, lat, step, img, d_pos, d_val, d_grad, out_f,
 
     plain_ms = run_plain_legs(args, pla, lat, d_pos, d_val, d_grad, out_f, out_r)
 
-    # build once, apply forward and reverse (what a caller that keeps the lattice gets)
-    lat.build(d_pos)
-    torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for _ in range(args.steps):
-        lat.apply(out_f, d_val, False)
-        lat.apply(out_r, d_grad, True)
-    torch.cuda.synchronize()
-    reuse_ms = 1e3 * (time.perf_counter() - t0) / args.steps
+    reuse = run_reuse_leg(args, pla, lat, d_pos, d_val, d_grad, out_f, out_r)
 
     # the op's boundary: the reference image comes in, not a positions array.  First as the
     # reference does it (feature kernel, then filter), then with the features built on the fly.
@@ -480,7 +501,7 @@ def run_side_legs(args, pla, synth, lat, step, img, d_pos, d_val, d_grad, out_f,
     double_ms = 1e3 * (time.perf_counter() - t0) / reps
     lat64.close()
 
-    return plain_ms, reuse_ms, op_ms, batch_ms, double_ms
+    return plain_ms, reuse, op_ms, batch_ms, double_ms
 
 
 def main():
@@ -499,6 +520,9 @@ def main():
                     help="only the legs without a grid hint (for profiling the ordering of plain lists)")
     ap.add_argument("--plain-legs", default="",
                     help="with --plain-only: the legs to run, comma-separated (default: all)")
+    ap.add_argument("--reuse-only", action="store_true",
+                    help="only the timed steps and the build-once / apply-many leg (for profiling the "
+                         "kernels of pl_build's lists and of pl_apply)")
     ap.add_argument("--configs-only", action="store_true",
                     help="only the leg that runs every BASELINE configuration at full size, without "
                          "the CPU reference (what a rocprofv3 run for the kernels of those "
@@ -579,10 +603,13 @@ def main():
         print("bench.py: the loaded library was built from sources %s, the tree holds %s: headline "
               "only; rebuild with `python permutohedral_lattice_amd/build.py`"
               % (library_sources, tree_sources), file=sys.stderr)
-    plain_ms, reuse_ms, double_ms = {}, 0.0, 0.0
+    plain_ms, reuse, double_ms = {}, {}, 0.0
     op_ms, batch_ms, batch = {}, {}, 4
+    if args.reuse_only:
+        print(json.dumps({"reuse": run_reuse_leg(args, pla, lat, d_pos, d_val, d_grad, out_f, out_r)}))
+        return
     if side_legs:
-        plain_ms, reuse_ms, op_ms, batch_ms, double_ms = run_side_legs(args, pla, synth, lat, step, img, d_pos,
+        plain_ms, reuse, op_ms, batch_ms, double_ms = run_side_legs(args, pla, synth, lat, step, img, d_pos,
                                                             d_val, d_grad, out_f, out_r, side, batch)
 
     # per-kernel durations from HIP events on the lattice's stream
@@ -645,9 +672,11 @@ def main():
                              "ms_per_step": {k: round(v, 4) for k, v in plain_ms.items()},
                              "value": {k: round(pixels_per_step / (v * 1e-3) / 1e6, 3)
                                        for k, v in plain_ms.items()}},
-            "reuse": {"what": "build once, apply forward + reverse per step",
-                      "ms_per_step": round(reuse_ms, 4),
-                      "value": round(pixels_per_step / (reuse_ms * 1e-3) / 1e6, 3)},
+            "reuse": {"what": "build once (build_ms), apply forward + reverse per step: with the per-vertex "
+                              "lists pl_build writes, so that an apply splats by gathering, and without",
+                      "ms_per_step": reuse["with_vertex_lists"]["ms_per_step"],
+                      "value": round(pixels_per_step / (reuse["with_vertex_lists"]["ms_per_step"] * 1e-3) / 1e6, 3),
+                      "modes": reuse},
             "op_level": {"what": "reference image in, forward + reverse per step: feature kernel + "
                                  "filter(), filter_image() (features built inside the first kernel), and "
                                  "lattice_filter(...).backward(...) (backward applies forward's lattice)",

@@ -326,7 +326,7 @@ int ensure_vertex_lists(pl_lattice *h) {
     l.block_sums = (unsigned *)h->dmalloc(sizeof(unsigned) * 2 * (plk::vertex_list_scan_blocks((int)mv) + 1));
     l.chunks.chunk_start = (unsigned *)h->dmalloc(sizeof(unsigned) * (mv + 1));
     l.chunks.chunk = (plk::ListChunk *)h->dmalloc(sizeof(plk::ListChunk) * max_chunks);
-    l.chunks.long_lists = (unsigned *)h->dmalloc(sizeof(unsigned) * max_long);
+    l.chunks.long_lists = (plk::LongList *)h->dmalloc(sizeof(plk::LongList) * max_long);
     l.chunks.partial_rows = (float *)h->dmalloc(sizeof(float) * max_chunks * (size_t)h->vd);
     if (!l.start || !l.entries || !l.count || !l.places || !l.block_sums || !l.chunks.chunk_start ||
         !l.chunks.chunk || !l.chunks.long_lists || !l.chunks.partial_rows)
@@ -334,6 +334,7 @@ int ensure_vertex_lists(pl_lattice *h) {
     l.chunks.info = l.count + mv;
     l.chunks.max_chunks = (unsigned)max_chunks;
     l.chunks.max_long = (unsigned)max_long;
+    l.chunks.rows = plk::list_chunk_rows(h->vd);
     h->lists_for_vertices = mv;
     l.capacity = h->replay_capacity;
     return PL_OK;
@@ -1301,8 +1302,8 @@ int pl_get_info(pl_handle h, int what, long *value) {
                                        (h->f64 ? sizeof(double) : 0));
             if (h->lists_of_vertices.start)
                 b += sizeof(unsigned) * (3 * h->lists_for_vertices + 5 +
-                                         plk::vertex_list_scan_blocks((int)h->lists_for_vertices) +
-                                         h->lists_of_vertices.chunks.max_long) +
+                                         2 * (plk::vertex_list_scan_blocks((int)h->lists_for_vertices) + 1)) +
+                     sizeof(plk::LongList) * h->lists_of_vertices.chunks.max_long +
                      (size_t)h->lists_of_vertices.chunks.max_chunks * (sizeof(plk::ListChunk) + sizeof(float) * h->vd) +
                      h->lists_of_vertices.capacity * (sizeof(plk::ListEntry) + sizeof(unsigned));
             if (h->point_order) {

@@ -96,14 +96,35 @@ __global__ __launch_bounds__(kBlock) void k_list_places(PointMap map, ReplayEntr
 // and of the chunks the counts make, both in one pass of three launches: sums of blocks of
 // kScanItems items; a scan of those by one workgroup; the scan inside each block from its start.
 // The last launch also describes the chunk of every list that has one chunk and names the lists
-// that have several (in the order the atomics give; each of those is summed on its own), whose
+// that have several (workgroup by workgroup in the order the atomics give; each of those is
+// summed on its own), whose
 // chunks a small launch describes.  start[n], chunk_start[n]: the totals.
 // ------------------------------------------------------------------------------------------------
 constexpr int kScanPerThread = 8;
 constexpr int kScanItems = kBlock * kScanPerThread;
 
-__host__ __device__ inline unsigned chunks_of(unsigned count) {
-    return (count + (unsigned)kListChunk - 1u) / (unsigned)kListChunk;
+// c := a thread's kScanPerThread counts from count[first ..], 0 beyond n: two loads of four where
+// all exist (first is a multiple of 8), else each from an element that exists
+__device__ __forceinline__ void load_counts(const unsigned *__restrict__ count, size_t first, unsigned n,
+                                            unsigned (&c)[kScanPerThread]) {
+    static_assert(kScanPerThread == 8, "two loads of four");
+    if (first + kScanPerThread <= n) {
+        const uint4 lo = *reinterpret_cast<const uint4 *>(count + first);
+        const uint4 hi = *reinterpret_cast<const uint4 *>(count + first + 4);
+        c[0] = lo.x, c[1] = lo.y, c[2] = lo.z, c[3] = lo.w;
+        c[4] = hi.x, c[5] = hi.y, c[6] = hi.z, c[7] = hi.w;
+    } else {
+        unsigned x[kScanPerThread];
+#pragma unroll
+        for (int i = 0; i < kScanPerThread; ++i) x[i] = count[first + i < n ? first + i : 0];
+#pragma unroll
+        for (int i = 0; i < kScanPerThread; ++i) c[i] = first + i < n ? x[i] : 0u;
+    }
+}
+
+// (rows: a power of two)
+__host__ __device__ inline unsigned chunks_of(unsigned count, unsigned rows) {
+    return (count + rows - 1u) >> __builtin_ctz(rows);
 }
 
 // exclusive prefix sums of one pair of values per thread over the workgroup; *total: the sums of all
@@ -139,15 +160,16 @@ __device__ __forceinline__ uint2 block_exclusive_scan(uint2 x, uint2 *total) {
 // (also zeroes info[0], the number of long lists, which the last launch of the pass counts)
 __global__ __launch_bounds__(kBlock) void k_scan_block_sums(const unsigned *__restrict__ count,
                                                              unsigned n, uint2 *block_sums,
-                                                             unsigned *info) {
+                                                             unsigned *info, unsigned rows) {
     if (blockIdx.x == 0 && threadIdx.x == 0) info[0] = 0u;
     const size_t first = (size_t)blockIdx.x * kScanItems + (size_t)threadIdx.x * kScanPerThread;
+    unsigned c[kScanPerThread];
+    load_counts(count, first, n, c);
     uint2 sum = make_uint2(0u, 0u);
 #pragma unroll
     for (int i = 0; i < kScanPerThread; ++i) {
-        const unsigned c = first + i < n ? count[first + i] : 0u;
-        sum.x += c;
-        sum.y += chunks_of(c);
+        sum.x += c[i];
+        sum.y += chunks_of(c[i], rows);
     }
     uint2 total;
     (void)block_exclusive_scan(sum, &total);
@@ -174,16 +196,27 @@ __global__ __launch_bounds__(kBlock) void k_scan_starts(const unsigned *__restri
                                                          unsigned *start, ListChunks chunks) {
     const size_t first = (size_t)blockIdx.x * kScanItems + (size_t)threadIdx.x * kScanPerThread;
     unsigned c[kScanPerThread];
+    load_counts(count, first, n, c);
     uint2 sum = make_uint2(0u, 0u);
 #pragma unroll
     for (int i = 0; i < kScanPerThread; ++i) {
-        c[i] = first + i < n ? count[first + i] : 0u;
         sum.x += c[i];
-        sum.y += chunks_of(c[i]);
+        sum.y += chunks_of(c[i], chunks.rows);
     }
     uint2 total;
     const uint2 base = block_sums[blockIdx.x];
     const uint2 before = block_exclusive_scan(sum, &total);
+    // the workgroup's long lists take one run of places in long_lists, drawn with one atomic
+    // (an atomic per list would queue up on the one counter)
+    unsigned long_here = 0;
+#pragma unroll
+    for (int i = 0; i < kScanPerThread; ++i) long_here += chunks_of(c[i], chunks.rows) > 1u ? 1u : 0u;
+    uint2 long_total;
+    const uint2 long_before = block_exclusive_scan(make_uint2(long_here, 0u), &long_total);
+    __shared__ unsigned long_base;
+    if (threadIdx.x == 0) long_base = long_total.x ? atomicAdd(&chunks.info[0], long_total.x) : 0u;
+    __syncthreads();
+    unsigned long_at = long_base + long_before.x;
     unsigned entry = base.x + before.x, chunk = base.y + before.y;
 #pragma unroll
     for (int i = 0; i < kScanPerThread; ++i) {
@@ -191,12 +224,13 @@ __global__ __launch_bounds__(kBlock) void k_scan_starts(const unsigned *__restri
             const unsigned v = (unsigned)(first + i);
             start[v] = entry;
             chunks.chunk_start[v] = chunk;
-            const unsigned of_v = chunks_of(c[i]);
+            const unsigned of_v = chunks_of(c[i], chunks.rows);
             if (of_v == 1u && chunk < chunks.max_chunks) {
                 chunks.chunk[chunk] = ListChunk{entry, entry + c[i], v, 1u};
             } else if (of_v > 1u) {
-                const unsigned at = atomicAdd(&chunks.info[0], 1u);
-                if (at < chunks.max_long) chunks.long_lists[at] = v;
+                if (long_at < chunks.max_long)
+                    chunks.long_lists[long_at] = LongList{v, chunk, entry, entry + c[i]};
+                long_at += 1u;
             }
             entry += c[i];
             chunk += of_v;
@@ -211,21 +245,20 @@ __global__ __launch_bounds__(kBlock) void k_scan_starts(const unsigned *__restri
 }
 
 // The chunks of the lists that have several: a workgroup per list, a thread per chunk.
-__global__ __launch_bounds__(kBlock) void k_long_list_chunks(const unsigned *__restrict__ start,
-                                                              ListChunks chunks, unsigned *host_info) {
+__global__ __launch_bounds__(kBlock) void k_long_list_chunks(ListChunks chunks, unsigned *host_info) {
     const unsigned n_long = chunks.info[0] < chunks.max_long ? chunks.info[0] : chunks.max_long;
     if (host_info && blockIdx.x == 0 && threadIdx.x == 0) {
         host_info[0] = chunks.info[0];
         host_info[1] = chunks.info[1];
     }
     for (unsigned i = blockIdx.x; i < n_long; i += gridDim.x) {
-        const unsigned v = chunks.long_lists[i];
-        const unsigned from = chunks.chunk_start[v], to = chunks.chunk_start[v + 1];
-        const unsigned list_from = start[v], list_to = start[v + 1];
+        const LongList list = chunks.long_lists[i];
+        const unsigned v = list.vertex, from = list.chunk_from;
+        const unsigned list_from = list.from, list_to = list.to;
+        const unsigned to = from + chunks_of(list_to - list_from, chunks.rows);
         for (unsigned c = from + threadIdx.x; c < to && c < chunks.max_chunks; c += kBlock) {
-            const unsigned first = list_from + (c - from) * (unsigned)kListChunk;
-            const unsigned last =
-                list_to - first < (unsigned)kListChunk ? list_to : first + (unsigned)kListChunk;
+            const unsigned first = list_from + (c - from) * chunks.rows;
+            const unsigned last = list_to - first < chunks.rows ? list_to : first + chunks.rows;
             chunks.chunk[c] = ListChunk{first, last, v, 0u};
         }
     }
@@ -392,35 +425,45 @@ __global__ __launch_bounds__(kBlock) void k_splat_gather_channels(ListChunks chu
 }
 
 // The lists of more than one chunk: the vertex's row := the sum of its chunks' partial rows.  A
-// workgroup per list and block of 32 channels: thread (s, c) adds channel c of every eighth chunk,
-// four loads in flight, and the eight sums are added through LDS (the same order on every call).
-__global__ __launch_bounds__(kBlock) void k_sum_partial_rows(ListChunks chunks, int vd, float *values) {
-    __shared__ float part[kBlock / 32][32];
-    const unsigned n_long = chunks.info[0] < chunks.max_long ? chunks.info[0] : chunks.max_long;
-    const unsigned slot = threadIdx.x >> 5, sub = threadIdx.x & 31;
-    constexpr unsigned kSlots = kBlock / 32;
-    for (unsigned i = blockIdx.x; i < n_long; i += gridDim.x) {
-        const unsigned v = chunks.long_lists[i];
-        const unsigned from = chunks.chunk_start[v], to = chunks.chunk_start[v + 1];
+// wavefront per list and block of 32 channels: lane (h, c) adds channel c of every second chunk,
+// kSumInFlight loads in flight (one round of loads for a list of up to 2 * kSumInFlight chunks),
+// and the two halves are added at the end.  Which lane adds which chunks depends on the list
+// alone: the same order on every call.
+constexpr int kSumInFlight = 16;
+
+__global__ __launch_bounds__(kBlock) void k_sum_partial_rows(ListChunks chunks, unsigned n_long, int vd,
+                                                              float *values) {
+    const int lane = threadIdx.x & 63, half = lane >> 5, sub = lane & 31;
+    const unsigned waves = gridDim.x * (kBlock / 64);
+    for (unsigned i = blockIdx.x * (kBlock / 64) + (threadIdx.x >> 6); i < n_long; i += waves) {
+        const LongList list = chunks.long_lists[i];
+        const unsigned from = list.chunk_from;
+        unsigned to = from + chunks_of(list.to - list.from, chunks.rows);
+        if (to > chunks.max_chunks) to = chunks.max_chunks;
         for (int c0 = 0; c0 < vd; c0 += 32) {
-            const int c = c0 + (int)sub;
-            float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
-            for (unsigned k = from + slot; k < to; k += 4u * kSlots) {
+            const int c = c0 + sub;
+            float acc[kSumInFlight];
 #pragma unroll
-                for (int u = 0; u < 4; ++u) {
-                    const unsigned ku = k + kSlots * (unsigned)u;
-                    if (ku < to && c < vd) acc[u] += chunks.partial_rows[(size_t)ku * vd + c];
+            for (int u = 0; u < kSumInFlight; ++u) acc[u] = 0.0f;
+            for (unsigned k = from + (unsigned)half; k < to; k += 2u * kSumInFlight) {
+#pragma unroll
+                for (int u = 0; u < kSumInFlight; ++u) {
+                    // (every load is issued, from a row that exists, and counted or not
+                    // afterwards: loads under a condition would wait for one another)
+                    const unsigned ku = k + 2u * (unsigned)u;
+                    const bool counts = ku < to && c < vd;
+                    const float x = chunks.partial_rows[(size_t)(ku < to ? ku : from) * vd +
+                                                        (c < vd ? c : 0)];
+                    acc[u] += counts ? x : 0.0f;
                 }
             }
-            __syncthreads();   // (part may still be read from the turn before)
-            part[slot][sub] = (acc[0] + acc[1]) + (acc[2] + acc[3]);
-            __syncthreads();
-            if (slot == 0 && c < vd) {
-                float sum = 0.0f;
 #pragma unroll
-                for (unsigned k = 0; k < kSlots; ++k) sum += part[k][sub];
-                values[(size_t)v * vd + c] = sum;
-            }
+            for (int width = kSumInFlight / 2; width >= 1; width /= 2)
+#pragma unroll
+                for (int u = 0; u < width; ++u) acc[u] += acc[u + width];
+            float sum = acc[0];
+            sum += __shfl_xor(sum, 32);
+            if (half == 0 && c < vd) values[(size_t)list.vertex * vd + c] = sum;
         }
     }
 }
@@ -431,9 +474,9 @@ size_t vertex_list_scan_blocks(int max_vertices) {
     return ((size_t)max_vertices + kScanItems - 1) / kScanItems;
 }
 size_t vertex_list_max_chunks(int max_vertices, size_t rows) {
-    return (size_t)max_vertices + rows / (size_t)kListChunk + 1;
+    return (size_t)max_vertices + rows / 128 + 1;
 }
-size_t vertex_list_max_long(size_t rows) { return rows / (size_t)kListChunk + 1; }
+size_t vertex_list_max_long(size_t rows) { return rows / 128 + 1; }
 
 hipError_t build_vertex_lists(int pd, const PointMap &map, ReplayEntry *replay, const int *cell_vertex,
                               int max_vertices, const VertexLists &lists, unsigned *host_info,
@@ -451,15 +494,15 @@ hipError_t build_vertex_lists(int pd, const PointMap &map, ReplayEntry *replay, 
     const unsigned scan_blocks = (unsigned)vertex_list_scan_blocks(max_vertices);
     uint2 *block_sums = reinterpret_cast<uint2 *>(lists.block_sums);
     hipLaunchKernelGGL(k_scan_block_sums, dim3(scan_blocks), block, 0, s, lists.count, n, block_sums,
-                       lists.chunks.info);
+                       lists.chunks.info, lists.chunks.rows);
     hipLaunchKernelGGL(k_scan_of_block_sums, dim3(1), block, 0, s, block_sums, scan_blocks);
     hipLaunchKernelGGL(k_scan_starts, dim3(scan_blocks), block, 0, s, lists.count, n, block_sums,
                        lists.start, lists.chunks);
     // (how many lists have several chunks is known on the device only: a grid that covers a
     // usual number of them, the workgroups walk the rest)
-    const unsigned long_blocks = lists.chunks.max_long < 1024u ? lists.chunks.max_long : 1024u;
+    const unsigned long_blocks = lists.chunks.max_long < 256u ? lists.chunks.max_long : 256u;
     hipLaunchKernelGGL(k_long_list_chunks, dim3(long_blocks ? long_blocks : 1u), block, 0, s,
-                       lists.start, lists.chunks, host_info);
+                       lists.chunks, host_info);
     if (map.n_blocks) {
         const dim3 grid(map.n_blocks);
         PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_list_fill<PD + 1>), grid, block, 0, s, map, replay,
@@ -504,8 +547,8 @@ hipError_t splat_gather(int vd, const VertexLists &lists, unsigned n_chunks, uns
     }
 #undef PLK_GATHER
     if (n_long)
-        hipLaunchKernelGGL(k_sum_partial_rows, dim3(n_long), block, 0, s,
-                           lists.chunks, vd, values);
+        hipLaunchKernelGGL(k_sum_partial_rows, dim3(blocks_for(n_long, kBlock / 64)), block, 0, s,
+                           lists.chunks, n_long, vd, values);
     return hipGetLastError();
 }
 

@@ -274,11 +274,14 @@ hipError_t splat(int pd, int vd, const PointMap &map, const float *input, int in
 // The transpose of the replay matrix, for lattices that are applied many times (pl_gather.hip):
 // the rows that name vertex v are entries[start[v] .. start[v+1]), each the point and its weight.
 // Vertices must be numbered densely (number_vertices).  The unit of work of the splat that
-// gathers is a chunk of at most kListChunk rows of one list: the chunks of vertex v are
+// gathers is a chunk of at most ListChunks::rows rows of one list: the chunks of vertex v are
 // chunk_start[v] .. chunk_start[v+1], chunk c is described by chunk[c]; a list of several chunks is
 // summed into the partial rows of its chunks first (partial_rows[c * vd ..]) and is named in
 // long_lists.  info: {long lists, chunks in all}.
-constexpr int kListChunk = 128;
+// (a chunk of 256 rows for rows of up to four values, where no list of an image like the
+// benchmark's is longer; 128 for rows of many channels, whose chunks cost more per row)
+constexpr int kMaxListChunk = 256;
+inline unsigned list_chunk_rows(int vd) { return vd <= 4 ? 256u : 128u; }
 struct ListEntry {
     int point;
     float weight;
@@ -288,13 +291,19 @@ struct alignas(16) ListChunk {
     unsigned vertex;
     unsigned whole;          // 1: the chunk is all of its vertex's list
 };
+struct alignas(16) LongList {   // a list of several chunks
+    unsigned vertex;
+    unsigned chunk_from;     // its first chunk
+    unsigned from, to;       // its rows: entries[from .. to)
+};
 struct ListChunks {
     unsigned *chunk_start;   // [max_vertices + 1]
     ListChunk *chunk;        // [max_chunks]
-    unsigned *long_lists;    // [max_long]
+    LongList *long_lists;    // [max_long]
     float *partial_rows;     // [max_chunks * vd]
     unsigned *info;          // [2], the two words behind VertexLists::count
     unsigned max_chunks, max_long;
+    unsigned rows;           // rows of a chunk at most (list_chunk_rows)
 };
 struct VertexLists {
     unsigned *start;       // [max_vertices + 1]

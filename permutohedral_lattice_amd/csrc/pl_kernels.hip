@@ -59,10 +59,18 @@ __device__ __forceinline__ void load_features(const PointFeatures &f, int n, flo
         }
     }
     if (f.n_reference_channels > 0) {
+        // (every channel is asked for at once, from an element that exists, and taken or not
+        // afterwards: loads behind the condition would wait for one another)
         const float *row = f.reference + (size_t)n * f.n_reference_channels;
+        float channel[PD];
+#pragma unroll
+        for (int i = 0; i < PD; ++i) {
+            const int j = i - f.n_spatial_dims;
+            channel[i] = row[j >= 0 && j < f.n_reference_channels ? j : 0];
+        }
 #pragma unroll
         for (int i = 0; i < PD; ++i)
-            if (i >= f.n_spatial_dims) pos[i] = row[i - f.n_spatial_dims] / f.feature_std;
+            if (i >= f.n_spatial_dims) pos[i] = channel[i] / f.feature_std;
     }
 }
 
@@ -1012,21 +1020,28 @@ __global__ __launch_bounds__(kBlock) void k_neighbours(VertexTables vertices,
     constexpr int D1 = PD + 1;
     // After a merging build nothing has told the host yet how the build went: the segments' counts
     // are summed here, and what the next build will count in is cleared.
-    if (report && blockIdx.x == gridDim.x - 1 && threadIdx.x == 0) {
-        unsigned total = 0, fullest = 0;
+    // (by the first wavefront of the first workgroup that looks up neighbours, which starts with
+    // the launch: a lane per segment)
+    if (report && blockIdx.x == foreign_blocks && threadIdx.x < 64) {
+        static_assert(kMaxSegments <= 64, "a lane per segment");
         const int n_segments = report->n_segments;
-        for (int k = 0; k < n_segments; ++k) {
-            const unsigned c = report->segment_count[k].n;
-            total += c;
-            fullest = c > fullest ? c : fullest;
+        const unsigned c = (int)threadIdx.x < n_segments ? report->segment_count[threadIdx.x].n : 0u;
+        unsigned total = c, fullest = c;
+#pragma unroll
+        for (int off = 32; off >= 1; off >>= 1) {
+            total += __shfl_xor(total, off);
+            const unsigned other = __shfl_xor(fullest, off);
+            fullest = other > fullest ? other : fullest;
         }
-        report->vertices = total;
-        host_status->num_vertices = (int)total;
-        host_status->flags = report->flags;
-        host_status->max_segment = (int)fullest;
-        host_status->n_segments = n_segments;
-        host_status->foreign_rows = (int)(report->foreign_rows_sampled.n * kForeignSampling);
-        reset_counters(next_counters);
+        if (threadIdx.x == 0) {
+            report->vertices = total;
+            host_status->num_vertices = (int)total;
+            host_status->flags = report->flags;
+            host_status->max_segment = (int)fullest;
+            host_status->n_segments = n_segments;
+            host_status->foreign_rows = (int)(report->foreign_rows_sampled.n * kForeignSampling);
+            reset_counters(next_counters);
+        }
     }
     if (blockIdx.x < foreign_blocks) {
         const unsigned group = xcd_contiguous_block(blockIdx.x, foreign_blocks, 1);
