@@ -334,39 +334,47 @@ struct alignas(IN == 3 ? 4 : 4 * IN) InputRow {
 // IN: channels of an input row, VD - 1 (the last channel of the vertex row is the sum of the bare
 // weights) or VD
 template <int VD, int IN>
-__global__ __launch_bounds__(kBlock) void k_splat_gather(ListChunks chunks,
+__global__ __launch_bounds__(kBlock) void k_splat_gather(ListChunks chunks, unsigned n_chunks,
                                                           const ListEntry *__restrict__ entries,
                                                           const float *__restrict__ input,
                                                           float *values) {
     static_assert(VD >= 2 && VD <= 4 && (IN == VD || IN == VD - 1), "the rows are gathered in registers");
-    const unsigned n_chunks = chunks.info[1];
     const unsigned sub = threadIdx.x % kLanes;
     constexpr unsigned per_block = kBlock / kLanes;
+    constexpr unsigned kTurn = kLanes * kInFlight;
     // (chunks follow the vertex numbers, which follow the image: every XCD takes one contiguous
     // range of them, so that the input rows its chunks share stay in its L2)
     const unsigned first_block = xcd_contiguous_block(blockIdx.x, gridDim.x, 1);
     for (unsigned c0 = first_block * per_block; c0 < n_chunks; c0 += gridDim.x * per_block) {
         const ChunkWork work = chunk_work(c0 + threadIdx.x / kLanes, n_chunks, chunks, VD, values);
         float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+        // A turn's entries are asked for one turn ahead, together with the rows of the turn before:
+        // a turn then waits for one round trip to memory, not two.  (An entry past the end of the
+        // chunk reads the chunk's first and counts with weight zero.)
+        ListEntry e[kInFlight];
+#pragma unroll
+        for (int u = 0; u < kInFlight; ++u) {
+            const unsigned i = work.from + (unsigned)u * kLanes + sub;
+            e[u] = entries[i < work.to ? i : work.from];
+        }
         // (the lanes of a chunk leave the loop together: what they exchange below is complete)
-        for (unsigned turn = work.from; turn < work.to; turn += kLanes * kInFlight) {
-            ListEntry e[kInFlight];
-            bool valid[kInFlight];
-#pragma unroll
-            for (int u = 0; u < kInFlight; ++u) {
-                const unsigned i = turn + (unsigned)u * kLanes + sub;
-                valid[u] = i < work.to;
-                e[u] = entries[valid[u] ? i : work.from];
-            }
+        for (unsigned turn = work.from; turn < work.to; turn += kTurn) {
             InputRow<IN> x[kInFlight];
-#pragma unroll
-            for (int u = 0; u < kInFlight; ++u)
-                x[u] = reinterpret_cast<const InputRow<IN> *>(input)[e[u].point];
+            float w[kInFlight];
 #pragma unroll
             for (int u = 0; u < kInFlight; ++u) {
-                const float w = valid[u] ? e[u].weight : 0.0f;
+                x[u] = reinterpret_cast<const InputRow<IN> *>(input)[e[u].point];
+                w[u] = turn + (unsigned)u * kLanes + sub < work.to ? e[u].weight : 0.0f;
+            }
 #pragma unroll
-                for (int j = 0; j < VD; ++j) acc[j] += w * (j < IN ? x[u].c[j] : 1.0f);
+            for (int u = 0; u < kInFlight; ++u) {
+                const unsigned i = turn + kTurn + (unsigned)u * kLanes + sub;
+                e[u] = entries[i < work.to ? i : work.from];
+            }
+#pragma unroll
+            for (int u = 0; u < kInFlight; ++u) {
+#pragma unroll
+                for (int j = 0; j < VD; ++j) acc[j] += w[u] * (j < IN ? x[u].c[j] : 1.0f);
             }
         }
 #pragma unroll
@@ -381,45 +389,77 @@ __global__ __launch_bounds__(kBlock) void k_splat_gather(ListChunks chunks,
     }
 }
 
-// Any number of channels: W lanes per chunk (a power of two, 16..64, at least vd unless vd > 64),
-// lane c on channel c.  The lanes read W entries of the list at once, one each, and hand them
-// round; every lane then reads its channel of the rows they name, sixteen loads in flight.
-// Channels past the input are the homogeneous one.
-template <int W>
-__global__ __launch_bounds__(kBlock) void k_splat_gather_channels(ListChunks chunks, int vd,
+// More than four channels: L lanes per chunk (4, 8 or 16), lane i on the channels 4i .. 4i+3 of
+// every row of the chunk.  What bounds a gather of rows of many channels is the number of load
+// instructions (the memory pipeline takes 16 cycles to look at the 64 addresses of one, whatever
+// their width), so a lane reads its four channels of an input row with one 16-byte load; rows
+// need only be aligned to four bytes for that.  The lane on the row's last channels reads the
+// row's last four instead (no load leaves the row) and its sums are shifted back at the end.  The
+// lanes first read the whole chunk's entries, kChannelChunk / L each, and hand them round.
+// Channels past the input are the homogeneous one: the sum of the bare weights.
+constexpr int kChannelChunk = 128;   // rows of a chunk at most (list_chunk_rows for vd > 4)
+
+
+struct alignas(4) FourFloats {
+    float c[4];
+};
+__device__ __forceinline__ float pick(const float (&x)[4], int i) {
+    return i == 0 ? x[0] : i == 1 ? x[1] : i == 2 ? x[2] : x[3];
+}
+
+template <int L>
+__global__ __launch_bounds__(kBlock) void k_splat_gather_channels(ListChunks chunks, unsigned n_chunks,
+                                                                   int vd,
                                                                    const ListEntry *__restrict__ entries,
                                                                    const float *__restrict__ input,
                                                                    int in_channels, float *values) {
-    const unsigned n_chunks = chunks.info[1];
-    constexpr unsigned per_block = kBlock / W;
-    const int sub = threadIdx.x % W;
-    constexpr int kBatch = 16;
+    constexpr unsigned per_block = kBlock / L;
+    constexpr int E = kChannelChunk / L;          // entries per lane
+    constexpr int kBatch = 16;                    // rows in flight (8: 6 % slower, 32: 2 %)
+    const int sub = threadIdx.x % L;
     const unsigned first_block = xcd_contiguous_block(blockIdx.x, gridDim.x, 1);
     for (unsigned c0 = first_block * per_block; c0 < n_chunks; c0 += gridDim.x * per_block) {
-        const ChunkWork work = chunk_work(c0 + threadIdx.x / W, n_chunks, chunks, vd, values);
-        for (int ch0 = 0; ch0 < vd; ch0 += W) {
-            const int c = ch0 + sub;
-            float acc = 0.0f;
-            for (unsigned turn = work.from; turn < work.to; turn += W) {
-                const unsigned mine = turn + (unsigned)sub;
-                const ListEntry e = entries[mine < work.to ? mine : work.from];
-                const unsigned here = work.to - turn < (unsigned)W ? work.to - turn : (unsigned)W;
-                for (unsigned k0 = 0; k0 < here; k0 += kBatch) {
-                    float x[kBatch], w[kBatch];
+        const ChunkWork work = chunk_work(c0 + threadIdx.x / L, n_chunks, chunks, vd, values);
+        const unsigned rows = work.to - work.from;
+        // (entries past the end of the chunk: its first row, weight zero)
+        ListEntry e[E];
+#pragma unroll
+        for (int u = 0; u < E; ++u) {
+            const unsigned mine = work.from + (unsigned)(u * L + sub);
+            e[u] = entries[mine < work.to ? mine : work.from];
+            if (mine >= work.to) e[u].weight = 0.0f;
+        }
+        for (int ch0 = 0; ch0 < vd; ch0 += 4 * L) {
+            const int c = ch0 + 4 * sub;
+            const int start = c < in_channels ? (c < in_channels - 4 ? c : in_channels - 4) : 0;
+            float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f}, weights = 0.0f;
+#pragma unroll
+            for (int row0 = 0; row0 < kChannelChunk; row0 += kBatch) {
+                if ((unsigned)row0 < rows) {
+                    FourFloats x[kBatch];
+                    float w[kBatch];
 #pragma unroll
                     for (int k = 0; k < kBatch; ++k) {
-                        // (entries past the end of the chunk: its first row, weight zero)
-                        const bool in_list = k0 + k < here;
-                        const int src = in_list ? (int)(k0 + k) : 0;
-                        const int p = __shfl(e.point, src, W);
-                        w[k] = in_list ? __shfl(e.weight, src, W) : 0.0f;
-                        x[k] = c < in_channels ? input[(size_t)p * in_channels + c] : 1.0f;
+                        // (row row0 + k of the chunk is entry (row0 + k) / L of lane (row0 + k) % L)
+                        const int p = __shfl(e[(row0 + k) / L].point, (row0 + k) % L, L);
+                        w[k] = __shfl(e[(row0 + k) / L].weight, (row0 + k) % L, L);
+                        x[k] = *reinterpret_cast<const FourFloats *>(
+                            input + (size_t)p * in_channels + start);
                     }
 #pragma unroll
-                    for (int k = 0; k < kBatch; ++k) acc += w[k] * x[k];
+                    for (int k = 0; k < kBatch; ++k) {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) acc[j] += w[k] * x[k].c[j];
+                        weights += w[k];
+                    }
                 }
             }
-            if (work.row && c < vd) work.row[c] = acc;
+            if (work.row) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    if (c + j < vd)
+                        work.row[c + j] = c + j < in_channels ? pick(acc, c - start + j) : weights;
+            }
         }
     }
 }
@@ -520,28 +560,30 @@ hipError_t splat_gather(int vd, const VertexLists &lists, unsigned n_chunks, uns
     case VD:                                                                                        \
         if (in_channels == VD)                                                                      \
             hipLaunchKernelGGL((k_splat_gather<VD, VD>), dim3(blocks_for(n_chunks, kBlock / kLanes)),\
-                               block, 0, s, lists.chunks, lists.entries, input, values);\
+                               block, 0, s, lists.chunks, n_chunks, lists.entries, input, values);\
         else if (in_channels == VD - 1)                                                             \
             hipLaunchKernelGGL((k_splat_gather<VD, VD - 1>),                                         \
                                dim3(blocks_for(n_chunks, kBlock / kLanes)), block, 0, s,            \
-                               lists.chunks, lists.entries, input, values);            \
+                               lists.chunks, n_chunks, lists.entries, input, values);  \
         else                                                                                        \
             return hipErrorInvalidValue;                                                            \
         break;
     switch (vd) {
         PLK_GATHER(2) PLK_GATHER(3) PLK_GATHER(4)
         default:
+            if (lists.chunks.rows > (unsigned)kChannelChunk) return hipErrorInvalidValue;
+            if (in_channels < 4) return hipErrorInvalidValue;
             if (vd <= 16)
-                hipLaunchKernelGGL(k_splat_gather_channels<16>, dim3(blocks_for(n_chunks, kBlock / 16)),
-                                   block, 0, s, lists.chunks, vd, lists.entries, input,
+                hipLaunchKernelGGL(k_splat_gather_channels<4>, dim3(blocks_for(n_chunks, kBlock / 4)),
+                                   block, 0, s, lists.chunks, n_chunks, vd, lists.entries, input,
                                    in_channels, values);
             else if (vd <= 32)
-                hipLaunchKernelGGL(k_splat_gather_channels<32>, dim3(blocks_for(n_chunks, kBlock / 32)),
-                                   block, 0, s, lists.chunks, vd, lists.entries, input,
+                hipLaunchKernelGGL(k_splat_gather_channels<8>, dim3(blocks_for(n_chunks, kBlock / 8)),
+                                   block, 0, s, lists.chunks, n_chunks, vd, lists.entries, input,
                                    in_channels, values);
             else
-                hipLaunchKernelGGL(k_splat_gather_channels<64>, dim3(blocks_for(n_chunks, kBlock / 64)),
-                                   block, 0, s, lists.chunks, vd, lists.entries, input,
+                hipLaunchKernelGGL(k_splat_gather_channels<16>, dim3(blocks_for(n_chunks, kBlock / 16)),
+                                   block, 0, s, lists.chunks, n_chunks, vd, lists.entries, input,
                                    in_channels, values);
             break;
     }

@@ -1810,6 +1810,98 @@ __global__ __launch_bounds__(kBlock) void k_slice_channels(int vd, PointMap map,
             output[(size_t)n * out_ch + j0 + i] = normalize ? acc[i] * scale : acc[i];
 }
 
+// Nine to sixty-four channels: L lanes per point (4, 8 or 16), lane i on the channels 4i .. 4i+3.
+// What bounds the slice of rows of many channels is the number of load instructions, not bytes
+// (the memory pipeline looks at the 64 addresses of one for 16 cycles whatever their width): a
+// lane reads its four channels of a vertex row with one 16-byte load (rows need only be aligned to
+// four bytes for that), and the pd+1 replay rows of a point are read once, a corner per lane, and
+// handed round.  The lane on the row's last channels reads the row's last four instead, so that
+// no load leaves the row, and its sums are shifted back before they are stored.  Same sums in the
+// same order as k_slice_channels.
+struct alignas(4) FourFloats {
+    float c[4];
+};
+constexpr int kSlicePoints = 2;   // points per group of L lanes (1: 2 % slower, 4: 4 %)
+template <int D1, int L>
+__global__ __launch_bounds__(kBlock) void k_slice_quads(int vd, PointMap map, size_t T,
+                                                         const ReplayEntry *__restrict__ replay,
+                                                         const float *__restrict__ values,
+                                                         float *__restrict__ output, int normalize) {
+    // workgroup (x, y): kSlicePoints * 256 / L points of point block x, each group of L lanes
+    // kSlicePoints of them, with the loads of all in flight together (a point's loads alone
+    // leave the lanes waiting: what bounds the pass is then how many points are in flight)
+    constexpr int kGroups = kBlock / L;
+    constexpr int P = kSlicePoints;
+    constexpr int E = (D1 + L - 1) / L;     // replay rows a lane reads per point
+    const int sub = threadIdx.x % L;
+    unsigned vblock;   // as in k_slice_point
+    if (!block_of_points(map, 1, vblock)) return;
+    int n[P];
+    ReplayEntry mine[P][E];
+#pragma unroll
+    for (int q = 0; q < P; ++q) {
+        const unsigned slot = (blockIdx.y * P + q) * kGroups + threadIdx.x / L;
+        const size_t t = (size_t)vblock * kBlock + slot;
+        n[q] = point_of_thread(map, vblock, slot);   // (the same for all L lanes)
+#pragma unroll
+        for (int u = 0; u < E; ++u) {
+            const int r = u * L + sub;
+            mine[q][u] = replay[(size_t)(r < D1 ? r : 0) * T + t];
+        }
+    }
+    const int c = 4 * sub;
+    const int start = c < vd - 4 ? c : vd - 4;
+    FourFloats x[P][D1];
+    float w[P][D1];
+#pragma unroll
+    for (int q = 0; q < P; ++q) {
+#pragma unroll
+        for (int r = 0; r < D1; ++r) {
+            const int index = __shfl(mine[q][r / L].index, r % L, L);
+            w[q][r] = __shfl(mine[q][r / L].weight, r % L, L);
+            const bool present = index >= 0 && n[q] >= 0;
+            x[q][r] = *reinterpret_cast<const FourFloats *>(values + (size_t)(present ? index : 0) * vd +
+                                                            start);
+            if (!present) w[q][r] = 0.0f, x[q][r] = FourFloats{{0.0f, 0.0f, 0.0f, 0.0f}};
+        }
+    }
+    // the homogeneous channel vd-1 is with the lane (vd-1)/4
+    const int with = (vd - 1) / 4;
+    const int with_start = 4 * with < vd - 4 ? 4 * with : vd - 4;
+    const int at = vd - 1 - with_start;
+    const int out_ch = normalize ? vd - 1 : vd;
+    const int shift = c - start;
+#pragma unroll
+    for (int q = 0; q < P; ++q) {
+        float acc[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+        for (int r = 0; r < D1; ++r) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[j] += w[q][r] * x[q][r].c[j];
+        }
+        const float own = at == 0 ? acc[0] : at == 1 ? acc[1] : at == 2 ? acc[2] : acc[3];
+        const float hom = __shfl(own, with, L);
+        if (n[q] < 0) continue;
+        const float scale = normalize ? (float)(1.0 / (double)hom) : 1.0f;
+        float *out = output + (size_t)n[q] * out_ch + c;
+        if (shift == 0 && c + 4 <= out_ch) {
+            FourFloats y;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) y.c[j] = normalize ? acc[j] * scale : acc[j];
+            *reinterpret_cast<FourFloats *>(out) = y;
+        } else {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                if (c + j < out_ch) {
+                    const int i = shift + j;
+                    const float v = i == 0 ? acc[0] : i == 1 ? acc[1] : i == 2 ? acc[2] : acc[3];
+                    out[j] = normalize ? v * scale : v;
+                }
+            }
+        }
+    }
+}
+
 // ------------------------------------------------------------------------------------------------
 // Debug exports and the feature builder
 // ------------------------------------------------------------------------------------------------
@@ -2303,6 +2395,22 @@ hipError_t slice(int pd, int vd, const PointMap &map, const ReplayEntry *replay,
         PLK_SLICE(5) PLK_SLICE(6) PLK_SLICE(7) PLK_SLICE(8)
         default: {
             const int out_ch = normalize ? vd - 1 : vd;
+#define PLK_SLICE_QUADS(L)                                                                      \
+    PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_slice_quads<PD + 1, L>),                          \
+                                           dim3(map.n_blocks, L / kSlicePoints),                \
+                                           block, 0, s, vd, map, T, replay, values, output,     \
+                                           normalize))
+            if (vd <= 16) {
+                PLK_SLICE_QUADS(4);
+                break;
+            } else if (vd <= 32) {
+                PLK_SLICE_QUADS(8);
+                break;
+            } else if (vd <= 64) {
+                PLK_SLICE_QUADS(16);
+                break;
+            }
+#undef PLK_SLICE_QUADS
             PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_slice_channels<PD + 1>),
                                                    dim3(map.n_blocks, (out_ch + kSliceRun - 1) / kSliceRun), block, 0, s,
                                                    vd, map, T, replay, values, output, normalize));
