@@ -61,23 +61,34 @@ def measured_traffic(kernel_name, grid_threads, stem="bench_bilateral_1024_pd5_v
     return int(sum(table[key])), stamp
 
 
-def kernel_names(pd, vd):
-    """The kernels a filter() call of a grid of points runs for these dimensions, by stage."""
+def kernel_names(pd, vd, in_channels=None, gathered=False):
+    """The kernels a filter() call of a grid of points runs for these dimensions, by stage
+    (gathered: an apply of a lattice that pl_build gave per-vertex lists)."""
     fused = vd <= 4
     d1 = pd + 1
+    lanes = 4 if vd <= 16 else (8 if vd <= 32 else 16)
     if fused:
         blur = "k_blur3_row<%d, float>" % vd if pd == 2 else "k_blur2_row<%d, float>" % vd
         slice_k = "k_slice_point<%d, %d>" % (vd, d1)
     else:
         blur = "k_blur2_element<float>"
-        slice_k = "k_slice_point<%d, 0>" % vd if vd <= 8 else "k_slice_channels<%d>" % d1
+        if vd <= 8:
+            slice_k = "k_slice_point<%d, 0>" % vd
+        elif vd <= 64:
+            slice_k = "k_slice_quads<%d, %d>" % (d1, lanes)
+        else:
+            slice_k = "k_slice_channels<%d>" % d1
     width = 16 if vd <= 16 else (32 if vd <= 32 else 64)
+    if gathered:
+        splat = ("k_splat_gather<%d, %d>" % (vd, in_channels if in_channels else vd - 1) if fused
+                 else "k_splat_gather_channels<%d>" % lanes)
+    else:
+        splat = "k_splat_dpp<%d, %d>" % (vd, d1) if fused else "k_splat_channels<%d>" % width
     return {"build": "k_build_tile<%d, %d, float>" % (pd, vd if fused else 0),
-            "splat": "k_splat_dpp<%d, %d>" % (vd, d1) if fused else "k_splat_channels<%d>" % width,
-            "blur_axis": blur, "slice": slice_k}
+            "splat": splat, "blur_axis": blur, "slice": slice_k}
 
 
-def stage_report(lat, call, n, pd, vd, samples=5, fused_splat=True):
+def stage_report(lat, call, n, pd, vd, samples=5, fused_splat=True, gathered=False):
     """Per-stage milliseconds of `call()` (one filter or apply on `lat`) from HIP events on the
     lattice's stream, and the stage that takes longest with its share of the HBM roofline."""
     import permutohedral_lattice_amd as pla
@@ -93,7 +104,7 @@ def stage_report(lat, call, n, pd, vd, samples=5, fused_splat=True):
     alg = algorithmic_bytes(n, m, pd, vd)
     if vd <= 4 and fused_splat:
         alg["build"] += alg["splat"]      # filter() splats inside the build kernel
-    names = kernel_names(pd, vd)
+    names = kernel_names(pd, vd, gathered=gathered)
     candidates = [k for k in ("build", "splat", "slice") if stages[k] > 0.0]
     dominant = max(candidates, key=lambda k: stages[k])
     if stages["blur"] > stages[dominant]:
@@ -266,9 +277,9 @@ def run_configs(args, pla, synth, with_cpu):
     msg = torch.empty_like(q0)
     torch.cuda.synchronize()      # (the lattices work on streams of their own)
     st_bi, dom_bi = stage_report(mf.bilateral[0], lambda: mf.bilateral[0].apply(msg, q0, False), n, 5,
-                                 classes + 1, fused_splat=False)
+                                 classes + 1, fused_splat=False, gathered=True)
     st_sp, dom_sp = stage_report(mf.spatial[0], lambda: mf.spatial[0].apply(msg, q0, False), n, 2,
-                                 classes + 1, fused_splat=False)
+                                 classes + 1, fused_splat=False, gathered=True)
     # an apply moves what a filter moves less the positions and the keys (the lattice is there)
     def apply_bytes(m, pd, vd):
         return 4 * n * 2 * (vd - 1) + m * 4 * vd * (2 * (pd + 1) + 2)

@@ -196,7 +196,11 @@ class PermutohedralLattice:
             _lib.pl_destroy(self._h)
             self._h = None
 
-    __del__ = close
+    def __del__(self):
+        # (at interpreter exit the module's globals may be gone before the last lattice: the
+        # process's memory goes with it)
+        if _lib is not None:
+            self.close()
 
     # -- the reference's interface -------------------------------------------------------------
     def filter(self, output, input, positions, reverse=False):

@@ -606,7 +606,13 @@ struct SegmentWalk {
             runs = (unsigned)mine.n_segments / kXcds;
             run_first = xcd * runs;
             stride = segment_stride((uint32_t)max_vertices, mine.n_segments);
-            load_run();
+            if (runs == 1) {
+                // (the XCD's one segment is the line just read: no second round trip to memory)
+                first = xcd * stride;
+                count = mine.n < stride ? mine.n : stride;
+            } else {
+                load_run();
+            }
         } else {
             // (one run: after the numbering pass every line holds the total, after a build
             // with one segment the first)

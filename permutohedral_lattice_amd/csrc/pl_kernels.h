@@ -31,7 +31,7 @@ enum : int {
 // table has one segment.  An atomic on one address takes about 50 ns and the next one waits for
 // it, so this is for builds of a few thousand workgroups.  Otherwise the numbering is left to
 // number_vertices, which gives the numbers 0 .. vertices-1 (n_segments == 0).
-constexpr int kMaxSegments = 8;
+constexpr int kMaxSegments = 64;
 struct Counters {
     unsigned int vertices;   // total (may exceed what the table can hold)
     int flags;
