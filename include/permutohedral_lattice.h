@@ -278,6 +278,22 @@ int pl_filter_image_begin(pl_handle h, float *output, const float *input, const 
 int pl_filter_end(pl_handle h);
 
 /*
+ * pl_build / pl_build_image in two halves, for callers that build several lattices at a time
+ * (each on a stream of its own): *_begin enqueues the build and returns at once; pl_build_end
+ * waits for the build's report, repeats the build with a larger hash table should it have turned
+ * out too small, and returns when the lattice is ready for pl_apply.  The arguments of *_begin
+ * must stay valid until pl_build_end; between the two only pl_build_end and pl_destroy may be
+ * called on the handle (anything else returns PL_ESTATE, also pl_filter_end).  pl_build_end with
+ * nothing in flight returns PL_OK.  No counterpart in the reference, which builds inside every
+ * filter call (src/LatticeFilterKernel.cpp:79).
+ */
+int pl_build_begin(pl_handle h, const float *positions);
+int pl_build_image_begin(pl_handle h, const float *reference, int n_reference_channels,
+                         int n_spatial_dims, const int *spatial_dims, float spatial_std,
+                         float feature_std);
+int pl_build_end(pl_handle h);
+
+/*
  * The LatticeFilter op on channels-last device tensors input[B, s_1..s_k, C_in],
  * reference[B, s_1..s_k, C_ref] -> output (shape of input).  bilateral: features are
  * (coords/theta_alpha, reference/theta_beta); otherwise coords/theta_gamma and the reference is

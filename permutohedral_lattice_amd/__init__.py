@@ -42,7 +42,8 @@ EXPORTS = (
     "pl_supported", "pl_strerror", "pl_last_hip_error", "pl_library_info", "pl_create", "pl_destroy", "pl_filter",
     "pl_filter_static", "pl_build", "pl_apply", "pl_set_point_grid", "pl_get_point_grid", "pl_num_vertices", "pl_set_option", "pl_get_info", "pl_stage_ms", "pl_debug_simplex",
     "pl_debug_keys", "pl_debug_values", "pl_debug_replay", "pl_compute_positions", "pl_filter_image", "pl_build_image",
-    "pl_filter_begin", "pl_filter_image_begin", "pl_filter_end", "pl_lattice_filter_op",
+    "pl_filter_begin", "pl_filter_image_begin", "pl_filter_end",
+    "pl_build_begin", "pl_build_image_begin", "pl_build_end", "pl_lattice_filter_op",
     "pl_set_op_concurrency",
     "pl_create_f64", "pl_filter_f64", "pl_build_f64", "pl_apply_f64", "pl_debug_simplex_f64",
     "pl_compute_positions_f64", "pl_lattice_filter_op_f64",
@@ -109,6 +110,9 @@ def _load(path=LIB_PATH):
     lib.pl_filter_begin.argtypes = [vp, vp, vp, vp, ci]
     lib.pl_filter_image_begin.argtypes = [vp, vp, vp, vp, ci, ci, C.POINTER(ci), cf, cf, ci]
     lib.pl_filter_end.argtypes = [vp]
+    lib.pl_build_begin.argtypes = [vp, vp]
+    lib.pl_build_image_begin.argtypes = [vp, vp, ci, ci, C.POINTER(ci), cf, cf]
+    lib.pl_build_end.argtypes = [vp]
     lib.pl_set_op_concurrency.argtypes = [ci]
     lib.pl_lattice_filter_op.argtypes = [vp, vp, vp, ci, ci, C.POINTER(ci), ci, ci, ci, cf, cf, cf,
                                          ci, vp, vp]
@@ -231,6 +235,18 @@ class PermutohedralLattice:
         call = _lib.pl_build_f64 if self._f64 else _lib.pl_build
         _check(call(self._h, self._t(positions, "positions", self.N * self.pd)), "pl_build")
 
+    def build_begin(self, positions):
+        """``build`` in two halves: enqueue, and ``build_end`` waits and checks (so that several
+        lattices, each on a stream of its own, are built side by side)."""
+        self._float_only("build_begin")
+        self._in_flight = (positions,)   # keep the tensor alive until build_end
+        _check(_lib.pl_build_begin(self._h, _dev_f32(positions, "positions", self.N * self.pd)),
+               "pl_build_begin")
+
+    def build_end(self):
+        _check(_lib.pl_build_end(self._h), "pl_build_end")
+        self._in_flight = None
+
     def apply(self, output, input, reverse=False):
         ch = self.vd - 1 if self._normalize else self.vd
         call = _lib.pl_apply_f64 if self._f64 else _lib.pl_apply
@@ -264,6 +280,13 @@ class PermutohedralLattice:
         ref, rc, k, dims = self._image_args(reference, spatial_dims)
         _check(_lib.pl_build_image(self._h, ref, rc, k, dims, float(spatial_std), float(feature_std)),
                "pl_build_image")
+
+    def build_image_begin(self, reference, spatial_dims, spatial_std, feature_std=1.0):
+        """``build_image`` enqueued; ``build_end`` completes it."""
+        ref, rc, k, dims = self._image_args(reference, spatial_dims)
+        self._in_flight = (reference,)
+        _check(_lib.pl_build_image_begin(self._h, ref, rc, k, dims, float(spatial_std),
+                                         float(feature_std)), "pl_build_image_begin")
 
     def set_point_grid(self, dims):
         """Hint: the N points form a row-major grid of these extents (None removes the hint)."""

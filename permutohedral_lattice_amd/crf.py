@@ -59,11 +59,15 @@ class MeanField:
         rc = int(guide.shape[-1])
         theta_alpha, theta_beta, theta_gamma = self.thetas
         self._side_streams_wait_for_caller()
+        # all builds are enqueued, each on its lattice's stream, before the first is waited for: a
+        # build is a chain of a dozen short kernels, and 2 x batch of them run side by side
         for b in range(self.batch):
-            self.bilateral[b].build_image(self.guide[b].reshape(self.n, rc), self.sdims,
-                                          theta_alpha, theta_beta)
-            self.spatial[b].build_image(None, self.sdims, theta_gamma)
-        # (a build returns when its lattice is complete: nothing to wait for here)
+            self.bilateral[b].build_image_begin(self.guide[b].reshape(self.n, rc), self.sdims,
+                                                theta_alpha, theta_beta)
+            self.spatial[b].build_image_begin(None, self.sdims, theta_gamma)
+        for lat in self.bilateral + self.spatial:
+            lat.build_end()
+        # (a build has ended when its lattice is complete: nothing to wait for here)
 
     def _side_streams_wait_for_caller(self):
         """What the caller's stream has been given so far is complete before any lattice's stream

@@ -188,6 +188,8 @@ struct pl_lattice {
     // a filter call that has been enqueued but not yet checked on the host (pl_filter_*_begin)
     struct Pending {
         bool active = false;
+        bool build_only = false;       // pl_build_*_begin: no apply behind the build
+        bool lists = false;            // ... and the per-vertex lists behind it
         plk::PointFeatures features{};
         const double *positions64 = nullptr;
         void *output = nullptr;
@@ -1065,8 +1067,31 @@ int features_from_image(pl_lattice *h, const float *reference, int n_reference_c
     return PL_OK;
 }
 
-int build_lattice(pl_lattice *h, const plk::PointFeatures &features,
-                  const double *positions64 = nullptr) {
+// pl_build in two halves, as pl_filter below: begin enqueues the build, and behind it the lists
+// of a lattice that keeps them, and returns; end waits for the build's report, repeats the build
+// with a larger table where it did not fit, and reads how many chunks the lists have.
+int enqueue_build_only(pl_lattice *h, const plk::PointFeatures &features, const double *positions64,
+                       uint32_t cells, bool lists) {
+    int rc = enqueue_build(h, features, positions64, cells, nullptr);
+    if (rc != PL_OK) return rc;
+    if (lists) {
+        // The lattice is there to be applied: per vertex the list of the rows that name it, so
+        // that every apply splats by gathering (float values; a build without a splat numbers its
+        // vertices densely).  Enqueued before the host waits for the build's report.
+        rc = ensure_vertex_lists(h);
+        if (rc != PL_OK) return rc;
+        PL_HIP(plk::build_vertex_lists(h->pd, h->map, h->replay,
+                                       h->replay_holds_cells ? h->cell_vertex : nullptr,
+                                       h->max_vertices(), h->lists_of_vertices,
+                                       reinterpret_cast<unsigned *>(h->h_status + 1), h->stream));
+        h->replay_holds_cells = false;
+    }
+    return PL_OK;
+}
+
+int build_begin(pl_lattice *h, const plk::PointFeatures &features,
+                const double *positions64 = nullptr) {
+    if (h->pending.active) return PL_ESTATE;
     h->built = false;
     h->M = 0;
     for (int i = 0; i <= EV_NBR; ++i) h->ev_recorded[i] = false;
@@ -1074,31 +1099,36 @@ int build_lattice(pl_lattice *h, const plk::PointFeatures &features,
         h->built = h->verified = true;
         return PL_OK;
     }
-    // The lattice is there to be applied: per vertex the list of the rows that name it, so that
-    // every apply splats by gathering (float values; a build without a splat numbers its vertices
-    // densely).  The lists are enqueued behind the build, before the host waits for its report.
     const bool lists = h->vertex_lists && !h->f64 && !h->status_on_device;
-    uint32_t cells = initial_cells(h);
+    const int rc = enqueue_build_only(h, features, positions64, initial_cells(h), lists);
+    if (rc != PL_OK) return rc;
+    h->pending.active = true;
+    h->pending.build_only = true;
+    h->pending.lists = lists;
+    h->pending.features = features;
+    h->pending.positions64 = positions64;
+    return PL_OK;
+}
+
+int build_end(pl_lattice *h) {
+    if (!h->pending.active) return PL_OK;   // nothing in flight (or an empty lattice)
+    if (!h->pending.build_only) return PL_ESTATE;
+    const bool lists = h->pending.lists;
     for (;;) {
-        int rc = enqueue_build(h, features, positions64, cells, nullptr);
-        if (rc != PL_OK) return rc;
-        if (lists) {
-            rc = ensure_vertex_lists(h);
-            if (rc != PL_OK) return rc;
-            PL_HIP(plk::build_vertex_lists(h->pd, h->map, h->replay,
-                                           h->replay_holds_cells ? h->cell_vertex : nullptr,
-                                           h->max_vertices(), h->lists_of_vertices,
-                                           reinterpret_cast<unsigned *>(h->h_status + 1), h->stream));
-            h->replay_holds_cells = false;
-        }
-        rc = verify_build(h, &cells);
+        uint32_t cells = 0;
+        int rc = verify_build(h, &cells);
         if (rc == PL_OK) break;
-        if (!cells) return rc;
+        if (cells) rc = enqueue_build_only(h, h->pending.features, h->pending.positions64, cells, lists);
+        if (!cells || rc != PL_OK) {
+            h->pending.active = false;
+            return rc;
+        }
     }
+    h->pending.active = false;
     if (lists && h->n_segments == 0) {
         // (how many chunks there are, and whether any list has several, sizes every apply's
-        // launches: read once here, where the caller is building and expects to wait)
-        // (the last kernel of the lists wrote them behind the build's status, in pinned memory)
+        // launches: the last kernel of the lists wrote them behind the build's status, in pinned
+        // memory; read once here, where the caller is building and expects to wait)
         PL_HIP(hipStreamSynchronize(h->stream));
         const volatile unsigned *info = reinterpret_cast<const volatile unsigned *>(h->h_status + 1);
         const plk::ListChunks &c = h->lists_of_vertices.chunks;
@@ -1107,6 +1137,12 @@ int build_lattice(pl_lattice *h, const plk::PointFeatures &features,
         h->lists_valid = true;
     }
     return PL_OK;
+}
+
+int build_lattice(pl_lattice *h, const plk::PointFeatures &features,
+                  const double *positions64 = nullptr) {
+    const int rc = build_begin(h, features, positions64);
+    return rc == PL_OK ? build_end(h) : rc;
 }
 
 // pl_filter in two halves.  begin: build and apply are enqueued together and the call returns.
@@ -1130,6 +1166,7 @@ int filter_begin(pl_lattice *h, void *output, const void *input,
     rc = enqueue_apply(h, output, input, reverse);
     if (rc != PL_OK) return rc;
     h->pending.active = true;
+    h->pending.build_only = false;
     h->pending.features = features;
     h->pending.positions64 = positions64;
     h->pending.output = output;
@@ -1140,6 +1177,7 @@ int filter_begin(pl_lattice *h, void *output, const void *input,
 
 int filter_end(pl_lattice *h) {
     if (!h->pending.active) return PL_OK;   // nothing in flight (or an empty lattice)
+    if (h->pending.build_only) return PL_ESTATE;
     for (;;) {
         uint32_t cells = 0;
         int rc = verify_build(h, &cells);
@@ -1185,6 +1223,32 @@ int pl_build_image(pl_handle h, const float *reference, int n_reference_channels
     const int rc = features_from_image(h, reference, n_reference_channels, n_spatial_dims,
                                        spatial_dims, spatial_std, feature_std, &features);
     return rc == PL_OK ? build_lattice(h, features) : rc;
+}
+
+int pl_build_begin(pl_handle h, const float *positions) {
+    if (!h || (!positions && h->N > 0)) return PL_EINVAL;
+    if (h->f64) return PL_EINVAL;   // a lattice of doubles: use the *_f64 entry points
+    if (h->pending.active) return PL_ESTATE;
+    const int rc = guess_point_grid(h, positions);
+    if (rc != PL_OK) return rc;
+    return build_begin(h, features_from_positions(positions));
+}
+
+int pl_build_image_begin(pl_handle h, const float *reference, int n_reference_channels,
+                         int n_spatial_dims, const int *spatial_dims, float spatial_std,
+                         float feature_std) {
+    if (!h) return PL_EINVAL;
+    if (h->f64) return PL_EINVAL;   // a lattice of doubles: use the *_f64 entry points
+    if (h->pending.active) return PL_ESTATE;
+    plk::PointFeatures features;
+    const int rc = features_from_image(h, reference, n_reference_channels, n_spatial_dims,
+                                       spatial_dims, spatial_std, feature_std, &features);
+    return rc == PL_OK ? build_begin(h, features) : rc;
+}
+
+int pl_build_end(pl_handle h) {
+    if (!h) return PL_EINVAL;
+    return build_end(h);
 }
 
 int pl_apply(pl_handle h, float *output, const float *input, int reverse) {

@@ -87,6 +87,57 @@ def test_end_repeats_the_call_when_the_table_was_too_small():
     close(out.cpu().numpy(), want)
 
 
+def test_several_lattices_built_side_by_side_then_applied():
+    """pl_build_begin / pl_build_image_begin on lattices with streams of their own, then
+    pl_build_end on each: applies give what filter gives (the oracle), also for a table that had to
+    grow in between, and with or without the per-vertex lists."""
+    h = w = 96
+    n = h * w
+    cases = []
+    for seed, reverse, image, lists in ((51, False, False, 1), (52, True, True, 1), (53, False, True, 0),
+                                        (54, True, False, 0)):
+        img = synth.blob_image(h, w, seed=seed)
+        pos = synth.bilateral_positions(img, 6.0, 0.1)
+        val = synth.uniform_image((n, 3), seed + 100)
+        cases.append((img, pos, val, reverse, image, lists,
+                      oracle.Lattice(5, 4, n).filter(val, pos, reverse)))
+    streams = [torch.cuda.Stream() for _ in cases]
+    lattices, keep = [], []
+    torch.cuda.synchronize()
+    for k, ((img, pos, val, reverse, image, lists, _), s) in enumerate(zip(cases, streams)):
+        lat = pla.PermutohedralLattice(5, 4, n, stream=s)
+        lat.set_option(pla.PL_OPT_VERTEX_LISTS, lists)
+        if k == 1:
+            lat.set_option(pla.PL_OPT_TABLE_CELLS, 2048)       # too small: build_end repeats the build
+        d_val = dev(val)
+        d_img, d_pos = dev(img.reshape(n, 3)), dev(pos)
+        torch.cuda.synchronize()          # the uploads ran on the current stream
+        if image:
+            lat.build_image_begin(d_img, (h, w), 6.0, 0.1)
+        else:
+            lat.set_point_grid((h, w))
+            lat.build_begin(d_pos)
+        lattices.append(lat)
+        keep.append((d_val, d_img, d_pos))
+    with pytest.raises(pla.PermutohedralError) as e:
+        lattices[0].filter_end()           # a build is in flight, not a filter
+    assert e.value.status == pla.PL_ESTATE
+    with pytest.raises(pla.PermutohedralError) as e:
+        lattices[0].apply(torch.empty((n, 3), device="cuda"), keep[0][0])
+    assert e.value.status == pla.PL_ESTATE
+    for lat in lattices:
+        lat.build_end()
+    lattices[0].build_end()                # nothing in flight: fine
+    for lat, (d_val, _, _), (_, _, _, reverse, _, _, want) in zip(lattices, keep, cases):
+        out = torch.empty((n, 3), dtype=torch.float32, device="cuda")
+        lat.apply(out, d_val, reverse)
+        torch.cuda.synchronize()
+        close(out.cpu().numpy(), want)
+        lat.apply(out, d_val, reverse)     # and again
+        torch.cuda.synchronize()
+        close(out.cpu().numpy(), want)
+
+
 @pytest.mark.parametrize("batch", [1, 3, 6])
 def test_op_results_do_not_depend_on_the_number_of_items_in_flight(batch):
     h, w = 72, 88
