@@ -333,6 +333,8 @@ int ensure_vertex_lists(pl_lattice *h) {
     if (!l.start || !l.entries || !l.count || !l.places || !l.block_sums || !l.chunks.chunk_start ||
         !l.chunks.chunk || !l.chunks.long_lists || !l.chunks.partial_rows)
         return PL_ENOMEM;
+    // (the counts start at zero and every build leaves them so)
+    PL_HIP(plk::fill_zero(reinterpret_cast<float *>(l.count), mv + 2, h->stream));
     l.chunks.info = l.count + mv;
     l.chunks.max_chunks = (unsigned)max_chunks;
     l.chunks.max_long = (unsigned)max_long;

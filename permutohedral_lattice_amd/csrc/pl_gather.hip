@@ -176,41 +176,37 @@ __global__ __launch_bounds__(kBlock) void k_scan_block_sums(const unsigned *__re
     if (threadIdx.x == 0) block_sums[blockIdx.x] = total;
 }
 
-// block_sums[0 .. n_blocks) := their exclusive prefix sums, block_sums[n_blocks] := the totals
-__global__ __launch_bounds__(kBlock) void k_scan_of_block_sums(uint2 *block_sums, unsigned n_blocks) {
-    uint2 carry = make_uint2(0u, 0u);
-    for (unsigned first = 0; first < n_blocks; first += kBlock) {
-        const unsigned i = first + threadIdx.x;
-        const uint2 x = i < n_blocks ? block_sums[i] : make_uint2(0u, 0u);
-        uint2 total;
-        const uint2 before = block_exclusive_scan(x, &total);
-        if (i < n_blocks) block_sums[i] = make_uint2(carry.x + before.x, carry.y + before.y);
-        carry.x += total.x;
-        carry.y += total.y;
-    }
-    if (threadIdx.x == 0) block_sums[n_blocks] = carry;
-}
-
-__global__ __launch_bounds__(kBlock) void k_scan_starts(const unsigned *__restrict__ count, unsigned n,
+// Every workgroup adds up the sums of the blocks before its own (a few hundred pairs: cheaper than
+// a launch that scans them), scans its block from there, and writes per vertex the start of its
+// list and of its chunks and the descriptor of its first chunk; a list of several chunks is also
+// recorded in long_lists (the workgroup's long lists take one run of places there, drawn with one
+// atomic: an atomic per list would queue up on the one counter).  The counts are left at
+// zero, as the next build's k_list_places must find them.
+__global__ __launch_bounds__(kBlock) void k_scan_starts(unsigned *count, unsigned n,
                                                          const uint2 *__restrict__ block_sums,
                                                          unsigned *start, ListChunks chunks) {
     const size_t first = (size_t)blockIdx.x * kScanItems + (size_t)threadIdx.x * kScanPerThread;
     unsigned c[kScanPerThread];
     load_counts(count, first, n, c);
-    uint2 sum = make_uint2(0u, 0u);
-#pragma unroll
-    for (int i = 0; i < kScanPerThread; ++i) {
-        sum.x += c[i];
-        sum.y += chunks_of(c[i], chunks.rows);
+    uint2 before_block = make_uint2(0u, 0u);
+    for (unsigned i = threadIdx.x; i < blockIdx.x; i += kBlock) {
+        const uint2 s = block_sums[i];
+        before_block.x += s.x;
+        before_block.y += s.y;
     }
-    uint2 total;
-    const uint2 base = block_sums[blockIdx.x];
-    const uint2 before = block_exclusive_scan(sum, &total);
-    // the workgroup's long lists take one run of places in long_lists, drawn with one atomic
-    // (an atomic per list would queue up on the one counter)
+    uint2 base;
+    (void)block_exclusive_scan(before_block, &base);
+    uint2 sum = make_uint2(0u, 0u);
     unsigned long_here = 0;
 #pragma unroll
-    for (int i = 0; i < kScanPerThread; ++i) long_here += chunks_of(c[i], chunks.rows) > 1u ? 1u : 0u;
+    for (int i = 0; i < kScanPerThread; ++i) {
+        const unsigned of_v = chunks_of(c[i], chunks.rows);
+        sum.x += c[i];
+        sum.y += of_v;
+        long_here += of_v > 1u ? 1u : 0u;
+    }
+    uint2 total;
+    const uint2 before = block_exclusive_scan(sum, &total);
     uint2 long_total;
     const uint2 long_before = block_exclusive_scan(make_uint2(long_here, 0u), &long_total);
     __shared__ unsigned long_base;
@@ -224,6 +220,7 @@ __global__ __launch_bounds__(kBlock) void k_scan_starts(const unsigned *__restri
             const unsigned v = (unsigned)(first + i);
             start[v] = entry;
             chunks.chunk_start[v] = chunk;
+            if (c[i]) count[v] = 0u;
             const unsigned of_v = chunks_of(c[i], chunks.rows);
             if (of_v == 1u && chunk < chunks.max_chunks) {
                 chunks.chunk[chunk] = ListChunk{entry, entry + c[i], v, 1u};
@@ -231,36 +228,20 @@ __global__ __launch_bounds__(kBlock) void k_scan_starts(const unsigned *__restri
                 if (long_at < chunks.max_long)
                     chunks.long_lists[long_at] = LongList{v, chunk, entry, entry + c[i]};
                 long_at += 1u;
+                // (its first chunk; the others are described by the rows that open them, in
+                // k_list_fill)
+                if (chunk < chunks.max_chunks)
+                    chunks.chunk[chunk] = ListChunk{entry, entry + chunks.rows, v, 0u};
             }
             entry += c[i];
             chunk += of_v;
         }
     }
     if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 0) {
-        const uint2 all = block_sums[gridDim.x];
+        const uint2 all = make_uint2(base.x + total.x, base.y + total.y);
         start[n] = all.x;
         chunks.chunk_start[n] = all.y;
         chunks.info[1] = all.y < chunks.max_chunks ? all.y : chunks.max_chunks;
-    }
-}
-
-// The chunks of the lists that have several: a workgroup per list, a thread per chunk.
-__global__ __launch_bounds__(kBlock) void k_long_list_chunks(ListChunks chunks, unsigned *host_info) {
-    const unsigned n_long = chunks.info[0] < chunks.max_long ? chunks.info[0] : chunks.max_long;
-    if (host_info && blockIdx.x == 0 && threadIdx.x == 0) {
-        host_info[0] = chunks.info[0];
-        host_info[1] = chunks.info[1];
-    }
-    for (unsigned i = blockIdx.x; i < n_long; i += gridDim.x) {
-        const LongList list = chunks.long_lists[i];
-        const unsigned v = list.vertex, from = list.chunk_from;
-        const unsigned list_from = list.from, list_to = list.to;
-        const unsigned to = from + chunks_of(list_to - list_from, chunks.rows);
-        for (unsigned c = from + threadIdx.x; c < to && c < chunks.max_chunks; c += kBlock) {
-            const unsigned first = list_from + (c - from) * chunks.rows;
-            const unsigned last = list_to - first < chunks.rows ? list_to : first + chunks.rows;
-            chunks.chunk[c] = ListChunk{first, last, v, 0u};
-        }
     }
 }
 
@@ -273,7 +254,14 @@ __global__ __launch_bounds__(kBlock) void k_list_fill(PointMap map,
                                                        const unsigned *__restrict__ places,
                                                        const unsigned *__restrict__ start,
                                                        ListEntry *entries, int max_vertices,
-                                                       size_t capacity) {
+                                                       size_t capacity, ListChunks chunks,
+                                                       unsigned *host_info) {
+    // (the last launch of the pass: how many lists have several chunks, and the chunks in all, for
+    // the host, which sizes every apply's launches by them)
+    if (host_info && blockIdx.x == 0 && threadIdx.x == 0) {
+        host_info[0] = chunks.info[0];
+        host_info[1] = chunks.info[1];
+    }
     unsigned vblock;
     if (!block_of_points(map, 1, vblock)) return;
     const size_t t = (size_t)vblock * kBlock + threadIdx.x;
@@ -293,8 +281,17 @@ __global__ __launch_bounds__(kBlock) void k_list_fill(PointMap map,
 #pragma unroll
     for (int r = 0; r < D1; ++r) {
         const size_t at = (size_t)first[r] + place[r];
-        if ((unsigned)e[r].index < (unsigned)max_vertices && at < capacity)
+        if ((unsigned)e[r].index < (unsigned)max_vertices && at < capacity) {
             entries[at] = ListEntry{n, e[r].weight};
+            // the row that opens a further chunk of its list describes that chunk
+            if (place[r] != 0u && (place[r] & (chunks.rows - 1u)) == 0u) {
+                const unsigned v = (unsigned)e[r].index;
+                const unsigned c = chunks.chunk_start[v] + (place[r] >> __builtin_ctz(chunks.rows));
+                const unsigned from = (unsigned)at, end = start[v + 1u];
+                if (c < chunks.max_chunks)
+                    chunks.chunk[c] = ListChunk{from, end - from < chunks.rows ? end : from + chunks.rows, v, 0u};
+            }
+        }
     }
 }
 
@@ -521,34 +518,21 @@ size_t vertex_list_max_long(size_t rows) { return rows / 128 + 1; }
 hipError_t build_vertex_lists(int pd, const PointMap &map, ReplayEntry *replay, const int *cell_vertex,
                               int max_vertices, const VertexLists &lists, unsigned *host_info,
                               hipStream_t s) {
-    if (max_vertices <= 0) return hipSuccess;
-    hipError_t err = fill_zero(reinterpret_cast<float *>(lists.count), (size_t)max_vertices, s);
-    if (err != hipSuccess) return err;
-    const dim3 block(kBlock);
-    if (map.n_blocks) {
-        const dim3 grid(map.n_blocks);
-        PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_list_places<PD + 1>), grid, block, 0, s, map, replay,
-                                               cell_vertex, lists.count, lists.places, max_vertices));
-    }
+    if (max_vertices <= 0 || map.n_blocks == 0) return hipSuccess;
+    // (lists.count is all zeros: filled so when it was allocated, left so by every k_scan_starts)
+    const dim3 block(kBlock), grid(map.n_blocks);
+    PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_list_places<PD + 1>), grid, block, 0, s, map, replay,
+                                           cell_vertex, lists.count, lists.places, max_vertices));
     const unsigned n = (unsigned)max_vertices;
     const unsigned scan_blocks = (unsigned)vertex_list_scan_blocks(max_vertices);
     uint2 *block_sums = reinterpret_cast<uint2 *>(lists.block_sums);
     hipLaunchKernelGGL(k_scan_block_sums, dim3(scan_blocks), block, 0, s, lists.count, n, block_sums,
                        lists.chunks.info, lists.chunks.rows);
-    hipLaunchKernelGGL(k_scan_of_block_sums, dim3(1), block, 0, s, block_sums, scan_blocks);
     hipLaunchKernelGGL(k_scan_starts, dim3(scan_blocks), block, 0, s, lists.count, n, block_sums,
                        lists.start, lists.chunks);
-    // (how many lists have several chunks is known on the device only: a grid that covers a
-    // usual number of them, the workgroups walk the rest)
-    const unsigned long_blocks = lists.chunks.max_long < 256u ? lists.chunks.max_long : 256u;
-    hipLaunchKernelGGL(k_long_list_chunks, dim3(long_blocks ? long_blocks : 1u), block, 0, s,
-                       lists.chunks, host_info);
-    if (map.n_blocks) {
-        const dim3 grid(map.n_blocks);
-        PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_list_fill<PD + 1>), grid, block, 0, s, map, replay,
-                                               lists.places, lists.start, lists.entries, max_vertices,
-                                               lists.capacity));
-    }
+    PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_list_fill<PD + 1>), grid, block, 0, s, map, replay,
+                                           lists.places, lists.start, lists.entries, max_vertices,
+                                           lists.capacity, lists.chunks, host_info));
     return hipGetLastError();
 }
 
