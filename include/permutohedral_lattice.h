@@ -80,7 +80,8 @@ typedef enum pl_option {
                                float additions; for measuring the difference).  Float lattices. */
     PL_OPT_NUMBER_SEGMENTS = 11, /* 0 (default): a build that numbers its vertices itself draws the numbers
                                from 8 counters (one per eighth of the image), or from 64 when it has more
-                               than 8192 workgroups; 8 or 64: always that many, table size permitting
+                               than 8192 workgroups; 8 or 64: always that many, table size permitting;
+                               -1: no build numbers its vertices itself, the numbering pass runs
                                (same results; for tests and measurements) */
     PL_OPT_ORDER_POINTS = 9 /* 1 (default): points that are a plain list (no grid given or found, at
                                least 4096 of them) are worked on in an order in which neighbours in

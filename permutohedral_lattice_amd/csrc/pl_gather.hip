@@ -12,8 +12,9 @@
 //
 // Lists differ in length by orders of magnitude (a wide kernel over a flat part of an image gives
 // one vertex ten thousand rows while most have twenty), so the unit of work is a chunk of at most
-// kListChunk rows of one list: a list of one chunk is summed straight into the value table, the
-// chunks of a longer list into partial rows that a second, small launch adds up.
+// ListChunks::rows rows of one list (list_chunk_rows): a list of one chunk is summed straight into
+// the value table, the chunks of a longer list into partial rows that a second, small launch adds
+// up.
 //
 // This translation unit needs no -ffp-contract=off (nothing here decides an integer), but is
 // compiled with the same flags as the others.
@@ -93,12 +94,12 @@ __global__ __launch_bounds__(kBlock) void k_list_places(PointMap map, ReplayEntr
 // ------------------------------------------------------------------------------------------------
 // Lists, step 2: where every vertex's list starts, and where its chunks start: exclusive prefix
 // sums over all n vertex numbers of the table (numbers without a vertex count zero) of the counts
-// and of the chunks the counts make, both in one pass of three launches: sums of blocks of
-// kScanItems items; a scan of those by one workgroup; the scan inside each block from its start.
-// The last launch also describes the chunk of every list that has one chunk and names the lists
-// that have several (workgroup by workgroup in the order the atomics give; each of those is
-// summed on its own), whose
-// chunks a small launch describes.  start[n], chunk_start[n]: the totals.
+// and of the chunks the counts make, both in one pass of two launches: sums of blocks of
+// kScanItems items; then the scan inside each block, every workgroup adding up the sums of the
+// blocks before its own.  The second launch also describes the first chunk of every list and
+// names the lists that have several (workgroup by workgroup in the order the atomics give; each
+// of those is summed on its own); their further chunks are described in step 3.  start[n],
+// chunk_start[n]: the totals.
 // ------------------------------------------------------------------------------------------------
 constexpr int kScanPerThread = 8;
 constexpr int kScanItems = kBlock * kScanPerThread;
