@@ -46,6 +46,17 @@ CASES = [
     ("spatial_pd2_vd2", 2, 2, (128, 128)),
     ("crf_pd5_vd70", 5, 70, (24, 24)),
     ("crf_pd5_vd9", 5, 9, (32, 40)),
+    # every width of the four-channels-per-lane kernels and their edges: 4 lanes (5..16 channels),
+    # 8 (17..32), 16 (33..64), more than 64; input rows of a multiple of four floats and not
+    ("crf_pd5_vd5", 5, 5, (32, 32)),
+    ("crf_pd3_vd13", 3, 13, (40, 24)),
+    ("crf_pd5_vd16", 5, 16, (24, 24)),
+    ("crf_pd5_vd17", 5, 17, (24, 24)),
+    ("spatial_pd2_vd32", 2, 32, (32, 32)),
+    ("spatial_pd2_vd33", 2, 33, (32, 32)),
+    ("crf_pd5_vd48", 5, 48, (24, 24)),
+    ("spatial_pd2_vd64", 2, 64, (24, 24)),
+    ("spatial_pd2_vd65", 2, 65, (24, 24)),
 ]
 
 
@@ -54,6 +65,8 @@ def _inputs(name, pd, vd, shape):
     rng = np.random.default_rng(zlib.crc32(name.encode()) % 1000)
     if pd == 2:
         pos = synth.spatial_positions(shape, 3.0)
+    elif pd == 3:
+        pos = synth.bilateral_positions(synth.blob_image(h, w, seed=7)[..., :1] * 255.0, 20.0, 13.0)
     elif vd > 4:
         pos = synth.bilateral_positions(synth.blob_image(h, w, seed=7) * 255.0, 80.0, 13.0)
     else:
@@ -75,6 +88,35 @@ def test_apply_from_vertex_lists_matches_oracle_and_atomic_splat(name, pd, vd, s
     assert np.isfinite(got).all()
     assert np.abs(got - want).max() <= MAX_ABS_TOL and rel_l2(got, want) <= REL_L2_TOL
     assert np.abs(got - plain).max() <= 1e-5
+
+
+@pytest.mark.parametrize("pd,vd,shape", [(5, 22, (48, 48)), (2, 13, (40, 40)), (5, 4, (64, 48)),
+                                         (2, 36, (24, 24)), (5, 8, (32, 32))])
+def test_apply_without_normalisation_takes_input_rows_of_vd_channels(pd, vd, shape):
+    """PL_OPT_NORMALIZE = 0: the input carries all vd channels and the output is the bare sum
+    (the gathers and the slice then read and write rows of vd floats, not vd - 1)."""
+    h, w = shape
+    n = h * w
+    rng = np.random.default_rng(vd)
+    pos = (synth.spatial_positions(shape, 3.0) if pd == 2 else
+           synth.bilateral_positions(synth.blob_image(h, w, seed=3) * 255.0, 60.0, 13.0))
+    val = rng.uniform(0, 1, (n, vd)).astype(np.float32)
+    outs = []
+    for lists in (1, 0):
+        lat = pla.PermutohedralLattice(pd, vd, n)
+        lat.set_option(pla.PL_OPT_VERTEX_LISTS, lists)
+        lat.set_option(pla.PL_OPT_NORMALIZE, 0)
+        lat.set_point_grid(shape)
+        lat.build(_dev(pos))
+        out = torch.full((n, vd), float("nan"), dtype=torch.float32, device="cuda")
+        lat.apply(out, _dev(val), False)
+        torch.cuda.synchronize()
+        outs.append(out.cpu().numpy())
+    want = oracle.Lattice(pd, vd, n).filter_raw(val, pos, False)
+    scale = max(1.0, np.abs(want).max())
+    assert np.isfinite(outs[0]).all()
+    assert np.abs(outs[0] - want).max() <= MAX_ABS_TOL * scale and rel_l2(outs[0], want) <= REL_L2_TOL
+    assert np.abs(outs[0] - outs[1]).max() <= 1e-5 * scale
 
 
 def test_vertex_values_after_the_gathering_splat():
