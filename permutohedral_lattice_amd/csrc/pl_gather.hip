@@ -395,7 +395,7 @@ __global__ __launch_bounds__(kBlock) void k_splat_gather(ListChunks chunks, unsi
 // row's last four instead (no load leaves the row) and its sums are shifted back at the end.  The
 // lanes first read the whole chunk's entries, kChannelChunk / L each, and hand them round.
 // Channels past the input are the homogeneous one: the sum of the bare weights.
-constexpr int kChannelChunk = 128;   // rows of a chunk at most (list_chunk_rows for vd > 4)
+constexpr int kChannelChunk = (int)kListChunkManyChannels;   // rows of a chunk at most (vd > 4)
 
 
 struct alignas(4) FourFloats {
@@ -512,9 +512,10 @@ size_t vertex_list_scan_blocks(int max_vertices) {
     return ((size_t)max_vertices + kScanItems - 1) / kScanItems;
 }
 size_t vertex_list_max_chunks(int max_vertices, size_t rows) {
-    return (size_t)max_vertices + rows / 128 + 1;
+    // (every vertex's list ends in a chunk that may be short; the rest are full ones)
+    return (size_t)max_vertices + rows / kListChunkManyChannels + 1;
 }
-size_t vertex_list_max_long(size_t rows) { return rows / 128 + 1; }
+size_t vertex_list_max_long(size_t rows) { return rows / kListChunkManyChannels + 1; }
 
 hipError_t build_vertex_lists(int pd, const PointMap &map, ReplayEntry *replay, const int *cell_vertex,
                               int max_vertices, const VertexLists &lists, unsigned *host_info,

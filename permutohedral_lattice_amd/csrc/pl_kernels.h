@@ -280,8 +280,8 @@ hipError_t splat(int pd, int vd, const PointMap &map, const float *input, int in
 // long_lists.  info: {long lists, chunks in all}.
 // (a chunk of 256 rows for rows of up to four values, where no list of an image like the
 // benchmark's is longer; 128 for rows of many channels, whose chunks cost more per row)
-constexpr int kMaxListChunk = 256;
-inline unsigned list_chunk_rows(int vd) { return vd <= 4 ? 256u : 128u; }
+constexpr unsigned kListChunkFewChannels = 256, kListChunkManyChannels = 128;
+inline unsigned list_chunk_rows(int vd) { return vd <= 4 ? kListChunkFewChannels : kListChunkManyChannels; }
 struct ListEntry {
     int point;
     float weight;
