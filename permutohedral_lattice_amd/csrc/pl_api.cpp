@@ -9,6 +9,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
+#include <chrono>
 #include <cmath>
 #include <cstdint>
 #include <cstring>
@@ -125,7 +127,7 @@ struct pl_lattice {
     plk::Counters *d_counters = nullptr;   // two sets, used by alternate builds
     int counter_set = 0;                   // the set of the last build
     plk::HostStatus *h_status = nullptr;   // pinned, written by the device
-    hipEvent_t status_written = nullptr;   // recorded behind the kernel that writes h_status
+    unsigned status_sequence = 0;          // the number of the last build enqueued: what its report carries
     // a lattice in the library's static scratch (pl_filter_static) owns no pinned memory and no
     // event: h_status is device memory there, copied to the host when the build is verified
     bool status_on_device = false;
@@ -460,6 +462,9 @@ int enqueue_build(pl_lattice *h, const plk::PointFeatures &features, const doubl
                               h->stream));
         h->cell_values_clean = true;
     }
+    // (what this build's report will carry; never 0, which is what a fresh status holds)
+    h->status_sequence = h->status_sequence + 1u ? h->status_sequence + 1u : 1u;
+    const plk::HostReport report_to{h->h_status, h->status_sequence};
     h->mark(EV_T0);
     h->stage_ran[0] = h->map.mode == 1 || !h->table_clean || cells != h->n_cells;
     h->stage_ran[1] = true;
@@ -530,9 +535,8 @@ int enqueue_build(pl_lattice *h, const plk::PointFeatures &features, const doubl
                                     (unsigned)h->n_chunks, vertices,
                                     h->values[0], h->f64 ? 2 * h->vd : h->vd,
                                     fused ? h->cell_values : nullptr, h->counters(),
-                                    h->d_counters + previous_set, h->h_status, wide, h->stream));
+                                    h->d_counters + previous_set, report_to, wide, h->stream));
     }
-    if (!numbers_in_build && !h->status_on_device) PL_HIP(hipEventRecord(h->status_written, h->stream));
     h->mark(EV_IDS);
     // (the rows a build that numbered its vertices listed for vertices of other workgroups join
     // the value table here, and its counts reach the host from here)
@@ -540,8 +544,7 @@ int enqueue_build(pl_lattice *h, const plk::PointFeatures &features, const doubl
                            h->launch_vertices(), numbers_in_build && fused ? &lists : nullptr,
                            h->map.n_blocks, h->values[0], h->vd, h->f64,
                            numbers_in_build ? h->counters() : nullptr,
-                           h->d_counters + previous_set, h->h_status, wide, h->stream));
-    if (numbers_in_build && !h->status_on_device) PL_HIP(hipEventRecord(h->status_written, h->stream));
+                           h->d_counters + previous_set, report_to, wide, h->stream));
     h->mark(EV_NBR);
     h->replay_holds_cells = true;
     h->values_zeroed = !fused;
@@ -711,7 +714,22 @@ int verify_build(pl_lattice *h, uint32_t *retry_cells) {
         PL_HIP(hipMemcpyAsync(&status, h->h_status, sizeof(status), hipMemcpyDeviceToHost, h->stream));
         PL_HIP(hipStreamSynchronize(h->stream));
     } else {
-        PL_HIP(hipEventSynchronize(h->status_written));
+        // The kernel that reports writes the build's number last, behind a system-wide fence, into
+        // pinned memory: the host polls that word.  (An event recorded between the reporting
+        // kernel and the blur kept the blur from starting for 6 us, and the host learned of the
+        // build only when the reporting kernel had ended; now it knows when that kernel starts.)
+        // Should the word never come -- a launch that failed -- the wait for the stream says why.
+        const volatile unsigned *word = &h->h_status->sequence;
+        const auto started = std::chrono::steady_clock::now();
+        for (unsigned spins = 1; *word != h->status_sequence; ++spins) {
+            if ((spins & 0xfffu) == 0 &&
+                std::chrono::steady_clock::now() - started > std::chrono::seconds(2)) {
+                PL_HIP(hipStreamSynchronize(h->stream));
+                if (*word != h->status_sequence) return PL_EHIP;
+                break;
+            }
+        }
+        std::atomic_thread_fence(std::memory_order_acquire);
         status = *h->h_status;
     }
     const int flags = status.flags;
@@ -861,9 +879,7 @@ static int create_lattice(int pd, int vd, int N, bool f64, pl_stream stream, con
         rc = PL_EHIP;
     if (rc == PL_OK &&
         hip_failed(hipHostMalloc((void **)&h->h_status, sizeof(plk::HostStatus) + 2 * sizeof(unsigned),
-                                 hipHostMallocDefault)))
-        rc = PL_EHIP;
-    if (rc == PL_OK && hip_failed(hipEventCreateWithFlags(&h->status_written, hipEventDisableTiming)))
+                                 hipHostMallocCoherent)))
         rc = PL_EHIP;
     if (rc != PL_OK) {
         pl_destroy(h);
@@ -871,6 +887,7 @@ static int create_lattice(int pd, int vd, int N, bool f64, pl_stream stream, con
     }
     h->h_status->num_vertices = 0;
     h->h_status->flags = 0;
+    h->h_status->sequence = 0;
     *out = h;
     return PL_OK;
 }
@@ -905,7 +922,6 @@ int pl_destroy(pl_handle h) {
     h->dfree(h->locality_words);
     h->dfree(h->bin_rank);
     if (h->h_status) (void)hipHostFree(h->h_status);
-    if (h->status_written) (void)hipEventDestroy(h->status_written);
     for (int i = 0; i < EV_COUNT; ++i)
         if (h->ev[i]) (void)hipEventDestroy(h->ev[i]);
     delete h;

@@ -72,6 +72,16 @@ struct HostStatus {
     int max_segment;   // vertices in the fullest segment (num_vertices when there are none)
     int n_segments;
     int foreign_rows;  // CreatedLists rows of a build that numbered its vertices (an estimate)
+    // written last, behind a system-wide fence: the number of the build the fields above belong
+    // to.  The host, which holds the struct in pinned memory, polls this word instead of waiting
+    // for an event behind the kernel (an event between two kernels of a stream keeps the second
+    // from starting for some microseconds).
+    unsigned sequence;
+};
+// Where a build reports to, and as which build.
+struct HostReport {
+    HostStatus *status;
+    unsigned sequence;
 };
 
 // Per-vertex and per-cell tables of a lattice (all sized by the hash table): vertex v has key
@@ -243,7 +253,7 @@ hipError_t build_f64(int pd, const Points64 &points, const PointMap &map, uint64
 hipError_t number_vertices(int pd, const PointMap &map, const CreatedLists &lists,
                            int *next_chunk_count, unsigned n_chunks, const VertexTables &vertices,
                            float *values, int vd, float *cell_values, Counters *counters, Counters *next_counters,
-                           HostStatus *host_status, bool wide_keys, hipStream_t s);
+                           HostReport host_report, bool wide_keys, hipStream_t s);
 
 // neighbours[a*max_vertices+v] := vertex indices of v's two neighbours along blur axis a, for v
 // below the vertex count; entries of absent neighbours keep their -1.
@@ -260,7 +270,7 @@ hipError_t neighbours(int pd, const VertexTables &vertices, const Counters *coun
                       const uint64_t *cell_keys, uint32_t n_cells, int launch_vertices,
                       const CreatedLists *foreign_rows, unsigned n_lists, void *values, int vd,
                       bool values_are_double, Counters *report, Counters *next_counters,
-                      HostStatus *host_status, bool wide_keys, hipStream_t s);
+                      HostReport host_report, bool wide_keys, hipStream_t s);
 
 hipError_t fill_zero(float *p, size_t n, hipStream_t s);
 

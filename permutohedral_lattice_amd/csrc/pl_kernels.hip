@@ -882,7 +882,8 @@ __global__ __launch_bounds__(64) void k_number_vertices(CreatedLists lists, int 
                                                         VertexTables vertices, float *values, int vd,
                                                         float *cell_values, Counters *counters,
                                                         Counters *next_counters,
-                                                        HostStatus *host_status) {
+                                                        HostReport host_report) {
+    HostStatus *host_status = host_report.status;
     // (an XCD takes the lists of one contiguous range of tiles: their cells are in its part of the
     // table and their vertex numbers in one range)
     const unsigned b = xcd_contiguous_block(blockIdx.x, gridDim.x, 1);
@@ -925,6 +926,9 @@ __global__ __launch_bounds__(64) void k_number_vertices(CreatedLists lists, int 
             host_status->max_segment = (int)m;
             host_status->n_segments = 0;
             host_status->foreign_rows = 0;
+            __threadfence_system();
+            __hip_atomic_store(&host_status->sequence, host_report.sequence, __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_SYSTEM);
             reset_counters(next_counters);
         }
         for (unsigned i = lane; i < n_chunks; i += 64) next_chunk_count[i] = 0;
@@ -1016,8 +1020,9 @@ __global__ __launch_bounds__(kBlock) void k_neighbours(VertexTables vertices,
                                                         CreatedLists lists, unsigned n_lists,
                                                         void *values, int vd, int values_are_double,
                                                         Counters *report, Counters *next_counters,
-                                                        HostStatus *host_status) {
+                                                        HostReport host_report) {
     constexpr int D1 = PD + 1;
+    HostStatus *host_status = host_report.status;
     // After a merging build nothing has told the host yet how the build went: the segments' counts
     // are summed here, and what the next build will count in is cleared.
     // (by the first wavefront of the first workgroup that looks up neighbours, which starts with
@@ -1040,6 +1045,9 @@ __global__ __launch_bounds__(kBlock) void k_neighbours(VertexTables vertices,
             host_status->max_segment = (int)fullest;
             host_status->n_segments = n_segments;
             host_status->foreign_rows = (int)(report->foreign_rows_sampled.n * kForeignSampling);
+            __threadfence_system();
+            __hip_atomic_store(&host_status->sequence, host_report.sequence, __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_SYSTEM);
             reset_counters(next_counters);
         }
     }
@@ -2156,18 +2164,18 @@ hipError_t number_vertices(int pd, const PointMap &map, const CreatedLists &list
                            int *next_chunk_count, unsigned n_chunks, const VertexTables &vertices,
                            float *values,
                            int vd, float *cell_values, Counters *counters, Counters *next_counters,
-                           HostStatus *host_status, bool wide_keys, hipStream_t s) {
+                           HostReport host_report, bool wide_keys, hipStream_t s) {
     if (map.n_blocks == 0) return hipErrorInvalidValue;
     if (wide_keys) {
         PLK_DISPATCH_WIDE_PD(pd, hipLaunchKernelGGL((k_number_vertices<PD + 1, true>), dim3(map.n_blocks),
                                                dim3(64), 0, s, lists, next_chunk_count, n_chunks,
                                                vertices, values, vd, cell_values, counters,
-                                               next_counters, host_status));
+                                               next_counters, host_report));
     } else {
         PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_number_vertices<PD + 1>), dim3(map.n_blocks),
                                                dim3(64), 0, s, lists, next_chunk_count, n_chunks,
                                                vertices, values, vd, cell_values, counters,
-                                               next_counters, host_status));
+                                               next_counters, host_report));
     }
     return hipGetLastError();
 }
@@ -2176,7 +2184,7 @@ hipError_t neighbours(int pd, const VertexTables &vertices, const Counters *coun
                       const uint64_t *cell_keys, uint32_t n_cells, int launch_vertices,
                       const CreatedLists *foreign_rows, unsigned n_lists, void *values, int vd,
                       bool values_are_double, Counters *report, Counters *next_counters,
-                      HostStatus *host_status, bool wide_keys, hipStream_t s) {
+                      HostReport host_report, bool wide_keys, hipStream_t s) {
     if (vertices.max_vertices <= 0) return hipErrorInvalidValue;
     const size_t items = (size_t)(pd + 1) * (size_t)launch_vertices;
     const unsigned foreign_blocks =
@@ -2188,7 +2196,7 @@ hipError_t neighbours(int pd, const VertexTables &vertices, const Counters *coun
                                            n_cells - 1u, foreign_blocks,                           \
                                            foreign_rows ? *foreign_rows : CreatedLists{}, n_lists, \
                                            values, vd, values_are_double ? 1 : 0, report,          \
-                                           next_counters, host_status))
+                                           next_counters, host_report))
     if (wide_keys) {
         PLK_NEIGHBOURS(true, PLK_DISPATCH_WIDE_PD);
     } else {
