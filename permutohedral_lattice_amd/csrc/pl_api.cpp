@@ -707,6 +707,25 @@ int enqueue_apply(pl_lattice *h, void *output_any, const void *input_any, int re
 // whether the table was large enough while the blur and the slice still run, and the caller's next
 // call is enqueued behind them without a gap).  PL_OK: it fitted, h->M is valid.
 // Otherwise *retry_cells is the table size to try next (0: give up with the returned status).
+// The kernels that report to the host write the number of the build they belong to last, behind a
+// system-wide fence, into pinned memory, and the host polls that word.  (An event recorded between
+// the reporting kernel and the next kept the next from starting for 6 us, and the host learned
+// of the report only when the reporting kernel had ended; now it knows when that kernel starts.)
+// Should the word never come -- a launch that failed -- the wait for the stream says why.
+int wait_for_report(pl_lattice *h, const volatile unsigned *word) {
+    const auto started = std::chrono::steady_clock::now();
+    for (unsigned spins = 1; *word != h->status_sequence; ++spins) {
+        if ((spins & 0xfffu) == 0 &&
+            std::chrono::steady_clock::now() - started > std::chrono::seconds(2)) {
+            PL_HIP(hipStreamSynchronize(h->stream));
+            if (*word != h->status_sequence) return PL_EHIP;
+            break;
+        }
+    }
+    std::atomic_thread_fence(std::memory_order_acquire);
+    return PL_OK;
+}
+
 int verify_build(pl_lattice *h, uint32_t *retry_cells) {
     *retry_cells = 0;
     plk::HostStatus status;
@@ -714,22 +733,8 @@ int verify_build(pl_lattice *h, uint32_t *retry_cells) {
         PL_HIP(hipMemcpyAsync(&status, h->h_status, sizeof(status), hipMemcpyDeviceToHost, h->stream));
         PL_HIP(hipStreamSynchronize(h->stream));
     } else {
-        // The kernel that reports writes the build's number last, behind a system-wide fence, into
-        // pinned memory: the host polls that word.  (An event recorded between the reporting
-        // kernel and the blur kept the blur from starting for 6 us, and the host learned of the
-        // build only when the reporting kernel had ended; now it knows when that kernel starts.)
-        // Should the word never come -- a launch that failed -- the wait for the stream says why.
-        const volatile unsigned *word = &h->h_status->sequence;
-        const auto started = std::chrono::steady_clock::now();
-        for (unsigned spins = 1; *word != h->status_sequence; ++spins) {
-            if ((spins & 0xfffu) == 0 &&
-                std::chrono::steady_clock::now() - started > std::chrono::seconds(2)) {
-                PL_HIP(hipStreamSynchronize(h->stream));
-                if (*word != h->status_sequence) return PL_EHIP;
-                break;
-            }
-        }
-        std::atomic_thread_fence(std::memory_order_acquire);
+        const int rc = wait_for_report(h, &h->h_status->sequence);
+        if (rc != PL_OK) return rc;
         status = *h->h_status;
     }
     const int flags = status.flags;
@@ -878,7 +883,7 @@ static int create_lattice(int pd, int vd, int N, bool f64, pl_stream stream, con
                                                  2 * sizeof(plk::Counters) / sizeof(float), h->stream)))
         rc = PL_EHIP;
     if (rc == PL_OK &&
-        hip_failed(hipHostMalloc((void **)&h->h_status, sizeof(plk::HostStatus) + 2 * sizeof(unsigned),
+        hip_failed(hipHostMalloc((void **)&h->h_status, sizeof(plk::HostStatus) + 3 * sizeof(unsigned),
                                  hipHostMallocCoherent)))
         rc = PL_EHIP;
     if (rc != PL_OK) {
@@ -888,6 +893,7 @@ static int create_lattice(int pd, int vd, int N, bool f64, pl_stream stream, con
     h->h_status->num_vertices = 0;
     h->h_status->flags = 0;
     h->h_status->sequence = 0;
+    reinterpret_cast<unsigned *>(h->h_status + 1)[2] = 0;   // (the lists' report, behind the status)
     *out = h;
     return PL_OK;
 }
@@ -1101,7 +1107,8 @@ int enqueue_build_only(pl_lattice *h, const plk::PointFeatures &features, const 
         PL_HIP(plk::build_vertex_lists(h->pd, h->map, h->replay,
                                        h->replay_holds_cells ? h->cell_vertex : nullptr,
                                        h->max_vertices(), h->lists_of_vertices,
-                                       reinterpret_cast<unsigned *>(h->h_status + 1), h->stream));
+                                       reinterpret_cast<unsigned *>(h->h_status + 1),
+                                       h->status_sequence, h->stream));
         h->replay_holds_cells = false;
     }
     return PL_OK;
@@ -1147,8 +1154,9 @@ int build_end(pl_lattice *h) {
         // (how many chunks there are, and whether any list has several, sizes every apply's
         // launches: the last kernel of the lists wrote them behind the build's status, in pinned
         // memory; read once here, where the caller is building and expects to wait)
-        PL_HIP(hipStreamSynchronize(h->stream));
         const volatile unsigned *info = reinterpret_cast<const volatile unsigned *>(h->h_status + 1);
+        const int rc = wait_for_report(h, info + 2);
+        if (rc != PL_OK) return rc;
         const plk::ListChunks &c = h->lists_of_vertices.chunks;
         h->long_lists = info[0] < c.max_long ? info[0] : c.max_long;
         h->list_chunks = info[1] < c.max_chunks ? info[1] : c.max_chunks;

@@ -256,12 +256,15 @@ __global__ __launch_bounds__(kBlock) void k_list_fill(PointMap map,
                                                        const unsigned *__restrict__ start,
                                                        ListEntry *entries, int max_vertices,
                                                        size_t capacity, ListChunks chunks,
-                                                       unsigned *host_info) {
+                                                       unsigned *host_info, unsigned sequence) {
     // (the last launch of the pass: how many lists have several chunks, and the chunks in all, for
-    // the host, which sizes every apply's launches by them)
+    // the host, which sizes every apply's launches by them; then, behind a system-wide fence, the
+    // number of the build they belong to, which the host polls for)
     if (host_info && blockIdx.x == 0 && threadIdx.x == 0) {
         host_info[0] = chunks.info[0];
         host_info[1] = chunks.info[1];
+        __threadfence_system();
+        __hip_atomic_store(&host_info[2], sequence, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
     }
     unsigned vblock;
     if (!block_of_points(map, 1, vblock)) return;
@@ -519,7 +522,7 @@ size_t vertex_list_max_long(size_t rows) { return rows / kListChunkManyChannels 
 
 hipError_t build_vertex_lists(int pd, const PointMap &map, ReplayEntry *replay, const int *cell_vertex,
                               int max_vertices, const VertexLists &lists, unsigned *host_info,
-                              hipStream_t s) {
+                              unsigned sequence, hipStream_t s) {
     if (max_vertices <= 0 || map.n_blocks == 0) return hipSuccess;
     // (lists.count is all zeros: filled so when it was allocated, left so by every k_scan_starts)
     const dim3 block(kBlock), grid(map.n_blocks);
@@ -534,7 +537,7 @@ hipError_t build_vertex_lists(int pd, const PointMap &map, ReplayEntry *replay, 
                        lists.start, lists.chunks);
     PLK_DISPATCH_PD(pd, hipLaunchKernelGGL((k_list_fill<PD + 1>), grid, block, 0, s, map, replay,
                                            lists.places, lists.start, lists.entries, max_vertices,
-                                           lists.capacity, lists.chunks, host_info));
+                                           lists.capacity, lists.chunks, host_info, sequence));
     return hipGetLastError();
 }
 

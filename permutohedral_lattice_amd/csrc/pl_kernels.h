@@ -329,10 +329,11 @@ size_t vertex_list_max_chunks(int max_vertices, size_t rows);
 size_t vertex_list_max_long(size_t rows);
 // cell_vertex != nullptr: the replay rows still hold hash cells; they are translated and written
 // back.  When the stream has run this, lists.chunks.info holds the numbers splat_gather wants,
-// and so do the two words at host_info (memory the device can write, read by the host).
+// and so do the first two of the three words at host_info (pinned memory the host reads); the
+// third is `sequence`, written last by the pass's last launch as that launch starts.
 hipError_t build_vertex_lists(int pd, const PointMap &map, ReplayEntry *replay, const int *cell_vertex,
                               int max_vertices, const VertexLists &lists, unsigned *host_info,
-                              hipStream_t s);
+                              unsigned sequence, hipStream_t s);
 // Stage 3 from the lists: values[v] := sum over v's entries of weight * input row (every vertex's
 // row is written whole; no zero fill needed).  n_chunks, n_long: lists.chunks.info as the build of
 // the lists left it (a second launch adds up the lists of several chunks when there are any).
