@@ -897,16 +897,27 @@ __global__ __launch_bounds__(64) void k_number_vertices(CreatedLists lists, int 
     // not (the list's memory is there).  With a load behind each condition the pass waited for
     // five memory round trips in a row; now for two, the entries and then their rows of sums.
     static_assert(kBlocksPerChunk == 64, "one lane per workgroup of the chunk");
-    const bool has_chunk = (unsigned)lane < chunk;
-    int before = lists.chunk_count[has_chunk ? lane : 0];
+    // (the sums of up to 512 chunks -- a volume of eight million voxels has that many -- in eight
+    // loads per lane that are all in flight together)
+    constexpr int kChunkLoads = 8;
+    int part[kChunkLoads];
+#pragma unroll
+    for (int u = 0; u < kChunkLoads; ++u) {
+        const unsigned i = (unsigned)lane + 64u * (unsigned)u;
+        part[u] = lists.chunk_count[i < chunk ? i : 0];
+    }
     const unsigned sibling = chunk * kBlocksPerChunk + lane;
     int sibling_count = lists.block_count[sibling < b ? sibling : b];
     const int count = lists.block_count[b];
     uint4 first_entry = lists.entries[list + (WIDE ? 2 * lane + 1 : lane)];
-    asm volatile("" : "+v"(before), "+v"(sibling_count), "+v"(first_entry.x), "+v"(first_entry.y),
-                 "+v"(first_entry.z));
-    before = has_chunk ? before : 0;
-    for (unsigned i = lane + 64; i < chunk; i += 64) before += lists.chunk_count[i];
+    asm volatile("" : "+v"(sibling_count), "+v"(first_entry.x), "+v"(first_entry.y), "+v"(first_entry.z));
+#pragma unroll
+    for (int u = 0; u < kChunkLoads; ++u) asm volatile("" : "+v"(part[u]));
+    int before = 0;
+#pragma unroll
+    for (int u = 0; u < kChunkLoads; ++u)
+        before += (unsigned)lane + 64u * (unsigned)u < chunk ? part[u] : 0;
+    for (unsigned i = lane + 64 * kChunkLoads; i < chunk; i += 64) before += lists.chunk_count[i];
     before += sibling < b ? sibling_count : 0;
 #pragma unroll
     for (int off = 32; off >= 1; off >>= 1) before += __shfl_xor(before, off);
