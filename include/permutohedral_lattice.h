@@ -131,9 +131,9 @@ int pl_destroy(pl_handle h);
  * Stands in for filter(output, input, positions, reverse)
  * (src/PermutohedralLatticeCPU.h:442-446, src/PermutohedralLatticeGPU.cuh:453-479).
  * Equivalent to pl_build followed by pl_apply.  Everything is enqueued at once; the call returns
- * when the build has reported whether its hash table was large enough (one wait for an event
- * behind the build's kernels; if it was not, the call is repeated with a larger table), while
- * the blur and the slice may still be running.  The output is complete in the order of the
+ * when the build has reported whether its hash table was large enough (the calling thread
+ * polls a word in pinned memory that the kernel behind the build writes; if the table was too
+ * small, the call is repeated with a larger one), while the rest of the call may still be running.  The output is complete in the order of the
  * lattice's stream, as with the reference's GPU path.
  */
 int pl_filter(pl_handle h, float *output, const float *input, const float *positions, int reverse);
